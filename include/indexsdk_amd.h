@@ -1,0 +1,151 @@
+/*
+ * C ABI of the MI355X-native IVFPQ / Flat search path.
+ *
+ * This is the drop-in boundary for the search hot path of Ascend IndexSDK's Faiss-style
+ * AscendIndexIVFPQ / AscendIndexFlat / AscendIndexInt8Flat classes: plain pointers and sizes,
+ * no C++ or framework types.  Each entry point names the reference interface it stands in for
+ * (paths relative to the reference root; FR/ = feature_retrieval/src/ascendfaiss/).
+ *
+ * Conventions
+ *   - every function returns an int status: 0 = ok, otherwise a code with the numeric values of
+ *     the reference's APP_ERROR enum (FR/common/ErrorCode.h:26-73); ixa_last_error() returns the
+ *     message of the last failure on the calling thread.  The reference's public layer turns such
+ *     codes into faiss::FaissException; the C++ wrappers in include/ascend do the same.
+ *   - host pointers are caller-owned, row-major, no alignment requirement; outputs are
+ *     pre-allocated by the caller (n * k elements), as in faiss::Index::search.
+ *   - the *_device variants take DEVICE pointers (16-byte aligned, row-major) and leave their
+ *     results in device memory; they synchronise the index's stream before returning.
+ *   - metric: 0 = inner product, 1 = L2 (faiss::MetricType values).
+ *   - missing results: label -1, distance FLT_MAX for L2 and -FLT_MAX for inner product
+ *     (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2202-2219; FR/ascend/impl/AscendIndexImpl.cpp:587-650).
+ *   - one index object may be used by one thread at a time (the reference's default mode,
+ *     FR/ascend/impl/AscendIndexImpl.h:215-237 without MX_INDEX_MULTITHREAD).
+ *   - there is no CPU fallback: every entry point fails with IXA_ERR_INDEX_NOT_INIT when no
+ *     HIP device is present.
+ */
+#ifndef INDEXSDK_AMD_H
+#define INDEXSDK_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define IXA_OK 0
+#define IXA_ERR_BAD_ALLOC 1001        /* APP_ERR_ACL_BAD_ALLOC */
+#define IXA_ERR_OP_EXEC_FAILED 1017   /* APP_ERR_ACL_OP_EXEC_FAILED */
+#define IXA_ERR_INVALID_PARAM 2001    /* APP_ERR_INVALID_PARAM */
+#define IXA_ERR_NOT_IMPLEMENT 2008    /* APP_ERR_NOT_IMPLEMENT */
+#define IXA_ERR_ILLEGAL_OPERATION 2009
+#define IXA_ERR_INNER_ERROR 2010      /* APP_ERR_INNER_ERROR */
+#define IXA_ERR_INDEX_NOT_INIT 2016   /* APP_ERR_INDEX_NOT_INIT */
+
+#define IXA_METRIC_INNER_PRODUCT 0
+#define IXA_METRIC_L2 1
+
+/* Message of the last failed call on this thread ("" if none). */
+const char *ixa_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * IVFPQ
+ * ------------------------------------------------------------------------------------------- */
+
+typedef struct ivfpq_index ivfpq_index_t;
+
+/* Mirrors AscendIndexIVFPQConfig / AscendIndexIVFConfig (FR/ascend/AscendIndexIVFPQ.h:32-68,
+ * FR/ascend/AscendIndexIVF.h:37-72); fields that only make sense on Ascend hardware (deviceList,
+ * useDistributedCoarse, enableQueryParallelSearch) have no counterpart on one GPU. */
+typedef struct ivfpq_config {
+    int32_t niter;                  /* cp.niter of the coarse k-means; reference CPU mode uses 25 */
+    int32_t pq_niter;               /* pqNiter; -1 = niter */
+    int32_t spherical;              /* cp.spherical; 0 = plain Lloyd (default here), 1 = reference default */
+    int32_t train_samples_per_list; /* trainSamplesPerList */
+    int64_t max_train_samples;      /* maxTrainSamples */
+    int32_t lut_fp16;               /* 1 = store the per-query LUT as IEEE half (accumulate in fp32) */
+    int32_t code_layout;            /* -1 = choose, 0 = row-major codes, 1 = bank-rotated (M in {32,64,96}) */
+    int64_t scratch_bytes;          /* resourceSize: bound of the coarse-score scratch in HBM */
+    uint64_t seed;                  /* sampling / initialisation seed */
+    int32_t strict_reference_params;/* 1 = enforce the reference whitelists d in {128}, nlist in
+                                       {1024..16384, 262144, 524288}, M in {2,4,8,16,32} */
+    int32_t reserved;
+} ivfpq_config_t;
+
+/* Fills *cfg with the defaults. */
+void ivfpq_config_default(ivfpq_config_t *cfg);
+
+/* AscendIndexIVFPQ(dims, metric, nlist, msubs, nbits, config)  FR/ascend/AscendIndexIVFPQ.h:74-75;
+ * parameter checks and messages of checkParams, FR/ascend/impl/AscendIndexIVFPQImpl.cpp:510-525.
+ * cfg may be NULL. */
+int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,
+                 ivfpq_index_t **out);
+/* ~AscendIndexIVFPQ */
+int ivfpq_destroy(ivfpq_index_t *h);
+
+/* AscendIndexIVFPQ::train(n, x)  FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1144-1252 */
+int ivfpq_train(ivfpq_index_t *h, int64_t n, const float *x);
+int ivfpq_train_device(ivfpq_index_t *h, int64_t n, const float *x_dev);
+
+/* Stands in for copyFrom(const faiss::IndexIVFPQ*) (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:392-425):
+ * injects trained quantizers.  centroids[nlist*d], codebook[msubs*256*dsub] laid out like
+ * faiss pq.centroids.  Codes added later are computed on the RAW vector (by_residual = false). */
+int ivfpq_set_trained(ivfpq_index_t *h, const float *centroids, const float *codebook);
+/* Stands in for copyTo(faiss::IndexIVFPQ*) (:453-508), quantizer part; either output may be NULL. */
+int ivfpq_get_trained(const ivfpq_index_t *h, float *centroids, float *codebook);
+int ivfpq_is_trained(const ivfpq_index_t *h, int *out);
+
+/* AscendIndex::add / add_with_ids  FR/ascend/AscendIndex.h:66-71, AscendIndexIVFPQImpl.cpp:694-864.
+ * ids == NULL numbers the vectors ntotal, ntotal+1, ... */
+int ivfpq_add_with_ids(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids);
+int ivfpq_add_with_ids_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int64_t *ids_dev);
+/* ascend::IndexIVFPQ::addPQCodes(listId, n, codes, ids)  FR/ascenddaemon/impl/IndexIVFPQ.cpp:210-235;
+ * codes row-major [n][msubs]. */
+int ivfpq_add_codes(ivfpq_index_t *h, int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids);
+
+/* AscendIndexIVF::setNumProbes / getNumProbes  FR/ascend/AscendIndexIVF.h:96-99 */
+int ivfpq_set_nprobe(ivfpq_index_t *h, int nprobe);
+int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out);
+
+/* AscendIndex::search(n, x, k, distances, labels)  FR/ascend/AscendIndex.h:79-80 ->
+ * ascend::IndexIVFPQ::searchImpl  FR/ascenddaemon/impl/IndexIVFPQ.cpp:2373-2411 */
+int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
+int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
+                        int64_t *labels_dev);
+
+/* Coarse assignment used by add (nearest centroid under L2), FR/ascend/impl/AscendIndexIVFPQImpl.cpp:603-672;
+ * out[n]. */
+int ivfpq_assign(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out_list_ids);
+/* L1 level of search: the nprobe best lists per query, best first
+ * (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2104-2164); out_ids[n*nprobe], out_dist may be NULL. */
+int ivfpq_coarse_probe(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out_ids, float *out_dist);
+/* Host PQ encoder of the reference (AscendIndexIVFPQImpl.cpp:879-921) on the device; codes[n][msubs]. */
+int ivfpq_encode(ivfpq_index_t *h, int64_t n, const float *x, uint8_t *codes);
+
+/* AscendIndexIVF::getListLength / getListCodesAndIds  FR/ascend/AscendIndexIVF.h:108-111;
+ * codes[len*msubs] row-major, ids[len]; either may be NULL. */
+int ivfpq_list_length(const ivfpq_index_t *h, int64_t list, int64_t *out);
+int ivfpq_get_list(const ivfpq_index_t *h, int64_t list, uint8_t *codes, int64_t *ids);
+
+/* AscendIndexIVFPQ::remove_ids(n, ids)  FR/ascend/AscendIndexIVFPQ.h:90; *removed may be NULL. */
+int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *removed);
+/* AscendIndexIVF::reset()  FR/ascend/AscendIndexIVF.h:93: drops the lists, keeps the quantizers. */
+int ivfpq_reset(ivfpq_index_t *h);
+int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out);
+
+/* Device timings of the last ivfpq_search* call, measured with HIP events on the index's stream.
+ * No counterpart in the reference (it prints std::chrono timers when verbose). */
+typedef struct ivfpq_search_stats {
+    double scanned_codes; /* sum of the lengths of all probed lists */
+    double ms_coarse;     /* stage 1: scores + selection + refine */
+    double ms_scan;       /* fused LUT + ADC scan + top-k (+ merge kernel when nsplit > 1) */
+    double ms_total;
+    double scan_launches; /* kernel launches covered by ms_scan */
+    double nsplit;        /* workgroups per query in the scan */
+} ivfpq_search_stats_t;
+int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INDEXSDK_AMD_H */

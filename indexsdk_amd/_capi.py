@@ -1,0 +1,112 @@
+"""ctypes binding of ``libindexsdk_amd.so`` (the C ABI declared in ``include/indexsdk_amd.h``).
+
+The library is built in-tree by ``indexsdk_amd/csrc/build.sh``; importing this module never
+compiles anything and never falls back to a CPU implementation: if the shared object is missing,
+``load()`` raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libindexsdk_amd.so")
+
+c_f32p = ctypes.POINTER(ctypes.c_float)
+c_i64p = ctypes.POINTER(ctypes.c_int64)
+c_i32p = ctypes.POINTER(ctypes.c_int32)
+c_u8p = ctypes.POINTER(ctypes.c_uint8)
+c_i8p = ctypes.POINTER(ctypes.c_int8)
+
+
+class IvfpqConfig(ctypes.Structure):
+    _fields_ = [
+        ("niter", ctypes.c_int32),
+        ("pq_niter", ctypes.c_int32),
+        ("spherical", ctypes.c_int32),
+        ("train_samples_per_list", ctypes.c_int32),
+        ("max_train_samples", ctypes.c_int64),
+        ("lut_fp16", ctypes.c_int32),
+        ("code_layout", ctypes.c_int32),
+        ("scratch_bytes", ctypes.c_int64),
+        ("seed", ctypes.c_uint64),
+        ("strict_reference_params", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+class IvfpqSearchStats(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_double) for n in
+                ("scanned_codes", "ms_coarse", "ms_scan", "ms_total", "scan_launches", "nsplit")]
+
+
+class FlatSearchStats(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_double) for n in ("ms_score", "ms_select", "ms_total", "score_launches")]
+
+
+# every exported symbol of include/indexsdk_amd.h: name -> (restype, argtypes)
+_H = ctypes.c_void_p
+_SIGNATURES = {
+    "ixa_last_error": (ctypes.c_char_p, []),
+    "ivfpq_config_default": (None, [ctypes.POINTER(IvfpqConfig)]),
+    "ivfpq_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                    ctypes.POINTER(IvfpqConfig), ctypes.POINTER(_H)]),
+    "ivfpq_destroy": (ctypes.c_int, [_H]),
+    "ivfpq_train": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p]),
+    "ivfpq_train_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p]),
+    "ivfpq_set_trained": (ctypes.c_int, [_H, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_get_trained": (ctypes.c_int, [_H, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_is_trained": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int)]),
+    "ivfpq_add_with_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_add_with_ids_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_add_codes": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_set_nprobe": (ctypes.c_int, [_H, ctypes.c_int]),
+    "ivfpq_get_nprobe": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int)]),
+    "ivfpq_search": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                    ctypes.c_void_p]),
+    "ivfpq_search_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                           ctypes.c_void_p]),
+    "ivfpq_assign": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_coarse_probe": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_encode": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_list_length": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
+    "ivfpq_get_list": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_remove_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
+    "ivfpq_reset": (ctypes.c_int, [_H]),
+    "ivfpq_ntotal": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int64)]),
+    "ivfpq_last_search_stats": (ctypes.c_int, [_H, ctypes.POINTER(IvfpqSearchStats)]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library; raises OSError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError(f"{LIB_PATH} is missing: build it with indexsdk_amd/csrc/build.sh "
+                          "(there is no CPU fallback)")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def exported_names():
+    return list(_SIGNATURES)
+
+
+class IndexSdkError(RuntimeError):
+    """Raised for a non-zero status of the C ABI (the reference throws faiss::FaissException)."""
+
+    def __init__(self, code, message):
+        super().__init__(f"[{code}] {message}")
+        self.code = code
+        self.message = message
+
+
+def check(status):
+    if status != 0:
+        raise IndexSdkError(status, load().ixa_last_error().decode("utf-8", "replace"))

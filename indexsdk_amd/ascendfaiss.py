@@ -1,0 +1,175 @@
+"""Python face of the MI355X IVFPQ / Flat search path with the array contracts of the reference's
+SWIG module ``ascendfaiss`` (examples/faiss-python/ascendfaiss.py:63-104): ``index.train(xb)``,
+``index.add(xb)``, ``D, I = index.search(xq, k)`` on C-contiguous float32 ``[n, d]`` arrays,
+returning ``D`` float32 ``[n, k]`` and ``I`` int64 ``[n, k]``.  Everything runs through the C ABI.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _capi
+from ._capi import IndexSdkError  # noqa: F401  (re-export)
+
+METRIC_INNER_PRODUCT = 0
+METRIC_L2 = 1
+
+
+def _as(a, dtype, ndim, name):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    if a.ndim != ndim:
+        raise ValueError(f"{name} must have {ndim} dimensions, got shape {a.shape}")
+    return a
+
+
+def _ptr(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+class AscendIndexIVFPQConfig:
+    """AscendIndexIVFPQConfig (FR/ascend/AscendIndexIVFPQ.h:32-68) plus the knobs of this build."""
+
+    def __init__(self, **kw):
+        self._c = _capi.IvfpqConfig()
+        _capi.load().ivfpq_config_default(ctypes.byref(self._c))
+        aliases = {"trainSamplesPerList": "train_samples_per_list", "maxTrainSamples": "max_train_samples",
+                   "pqNiter": "pq_niter", "resourceSize": "scratch_bytes"}
+        for key, val in kw.items():
+            key = aliases.get(key, key)
+            if key not in dict(self._c._fields_):
+                raise TypeError(f"unknown config field {key}")
+            setattr(self._c, key, val)
+
+    def __getattr__(self, name):
+        return getattr(self.__dict__["_c"], name)
+
+
+class AscendIndexIVFPQ:
+    """AscendIndexIVFPQ(dims, metric, nlist, msubs, nbits, config) -- FR/ascend/AscendIndexIVFPQ.h:71-96."""
+
+    def __init__(self, dims, metric, nlist, msubs, nbits=8, config=None):
+        self._lib = _capi.load()
+        self._h = ctypes.c_void_p()
+        self.d, self.metric_type, self.nlist, self.msubs, self.nbits = dims, metric, nlist, msubs, nbits
+        cfg = ctypes.byref(config._c) if config is not None else None
+        _capi.check(self._lib.ivfpq_create(dims, metric, nlist, msubs, nbits, cfg, ctypes.byref(self._h)))
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            self._lib.ivfpq_destroy(h)
+            self._h = None
+
+    # ---- training -----------------------------------------------------------------------------
+    @property
+    def is_trained(self):
+        out = ctypes.c_int()
+        _capi.check(self._lib.ivfpq_is_trained(self._h, ctypes.byref(out)))
+        return bool(out.value)
+
+    @property
+    def ntotal(self):
+        out = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_ntotal(self._h, ctypes.byref(out)))
+        return out.value
+
+    def train(self, x):
+        x = _as(x, np.float32, 2, "x")
+        assert x.shape[1] == self.d
+        _capi.check(self._lib.ivfpq_train(self._h, x.shape[0], _ptr(x)))
+
+    def set_trained(self, centroids, codebook):
+        """Injects quantizers (the role of copyFrom); codebook is [msubs, 256, dsub]."""
+        c = _as(centroids, np.float32, 2, "centroids")
+        cb = np.ascontiguousarray(codebook, dtype=np.float32)
+        assert c.shape == (self.nlist, self.d) and cb.size == self.msubs * 256 * (self.d // self.msubs)
+        _capi.check(self._lib.ivfpq_set_trained(self._h, _ptr(c), _ptr(cb)))
+
+    def get_trained(self):
+        c = np.empty((self.nlist, self.d), dtype=np.float32)
+        cb = np.empty((self.msubs, 256, self.d // self.msubs), dtype=np.float32)
+        _capi.check(self._lib.ivfpq_get_trained(self._h, _ptr(c), _ptr(cb)))
+        return c, cb
+
+    # ---- add ----------------------------------------------------------------------------------
+    def add(self, x):
+        self.add_with_ids(x, None)
+
+    def add_with_ids(self, x, ids):
+        x = _as(x, np.float32, 2, "x")
+        assert x.shape[1] == self.d
+        idp = None
+        if ids is not None:
+            ids = _as(ids, np.int64, 1, "ids")
+            assert ids.shape[0] == x.shape[0]
+            idp = _ptr(ids)
+        _capi.check(self._lib.ivfpq_add_with_ids(self._h, x.shape[0], _ptr(x), idp))
+
+    def add_codes(self, list_id, codes, ids):
+        codes = _as(codes, np.uint8, 2, "codes")
+        ids = _as(ids, np.int64, 1, "ids")
+        assert codes.shape == (ids.shape[0], self.msubs)
+        _capi.check(self._lib.ivfpq_add_codes(self._h, list_id, ids.shape[0], _ptr(codes), _ptr(ids)))
+
+    # ---- search -------------------------------------------------------------------------------
+    def setNumProbes(self, nprobe):
+        _capi.check(self._lib.ivfpq_set_nprobe(self._h, nprobe))
+
+    def getNumProbes(self):
+        out = ctypes.c_int()
+        _capi.check(self._lib.ivfpq_get_nprobe(self._h, ctypes.byref(out)))
+        return out.value
+
+    def search(self, x, k):
+        x = _as(x, np.float32, 2, "x")
+        assert x.shape[1] == self.d
+        D = np.empty((x.shape[0], k), dtype=np.float32)
+        I = np.empty((x.shape[0], k), dtype=np.int64)
+        _capi.check(self._lib.ivfpq_search(self._h, x.shape[0], _ptr(x), k, _ptr(D), _ptr(I)))
+        return D, I
+
+    def assign(self, x):
+        x = _as(x, np.float32, 2, "x")
+        out = np.empty(x.shape[0], dtype=np.int64)
+        _capi.check(self._lib.ivfpq_assign(self._h, x.shape[0], _ptr(x), _ptr(out)))
+        return out
+
+    def coarse_probe(self, x):
+        x = _as(x, np.float32, 2, "x")
+        nprobe = self.getNumProbes()
+        ids = np.empty((x.shape[0], nprobe), dtype=np.int64)
+        dist = np.empty((x.shape[0], nprobe), dtype=np.float32)
+        _capi.check(self._lib.ivfpq_coarse_probe(self._h, x.shape[0], _ptr(x), _ptr(ids), _ptr(dist)))
+        return ids, dist
+
+    def encode(self, x):
+        x = _as(x, np.float32, 2, "x")
+        codes = np.empty((x.shape[0], self.msubs), dtype=np.uint8)
+        _capi.check(self._lib.ivfpq_encode(self._h, x.shape[0], _ptr(x), _ptr(codes)))
+        return codes
+
+    # ---- lists --------------------------------------------------------------------------------
+    def getListLength(self, list_id):
+        out = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_list_length(self._h, list_id, ctypes.byref(out)))
+        return out.value
+
+    def getListCodesAndIds(self, list_id):
+        n = self.getListLength(list_id)
+        codes = np.empty((n, self.msubs), dtype=np.uint8)
+        ids = np.empty(n, dtype=np.int64)
+        _capi.check(self._lib.ivfpq_get_list(self._h, list_id, _ptr(codes), _ptr(ids)))
+        return codes, ids
+
+    def remove_ids(self, ids):
+        ids = _as(ids, np.int64, 1, "ids")
+        out = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_remove_ids(self._h, ids.shape[0], _ptr(ids), ctypes.byref(out)))
+        return out.value
+
+    def reset(self):
+        _capi.check(self._lib.ivfpq_reset(self._h))
+
+    def last_search_stats(self):
+        s = _capi.IvfpqSearchStats()
+        _capi.check(self._lib.ivfpq_last_search_stats(self._h, ctypes.byref(s)))
+        return {n: getattr(s, n) for n, _ in s._fields_}

@@ -1,0 +1,203 @@
+// extern "C" surface of the library (declared in include/indexsdk_amd.h).  Every entry point
+// catches C++ exceptions, stores the message for ixa_last_error() and returns the status code.
+#include "../../include/indexsdk_amd.h"
+
+#include <cstring>
+#include <new>
+#include <string>
+
+#include "ivfpq_index.h"
+
+struct ivfpq_index {
+    ixa::IvfpqIndex impl;
+    ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
+        : impl(d, metric, nlist, M, nbits, c)
+    {
+    }
+};
+
+namespace {
+
+thread_local std::string g_last_error;
+
+template <typename F>
+int guarded(F &&f)
+{
+    try {
+        f();
+        return IXA_OK;
+    } catch (const ixa::Error &e) {
+        g_last_error = e.what();
+        return e.code;
+    } catch (const std::bad_alloc &) {
+        g_last_error = "host allocation failed";
+        return IXA_ERR_BAD_ALLOC;
+    } catch (const std::exception &e) {
+        g_last_error = e.what();
+        return IXA_ERR_INNER_ERROR;
+    }
+}
+
+#define IXA_HANDLE(h) IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.")
+
+}  // namespace
+
+extern "C" {
+
+#define IXA_EXPORT __attribute__((visibility("default")))
+
+IXA_EXPORT const char *ixa_last_error(void) { return g_last_error.c_str(); }
+
+IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
+{
+    if (!cfg) {
+        return;
+    }
+    const ixa::IvfpqConfig d;
+    std::memset(cfg, 0, sizeof(*cfg));
+    cfg->niter = d.niter;
+    cfg->pq_niter = d.pq_niter;
+    cfg->spherical = d.spherical;
+    cfg->train_samples_per_list = d.train_samples_per_list;
+    cfg->max_train_samples = d.max_train_samples;
+    cfg->lut_fp16 = d.lut_fp16;
+    cfg->code_layout = d.code_layout;
+    cfg->scratch_bytes = d.scratch_bytes;
+    cfg->seed = d.seed;
+    cfg->strict_reference_params = d.strict_reference_params;
+}
+
+IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,
+                            ivfpq_index_t **out)
+{
+    return guarded([&] {
+        IXA_REQUIRE(out != nullptr, ixa::kErrInvalidParam, "out can not be nullptr.");
+        *out = nullptr;
+        ixa::IvfpqConfig c;
+        if (cfg) {
+            IXA_REQUIRE(cfg->niter >= 0 && cfg->train_samples_per_list >= 1 && cfg->max_train_samples >= 1 &&
+                            cfg->scratch_bytes >= (1 << 20) && cfg->code_layout >= -1 && cfg->code_layout <= 1,
+                        ixa::kErrInvalidParam, "invalid ivfpq_config_t field");
+            c.niter = cfg->niter;
+            c.pq_niter = cfg->pq_niter;
+            c.spherical = cfg->spherical;
+            c.train_samples_per_list = cfg->train_samples_per_list;
+            c.max_train_samples = cfg->max_train_samples;
+            c.lut_fp16 = cfg->lut_fp16;
+            c.code_layout = cfg->code_layout;
+            c.scratch_bytes = cfg->scratch_bytes;
+            c.seed = cfg->seed;
+            c.strict_reference_params = cfg->strict_reference_params;
+        }
+        *out = new ivfpq_index(d, metric, nlist, msubs, nbits, c);
+    });
+}
+
+IXA_EXPORT int ivfpq_destroy(ivfpq_index_t *h)
+{
+    return guarded([&] { delete h; });
+}
+
+IXA_EXPORT int ivfpq_train(ivfpq_index_t *h, int64_t n, const float *x)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.train(n, x, false); });
+}
+IXA_EXPORT int ivfpq_train_device(ivfpq_index_t *h, int64_t n, const float *x)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.train(n, x, true); });
+}
+IXA_EXPORT int ivfpq_set_trained(ivfpq_index_t *h, const float *centroids, const float *codebook)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.set_trained(centroids, codebook); });
+}
+IXA_EXPORT int ivfpq_get_trained(const ivfpq_index_t *h, float *centroids, float *codebook)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.get_trained(centroids, codebook); });
+}
+IXA_EXPORT int ivfpq_is_trained(const ivfpq_index_t *h, int *out)
+{
+    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.is_trained(); });
+}
+IXA_EXPORT int ivfpq_add_with_ids(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.add(n, x, ids, false); });
+}
+IXA_EXPORT int ivfpq_add_with_ids_device(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.add(n, x, ids, true); });
+}
+IXA_EXPORT int ivfpq_add_codes(ivfpq_index_t *h, int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.add_codes(list, n, codes, ids); });
+}
+IXA_EXPORT int ivfpq_set_nprobe(ivfpq_index_t *h, int nprobe)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.set_nprobe(nprobe); });
+}
+IXA_EXPORT int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out)
+{
+    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.nprobe(); });
+}
+IXA_EXPORT int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+}
+IXA_EXPORT int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances,
+                                   int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
+}
+IXA_EXPORT int ivfpq_assign(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.assign(n, x, out, false); });
+}
+IXA_EXPORT int ivfpq_coarse_probe(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out_ids, float *out_dist)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.coarse_probe(n, x, out_ids, out_dist, false); });
+}
+IXA_EXPORT int ivfpq_encode(ivfpq_index_t *h, int64_t n, const float *x, uint8_t *codes)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.encode(n, x, codes, false); });
+}
+IXA_EXPORT int ivfpq_list_length(const ivfpq_index_t *h, int64_t list, int64_t *out)
+{
+    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.list_length(list); });
+}
+IXA_EXPORT int ivfpq_get_list(const ivfpq_index_t *h, int64_t list, uint8_t *codes, int64_t *ids)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.get_list(list, codes, ids); });
+}
+IXA_EXPORT int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *removed)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        const int64_t r = h->impl.remove_ids(n, ids);
+        if (removed) {
+            *removed = r;
+        }
+    });
+}
+IXA_EXPORT int ivfpq_reset(ivfpq_index_t *h)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.reset(); });
+}
+IXA_EXPORT int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out)
+{
+    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.ntotal(); });
+}
+IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");
+        const ixa::SearchStats &s = h->impl.stats();
+        out->scanned_codes = s.scanned_codes;
+        out->ms_coarse = s.ms_coarse;
+        out->ms_scan = s.ms_scan;
+        out->ms_total = s.ms_total;
+        out->scan_launches = s.scan_launches;
+        out->nsplit = s.nsplit;
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,399 @@
+// Stage 1 of IVFPQ search and the brute-force Flat fp32 path: query x centroid scores on the
+// fp32 matrix cores, per-row selection of the best candidates, and an exact re-evaluation of the
+// selected candidates in the canonical scalar arithmetic.
+//
+// Replaces, for one GPU, the reference's L1 level (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2104-2164):
+//   op DistanceFlatL2MinsAtFP32 (FR/ops/ascendc/op_kernel/distance_flat_l2_mins_at_fp32.cpp:191-210)
+//   op TopkFlatFp32             (FR/ops/cpukernel/impl/topk_flat_fp32_cpu_kernel.cpp:223-384)
+//
+// "score" everywhere is the value to minimise: the expanded-form L2 distance
+// (|q|^2 + |c|^2) - 2 q.c, or the negated inner product.
+#include "coarse.h"
+
+#include "topk.h"
+
+namespace ixa {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// ------------------------------------------------------------------------------------------------
+// |x_i|^2 accumulated left to right in fp32 (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1114-1126).
+// One lane per row: the order of additions is part of the contract, so a row is never split.
+__global__ __launch_bounds__(256) void sqnorm_rows_kernel(const float *__restrict__ x, int64_t n, int d,
+                                                          float *__restrict__ out)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const float *row = x + i * d;
+    float s = 0.0f;
+    for (int j = 0; j < d; j++) {
+        float v = row[j];
+        s = __fadd_rn(s, __fmul_rn(v, v));
+    }
+    out[i] = s;
+}
+
+void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_t s)
+{
+    if (n == 0) {
+        return;
+    }
+    hipLaunchKernelGGL(sqnorm_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, d, out);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Score tile kernel.  One workgroup (4 wavefronts) produces a 128 x 128 tile; each wavefront owns
+// a 64 x 64 quadrant as 2 x 2 blocks of v_mfma_f32_32x32x2_f32 (16 accumulator VGPRs per block).
+// Operand tiles are staged through LDS in K-steps of 16 with a padded row stride of 20 floats,
+// which makes the 128-bit operand reads of 16 consecutive rows hit disjoint banks.  The sum over
+// k is order-free, so each lane half (lane/32) owns 8 of the 16 k's of a step and feeds them to 8
+// consecutive MFMAs.
+constexpr int kTile = 128;
+constexpr int kKStep = 16;
+constexpr int kLdsStride = 20;
+
+template <bool VEC4>
+__device__ __forceinline__ float4 load_k4(const float *row, int k, int d)
+{
+    if (VEC4) {
+        if (k < d) {
+            return *reinterpret_cast<const float4 *>(row + k);
+        }
+        return make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float4 v;
+    v.x = k + 0 < d ? row[k + 0] : 0.f;
+    v.y = k + 1 < d ? row[k + 1] : 0.f;
+    v.z = k + 2 < d ? row[k + 2] : 0.f;
+    v.w = k + 3 < d ? row[k + 3] : 0.f;
+    return v;
+}
+
+template <bool VEC4>
+__global__ __launch_bounds__(256) void score_tile_kernel(const float *__restrict__ Q, int64_t nq,
+                                                         const float *__restrict__ C, int64_t nc, int d,
+                                                         const float *__restrict__ qn, const float *__restrict__ cn,
+                                                         int metric, float *__restrict__ out, int64_t ldo,
+                                                         int tiles_n)
+{
+    __shared__ float As[2][kTile * kLdsStride];
+    __shared__ float Bs[2][kTile * kLdsStride];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const int64_t i0 = tile_m * kTile, j0 = tile_n * kTile;
+
+    // global -> register mapping: a tile step is 128 rows x 4 float4; thread t moves float4 t, t+256
+    const int lrow0 = tid >> 2, lrow1 = (tid + 256) >> 2, lkq = (tid & 3) * 4;
+    const int64_t qa0 = i0 + lrow0 < nq ? i0 + lrow0 : nq - 1, qa1 = i0 + lrow1 < nq ? i0 + lrow1 : nq - 1;
+    const int64_t cb0 = j0 + lrow0 < nc ? j0 + lrow0 : nc - 1, cb1 = j0 + lrow1 < nc ? j0 + lrow1 : nc - 1;
+    const float *qrow0 = Q + qa0 * d, *qrow1 = Q + qa1 * d;
+    const float *crow0 = C + cb0 * d, *crow1 = C + cb1 * d;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[a][b][r] = 0.f;
+            }
+        }
+    }
+
+    const int nk = (d + kKStep - 1) / kKStep;
+    float4 ra0 = load_k4<VEC4>(qrow0, lkq, d), ra1 = load_k4<VEC4>(qrow1, lkq, d);
+    float4 rb0 = load_k4<VEC4>(crow0, lkq, d), rb1 = load_k4<VEC4>(crow1, lkq, d);
+    *reinterpret_cast<float4 *>(&As[0][lrow0 * kLdsStride + lkq]) = ra0;
+    *reinterpret_cast<float4 *>(&As[0][lrow1 * kLdsStride + lkq]) = ra1;
+    *reinterpret_cast<float4 *>(&Bs[0][lrow0 * kLdsStride + lkq]) = rb0;
+    *reinterpret_cast<float4 *>(&Bs[0][lrow1 * kLdsStride + lkq]) = rb1;
+    __syncthreads();
+
+    for (int ks = 0; ks < nk; ks++) {
+        const int buf = ks & 1;
+        if (ks + 1 < nk) {
+            const int k = (ks + 1) * kKStep + lkq;
+            ra0 = load_k4<VEC4>(qrow0, k, d);
+            ra1 = load_k4<VEC4>(qrow1, k, d);
+            rb0 = load_k4<VEC4>(crow0, k, d);
+            rb1 = load_k4<VEC4>(crow1, k, d);
+        }
+        float a[2][8], b[2][8];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+            const float *pa = &As[buf][(wr * 64 + blk * 32 + l32) * kLdsStride + half * 8];
+            const float *pb = &Bs[buf][(wc * 64 + blk * 32 + l32) * kLdsStride + half * 8];
+            float4 a0 = *reinterpret_cast<const float4 *>(pa), a1 = *reinterpret_cast<const float4 *>(pa + 4);
+            float4 b0 = *reinterpret_cast<const float4 *>(pb), b1 = *reinterpret_cast<const float4 *>(pb + 4);
+            a[blk][0] = a0.x; a[blk][1] = a0.y; a[blk][2] = a0.z; a[blk][3] = a0.w;
+            a[blk][4] = a1.x; a[blk][5] = a1.y; a[blk][6] = a1.z; a[blk][7] = a1.w;
+            b[blk][0] = b0.x; b[blk][1] = b0.y; b[blk][2] = b0.z; b[blk][3] = b0.w;
+            b[blk][4] = b1.x; b[blk][5] = b1.y; b[blk][6] = b1.z; b[blk][7] = b1.w;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+#pragma unroll
+            for (int ra = 0; ra < 2; ra++) {
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    acc[ra][rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ra][t], b[rb][t], acc[ra][rb], 0, 0, 0);
+                }
+            }
+        }
+        if (ks + 1 < nk) {
+            const int nb = buf ^ 1;
+            *reinterpret_cast<float4 *>(&As[nb][lrow0 * kLdsStride + lkq]) = ra0;
+            *reinterpret_cast<float4 *>(&As[nb][lrow1 * kLdsStride + lkq]) = ra1;
+            *reinterpret_cast<float4 *>(&Bs[nb][lrow0 * kLdsStride + lkq]) = rb0;
+            *reinterpret_cast<float4 *>(&Bs[nb][lrow1 * kLdsStride + lkq]) = rb1;
+        }
+        __syncthreads();
+    }
+
+    // epilogue: accumulator register r of lane (half, l32) in block (ra, rb) is
+    //   row = 8 * (r / 4) + 4 * half + (r % 4),  col = l32   of that 32 x 32 block.
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+        const int64_t col = j0 + wc * 64 + rb * 32 + l32;
+        const float cnv = (metric == kMetricL2 && col < nc) ? cn[col] : 0.f;
+#pragma unroll
+        for (int ra = 0; ra < 2; ra++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t row = i0 + wr * 64 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (row < nq && col < nc) {
+                    float g = acc[ra][rb][r];
+                    float v;
+                    if (metric == kMetricL2) {
+                        v = __fadd_rn(qn[row], cnv);
+                        v = __fsub_rn(v, g);
+                        v = __fsub_rn(v, g);
+                    } else {
+                        v = -g;
+                    }
+                    out[row * ldo + col] = v;
+                }
+            }
+        }
+    }
+}
+
+void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                        const float *cn, int metric, float *out, int64_t ldo, hipStream_t s)
+{
+    if (nq == 0 || nc == 0) {
+        return;
+    }
+    const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nc + kTile - 1) / kTile;
+    IXA_REQUIRE(tiles_m * tiles_n < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
+    const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    if (vec4) {
+        hipLaunchKernelGGL(score_tile_kernel<true>, grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo,
+                           (int)tiles_n);
+    } else {
+        hipLaunchKernelGGL(score_tile_kernel<false>, grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo,
+                           (int)tiles_n);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-row selection of the ksel smallest scores of a materialised score row.  One workgroup per
+// row, four wavefront pools, block merge.  Output: ksel column indices per row (best first),
+// -1 where the row has fewer than ksel columns.
+__global__ __launch_bounds__(256) void select_rows_kernel(const float *__restrict__ scores, int64_t ld, int64_t nc,
+                                                          int ksel, int cap, int merge_n,
+                                                          int32_t *__restrict__ out_idx, int64_t col_base,
+                                                          key_t *__restrict__ out_keys)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // 4 * cap
+    key_t *merge = pools + 4 * cap;                                     // merge_n
+    float *bounds = reinterpret_cast<float *>(merge + merge_n);         // 4
+    int *counts = reinterpret_cast<int *>(bounds + 4);                  // 4
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *row = scores + (int64_t)blockIdx.x * ld;
+    if (tid < 4) {
+        bounds[tid] = __builtin_inff();
+    }
+    __syncthreads();
+    WavePool pool;
+    pool.init(pools + wave * cap, cap, ksel);
+    int iter = 0;
+    for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
+        int64_t c = base + lane;
+        float v = c < nc ? row[c] : __builtin_inff();
+        const bool compacted = pool.push(c < nc && v <= pool.bound, v, (uint32_t)c, lane);
+        if (compacted || (iter & 7) == 7) {
+            // after a compaction (or every 8th step) publish the bound and adopt the best one
+            if (lane == 0) {
+                bounds[wave] = pool.bound;
+            }
+            float b = fminf(fminf(bounds[0], bounds[1]), fminf(bounds[2], bounds[3]));
+            pool.bound = b < pool.bound ? b : pool.bound;
+        }
+    }
+    pool.compact(lane);
+    if (lane == 0) {
+        counts[wave] = pool.count;
+    }
+    __syncthreads();
+    for (int i = tid; i < merge_n; i += 256) {
+        int w = i / ksel, r = i - w * ksel;
+        merge[i] = (w < 4 && r < counts[w]) ? pools[w * cap + r] : kEmptyKey;
+    }
+    block_bitonic_sort(merge, merge_n, tid, 256);
+    for (int i = tid; i < ksel; i += 256) {
+        key_t kk = merge[i];
+        if (out_idx) {
+            out_idx[(int64_t)blockIdx.x * ksel + i] = kk == kEmptyKey ? -1 : (int32_t)key_index(kk);
+        }
+        if (out_keys) {
+            out_keys[(int64_t)blockIdx.x * ksel + i] =
+                kk == kEmptyKey ? kEmptyKey : (kk & 0xffffffff00000000ull) | (key_index(kk) + (uint32_t)col_base);
+        }
+    }
+}
+
+void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
+                        int64_t col_base, unsigned long long *out_keys, hipStream_t s)
+{
+    if (nrows == 0) {
+        return;
+    }
+    IXA_REQUIRE(ksel >= 1 && ksel <= 2048, kErrInvalidParam, "selection size %d out of range [1, 2048]", ksel);
+    const int cap = wave_pool_capacity(ksel);
+    const int merge_n = pow2_ceil(4 * ksel);
+    const size_t smem = (size_t)(4 * cap + merge_n) * sizeof(key_t) + 32;
+    IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "selection size %d needs %zu bytes of LDS", ksel, smem);
+    if (smem > 48 * 1024) {
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    }
+    hipLaunchKernelGGL(select_rows_kernel, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
+                       merge_n, out_idx, col_base, out_keys);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Exact re-evaluation.  Each lane recomputes ONE (query, candidate) score in the canonical order
+// (dot product left to right, no FMA, then (|q|^2 + |c|^2) - g - g), the candidates of a query are
+// sorted by (score, centroid id) and the best `nout` are written.  Because the MFMA pass only has
+// to deliver a superset of the true winners, the result equals the scalar arithmetic bit for bit.
+// A workgroup of 256 lanes serves 256 / P queries, P = padded candidate count (power of two).
+template <bool VEC4>
+__global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q, int64_t nq,
+                                                     const float *__restrict__ C, int d,
+                                                     const float *__restrict__ qn, const float *__restrict__ cn,
+                                                     int metric, const int32_t *__restrict__ cand, int ncand, int P,
+                                                     int nout, int32_t *__restrict__ out_ids,
+                                                     float *__restrict__ out_dist)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    key_t *keys = reinterpret_cast<key_t *>(smem_raw);
+    const int tid = threadIdx.x;
+    const int rows_per_block = P >= 256 ? 1 : 256 / P;
+    const int total = rows_per_block * P;  // >= 256, power of two
+    for (int e = tid; e < total; e += 256) {
+        const int sub = e / P, t = e - sub * P;
+        const int64_t row = (int64_t)blockIdx.x * rows_per_block + sub;
+        key_t key = kEmptyKey;
+        if (row < nq && t < ncand) {
+            const int32_t c = cand[row * ncand + t];
+            if (c >= 0) {
+                const float *q = Q + row * d;
+                const float *cv = C + (int64_t)c * d;
+                float g = 0.f;
+                if (VEC4) {
+                    for (int j = 0; j < d; j += 4) {
+                        float4 a = *reinterpret_cast<const float4 *>(q + j);
+                        float4 b = *reinterpret_cast<const float4 *>(cv + j);
+                        g = __fadd_rn(g, __fmul_rn(a.x, b.x));
+                        g = __fadd_rn(g, __fmul_rn(a.y, b.y));
+                        g = __fadd_rn(g, __fmul_rn(a.z, b.z));
+                        g = __fadd_rn(g, __fmul_rn(a.w, b.w));
+                    }
+                } else {
+                    for (int j = 0; j < d; j++) {
+                        g = __fadd_rn(g, __fmul_rn(q[j], cv[j]));
+                    }
+                }
+                float v;
+                if (metric == kMetricL2) {
+                    v = __fadd_rn(qn[row], cn[c]);
+                    v = __fsub_rn(v, g);
+                    v = __fsub_rn(v, g);
+                } else {
+                    v = -g;
+                }
+                key = make_key(v, (uint32_t)c);
+            }
+        }
+        keys[e] = key;
+    }
+    // segmented bitonic sort: every P-aligned segment ascending
+    for (int size = 2; size <= P; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int t = tid; t < (total >> 1); t += 256) {
+                int i = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
+                int j = i + stride;
+                bool up = ((i & (P - 1)) & size) == 0;
+                key_t a = keys[i], b = keys[j];
+                if ((a > b) == up) {
+                    keys[i] = b;
+                    keys[j] = a;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < rows_per_block * nout; e += 256) {
+        const int sub = e / nout, t = e - sub * nout;
+        const int64_t row = (int64_t)blockIdx.x * rows_per_block + sub;
+        if (row >= nq) {
+            continue;
+        }
+        key_t kk = keys[sub * P + t];
+        const bool ok = kk != kEmptyKey;
+        out_ids[row * nout + t] = ok ? (int32_t)key_index(kk) : -1;
+        if (out_dist) {
+            float v = key_score(kk);
+            const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+            out_dist[row * nout + t] = ok ? (metric == kMetricL2 ? v : -v) : pad;
+        }
+    }
+}
+
+void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,
+                   const int32_t *cand, int ncand, int nout, int32_t *out_ids, float *out_dist, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    IXA_REQUIRE(ncand >= 1 && ncand <= 4096 && nout <= ncand, kErrInvalidParam,
+                "refine candidate count %d out of range [1, 4096]", ncand);
+    const int P = pow2_ceil(ncand < 2 ? 2 : ncand);
+    const int rows_per_block = P >= 256 ? 1 : 256 / P;
+    const unsigned grid = (unsigned)((nq + rows_per_block - 1) / rows_per_block);
+    const size_t smem = (size_t)rows_per_block * P * sizeof(key_t);
+    const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    if (vec4) {
+        hipLaunchKernelGGL(refine_kernel<true>, dim3(grid), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, cand,
+                           ncand, P, nout, out_ids, out_dist);
+    } else {
+        hipLaunchKernelGGL(refine_kernel<false>, dim3(grid), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, cand,
+                           ncand, P, nout, out_ids, out_dist);
+    }
+}
+
+}  // namespace ixa

@@ -1,0 +1,107 @@
+// Device-resident IVFPQ index for one MI355X: the counterpart of the reference's per-device
+// ascend::IndexIVFPQ (FR/ascenddaemon/impl/IndexIVFPQ.h:47-116, 230-278) together with the host
+// orchestration of AscendIndexIVFPQImpl (FR/ascend/impl/AscendIndexIVFPQImpl.cpp).
+#pragma once
+#include <cstdint>
+#include <vector>
+
+#include "common.h"
+
+namespace ixa {
+
+struct IvfpqConfig {
+    int niter = 25;                   // coarse k-means iterations (reference CPU mode: 25)
+    int pq_niter = -1;                // sub-quantizer k-means iterations; -1 = niter (pqNiter)
+    int spherical = 0;                // 1 = L2-normalise centroids after every update (reference default)
+    int train_samples_per_list = 256; // rows sampled per coarse centroid (trainSamplesPerList)
+    int64_t max_train_samples = 10000000;  // maxTrainSamples
+    int lut_fp16 = 0;                 // LUT entries stored as IEEE half
+    int code_layout = -1;             // -1 = pick (rot32 when M % 32 == 0), 0 = row, 1 = rot32
+    int64_t scratch_bytes = (int64_t)1 << 30;  // budget of the coarse score scratch
+    uint64_t seed = 1234;
+    int strict_reference_params = 0;  // 1 = enforce the reference's d / nlist / M whitelists
+};
+
+struct SearchStats {
+    double scanned_codes = 0;   // sum of probed list lengths of the last search
+    double ms_coarse = 0;       // stage 1 (scores, selection, refine)
+    double ms_scan = 0;         // fused LUT + ADC + top-k kernel (+ merge)
+    double ms_total = 0;        // device time of the whole search
+    double scan_launches = 0;   // kernel launches the ms_scan figure covers
+    double nsplit = 0;
+};
+
+class IvfpqIndex {
+public:
+    IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const IvfpqConfig &cfg);
+    ~IvfpqIndex();
+    IvfpqIndex(const IvfpqIndex &) = delete;
+    IvfpqIndex &operator=(const IvfpqIndex &) = delete;
+
+    int d() const { return d_; }
+    int M() const { return M_; }
+    int metric() const { return metric_; }
+    int64_t nlist() const { return nlist_; }
+    int64_t ntotal() const { return ntotal_; }
+    bool is_trained() const { return trained_; }
+    int nprobe() const { return nprobe_; }
+    void set_nprobe(int nprobe);
+    int code_layout() const { return layout_; }
+    hipStream_t stream() const { return stream_; }
+
+    // x may live on the host or on the device (on_device says which).
+    void train(int64_t n, const float *x, bool on_device);
+    void set_trained(const float *centroids, const float *codebook);   // host pointers
+    void get_trained(float *centroids, float *codebook) const;          // host pointers, either may be null
+    void add(int64_t n, const float *x, const int64_t *ids, bool on_device);
+    void add_codes(int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids);  // host pointers
+    void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
+    void assign(int64_t n, const float *x, int64_t *out, bool on_device);               // out: host
+    void coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device);  // out: host
+    void encode(int64_t n, const float *x, uint8_t *codes, bool on_device);             // codes: host
+    int64_t list_length(int64_t list) const;
+    void get_list(int64_t list, uint8_t *codes, int64_t *ids) const;                    // host pointers
+    int64_t remove_ids(int64_t n, const int64_t *ids);
+    void reset();
+    const SearchStats &stats() const { return stats_; }
+
+private:
+    void check_trained() const;
+    void upload_trained(const float *centroids, const float *codebook);
+    // best `nout` lists of every row of device matrix x (canonical arithmetic), device outputs
+    void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
+                       float *out_dist);
+    void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev);
+    void sync_list_tables();
+    void kmeans_coarse(const std::vector<float> &sample, int64_t ns);
+    void kmeans_pq(const std::vector<float> &sample, int64_t ns);
+
+    int d_, M_, dsub_, metric_;
+    int nbits_;  // always 8 (256 codewords per sub-quantizer)
+    int64_t nlist_;
+    IvfpqConfig cfg_;
+    int layout_ = 0;
+    int nprobe_ = 64;
+    bool trained_ = false;
+    int64_t ntotal_ = 0;
+    hipStream_t stream_ = nullptr;
+    hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
+
+    DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
+    // arena
+    DeviceBuffer<uint8_t> codes_;
+    DeviceBuffer<int64_t> ids_;
+    DeviceBuffer<int64_t> list_off_dev_;
+    DeviceBuffer<int32_t> list_len_dev_;
+    std::vector<int64_t> list_off_;   // first slot of each list (host mirror), size nlist + 1
+    std::vector<int32_t> list_len_;
+    int64_t total_slots_ = 0;
+    // search workspaces (grown on demand, reused between calls)
+    DeviceBuffer<float> ws_x_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<int32_t> ws_cand_, ws_probes_;
+    DeviceBuffer<int64_t> ws_labels_;
+    DeviceBuffer<unsigned long long> ws_partial_, ws_counter_;
+    SearchStats stats_;
+};
+
+}  // namespace ixa

@@ -1,0 +1,778 @@
+// Host orchestration of the device-resident IVFPQ index (see ivfpq_index.h).
+#include "ivfpq_index.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+#include <random>
+#include <unordered_set>
+
+#include "coarse.h"
+#include "pq.h"
+#include "scan.h"
+
+namespace ixa {
+
+namespace {
+
+// Parameter whitelists of the reference (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:130-140).
+const int kRefDims[] = {128};
+const int kRefNlists[] = {1024, 2048, 4096, 8192, 16384, 262144, 524288};
+const int kRefMsubs[] = {2, 4, 8, 16, 32};
+
+template <size_t N>
+bool contains(const int (&a)[N], int64_t v)
+{
+    for (size_t i = 0; i < N; i++) {
+        if (a[i] == v) {
+            return true;
+        }
+    }
+    return false;
+}
+
+constexpr int64_t kMaxN = 1000000000;   // MAX_N, FR/ascend/AscendIndex.h
+constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this build (reference device limit: 320)
+constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
+
+// ---- arena kernels ------------------------------------------------------------------------------
+
+// Copies every list from the old arena to its place in the new one (16-byte units; a list's slot
+// range is a multiple of 64 slots, so both ends are 16-byte aligned for every M).
+__global__ __launch_bounds__(256) void copy_lists_kernel(const uint8_t *__restrict__ old_codes,
+                                                         const int64_t *__restrict__ old_ids,
+                                                         const int64_t *__restrict__ old_off,
+                                                         const int32_t *__restrict__ old_len,
+                                                         uint8_t *__restrict__ new_codes,
+                                                         int64_t *__restrict__ new_ids,
+                                                         const int64_t *__restrict__ new_off, int M)
+{
+    const int l = blockIdx.x;
+    const int len = old_len[l];
+    if (len == 0) {
+        return;
+    }
+    const int64_t so = old_off[l], dn = new_off[l];
+    const int64_t slots = ((int64_t)len + 63) / 64 * 64;
+    const uint4 *src = reinterpret_cast<const uint4 *>(old_codes + so * M);
+    uint4 *dst = reinterpret_cast<uint4 *>(new_codes + dn * M);
+    const int64_t n16 = slots * M / 16;
+    for (int64_t i = threadIdx.x; i < n16; i += 256) {
+        dst[i] = src[i];
+    }
+    for (int64_t i = threadIdx.x; i < len; i += 256) {
+        new_ids[dn + i] = old_ids[so + i];
+    }
+}
+
+// Places freshly encoded vectors: vector i goes to position pos[i] of list list_no[i].
+// layout 1 rotates the code bytes by the position inside the list (see scan.hip).
+__global__ __launch_bounds__(256) void scatter_new_kernel(int64_t n, const int32_t *__restrict__ list_no,
+                                                          const int32_t *__restrict__ pos,
+                                                          const uint8_t *__restrict__ codes_in,
+                                                          const int64_t *__restrict__ ids_in, int64_t id_base,
+                                                          const int64_t *__restrict__ new_off, int M, int layout,
+                                                          uint8_t *__restrict__ codes, int64_t *__restrict__ ids)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const int p = pos[i];
+    const int64_t slot = new_off[list_no[i]] + p;
+    const uint8_t *src = codes_in + i * M;
+    uint8_t *dst = codes + slot * M;
+    for (int j = 0; j < M; j++) {
+        const int m = layout == 1 ? ((j & ~31) | ((j + p) & 31)) : j;
+        dst[j] = src[m];
+    }
+    ids[slot] = ids_in ? ids_in[i] : id_base + i;
+}
+
+// Reads one list back in the public row-major form [len][M].
+__global__ __launch_bounds__(256) void gather_list_kernel(const uint8_t *__restrict__ codes, int64_t off, int len,
+                                                          int M, int layout, uint8_t *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (int64_t)len * M) {
+        return;
+    }
+    const int p = (int)(e / M), m = (int)(e % M);
+    // sub-quantizer m of position p is stored at byte j with (j + p) % 32 == m % 32 inside its 32-block
+    const int j = layout == 1 ? ((m & ~31) | ((m - p) & 31)) : m;
+    out[e] = codes[(off + p) * M + j];
+}
+
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ x, const int64_t *__restrict__ idx,
+                                                          int64_t n, int d, float *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * d) {
+        return;
+    }
+    out[e] = x[idx[e / d] * d + e % d];
+}
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+}  // namespace
+
+// -------------------------------------------------------------------------------------------------
+
+IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const IvfpqConfig &cfg)
+    : d_(d), M_(M), dsub_(0), metric_(metric), nbits_(nbits), nlist_(nlist), cfg_(cfg)
+{
+    // Messages keep the reference's wording (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:510-525) so that
+    // its unit tests' substring checks (FR/ut/TestAscendIndexUTIVFPQ.cpp:77-184) carry over.
+    IXA_REQUIRE(metric == kMetricL2 || metric == kMetricInnerProduct, kErrInvalidParam, "Unsupported metric type");
+    const bool strict = cfg.strict_reference_params != 0;
+    IXA_REQUIRE(d >= 1 && d <= 4096 && (!strict || contains(kRefDims, d)), kErrInvalidParam, "Unsupported dims: %d\n",
+                d);
+    IXA_REQUIRE(nlist >= 1 && nlist <= (1 << 20) && (!strict || contains(kRefNlists, nlist)), kErrInvalidParam,
+                "Unsupported nlists: %d\n", (int)nlist);
+    IXA_REQUIRE(M >= 1 && M <= 128 && d % M == 0 && (!strict || contains(kRefMsubs, M)), kErrInvalidParam,
+                "Unsupported msubs: %d\n", M);
+    IXA_REQUIRE(nbits == 8, kErrInvalidParam, "Unsupported nbits: %d\n", nbits);
+    dsub_ = d / M;
+    if (cfg.code_layout == 1) {
+        IXA_REQUIRE(M == 32 || M == 64 || M == 96, kErrInvalidParam,
+                    "code layout rot32 needs msubs in {32, 64, 96}, got %d", M);
+    }
+    layout_ = cfg.code_layout >= 0 ? cfg.code_layout : ((M == 32 || M == 64 || M == 96) ? 1 : 0);
+    nprobe_ = (int)std::min<int64_t>(64, nlist);
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    IXA_REQUIRE(e == hipSuccess && ndev > 0, kErrIndexNotInit,
+                "no HIP device available (%s): this library has no CPU path", hipGetErrorString(e));
+    IXA_HIP(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+    for (auto &ev : ev_) {
+        IXA_HIP(hipEventCreate(&ev));
+    }
+    list_off_.assign(nlist_ + 1, 0);
+    list_len_.assign(nlist_, 0);
+    sync_list_tables();
+}
+
+IvfpqIndex::~IvfpqIndex()
+{
+    if (stream_) {
+        (void)hipStreamSynchronize(stream_);
+    }
+    for (auto &ev : ev_) {
+        if (ev) {
+            (void)hipEventDestroy(ev);
+        }
+    }
+    if (stream_) {
+        (void)hipStreamDestroy(stream_);
+    }
+}
+
+void IvfpqIndex::set_nprobe(int nprobe)
+{
+    IXA_REQUIRE(nprobe >= 1, kErrInvalidParam, "nprobe must be >= 1, got %d", nprobe);
+    nprobe_ = (int)std::min<int64_t>(nprobe, nlist_);
+}
+
+void IvfpqIndex::check_trained() const
+{
+    IXA_REQUIRE(trained_, kErrIndexNotInit, "AscendIndexIVFPQ is not trained!");
+}
+
+void IvfpqIndex::sync_list_tables()
+{
+    list_off_dev_.upload(list_off_.data(), (size_t)nlist_, stream_);
+    list_len_dev_.upload(list_len_.data(), (size_t)nlist_, stream_);
+    IXA_HIP(hipStreamSynchronize(stream_));
+}
+
+// Centroid and codeword norms are produced on the device in the same left-to-right fp32 order the
+// reference uses on the host (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1114-1126).
+void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
+{
+    if (centroids) {
+        centroids_.upload(centroids, (size_t)nlist_ * d_, stream_);
+        cnorm_.resize((size_t)nlist_);
+        launch_sqnorm_rows(centroids_.data(), nlist_, d_, cnorm_.data(), stream_);
+    }
+    if (codebook) {
+        codebook_.upload(codebook, (size_t)M_ * 256 * dsub_, stream_);
+        cbnorm_.resize((size_t)M_ * 256);
+        launch_sqnorm_rows(codebook_.data(), (int64_t)M_ * 256, dsub_, cbnorm_.data(), stream_);
+    }
+    IXA_HIP(hipStreamSynchronize(stream_));
+}
+
+void IvfpqIndex::set_trained(const float *centroids, const float *codebook)
+{
+    IXA_REQUIRE(centroids && codebook, kErrInvalidParam, "centroids and codebook can not be nullptr.");
+    IXA_REQUIRE(ntotal_ == 0, kErrIllegalOperation, "set_trained on a non-empty index; call reset first");
+    upload_trained(centroids, codebook);
+    trained_ = true;
+}
+
+void IvfpqIndex::get_trained(float *centroids, float *codebook) const
+{
+    check_trained();
+    if (centroids) {
+        centroids_.download(centroids, (size_t)nlist_ * d_, stream_);
+    }
+    if (codebook) {
+        codebook_.download(codebook, (size_t)M_ * 256 * dsub_, stream_);
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Stage 1 driver: MFMA scores into a bounded scratch, per-row selection of nout + slack candidates,
+// exact refine.  Never materialises more than scratch_bytes of the n x nlist score matrix.
+void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
+                               float *out_dist)
+{
+    if (n == 0) {
+        return;
+    }
+    const int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
+    ws_qn_.resize((size_t)n);
+    launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
+    int64_t rows = cfg_.scratch_bytes / ((int64_t)nlist_ * 4);
+    rows = std::max<int64_t>(128, rows / 128 * 128);
+    rows = std::min<int64_t>(rows, round_up(n, 128));
+    ws_scores_.resize((size_t)rows * nlist_);
+    ws_cand_.resize((size_t)rows * ncand);
+    for (int64_t r0 = 0; r0 < n; r0 += rows) {
+        const int64_t nr = std::min(rows, n - r0);
+        launch_score_tiles(x_dev + r0 * d_, nr, centroids_.data(), nlist_, d_, ws_qn_.data() + r0, cnorm_.data(),
+                           select_metric, ws_scores_.data(), nlist_, stream_);
+        launch_select_rows(ws_scores_.data(), nr, nlist_, nlist_, ncand, ws_cand_.data(), 0, nullptr, stream_);
+        launch_refine(x_dev + r0 * d_, nr, centroids_.data(), d_, ws_qn_.data() + r0, cnorm_.data(), select_metric,
+                      ws_cand_.data(), ncand, nout, out_ids + r0 * nout, out_dist ? out_dist + r0 * nout : nullptr,
+                      stream_);
+    }
+}
+
+void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)
+{
+    check_trained();
+    IXA_REQUIRE(x && out, kErrInvalidParam, "x can not be nullptr.");
+    IXA_REQUIRE(n >= 0 && n < kMaxN, kErrInvalidParam, "n must be >= 0 and < %ld", (long)kMaxN);
+    std::vector<int32_t> tmp;
+    for (int64_t p0 = 0; p0 < n; p0 += kAddPage) {
+        const int64_t np = std::min(kAddPage, n - p0);
+        const float *xd = x + p0 * d_;
+        if (!on_device) {
+            ws_x_.upload(x + p0 * d_, (size_t)np * d_, stream_);
+            xd = ws_x_.data();
+        }
+        ws_probes_.resize((size_t)np);
+        coarse_select(xd, np, 1, kMetricL2, ws_probes_.data(), nullptr);
+        tmp.resize((size_t)np);
+        ws_probes_.download(tmp.data(), (size_t)np, stream_);
+        for (int64_t i = 0; i < np; i++) {
+            out[p0 + i] = tmp[(size_t)i];
+        }
+    }
+}
+
+void IvfpqIndex::coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device)
+{
+    check_trained();
+    IXA_REQUIRE(x && out_ids, kErrInvalidParam, "x can not be nullptr.");
+    const float *xd = x;
+    if (!on_device) {
+        ws_x_.upload(x, (size_t)n * d_, stream_);
+        xd = ws_x_.data();
+    }
+    ws_probes_.resize((size_t)n * nprobe_);
+    ws_dist_.resize((size_t)n * nprobe_);
+    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), ws_dist_.data());
+    std::vector<int32_t> tmp((size_t)n * nprobe_);
+    ws_probes_.download(tmp.data(), tmp.size(), stream_);
+    for (size_t i = 0; i < tmp.size(); i++) {
+        out_ids[i] = tmp[i];
+    }
+    if (out_dist) {
+        ws_dist_.download(out_dist, (size_t)n * nprobe_, stream_);
+    }
+}
+
+void IvfpqIndex::encode(int64_t n, const float *x, uint8_t *codes, bool on_device)
+{
+    check_trained();
+    IXA_REQUIRE(x && codes, kErrInvalidParam, "x can not be nullptr.");
+    DeviceBuffer<uint8_t> cd;
+    for (int64_t p0 = 0; p0 < n; p0 += kAddPage) {
+        const int64_t np = std::min(kAddPage, n - p0);
+        const float *xd = x + p0 * d_;
+        if (!on_device) {
+            ws_x_.upload(x + p0 * d_, (size_t)np * d_, stream_);
+            xd = ws_x_.data();
+        }
+        cd.resize((size_t)np * M_);
+        launch_pq_encode(xd, np, d_, M_, codebook_.data(), cd.data(), stream_);
+        cd.download(codes + p0 * M_, (size_t)np * M_, stream_);
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// add: coarse assignment (always L2, as the reference's add path: AscendIndexIVFPQImpl.cpp:603-672,
+// 701), PQ encode of the raw vector (:674-692, 879-921), then append to the lists in input order
+// (:715-805; ids default to ntotal + i, FR/ascend/impl/AscendIndexImpl.h:59-83).
+void IvfpqIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_device)
+{
+    check_trained();
+    IXA_REQUIRE(x, kErrInvalidParam, "x can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(ntotal_ + n < ((int64_t)1 << 32) - 64 * nlist_, kErrInvalidParam,
+                "index would exceed the 32-bit slot space");
+    DeviceBuffer<int32_t> list_no;
+    DeviceBuffer<uint8_t> codes;
+    DeviceBuffer<int64_t> ids_dev;
+    for (int64_t p0 = 0; p0 < n; p0 += kAddPage) {
+        const int64_t np = std::min(kAddPage, n - p0);
+        const float *xd = x + p0 * d_;
+        if (!on_device) {
+            ws_x_.upload(x + p0 * d_, (size_t)np * d_, stream_);
+            xd = ws_x_.data();
+        }
+        const int64_t *idd = nullptr;
+        if (ids) {
+            if (on_device) {
+                idd = ids + p0;
+            } else {
+                ids_dev.upload(ids + p0, (size_t)np, stream_);
+                idd = ids_dev.data();
+            }
+        }
+        list_no.resize((size_t)np);
+        coarse_select(xd, np, 1, kMetricL2, list_no.data(), nullptr);
+        codes.resize((size_t)np * M_);
+        launch_pq_encode(xd, np, d_, M_, codebook_.data(), codes.data(), stream_);
+        append(np, list_no.data(), codes.data(), idd);
+    }
+}
+
+void IvfpqIndex::add_codes(int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids)
+{
+    check_trained();
+    IXA_REQUIRE(list >= 0 && list < nlist_, kErrInvalidParam, "the listId is %ld, out of numLists(%ld)", (long)list,
+                (long)nlist_);
+    IXA_REQUIRE(n >= 0 && (n == 0 || (codes && ids)), kErrInvalidParam, "codes and ids can not be nullptr.");
+    if (n == 0) {
+        return;
+    }
+    std::vector<int32_t> ln((size_t)n, (int32_t)list);
+    DeviceBuffer<int32_t> list_no;
+    DeviceBuffer<uint8_t> cd;
+    DeviceBuffer<int64_t> idd;
+    list_no.upload(ln.data(), (size_t)n, stream_);
+    cd.upload(codes, (size_t)n * M_, stream_);
+    idd.upload(ids, (size_t)n, stream_);
+    append(n, list_no.data(), cd.data(), idd.data());
+}
+
+void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev)
+{
+    std::vector<int32_t> list_no((size_t)n), pos((size_t)n);
+    IXA_HIP(hipMemcpyAsync(list_no.data(), list_no_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream_));
+    IXA_HIP(hipStreamSynchronize(stream_));
+    std::vector<int32_t> new_len(list_len_);
+    for (int64_t i = 0; i < n; i++) {
+        const int32_t l = list_no[(size_t)i];
+        IXA_REQUIRE(l >= 0 && l < nlist_, kErrInner, "coarse assignment produced list %d", l);
+        pos[(size_t)i] = new_len[(size_t)l]++;
+    }
+    std::vector<int64_t> new_off((size_t)nlist_ + 1, 0);
+    for (int64_t l = 0; l < nlist_; l++) {
+        new_off[(size_t)l + 1] = new_off[(size_t)l] + round_up(new_len[(size_t)l], 64);
+    }
+    const int64_t slots = new_off[(size_t)nlist_];
+    IXA_REQUIRE(slots < ((int64_t)1 << 32) - 1, kErrInvalidParam, "index exceeds the 32-bit slot space");
+
+    DeviceBuffer<uint8_t> new_codes((size_t)std::max<int64_t>(slots, 64) * M_);
+    DeviceBuffer<int64_t> new_ids((size_t)std::max<int64_t>(slots, 64));
+    DeviceBuffer<int64_t> new_off_dev;
+    DeviceBuffer<int32_t> pos_dev;
+    new_off_dev.upload(new_off.data(), (size_t)nlist_, stream_);
+    pos_dev.upload(pos.data(), (size_t)n, stream_);
+    IXA_HIP(hipMemsetAsync(new_codes.data(), 0, new_codes.bytes(), stream_));
+    IXA_HIP(hipMemsetAsync(new_ids.data(), 0xff, new_ids.bytes(), stream_));
+    if (ntotal_ > 0) {
+        hipLaunchKernelGGL(copy_lists_kernel, dim3((unsigned)nlist_), dim3(256), 0, stream_, codes_.data(),
+                           ids_.data(), list_off_dev_.data(), list_len_dev_.data(), new_codes.data(), new_ids.data(),
+                           new_off_dev.data(), M_);
+    }
+    hipLaunchKernelGGL(scatter_new_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, n, list_no_dev, pos_dev.data(),
+                       codes_dev, ids_dev, ntotal_, new_off_dev.data(), M_, layout_, new_codes.data(), new_ids.data());
+    IXA_HIP(hipStreamSynchronize(stream_));
+    codes_ = std::move(new_codes);
+    ids_ = std::move(new_ids);
+    list_off_ = std::move(new_off);
+    list_len_ = std::move(new_len);
+    total_slots_ = slots;
+    ntotal_ += n;
+    sync_list_tables();
+}
+
+int64_t IvfpqIndex::list_length(int64_t list) const
+{
+    IXA_REQUIRE(list >= 0 && list < nlist_, kErrInvalidParam, "the listId is %ld, out of numLists(%ld)", (long)list,
+                (long)nlist_);
+    return list_len_[(size_t)list];
+}
+
+void IvfpqIndex::get_list(int64_t list, uint8_t *codes, int64_t *ids) const
+{
+    const int64_t len = list_length(list);
+    if (len == 0) {
+        return;
+    }
+    const int64_t off = list_off_[(size_t)list];
+    if (codes) {
+        DeviceBuffer<uint8_t> tmp((size_t)len * M_);
+        hipLaunchKernelGGL(gather_list_kernel, dim3(blocks_for(len * M_)), dim3(256), 0, stream_, codes_.data(), off,
+                           (int)len, M_, layout_, tmp.data());
+        tmp.download(codes, (size_t)len * M_, stream_);
+    }
+    if (ids) {
+        IXA_HIP(hipMemcpyAsync(ids, ids_.data() + off, (size_t)len * 8, hipMemcpyDeviceToHost, stream_));
+        IXA_HIP(hipStreamSynchronize(stream_));
+    }
+}
+
+// remove_ids: every list is filtered in place keeping the order of the survivors
+// (FR/ascenddaemon/impl/IndexIVFPQ.cpp:346-506).  Host-mediated: the arena is read back, filtered
+// and re-appended list by list.
+int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
+{
+    IXA_REQUIRE(n >= 0 && (n == 0 || ids), kErrInvalidParam, "ids can not be nullptr.");
+    if (n == 0 || ntotal_ == 0) {
+        return 0;
+    }
+    std::unordered_set<int64_t> del(ids, ids + n);
+    std::vector<int64_t> all_ids((size_t)total_slots_);
+    IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
+    IXA_HIP(hipStreamSynchronize(stream_));
+    std::vector<int32_t> keep_list;
+    std::vector<int64_t> keep_ids;
+    std::vector<uint8_t> keep_codes, buf;
+    int64_t removed = 0;
+    for (int64_t l = 0; l < nlist_; l++) {
+        const int64_t len = list_len_[(size_t)l], off = list_off_[(size_t)l];
+        if (len == 0) {
+            continue;
+        }
+        bool any = false;
+        for (int64_t i = 0; i < len && !any; i++) {
+            any = del.count(all_ids[(size_t)(off + i)]) != 0;
+        }
+        buf.resize((size_t)len * M_);
+        get_list(l, buf.data(), nullptr);
+        for (int64_t i = 0; i < len; i++) {
+            const int64_t id = all_ids[(size_t)(off + i)];
+            if (any && del.count(id)) {
+                removed++;
+                continue;
+            }
+            keep_list.push_back((int32_t)l);
+            keep_ids.push_back(id);
+            keep_codes.insert(keep_codes.end(), buf.begin() + i * M_, buf.begin() + (i + 1) * M_);
+        }
+    }
+    if (removed == 0) {
+        return 0;
+    }
+    reset();
+    if (!keep_ids.empty()) {
+        DeviceBuffer<int32_t> ln;
+        DeviceBuffer<uint8_t> cd;
+        DeviceBuffer<int64_t> idd;
+        ln.upload(keep_list.data(), keep_list.size(), stream_);
+        cd.upload(keep_codes.data(), keep_codes.size(), stream_);
+        idd.upload(keep_ids.data(), keep_ids.size(), stream_);
+        append((int64_t)keep_ids.size(), ln.data(), cd.data(), idd.data());
+    }
+    return removed;
+}
+
+// reset keeps the trained quantizers and drops every list (FR/ascend/AscendIndexIVF.h: reset()).
+void IvfpqIndex::reset()
+{
+    IXA_HIP(hipStreamSynchronize(stream_));
+    codes_.release();
+    ids_.release();
+    list_off_.assign((size_t)nlist_ + 1, 0);
+    list_len_.assign((size_t)nlist_, 0);
+    total_slots_ = 0;
+    ntotal_ = 0;
+    sync_list_tables();
+}
+
+// -------------------------------------------------------------------------------------------------
+// search (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2351-2411): the whole batch goes through three
+// launches on one stream -- no per-8-query batching, no host round trip for the probe lists.
+void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
+{
+    check_trained();
+    IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+
+    const float *xd = x;
+    if (!on_device) {
+        ws_x_.upload(x, (size_t)n * d_, stream_);
+        xd = ws_x_.data();
+    }
+    float *dd = dist;
+    int64_t *ld = labels;
+    if (!on_device) {
+        ws_dist_.resize((size_t)n * k);
+        ws_labels_.resize((size_t)n * k);
+        dd = ws_dist_.data();
+        ld = ws_labels_.data();
+    }
+    ws_probes_.resize((size_t)n * nprobe_);
+    ws_counter_.resize(1);
+
+    IXA_HIP(hipEventRecord(ev_[0], stream_));
+    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr);
+    IXA_HIP(hipEventRecord(ev_[1], stream_));
+
+    ScanParams p{};
+    p.queries = xd;
+    p.probes = ws_probes_.data();
+    p.nprobe = nprobe_;
+    p.codebook = codebook_.data();
+    p.cb_norms = cbnorm_.data();
+    p.d = d_;
+    p.M = M_;
+    p.dsub = dsub_;
+    p.metric = metric_;
+    p.lut_fp16 = cfg_.lut_fp16;
+    p.codes = codes_.data();
+    p.ids = ids_.data();
+    p.list_off = list_off_dev_.data();
+    p.list_len = list_len_dev_.data();
+    p.code_layout = layout_;
+    p.k = (int)k;
+    // enough workgroups to fill 256 CUs several times over, bounded by what one merge pass can hold
+    int nsplit = 1;
+    if (n < 2048) {
+        nsplit = (int)std::min<int64_t>((2048 + n - 1) / n, nprobe_);
+        nsplit = (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));
+    }
+    p.nsplit = nsplit;
+    if (nsplit > 1) {
+        ws_partial_.resize((size_t)n * nsplit * k);
+        p.partial = ws_partial_.data();
+    }
+    p.out_dist = dd;
+    p.out_labels = ld;
+    launch_scan(p, n, stream_);
+    IXA_HIP(hipEventRecord(ev_[2], stream_));
+
+    IXA_HIP(hipMemsetAsync(ws_counter_.data(), 0, 8, stream_));
+    launch_count_scanned(ws_probes_.data(), n * nprobe_, list_len_dev_.data(), ws_counter_.data(), stream_);
+    unsigned long long scanned = 0;
+    ws_counter_.download(&scanned, 1, stream_);
+    if (!on_device) {
+        ws_dist_.download(dist, (size_t)n * k, stream_);
+        ws_labels_.download(labels, (size_t)n * k, stream_);
+    }
+    float ms01 = 0, ms12 = 0;
+    IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
+    IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+    stats_.scanned_codes = (double)scanned;
+    stats_.ms_coarse = ms01;
+    stats_.ms_scan = ms12;
+    stats_.ms_total = ms01 + ms12;
+    stats_.scan_launches = nsplit > 1 ? 2 : 1;
+    stats_.nsplit = nsplit;
+}
+
+// -------------------------------------------------------------------------------------------------
+// Training.  The reference delegates to faiss::Clustering (CPU mode) or runs device assignment with
+// a host centroid update (NPU mode: FR/ascendhost/src/impl/AscendClusteringImpl.cpp:686-762); this
+// build does the latter: assignment on the GPU (stage-1 kernels, PQ encode kernel), centroid update
+// on the host in float64.  Sampling follows computeTrainTotalSize / sampleTrainData
+// (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:51-112).  Plain Lloyd unless cfg.spherical.
+
+void IvfpqIndex::train(int64_t n, const float *x, bool on_device)
+{
+    IXA_REQUIRE(x, kErrInvalidParam, "x can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    if (trained_) {
+        return;  // same as the reference: training a trained index is a no-op
+    }
+    IXA_REQUIRE(n >= nlist_ && n >= 256, kErrInvalidParam,
+                "need at least max(nlist, 256) = %ld training vectors, got %ld", (long)std::max<int64_t>(nlist_, 256),
+                (long)n);
+    int64_t ns = std::min<int64_t>({(int64_t)nlist_ * cfg_.train_samples_per_list, n, cfg_.max_train_samples});
+    ns = std::max<int64_t>(ns, std::min<int64_t>(n, std::max<int64_t>(nlist_, 256 * 40)));
+    std::vector<float> sample((size_t)ns * d_);
+    std::vector<int64_t> idx((size_t)n);
+    std::iota(idx.begin(), idx.end(), 0);
+    if (ns < n) {
+        std::mt19937_64 gen(cfg_.seed);
+        std::shuffle(idx.begin(), idx.end(), gen);
+        idx.resize((size_t)ns);
+    }
+    if (on_device) {
+        DeviceBuffer<int64_t> idx_dev;
+        DeviceBuffer<float> out((size_t)ns * d_);
+        idx_dev.upload(idx.data(), (size_t)ns, stream_);
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for(ns * d_)), dim3(256), 0, stream_, x, idx_dev.data(), ns,
+                           d_, out.data());
+        out.download(sample.data(), sample.size(), stream_);
+    } else {
+        for (int64_t i = 0; i < ns; i++) {
+            std::memcpy(&sample[(size_t)i * d_], x + idx[(size_t)i] * d_, sizeof(float) * (size_t)d_);
+        }
+    }
+    kmeans_coarse(sample, ns);
+    kmeans_pq(sample, ns);
+    trained_ = true;
+}
+
+namespace {
+
+// Re-seeds empty clusters by splitting the most populated one (symmetric perturbation).
+void split_empty(std::vector<float> &cent, std::vector<int64_t> &cnt, int64_t k, int dim)
+{
+    for (int64_t c = 0; c < k; c++) {
+        if (cnt[(size_t)c] != 0) {
+            continue;
+        }
+        const int64_t big = std::max_element(cnt.begin(), cnt.begin() + k) - cnt.begin();
+        for (int t = 0; t < dim; t++) {
+            const float v = cent[(size_t)(big * dim + t)];
+            const float eps = (t & 1) ? 1.0f / 1024 : -1.0f / 1024;
+            cent[(size_t)(c * dim + t)] = v * (1.0f + eps);
+            cent[(size_t)(big * dim + t)] = v * (1.0f - eps);
+        }
+        cnt[(size_t)c] = cnt[(size_t)big] / 2;
+        cnt[(size_t)big] -= cnt[(size_t)c];
+    }
+}
+
+void normalise_rows(std::vector<float> &cent, int64_t k, int dim)
+{
+    for (int64_t c = 0; c < k; c++) {
+        double nn = 0;
+        for (int t = 0; t < dim; t++) {
+            nn += (double)cent[(size_t)(c * dim + t)] * cent[(size_t)(c * dim + t)];
+        }
+        nn = std::sqrt(nn);
+        if (nn > 0) {
+            for (int t = 0; t < dim; t++) {
+                cent[(size_t)(c * dim + t)] = (float)(cent[(size_t)(c * dim + t)] / nn);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+void IvfpqIndex::kmeans_coarse(const std::vector<float> &sample, int64_t ns)
+{
+    std::vector<int64_t> pick((size_t)ns);
+    std::iota(pick.begin(), pick.end(), 0);
+    std::mt19937_64 gen(cfg_.seed + 1);
+    std::shuffle(pick.begin(), pick.end(), gen);
+    std::vector<float> cent((size_t)nlist_ * d_);
+    for (int64_t c = 0; c < nlist_; c++) {
+        std::memcpy(&cent[(size_t)c * d_], &sample[(size_t)pick[(size_t)c] * d_], sizeof(float) * (size_t)d_);
+    }
+    DeviceBuffer<float> xs;
+    xs.upload(sample.data(), sample.size(), stream_);
+    DeviceBuffer<int32_t> asg((size_t)ns);
+    std::vector<int32_t> h_asg((size_t)ns);
+    std::vector<double> acc((size_t)nlist_ * d_);
+    std::vector<int64_t> cnt((size_t)nlist_);
+    for (int it = 0; it < cfg_.niter; it++) {
+        upload_trained(cent.data(), nullptr);
+        coarse_select(xs.data(), ns, 1, kMetricL2, asg.data(), nullptr);
+        asg.download(h_asg.data(), (size_t)ns, stream_);
+        std::fill(acc.begin(), acc.end(), 0.0);
+        std::fill(cnt.begin(), cnt.end(), 0);
+        for (int64_t i = 0; i < ns; i++) {
+            const int64_t a = h_asg[(size_t)i];
+            cnt[(size_t)a]++;
+            double *dst = &acc[(size_t)a * d_];
+            const float *src = &sample[(size_t)i * d_];
+            for (int t = 0; t < d_; t++) {
+                dst[t] += src[t];
+            }
+        }
+        for (int64_t c = 0; c < nlist_; c++) {
+            if (cnt[(size_t)c] > 0) {
+                for (int t = 0; t < d_; t++) {
+                    cent[(size_t)c * d_ + t] = (float)(acc[(size_t)c * d_ + t] / (double)cnt[(size_t)c]);
+                }
+            }
+        }
+        split_empty(cent, cnt, nlist_, d_);
+        if (cfg_.spherical) {
+            normalise_rows(cent, nlist_, d_);
+        }
+    }
+    upload_trained(cent.data(), nullptr);
+}
+
+void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
+{
+    const int niter = cfg_.pq_niter >= 0 ? cfg_.pq_niter : cfg_.niter;
+    std::vector<float> cb((size_t)M_ * 256 * dsub_);
+    std::mt19937_64 gen(cfg_.seed + 2);
+    for (int m = 0; m < M_; m++) {
+        std::vector<int64_t> pick((size_t)ns);
+        std::iota(pick.begin(), pick.end(), 0);
+        std::shuffle(pick.begin(), pick.end(), gen);
+        for (int k = 0; k < 256; k++) {
+            std::memcpy(&cb[((size_t)m * 256 + k) * dsub_], &sample[(size_t)pick[(size_t)(k % ns)] * d_ + m * dsub_],
+                        sizeof(float) * (size_t)dsub_);
+        }
+    }
+    DeviceBuffer<float> xs;
+    xs.upload(sample.data(), sample.size(), stream_);
+    DeviceBuffer<uint8_t> codes((size_t)ns * M_);
+    std::vector<uint8_t> h_codes((size_t)ns * M_);
+    std::vector<double> acc((size_t)M_ * 256 * dsub_);
+    std::vector<int64_t> cnt((size_t)M_ * 256);
+    for (int it = 0; it < niter; it++) {
+        upload_trained(nullptr, cb.data());
+        launch_pq_encode(xs.data(), ns, d_, M_, codebook_.data(), codes.data(), stream_);
+        codes.download(h_codes.data(), h_codes.size(), stream_);
+        std::fill(acc.begin(), acc.end(), 0.0);
+        std::fill(cnt.begin(), cnt.end(), 0);
+        for (int64_t i = 0; i < ns; i++) {
+            for (int m = 0; m < M_; m++) {
+                const size_t slot = (size_t)m * 256 + h_codes[(size_t)i * M_ + m];
+                cnt[slot]++;
+                for (int t = 0; t < dsub_; t++) {
+                    acc[slot * dsub_ + t] += sample[(size_t)i * d_ + m * dsub_ + t];
+                }
+            }
+        }
+        for (int m = 0; m < M_; m++) {
+            std::vector<float> sub(cb.begin() + (size_t)m * 256 * dsub_, cb.begin() + (size_t)(m + 1) * 256 * dsub_);
+            std::vector<int64_t> sc(cnt.begin() + (size_t)m * 256, cnt.begin() + (size_t)(m + 1) * 256);
+            for (int k = 0; k < 256; k++) {
+                if (sc[(size_t)k] > 0) {
+                    for (int t = 0; t < dsub_; t++) {
+                        sub[(size_t)k * dsub_ + t] =
+                            (float)(acc[((size_t)m * 256 + k) * dsub_ + t] / (double)sc[(size_t)k]);
+                    }
+                }
+            }
+            split_empty(sub, sc, 256, dsub_);
+            if (cfg_.spherical) {
+                normalise_rows(sub, 256, dsub_);
+            }
+            std::copy(sub.begin(), sub.end(), cb.begin() + (size_t)m * 256 * dsub_);
+        }
+    }
+    upload_trained(nullptr, cb.data());
+}
+
+}  // namespace ixa

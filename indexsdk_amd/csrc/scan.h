@@ -1,0 +1,42 @@
+// Host launcher of the fused LUT + ADC scan + top-k kernel.
+#pragma once
+#include "common.h"
+
+namespace ixa {
+
+struct ScanParams {
+    // query side
+    const float *queries;      // [nq][d]
+    const int32_t *probes;     // [nq][nprobe] list ids, best first, -1 = none
+    int nprobe;
+    // trained state
+    const float *codebook;     // [M][256][dsub]
+    const float *cb_norms;     // [M][256]  |codeword|^2, left-to-right fp32
+    int d, M, dsub, metric;
+    int lut_fp16;              // 1: LUT entries rounded to IEEE half (RNE), accumulated in fp32
+    // inverted lists (arena)
+    const uint8_t *codes;
+    const int64_t *ids;
+    const int64_t *list_off;   // first slot of each list
+    const int32_t *list_len;   // valid entries of each list
+    int code_layout;           // 0 = row, 1 = rot32
+    // selection
+    int k;
+    int nsplit;                // workgroups per query; > 1 needs `partial`
+    unsigned long long *partial;  // [nq][nsplit][k] keys
+    float *out_dist;           // [nq][k]
+    int64_t *out_labels;       // [nq][k]
+    // filled by plan_scan()
+    int cap, merge_n, off_query, off_pools, off_merge, off_misc;
+};
+
+// Computes the LDS plan of a launch; returns the dynamic LDS bytes it needs.
+size_t plan_scan(ScanParams &p);
+
+void launch_scan(ScanParams p, int64_t nq, hipStream_t s);
+
+// *out += sum over probes of list_len[probe]  (probe < 0 contributes nothing).
+void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, unsigned long long *out,
+                          hipStream_t s);
+
+}  // namespace ixa

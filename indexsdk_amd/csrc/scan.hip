@@ -1,0 +1,334 @@
+// Stages 2-4 of IVFPQ search fused into one kernel: per-query PQ lookup table built straight into
+// LDS, ADC scan of the probed inverted lists, wavefront-level top-k, workgroup merge.
+//
+// Replaces, for one GPU, the reference's L2 and L3 levels
+// (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2151, 2166-2349):
+//   op AscendcIvfpqSubspaceDistance  (FR/ops/ascendc/op_kernel/ascendc_ivfpq_subspace_distance.cpp:419-463)
+//   op AscendcIvfpqSearchDistanceL2  (FR/ops/ascendc/op_kernel/ascendc_ivfpq_search_distance_topk.h:39-93, 556-810)
+//   op TopkIvfpqL3                   (FR/ops/cpukernel/impl/topk_ivfpq_l3_cpu_kernel.cpp:176-250)
+// The reference round-trips the LUT and a [B,128,262144] distance scratch through global memory and
+// selects a fixed top-320; here the LUT never leaves LDS, no distance is ever written to HBM and
+// the selection is exactly top-k.
+//
+// Layout of one inverted list in the code arena: list l owns slots [list_off[l], list_off[l] +
+// roundup64(list_len[l])); slot s holds M code bytes at codes + s*M and its id at ids[s].
+// Code layout 0 ("row"): byte j of a slot is sub-quantizer j.
+// Code layout 1 ("rot32", M % 32 == 0): byte j of the slot at list position p holds sub-quantizer
+//   32*(j/32) + ((j + p) % 32).  With the LUT stored k-major (word k*M + m) the 32 lanes of a half
+//   wavefront then read 32 different sub-quantizers, i.e. 32 different LDS banks, at every step,
+//   whatever their code values are.
+#include "scan.h"
+
+#include <hip/hip_fp16.h>
+
+#include "topk.h"
+
+namespace ixa {
+
+template <typename T>
+__device__ __forceinline__ T to_lut(float v);
+template <>
+__device__ __forceinline__ float to_lut<float>(float v)
+{
+    return v;
+}
+template <>
+__device__ __forceinline__ __half to_lut<__half>(float v)
+{
+    return __float2half_rn(v);
+}
+__device__ __forceinline__ float from_lut(float v) { return v; }
+__device__ __forceinline__ float from_lut(__half v) { return __half2float(v); }
+
+// MT > 0: compile-time number of sub-quantizers; MT == 0: run-time p.M with byte loads.
+template <int MT, typename LutT, int LAYOUT>
+__global__ __launch_bounds__(256) void ivfpq_scan_kernel(ScanParams p)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int M = MT > 0 ? MT : p.M;
+    LutT *lut = reinterpret_cast<LutT *>(smem_raw);
+    float *qs = reinterpret_cast<float *>(smem_raw + p.off_query);
+    key_t *pools = reinterpret_cast<key_t *>(smem_raw + p.off_pools);
+    key_t *merge = reinterpret_cast<key_t *>(smem_raw + p.off_merge);
+    float *bounds = reinterpret_cast<float *>(smem_raw + p.off_misc);
+    int *counts = reinterpret_cast<int *>(bounds + 4);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t q = blockIdx.x / p.nsplit;
+    const int split = blockIdx.x % p.nsplit;
+
+    // ---- stage 2: LUT into LDS.  Lane t owns codeword k = t of every sub-quantizer.
+    for (int j = tid; j < p.d; j += 256) {
+        qs[j] = p.queries[q * p.d + j];
+    }
+    if (tid < 4) {
+        bounds[tid] = __builtin_inff();
+    }
+    __syncthreads();
+    {
+        const int dsub = p.dsub;
+        for (int m = 0; m < M; m++) {
+            const float *qm = qs + m * dsub;
+            const float *cw = p.codebook + ((int64_t)m * 256 + tid) * dsub;
+            float ip = 0.f, qn = 0.f;
+            for (int t = 0; t < dsub; t++) {
+                float qv = qm[t];
+                ip = __fadd_rn(ip, __fmul_rn(qv, cw[t]));
+                qn = __fadd_rn(qn, __fmul_rn(qv, qv));
+            }
+            float v;
+            if (p.metric == kMetricL2) {
+                v = __fadd_rn(__fadd_rn(p.cb_norms[m * 256 + tid], qn), __fmul_rn(ip, -2.0f));
+            } else {
+                v = -ip;  // minimise the negated inner product
+            }
+            const int slot = LAYOUT == 1 ? tid * M + m : m * 256 + tid;
+            lut[slot] = to_lut<LutT>(v);
+        }
+    }
+    __syncthreads();
+
+    // ---- stages 3 + 4: scan the probed lists; each wavefront takes every 4th 64-code group.
+    WavePool pool;
+    pool.init(pools + wave * p.cap, p.cap, p.k);
+    const int l32 = lane & 31;
+    for (int r = split; r < p.nprobe; r += p.nsplit) {
+        const int l = p.probes[q * p.nprobe + r];
+        if (l < 0) {
+            continue;
+        }
+        const int len = p.list_len[l];
+        const int64_t off = p.list_off[l];
+        for (int base = wave * 64; base < len; base += 256) {
+            const int pos = base + lane;
+            const int64_t slot = off + pos;
+            const uint8_t *cp = p.codes + slot * M;
+            float s = 0.f;
+            if (MT == 0) {
+                for (int m = 0; m < M; m++) {
+                    s = __fadd_rn(s, from_lut(lut[m * 256 + cp[m]]));
+                }
+            } else {
+                constexpr int NW = MT > 0 ? (MT + 3) / 4 : 1;
+                uint32_t w[NW];
+                if (MT % 16 == 0) {
+#pragma unroll
+                    for (int v = 0; v < MT / 16; v++) {
+                        uint4 u = reinterpret_cast<const uint4 *>(cp)[v];
+                        w[4 * v + 0] = u.x;
+                        w[4 * v + 1] = u.y;
+                        w[4 * v + 2] = u.z;
+                        w[4 * v + 3] = u.w;
+                    }
+                } else if (MT % 8 == 0) {
+#pragma unroll
+                    for (int v = 0; v < MT / 8; v++) {
+                        uint2 u = reinterpret_cast<const uint2 *>(cp)[v];
+                        w[2 * v + 0] = u.x;
+                        w[2 * v + 1] = u.y;
+                    }
+                } else if (MT % 4 == 0) {
+#pragma unroll
+                    for (int v = 0; v < MT / 4; v++) {
+                        w[v] = reinterpret_cast<const uint32_t *>(cp)[v];
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < NW; v++) {
+                        w[v] = 0;
+                    }
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        w[m >> 2] |= (uint32_t)cp[m] << (8 * (m & 3));
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    const uint32_t code = (w[m >> 2] >> (8 * (m & 3))) & 0xffu;
+                    if (LAYOUT == 1) {
+                        const int mm = (m & ~31) | ((m + l32) & 31);
+                        s = __fadd_rn(s, from_lut(lut[code * MT + mm]));
+                    } else {
+                        s = __fadd_rn(s, from_lut(lut[m * 256 + code]));
+                    }
+                }
+            }
+            const bool compacted = pool.push(pos < len && s <= pool.bound, s, (uint32_t)slot, lane);
+            if (compacted) {
+                if (lane == 0) {
+                    bounds[wave] = pool.bound;
+                }
+            }
+        }
+        // adopt the tightest bound any wavefront of this workgroup has published
+        float b = fminf(fminf(bounds[0], bounds[1]), fminf(bounds[2], bounds[3]));
+        pool.bound = b < pool.bound ? b : pool.bound;
+    }
+    pool.compact(lane);
+    if (lane == 0) {
+        counts[wave] = pool.count;
+    }
+    __syncthreads();  // everyone is done with the LUT: its space may now hold the merge array
+
+    for (int i = tid; i < p.merge_n; i += 256) {
+        int w = i / p.k, r = i - w * p.k;
+        merge[i] = (w < 4 && r < counts[w]) ? pools[w * p.cap + r] : kEmptyKey;
+    }
+    block_bitonic_sort(merge, p.merge_n, tid, 256);
+
+    if (p.nsplit > 1) {
+        key_t *dst = p.partial + ((int64_t)q * p.nsplit + split) * p.k;
+        for (int i = tid; i < p.k; i += 256) {
+            dst[i] = merge[i];
+        }
+        return;
+    }
+    for (int i = tid; i < p.k; i += 256) {
+        const key_t kk = merge[i];
+        const bool ok = kk != kEmptyKey;
+        const float v = key_score(kk);
+        const float pad = p.metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+        p.out_dist[q * p.k + i] = ok ? (p.metric == kMetricL2 ? v : -v) : pad;
+        p.out_labels[q * p.k + i] = ok ? p.ids[key_index(kk)] : -1;
+    }
+}
+
+// Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3).
+__global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restrict__ partial, int nsplit, int k,
+                                                          int merge_n, int metric, const int64_t *__restrict__ ids,
+                                                          float *__restrict__ out_dist,
+                                                          int64_t *__restrict__ out_labels)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    key_t *merge = reinterpret_cast<key_t *>(smem_raw);
+    const int tid = threadIdx.x;
+    const int64_t q = blockIdx.x;
+    const int total = nsplit * k;
+    for (int i = tid; i < merge_n; i += 256) {
+        merge[i] = i < total ? partial[q * total + i] : kEmptyKey;
+    }
+    block_bitonic_sort(merge, merge_n, tid, 256);
+    for (int i = tid; i < k; i += 256) {
+        const key_t kk = merge[i];
+        const bool ok = kk != kEmptyKey;
+        const float v = key_score(kk);
+        const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+        out_dist[q * k + i] = ok ? (metric == kMetricL2 ? v : -v) : pad;
+        out_labels[q * k + i] = ok ? ids[key_index(kk)] : -1;
+    }
+}
+
+// Sum of the lengths of all probed lists (the number of codes the scan visits).
+__global__ __launch_bounds__(256) void count_scanned_kernel(const int32_t *__restrict__ probes, int64_t n,
+                                                            const int32_t *__restrict__ list_len,
+                                                            unsigned long long *__restrict__ out)
+{
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    unsigned long long v = 0;
+    if (i < n) {
+        int l = probes[i];
+        v = l >= 0 ? (unsigned long long)list_len[l] : 0ull;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        v += __shfl_down(v, o);
+    }
+    if ((threadIdx.x & 63) == 0 && v) {
+        atomicAdd(out, v);
+    }
+}
+
+void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, unsigned long long *out,
+                          hipStream_t s)
+{
+    if (n == 0) {
+        return;
+    }
+    hipLaunchKernelGGL(count_scanned_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, probes, n, list_len,
+                       out);
+}
+
+template <int MT, typename LutT, int LAYOUT>
+static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
+{
+    auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT>;
+    if (smem > 48 * 1024) {
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(256), smem, s, p);
+}
+
+template <typename LutT>
+static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
+{
+    if (p.code_layout == 1) {
+        switch (p.M) {
+            case 32: return launch_one<32, LutT, 1>(p, nq, smem, s);
+            case 64: return launch_one<64, LutT, 1>(p, nq, smem, s);
+            case 96: return launch_one<96, LutT, 1>(p, nq, smem, s);
+            default: fail(kErrInner, "rot32 code layout needs M in {32, 64, 96}, got %d", p.M);
+        }
+    }
+    switch (p.M) {
+        case 4: return launch_one<4, LutT, 0>(p, nq, smem, s);
+        case 8: return launch_one<8, LutT, 0>(p, nq, smem, s);
+        case 16: return launch_one<16, LutT, 0>(p, nq, smem, s);
+        case 32: return launch_one<32, LutT, 0>(p, nq, smem, s);
+        case 48: return launch_one<48, LutT, 0>(p, nq, smem, s);
+        case 64: return launch_one<64, LutT, 0>(p, nq, smem, s);
+        case 96: return launch_one<96, LutT, 0>(p, nq, smem, s);
+        default: return launch_one<0, LutT, 0>(p, nq, smem, s);
+    }
+}
+
+size_t plan_scan(ScanParams &p)
+{
+    const size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
+    p.cap = wave_pool_capacity(p.k);
+    p.merge_n = pow2_ceil(4 * p.k);
+    size_t off = round_up((int64_t)lut_bytes, 16);
+    p.off_query = (int)off;
+    off += round_up((int64_t)p.d * 4, 16);
+    p.off_pools = (int)off;
+    off += (size_t)4 * p.cap * sizeof(key_t);
+    const size_t merge_bytes = (size_t)p.merge_n * sizeof(key_t);
+    if (merge_bytes <= (size_t)p.off_pools) {
+        p.off_merge = 0;  // reuse the LUT (+ query) space once the scan is over
+    } else {
+        p.off_merge = (int)off;
+        off += merge_bytes;
+    }
+    p.off_misc = (int)off;
+    off += 64;
+    return off;
+}
+
+void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    const size_t smem = plan_scan(p);
+    IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam,
+                "IVFPQ scan needs %zu bytes of LDS (M=%d, k=%d, %s LUT); the limit is 163840", smem, p.M, p.k,
+                p.lut_fp16 ? "fp16" : "fp32");
+    IXA_REQUIRE(nq * p.nsplit < ((int64_t)1 << 31), kErrInvalidParam, "scan grid too large");
+    if (p.lut_fp16) {
+        dispatch_m<__half>(p, nq, smem, s);
+    } else {
+        dispatch_m<float>(p, nq, smem, s);
+    }
+    if (p.nsplit > 1) {
+        const int merge_n = pow2_ceil(p.nsplit * p.k);
+        const size_t msmem = (size_t)merge_n * sizeof(key_t);
+        IXA_REQUIRE(msmem <= 160 * 1024, kErrInner, "merge of %d x %d candidates exceeds LDS", p.nsplit, p.k);
+        if (msmem > 48 * 1024) {
+            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(ivfpq_merge_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem));
+        }
+        hipLaunchKernelGGL(ivfpq_merge_kernel, dim3((unsigned)nq), dim3(256), msmem, s, p.partial, p.nsplit, p.k,
+                           merge_n, p.metric, p.ids, p.out_dist, p.out_labels);
+    }
+}
+
+}  // namespace ixa

@@ -1,0 +1,191 @@
+"""GPU parity tests of the IVFPQ path: HIP library (through the C ABI) against the CPU oracle.
+
+Bars: coarse assignment, probe lists and PQ codes bit-exact; distances within 1e-4 relative with
+an fp32 LUT (1e-2 with an fp16 LUT); top-k ids identical except where oracle distances tie within
+that tolerance.
+"""
+import numpy as np
+import pytest
+
+from tests.parity import FLT_MAX, assert_topk_parity
+
+pytestmark = pytest.mark.gpu
+
+TOL_FP32 = 1e-4
+TOL_FP16 = 1e-2
+
+
+@pytest.fixture(scope="module")
+def ix():
+    import indexsdk_amd
+    return indexsdk_amd
+
+
+def make_data(seed, n, nq, d, comp=32, sigma=0.3):
+    rng = np.random.default_rng(seed)
+    centres = rng.standard_normal((comp, d)).astype(np.float32)
+    x = (centres[rng.integers(0, comp, n)] + sigma * rng.standard_normal((n, d))).astype(np.float32)
+    q = (centres[rng.integers(0, comp, nq)] + sigma * rng.standard_normal((nq, d))).astype(np.float32)
+    return x, q
+
+
+def build_pair(ix, oracle, seed, n, nq, d, nlist, M, metric, layout=-1, lut_fp16=0, niter=4):
+    """Oracle-trained quantizers injected into both sides; base added through the GPU add path."""
+    x, q = make_data(seed, n, nq, d)
+    if metric == ix.METRIC_INNER_PRODUCT:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    cent, _ = oracle.kmeans(x[: min(n, 20 * nlist)], nlist, niter=niter, seed=seed)
+    cb = oracle.train_pq(x[: min(n, 5000)], M, niter=niter, seed=seed)
+    ids = np.random.default_rng(seed + 1).permutation(10 * n)[:n].astype(np.int64)
+    ref = oracle.CsrIndex.build(d, M, metric, cent, cb, x, ids)
+    cfg = ix.AscendIndexIVFPQConfig(code_layout=layout, lut_fp16=lut_fp16)
+    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, cfg)
+    gpu.set_trained(cent, cb)
+    gpu.add_with_ids(x, ids)
+    return gpu, ref, x, q, ids
+
+
+def test_assign_encode_lists_bit_exact(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 21, 20000, 10, 128, 64, 16, ix.METRIC_L2)
+    assert gpu.ntotal == 20000
+    assert np.array_equal(gpu.assign(x[:3000]), oracle.assign(x[:3000], ref.cent))
+    assert np.array_equal(gpu.encode(x[:3000]), oracle.pq_encode(x[:3000], ref.codebook))
+    total = 0
+    for l in range(ref.nlist):
+        codes, lid = gpu.getListCodesAndIds(l)
+        b, e = ref.list_off[l], ref.list_off[l + 1]
+        assert gpu.getListLength(l) == e - b
+        assert np.array_equal(lid, ref.ids[b:e]), f"list {l}: ids / insertion order differ"
+        assert np.array_equal(codes, ref.codes[b:e]), f"list {l}: codes differ"
+        total += e - b
+    assert total == 20000
+
+
+@pytest.mark.parametrize("metric_name", ["L2", "IP"])
+@pytest.mark.parametrize("nprobe", [1, 8, 64])
+def test_coarse_probe_bit_exact(ix, oracle, metric_name, nprobe):
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 22, 6000, 300, 96, 200, 8, metric)
+    gpu.setNumProbes(nprobe)
+    gi, gd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, ref.cent, nprobe, metric)
+    assert np.array_equal(gi, oi)
+    assert np.array_equal(gd.view(np.uint32), od.view(np.uint32))
+
+
+@pytest.mark.parametrize("d,M,nlist,layout", [(128, 16, 64, 0), (128, 32, 64, 0), (128, 32, 64, 1), (96, 48, 32, 0),
+                                              (64, 8, 16, 0), (60, 12, 16, 0), (192, 96, 16, 1), (128, 64, 16, 1)])
+def test_search_l2_fp32(ix, oracle, d, M, nlist, layout):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 23, 12000, 150, d, nlist, M, ix.METRIC_L2, layout=layout)
+    for nprobe, k in ((4, 10), (nlist, 100)):
+        gpu.setNumProbes(nprobe)
+        D, I = gpu.search(q, k)
+        Dr, Ir = ref.search(q, k, nprobe)
+        assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+        if layout == 0:
+            # row layout accumulates m = 0..M-1 like the oracle: distances are bit-identical
+            assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+        assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
+
+
+def test_search_ip_fp16_lut(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 24, 8000, 100, 192, 32, 96, ix.METRIC_INNER_PRODUCT, lut_fp16=1)
+    gpu.setNumProbes(8)
+    D, I = gpu.search(q, 50)
+    Dr, Ir = ref.search(q, 50, 8, lut_fp16=True)
+    assert np.all(np.diff(D, axis=1) <= 0)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP16)
+
+
+def test_search_sentinels_k_larger_than_candidates(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 25, 600, 20, 64, 32, 8, ix.METRIC_L2)
+    gpu.setNumProbes(2)
+    D, I = gpu.search(q, 200)
+    Dr, Ir = ref.search(q, 200, 2)
+    assert (Ir == -1).any()
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    assert np.all(D[I == -1] == FLT_MAX)
+
+
+def test_search_empty_index_and_single_query(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 26, 3000, 5, 64, 16, 8, ix.METRIC_L2)
+    D, I = gpu.search(q[:1], 7)      # one query -> the scan splits the probes over several workgroups
+    Dr, Ir = ref.search(q[:1], 7, gpu.getNumProbes())
+    assert_topk_parity(oracle, ref, q[:1], D, I, Dr, Ir, TOL_FP32)
+    gpu.reset()
+    assert gpu.ntotal == 0 and gpu.is_trained
+    D, I = gpu.search(q, 5)
+    assert np.all(I == -1) and np.all(D == FLT_MAX)
+
+
+def test_large_k(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 27, 30000, 40, 96, 32, 48, ix.METRIC_L2)
+    gpu.setNumProbes(16)
+    D, I = gpu.search(q, 1024)
+    Dr, Ir = ref.search(q, 1024, 16)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+
+
+def test_add_in_two_calls_add_codes_and_remove(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 28, 5000, 30, 64, 16, 32, ix.METRIC_L2)
+    cfg = ix.AscendIndexIVFPQConfig()
+    g2 = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 16, 32, 8, cfg)
+    g2.set_trained(ref.cent, ref.codebook)
+    g2.add_with_ids(x[:2000], ids[:2000])
+    g2.add_with_ids(x[2000:], ids[2000:])
+    for l in range(16):
+        a, b = gpu.getListCodesAndIds(l), g2.getListCodesAndIds(l)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    # addPQCodes path: rebuild a third index from the raw lists
+    g3 = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 16, 32, 8, cfg)
+    g3.set_trained(ref.cent, ref.codebook)
+    for l in range(16):
+        b, e = ref.list_off[l], ref.list_off[l + 1]
+        g3.add_codes(l, ref.codes[b:e], ref.ids[b:e])
+    D, I = gpu.search(q, 20)
+    D3, I3 = g3.search(q, 20)
+    assert np.array_equal(I, I3) and np.array_equal(D, D3)
+    # default ids = ntotal + i
+    g4 = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 16, 32, 8, cfg)
+    g4.set_trained(ref.cent, ref.codebook)
+    g4.add(x[:100])
+    g4.add(x[100:300])
+    got = np.sort(np.concatenate([g4.getListCodesAndIds(l)[1] for l in range(16)]))
+    assert np.array_equal(got, np.arange(300))
+    # remove: survivors keep their order
+    victims = ids[::3]
+    assert gpu.remove_ids(victims) == len(victims)
+    assert gpu.ntotal == 5000 - len(victims)
+    vs = set(victims.tolist())
+    for l in range(16):
+        b, e = ref.list_off[l], ref.list_off[l + 1]
+        keep = np.array([i not in vs for i in ref.ids[b:e]], dtype=bool)
+        codes, lid = gpu.getListCodesAndIds(l)
+        assert np.array_equal(lid, ref.ids[b:e][keep]) and np.array_equal(codes, ref.codes[b:e][keep])
+    D, I = gpu.search(q, 20)
+    assert not (set(I.ravel().tolist()) & vs)
+
+
+def test_train_on_gpu_then_parity_with_oracle_on_same_codebooks(ix, oracle):
+    x, q = make_data(29, 30000, 100, 64)
+    cfg = ix.AscendIndexIVFPQConfig(niter=6)
+    gpu = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 128, 16, 8, cfg)
+    assert not gpu.is_trained
+    with pytest.raises(ix.IndexSdkError, match="not trained"):
+        gpu.add(x[:10])
+    gpu.train(x)
+    assert gpu.is_trained
+    gpu.add(x)
+    cent, cb = gpu.get_trained()
+    ref = oracle.CsrIndex.build(64, 16, ix.METRIC_L2, cent, cb, x)
+    gpu.setNumProbes(16)
+    D, I = gpu.search(q, 10)
+    Dr, Ir = ref.search(q, 10, 16)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    # trained quantizer is usable: self queries come back first (reference ST invariant,
+    # FR/test/ascend/TestAscendIndexIVFPQ.cpp:150-166)
+    D, I = gpu.search(x[:500], 1)
+    assert (I[:, 0] == np.arange(500)).mean() > 0.9
+    lens = np.array([gpu.getListLength(l) for l in range(128)])
+    assert lens.sum() == 30000 and (lens > 0).mean() > 0.9
