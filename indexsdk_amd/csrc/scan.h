@@ -27,7 +27,7 @@ struct ScanParams {
     float *out_dist;           // [nq][k]
     int64_t *out_labels;       // [nq][k]
     // filled by plan_scan()
-    int cap, merge_n, off_query, off_pools, off_merge, off_misc;
+    int waves, cap, merge_n, table_n, off_query, off_pools, off_merge, off_table, off_misc;
 };
 
 // Computes the LDS plan of a launch; returns the dynamic LDS bytes it needs.

@@ -40,36 +40,76 @@ __device__ __forceinline__ __half to_lut<__half>(float v)
 __device__ __forceinline__ float from_lut(float v) { return v; }
 __device__ __forceinline__ float from_lut(__half v) { return __half2float(v); }
 
+// One 64-code group of a probed list, as a wavefront sees it.
+struct GroupRef {
+    uint32_t slot;  // arena slot of this lane's code
+    bool valid;     // lane is inside the list
+};
+
 // MT > 0: compile-time number of sub-quantizers; MT == 0: run-time p.M with byte loads.
-template <int MT, typename LutT, int LAYOUT>
-__global__ __launch_bounds__(256) void ivfpq_scan_kernel(ScanParams p)
+// W: wavefronts per workgroup (the workgroup serves one query, or one split of a query).
+template <int MT, typename LutT, int LAYOUT, int W>
+__global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int NT = W * 64;
     const int M = MT > 0 ? MT : p.M;
     LutT *lut = reinterpret_cast<LutT *>(smem_raw);
     float *qs = reinterpret_cast<float *>(smem_raw + p.off_query);
     key_t *pools = reinterpret_cast<key_t *>(smem_raw + p.off_pools);
     key_t *merge = reinterpret_cast<key_t *>(smem_raw + p.off_merge);
-    float *bounds = reinterpret_cast<float *>(smem_raw + p.off_misc);
-    int *counts = reinterpret_cast<int *>(bounds + 4);
+    float *bounds = reinterpret_cast<float *>(smem_raw + p.off_misc);   // W
+    int *counts = reinterpret_cast<int *>(bounds + W);                  // W
+    uint32_t *t_off = reinterpret_cast<uint32_t *>(smem_raw + p.off_table);  // first slot of local list i
+    int *t_len = reinterpret_cast<int *>(t_off + p.table_n);                  // its length
+    int *t_gend = t_len + p.table_n;                                          // groups up to and incl. list i
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t q = blockIdx.x / p.nsplit;
     const int split = blockIdx.x % p.nsplit;
 
-    // ---- stage 2: LUT into LDS.  Lane t owns codeword k = t of every sub-quantizer.
-    for (int j = tid; j < p.d; j += 256) {
+    // ---- list table of this workgroup: local list i = probe rank split + i * nsplit
+    const int nlocal = (p.nprobe - split + p.nsplit - 1) / p.nsplit;
+    for (int j = tid; j < p.d; j += NT) {
         qs[j] = p.queries[q * p.d + j];
     }
-    if (tid < 4) {
+    if (tid < W) {
         bounds[tid] = __builtin_inff();
     }
+    for (int i = tid; i < nlocal; i += NT) {
+        const int l = p.probes[q * p.nprobe + split + i * p.nsplit];
+        const int len = l >= 0 ? p.list_len[l] : 0;
+        t_len[i] = len;
+        t_off[i] = l >= 0 ? (uint32_t)p.list_off[l] : 0u;
+    }
     __syncthreads();
+    if (wave == 0) {
+        // inclusive prefix sum of the group counts, 64 lists at a time
+        int carry = 0;
+        for (int base = 0; base < nlocal; base += 64) {
+            const int i = base + lane;
+            int g = i < nlocal ? (t_len[i] + 63) >> 6 : 0;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                int up = __shfl_up(g, o);
+                if (lane >= o) {
+                    g += up;
+                }
+            }
+            if (i < nlocal) {
+                t_gend[i] = carry + g;
+            }
+            carry += __shfl(g, 63);
+        }
+    }
+
+    // ---- stage 2: LUT into LDS.  Thread t owns codeword k = t % 256 of every (NT/256)-th sub-quantizer.
     {
         const int dsub = p.dsub;
-        for (int m = 0; m < M; m++) {
+        const int kk = tid & 255;
+        for (int m = tid >> 8; m < M; m += NT / 256) {
             const float *qm = qs + m * dsub;
-            const float *cw = p.codebook + ((int64_t)m * 256 + tid) * dsub;
+            const float *cw = p.codebook + ((int64_t)m * 256 + kk) * dsub;
             float ip = 0.f, qn = 0.f;
             for (int t = 0; t < dsub; t++) {
                 float qv = qm[t];
@@ -78,91 +118,139 @@ __global__ __launch_bounds__(256) void ivfpq_scan_kernel(ScanParams p)
             }
             float v;
             if (p.metric == kMetricL2) {
-                v = __fadd_rn(__fadd_rn(p.cb_norms[m * 256 + tid], qn), __fmul_rn(ip, -2.0f));
+                v = __fadd_rn(__fadd_rn(p.cb_norms[m * 256 + kk], qn), __fmul_rn(ip, -2.0f));
             } else {
                 v = -ip;  // minimise the negated inner product
             }
-            const int slot = LAYOUT == 1 ? tid * M + m : m * 256 + tid;
+            const int slot = LAYOUT == 1 ? kk * M + m : m * 256 + kk;
             lut[slot] = to_lut<LutT>(v);
         }
     }
     __syncthreads();
 
-    // ---- stages 3 + 4: scan the probed lists; each wavefront takes every 4th 64-code group.
+    // ---- stages 3 + 4: the probed lists form one sequence of 64-code groups; wavefront w takes
+    // groups w, w + W, ... of that sequence, so the waves stay balanced whatever the list lengths.
     WavePool pool;
     pool.init(pools + wave * p.cap, p.cap, p.k);
     const int l32 = lane & 31;
-    for (int r = split; r < p.nprobe; r += p.nsplit) {
-        const int l = p.probes[q * p.nprobe + r];
-        if (l < 0) {
-            continue;
+    const int total = nlocal > 0 ? t_gend[nlocal - 1] : 0;
+    int li = 0;          // list the current group belongs to (monotone)
+    int gstart = 0;      // first group of that list
+
+    auto locate = [&](int G) -> GroupRef {
+        while (G >= t_gend[li]) {
+            gstart = t_gend[li];
+            li++;
         }
-        const int len = p.list_len[l];
-        const int64_t off = p.list_off[l];
-        for (int base = wave * 64; base < len; base += 256) {
-            const int pos = base + lane;
-            const int64_t slot = off + pos;
-            const uint8_t *cp = p.codes + slot * M;
-            float s = 0.f;
-            if (MT == 0) {
-                for (int m = 0; m < M; m++) {
-                    s = __fadd_rn(s, from_lut(lut[m * 256 + cp[m]]));
-                }
-            } else {
-                constexpr int NW = MT > 0 ? (MT + 3) / 4 : 1;
-                uint32_t w[NW];
-                if (MT % 16 == 0) {
+        const int pos = ((G - gstart) << 6) + lane;
+        GroupRef r;
+        r.slot = t_off[li] + (uint32_t)pos;
+        r.valid = pos < t_len[li];
+        return r;
+    };
+
+    constexpr int NW = MT > 0 ? (MT + 3) / 4 : 1;
+    auto load_codes = [&](uint32_t slot, uint32_t (&w)[NW]) {
+        if (MT == 0) {
+            return;
+        }
+        const uint8_t *cp = p.codes + (int64_t)slot * MT;
+        if (MT % 16 == 0) {
 #pragma unroll
-                    for (int v = 0; v < MT / 16; v++) {
-                        uint4 u = reinterpret_cast<const uint4 *>(cp)[v];
-                        w[4 * v + 0] = u.x;
-                        w[4 * v + 1] = u.y;
-                        w[4 * v + 2] = u.z;
-                        w[4 * v + 3] = u.w;
-                    }
-                } else if (MT % 8 == 0) {
-#pragma unroll
-                    for (int v = 0; v < MT / 8; v++) {
-                        uint2 u = reinterpret_cast<const uint2 *>(cp)[v];
-                        w[2 * v + 0] = u.x;
-                        w[2 * v + 1] = u.y;
-                    }
-                } else if (MT % 4 == 0) {
-#pragma unroll
-                    for (int v = 0; v < MT / 4; v++) {
-                        w[v] = reinterpret_cast<const uint32_t *>(cp)[v];
-                    }
-                } else {
-#pragma unroll
-                    for (int v = 0; v < NW; v++) {
-                        w[v] = 0;
-                    }
-#pragma unroll
-                    for (int m = 0; m < MT; m++) {
-                        w[m >> 2] |= (uint32_t)cp[m] << (8 * (m & 3));
-                    }
-                }
-#pragma unroll
-                for (int m = 0; m < MT; m++) {
-                    const uint32_t code = (w[m >> 2] >> (8 * (m & 3))) & 0xffu;
-                    if (LAYOUT == 1) {
-                        const int mm = (m & ~31) | ((m + l32) & 31);
-                        s = __fadd_rn(s, from_lut(lut[code * MT + mm]));
-                    } else {
-                        s = __fadd_rn(s, from_lut(lut[m * 256 + code]));
-                    }
-                }
+            for (int v = 0; v < MT / 16; v++) {
+                uint4 u = reinterpret_cast<const uint4 *>(cp)[v];
+                w[(4 * v + 0) % NW] = u.x;
+                w[(4 * v + 1) % NW] = u.y;
+                w[(4 * v + 2) % NW] = u.z;
+                w[(4 * v + 3) % NW] = u.w;
             }
-            const bool compacted = pool.push(pos < len && s <= pool.bound, s, (uint32_t)slot, lane);
+        } else if (MT % 8 == 0) {
+#pragma unroll
+            for (int v = 0; v < MT / 8; v++) {
+                uint2 u = reinterpret_cast<const uint2 *>(cp)[v];
+                w[(2 * v + 0) % NW] = u.x;
+                w[(2 * v + 1) % NW] = u.y;
+            }
+        } else if (MT % 4 == 0) {
+#pragma unroll
+            for (int v = 0; v < MT / 4; v++) {
+                w[v % NW] = reinterpret_cast<const uint32_t *>(cp)[v];
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < NW; v++) {
+                w[v] = 0;
+            }
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                w[(m >> 2) % NW] |= (uint32_t)cp[m] << (8 * (m & 3));
+            }
+        }
+    };
+
+    auto adc = [&](uint32_t slot, const uint32_t (&w)[NW]) -> float {
+        if (MT == 0) {
+            const uint8_t *cp = p.codes + (int64_t)slot * M;
+            float s = 0.f;
+            for (int m = 0; m < M; m++) {
+                s = __fadd_rn(s, from_lut(lut[m * 256 + cp[m]]));
+            }
+            return s;
+        }
+        if (LAYOUT == 1) {
+            // any association is within tolerance: four independent partial sums
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const uint32_t code = (w[(m >> 2) % NW] >> (8 * (m & 3))) & 0xffu;
+                const int mm = (m & ~31) | ((m + l32) & 31);
+                acc[m & 3] += from_lut(lut[code * MT + mm]);
+            }
+            return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        }
+        // row layout: m = 0..M-1 in sequence, the accumulation order of the reference's scalar path
+        float s = 0.f;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const uint32_t code = (w[(m >> 2) % NW] >> (8 * (m & 3))) & 0xffu;
+            s = __fadd_rn(s, from_lut(lut[m * 256 + code]));
+        }
+        return s;
+    };
+
+    if (wave < total) {
+        uint32_t wc[NW], wn[NW];
+        GroupRef cur = locate(wave);
+        load_codes(cur.slot, wc);
+        for (int G = wave; G < total; G += W) {
+            GroupRef nxt = cur;
+            const bool more = G + W < total;
+            if (more) {
+                nxt = locate(G + W);
+                load_codes(nxt.slot, wn);   // in flight while the current group is evaluated
+            }
+            const float s = adc(cur.slot, wc);
+            const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane);
             if (compacted) {
                 if (lane == 0) {
                     bounds[wave] = pool.bound;
                 }
             }
+            if (compacted || (G & (16 * W - 1)) < W) {
+                // adopt the tightest bound any wavefront of this workgroup has published
+                float b = bounds[0];
+#pragma unroll
+                for (int i = 1; i < W; i++) {
+                    b = fminf(b, bounds[i]);
+                }
+                pool.bound = b < pool.bound ? b : pool.bound;
+            }
+            cur = nxt;
+#pragma unroll
+            for (int v = 0; v < NW; v++) {
+                wc[v] = wn[v];
+            }
         }
-        // adopt the tightest bound any wavefront of this workgroup has published
-        float b = fminf(fminf(bounds[0], bounds[1]), fminf(bounds[2], bounds[3]));
-        pool.bound = b < pool.bound ? b : pool.bound;
     }
     pool.compact(lane);
     if (lane == 0) {
@@ -170,20 +258,20 @@ __global__ __launch_bounds__(256) void ivfpq_scan_kernel(ScanParams p)
     }
     __syncthreads();  // everyone is done with the LUT: its space may now hold the merge array
 
-    for (int i = tid; i < p.merge_n; i += 256) {
+    for (int i = tid; i < p.merge_n; i += NT) {
         int w = i / p.k, r = i - w * p.k;
-        merge[i] = (w < 4 && r < counts[w]) ? pools[w * p.cap + r] : kEmptyKey;
+        merge[i] = (w < W && r < counts[w]) ? pools[w * p.cap + r] : kEmptyKey;
     }
-    block_bitonic_sort(merge, p.merge_n, tid, 256);
+    block_bitonic_sort(merge, p.merge_n, tid, NT);
 
     if (p.nsplit > 1) {
         key_t *dst = p.partial + ((int64_t)q * p.nsplit + split) * p.k;
-        for (int i = tid; i < p.k; i += 256) {
+        for (int i = tid; i < p.k; i += NT) {
             dst[i] = merge[i];
         }
         return;
     }
-    for (int i = tid; i < p.k; i += 256) {
+    for (int i = tid; i < p.k; i += NT) {
         const key_t kk = merge[i];
         const bool ok = kk != kEmptyKey;
         const float v = key_score(kk);
@@ -250,12 +338,21 @@ void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_
 template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
-    auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT>;
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
+    if (p.waves == 8) {
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8>;
+        if (smem > 48 * 1024) {
+            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(512), smem, s, p);
+    } else {
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4>;
+        if (smem > 48 * 1024) {
+            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(256), smem, s, p);
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(256), smem, s, p);
 }
 
 template <typename LutT>
@@ -281,16 +378,18 @@ static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
     }
 }
 
-size_t plan_scan(ScanParams &p)
+static size_t plan_with_waves(ScanParams &p, int waves)
 {
     const size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
+    p.waves = waves;
     p.cap = wave_pool_capacity(p.k);
-    p.merge_n = pow2_ceil(4 * p.k);
+    p.merge_n = pow2_ceil(waves * p.k);
+    p.table_n = (p.nprobe + p.nsplit - 1) / p.nsplit;
     size_t off = round_up((int64_t)lut_bytes, 16);
     p.off_query = (int)off;
     off += round_up((int64_t)p.d * 4, 16);
     p.off_pools = (int)off;
-    off += (size_t)4 * p.cap * sizeof(key_t);
+    off += (size_t)waves * p.cap * sizeof(key_t);
     const size_t merge_bytes = (size_t)p.merge_n * sizeof(key_t);
     if (merge_bytes <= (size_t)p.off_pools) {
         p.off_merge = 0;  // reuse the LUT (+ query) space once the scan is over
@@ -298,9 +397,22 @@ size_t plan_scan(ScanParams &p)
         p.off_merge = (int)off;
         off += merge_bytes;
     }
+    p.off_table = (int)off;
+    off += round_up((int64_t)p.table_n * 12, 16);
     p.off_misc = (int)off;
-    off += 64;
+    off += 128;
     return off;
+}
+
+// Eight wavefronts per workgroup when three such workgroups still fit the 160 KB of a CU,
+// otherwise four.
+size_t plan_scan(ScanParams &p)
+{
+    size_t smem = plan_with_waves(p, 8);
+    if (smem * 3 > 160 * 1024) {
+        smem = plan_with_waves(p, 4);
+    }
+    return smem;
 }
 
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
