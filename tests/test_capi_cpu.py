@@ -1,0 +1,102 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the header declares,
+validates constructor parameters with the reference's messages, and refuses to run without a GPU
+(no CPU fallback).  No compute entry point is called here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "indexsdk_amd.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:ixa|ivfpq|flat|flat_i8)_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from indexsdk_amd import _capi
+    if not os.path.exists(_capi.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    _capi.load()
+    return _capi
+
+
+def test_header_declares_the_survey_boundary():
+    names = declared_functions()
+    for need in ["ivfpq_create", "ivfpq_destroy", "ivfpq_train", "ivfpq_set_trained", "ivfpq_add_with_ids",
+                 "ivfpq_add_codes", "ivfpq_set_nprobe", "ivfpq_get_nprobe", "ivfpq_search", "ivfpq_assign",
+                 "ivfpq_coarse_probe", "ivfpq_list_length", "ivfpq_get_list", "ivfpq_remove_ids", "ivfpq_reset",
+                 "ixa_last_error"]:
+        assert need in names
+
+
+def test_library_exports_every_declared_symbol(capi):
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    missing = [n for n in declared_functions() if not hasattr(lib, n)]
+    assert not missing, f"declared in the header but not exported: {missing}"
+    unbound = [n for n in declared_functions() if n not in capi.exported_names()]
+    assert not unbound, f"declared in the header but not bound in _capi.py: {unbound}"
+
+
+def _create(capi, d, metric, nlist, M, nbits, strict=0):
+    lib = capi.load()
+    cfg = capi.IvfpqConfig()
+    lib.ivfpq_config_default(ctypes.byref(cfg))
+    cfg.strict_reference_params = strict
+    h = ctypes.c_void_p()
+    rc = lib.ivfpq_create(d, metric, nlist, M, nbits, ctypes.byref(cfg), ctypes.byref(h))
+    return rc, lib.ixa_last_error().decode(), h
+
+
+# FR/ut/TestAscendIndexUTIVFPQ.cpp:77-184: constructor validation messages
+@pytest.mark.parametrize("args,strict,needle", [
+    ((64, 1, 1024, 4, 8), 1, "Unsupported dims"),
+    ((128, 1, 512, 4, 8), 1, "Unsupported nlists"),
+    ((128, 1, 262144, 3, 8), 1, "Unsupported msubs"),
+    ((128, 1, 524288, 3, 8), 1, "Unsupported msubs"),
+    ((128, 1, 1024, 4, 4), 1, "Unsupported nbits"),
+    ((128, 7, 1024, 4, 8), 1, "Unsupported metric type"),
+    ((128, 1, 1024, 3, 8), 0, "Unsupported msubs"),       # 3 does not divide 128
+    ((0, 1, 1024, 4, 8), 0, "Unsupported dims"),
+    ((128, 1, 0, 4, 8), 0, "Unsupported nlists"),
+])
+def test_constructor_rejects_bad_parameters(capi, args, strict, needle):
+    rc, msg, h = _create(capi, *args, strict=strict)
+    assert rc == 2001 and needle in msg and not h.value
+
+
+def test_large_nlist_passes_the_nlist_check(capi):
+    # FR/ut/TestAscendIndexUTIVFPQ.cpp:122-145
+    for nlist in (262144, 524288):
+        rc, msg, _ = _create(capi, 128, 1, nlist, 3, 8, strict=1)
+        assert "Unsupported nlists" not in msg and "Unsupported msubs" in msg
+
+
+def test_null_handle_and_null_out_are_errors_not_crashes(capi):
+    lib = capi.load()
+    assert lib.ivfpq_search(None, 1, None, 1, None, None) == 2001
+    assert "nullptr" in lib.ixa_last_error().decode()
+    assert lib.ivfpq_create(128, 1, 1024, 4, 8, None, None) == 2001
+    assert lib.ivfpq_destroy(None) == 0
+
+
+def test_no_cpu_fallback(capi):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    rc, msg, h = _create(capi, 128, 1, 1024, 4, 8)
+    assert rc == 2016 and "no CPU path" in msg and not h.value
+
+
+def test_product_never_imports_the_oracle():
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "indexsdk_amd")):
+        for f in files:
+            if f.endswith((".py", ".h", ".hip", ".cpp", ".sh")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"
