@@ -145,6 +145,59 @@ typedef struct ivfpq_search_stats {
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 
+/* ---------------------------------------------------------------------------------------------
+ * Flat (brute force): the coarse stage in isolation
+ * ------------------------------------------------------------------------------------------- */
+
+typedef struct flat_index flat_index_t;       /* fp32 vectors, L2 or inner product */
+typedef struct flat_i8_index flat_i8_index_t; /* int8 vectors, exact int32 L2 */
+
+typedef struct flat_search_stats {
+    double ms_score;       /* fp32: all score + selection launches of the last search */
+    double ms_select;      /* fp32: exact refine + label mapping */
+    double ms_total;
+    double score_launches; /* number of (query block, base chunk) score launches */
+} flat_search_stats_t;
+
+/* AscendIndexFlat(dims, metric, config)  FR/ascend/AscendIndexFlat.h:48-90.  scratch_bytes bounds the
+ * score scratch in HBM (the role of config.resourceSize); 0 = default (1 GiB).
+ * Distances are fp32 in the canonical expanded form (the reference returns fp16-rounded values:
+ * FR/ascend/impl/AscendIndexFlatImpl.cpp:444-446). */
+int flat_create(int d, int metric, int64_t scratch_bytes, flat_index_t **out);
+int flat_destroy(flat_index_t *h);
+/* AscendIndex::add / add_with_ids  FR/ascend/AscendIndex.h:66-71; ids == NULL numbers from ntotal. */
+int flat_add_with_ids(flat_index_t *h, int64_t n, const float *x, const int64_t *ids);
+int flat_add_with_ids_device(flat_index_t *h, int64_t n, const float *x_dev, const int64_t *ids_dev);
+/* AscendIndex::search  FR/ascend/AscendIndex.h:79-80 -> IndexFlatL2Aicpu::searchImpl
+ * (FR/ascendhost/src/index/IndexFlatL2Aicpu.cpp:157-306). */
+int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
+int flat_search_device(flat_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
+                       int64_t *labels_dev);
+/* AscendIndexFlat::getBase / getBaseSize  FR/ascend/AscendIndexFlat.h; rows [offset, offset + n). */
+int flat_get_base(const flat_index_t *h, int64_t offset, int64_t n, float *out);
+int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out);
+int flat_ntotal(const flat_index_t *h, int64_t *out);
+int flat_reset(flat_index_t *h);
+int flat_last_search_stats(const flat_index_t *h, flat_search_stats_t *out);
+
+/* AscendIndexInt8Flat(dims, metric, config)  FR/ascend/AscendIndexInt8.h:53-96 (L2 only here).
+ * Distances are the exact int32 values |q|^2 + |b|^2 - 2 q.b; the reference multiplies by
+ * 0.01 / min(d/64, max(d/128 + 1, 4)) and rounds to fp16
+ * (FR/ops/ascendc/op_kernel/ascendc_dist_int8_flat_l2.cpp:201-203, 491-500), which is not done here.
+ * Ties on distance resolve to the vector added first. */
+int flat_i8_create(int d, int metric, int64_t scratch_bytes, flat_i8_index_t **out);
+int flat_i8_destroy(flat_i8_index_t *h);
+int flat_i8_add_with_ids(flat_i8_index_t *h, int64_t n, const int8_t *x, const int64_t *ids);
+int flat_i8_add_with_ids_device(flat_i8_index_t *h, int64_t n, const int8_t *x_dev, const int64_t *ids_dev);
+/* AscendIndexInt8::search(n, const int8_t *x, k, distances, labels)  FR/ascend/AscendIndexInt8.h:70-72 */
+int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances, int64_t *labels);
+int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x_dev, int64_t k, int32_t *distances_dev,
+                          int64_t *labels_dev);
+int flat_i8_get_base(const flat_i8_index_t *h, int64_t offset, int64_t n, int8_t *out);
+int flat_i8_ntotal(const flat_i8_index_t *h, int64_t *out);
+int flat_i8_reset(flat_i8_index_t *h);
+int flat_i8_last_search_stats(const flat_i8_index_t *h, flat_search_stats_t *out);
+
 #ifdef __cplusplus
 }
 #endif

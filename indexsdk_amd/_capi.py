@@ -75,6 +75,23 @@ _SIGNATURES = {
     "ivfpq_last_search_stats": (ctypes.c_int, [_H, ctypes.POINTER(IvfpqSearchStats)]),
 }
 
+for _pfx, _dist in (("flat", ctypes.c_void_p), ("flat_i8", ctypes.c_void_p)):
+    _SIGNATURES.update({
+        f"{_pfx}_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.POINTER(_H)]),
+        f"{_pfx}_destroy": (ctypes.c_int, [_H]),
+        f"{_pfx}_add_with_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+        f"{_pfx}_add_with_ids_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+        f"{_pfx}_search": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, _dist,
+                                          ctypes.c_void_p]),
+        f"{_pfx}_search_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, _dist,
+                                                 ctypes.c_void_p]),
+        f"{_pfx}_get_base": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+        f"{_pfx}_ntotal": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int64)]),
+        f"{_pfx}_reset": (ctypes.c_int, [_H]),
+        f"{_pfx}_last_search_stats": (ctypes.c_int, [_H, ctypes.POINTER(FlatSearchStats)]),
+    })
+_SIGNATURES["flat_get_ids"] = (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p])
+
 _lib = None
 
 

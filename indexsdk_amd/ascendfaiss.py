@@ -173,3 +173,99 @@ class AscendIndexIVFPQ:
         s = _capi.IvfpqSearchStats()
         _capi.check(self._lib.ivfpq_last_search_stats(self._h, ctypes.byref(s)))
         return {n: getattr(s, n) for n, _ in s._fields_}
+
+
+class _FlatCommon:
+    _pfx = None
+    _dtype = None
+
+    def __init__(self, dims, metric=METRIC_L2, scratch_bytes=0):
+        self._lib = _capi.load()
+        self._h = ctypes.c_void_p()
+        self.d, self.metric_type = dims, metric
+        _capi.check(self._fn("create")(dims, metric, scratch_bytes, ctypes.byref(self._h)))
+
+    def _fn(self, name):
+        return getattr(self._lib, f"{self._pfx}_{name}")
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h:
+            self._fn("destroy")(h)
+            self._h = None
+
+    @property
+    def ntotal(self):
+        out = ctypes.c_int64()
+        _capi.check(self._fn("ntotal")(self._h, ctypes.byref(out)))
+        return out.value
+
+    is_trained = True
+
+    def add(self, x):
+        self.add_with_ids(x, None)
+
+    def add_with_ids(self, x, ids):
+        x = _as(x, self._dtype, 2, "x")
+        assert x.shape[1] == self.d
+        idp = None
+        if ids is not None:
+            ids = _as(ids, np.int64, 1, "ids")
+            assert ids.shape[0] == x.shape[0]
+            idp = _ptr(ids)
+        _capi.check(self._fn("add_with_ids")(self._h, x.shape[0], _ptr(x), idp))
+
+    def getBase(self, offset=0, n=None):
+        n = self.ntotal - offset if n is None else n
+        out = np.empty((n, self.d), dtype=self._dtype)
+        _capi.check(self._fn("get_base")(self._h, offset, n, _ptr(out)))
+        return out
+
+    def reset(self):
+        _capi.check(self._fn("reset")(self._h))
+
+    def last_search_stats(self):
+        s = _capi.FlatSearchStats()
+        _capi.check(self._fn("last_search_stats")(self._h, ctypes.byref(s)))
+        return {n: getattr(s, n) for n, _ in s._fields_}
+
+
+class AscendIndexFlat(_FlatCommon):
+    """AscendIndexFlat(dims, metric, config) -- FR/ascend/AscendIndexFlat.h:48-90; fp32 distances."""
+    _pfx = "flat"
+    _dtype = np.float32
+
+    def search(self, x, k):
+        x = _as(x, np.float32, 2, "x")
+        assert x.shape[1] == self.d
+        D = np.empty((x.shape[0], k), dtype=np.float32)
+        I = np.empty((x.shape[0], k), dtype=np.int64)
+        _capi.check(self._lib.flat_search(self._h, x.shape[0], _ptr(x), k, _ptr(D), _ptr(I)))
+        return D, I
+
+
+class AscendIndexFlatL2(AscendIndexFlat):
+    def __init__(self, dims, scratch_bytes=0):
+        super().__init__(dims, METRIC_L2, scratch_bytes)
+
+
+class AscendIndexInt8Flat(_FlatCommon):
+    """AscendIndexInt8Flat(dims, metric, config) -- FR/ascend/AscendIndexInt8.h:53-96; L2 only.
+    ``search_int32`` returns the exact int32 distances; ``search`` returns them as float32 like the
+    reference's signature (exact below 2**24, rounded to nearest above)."""
+    _pfx = "flat_i8"
+    _dtype = np.int8
+
+    def search_int32(self, x, k):
+        x = _as(x, np.int8, 2, "x")
+        assert x.shape[1] == self.d
+        D = np.empty((x.shape[0], k), dtype=np.int32)
+        I = np.empty((x.shape[0], k), dtype=np.int64)
+        _capi.check(self._lib.flat_i8_search(self._h, x.shape[0], _ptr(x), k, _ptr(D), _ptr(I)))
+        return D, I
+
+    def search(self, x, k):
+        D, I = self.search_int32(x, k)
+        Df = D.astype(np.float32)
+        Df[I == -1] = np.finfo(np.float32).max
+        return Df, I

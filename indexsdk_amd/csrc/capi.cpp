@@ -6,6 +6,7 @@
 #include <new>
 #include <string>
 
+#include "flat_index.h"
 #include "ivfpq_index.h"
 
 struct ivfpq_index {
@@ -14,6 +15,15 @@ struct ivfpq_index {
         : impl(d, metric, nlist, M, nbits, c)
     {
     }
+};
+
+struct flat_index {
+    ixa::FlatIndex impl;
+    flat_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
+};
+struct flat_i8_index {
+    ixa::FlatI8Index impl;
+    flat_i8_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
 };
 
 namespace {
@@ -198,6 +208,80 @@ IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stat
         out->scan_launches = s.scan_launches;
         out->nsplit = s.nsplit;
     });
+}
+
+// ---- Flat ---------------------------------------------------------------------------------------
+
+static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
+{
+    IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");
+    out->ms_score = s.ms_score;
+    out->ms_select = s.ms_select;
+    out->ms_total = s.ms_total;
+    out->score_launches = s.score_launches;
+}
+
+#define IXA_FLAT_COMMON(PFX, HT, ET)                                                                              \
+    IXA_EXPORT int PFX##_create(int d, int metric, int64_t scratch_bytes, HT **out)                              \
+    {                                                                                                             \
+        return guarded([&] {                                                                                      \
+            IXA_REQUIRE(out != nullptr, ixa::kErrInvalidParam, "out can not be nullptr.");                        \
+            *out = nullptr;                                                                                       \
+            *out = new HT(d, metric, scratch_bytes > 0 ? scratch_bytes : ((int64_t)1 << 30));                     \
+        });                                                                                                       \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_destroy(HT *h) { return guarded([&] { delete h; }); }                                    \
+    IXA_EXPORT int PFX##_add_with_ids(HT *h, int64_t n, const ET *x, const int64_t *ids)                         \
+    {                                                                                                             \
+        return guarded([&] { IXA_HANDLE(h); h->impl.add(n, x, ids, false); });                                    \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_add_with_ids_device(HT *h, int64_t n, const ET *x, const int64_t *ids)                  \
+    {                                                                                                             \
+        return guarded([&] { IXA_HANDLE(h); h->impl.add(n, x, ids, true); });                                     \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_get_base(const HT *h, int64_t offset, int64_t n, ET *out)                               \
+    {                                                                                                             \
+        return guarded([&] { IXA_HANDLE(h); h->impl.get_base(offset, n, out); });                                 \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_ntotal(const HT *h, int64_t *out)                                                        \
+    {                                                                                                             \
+        return guarded([&] {                                                                                      \
+            IXA_HANDLE(h);                                                                                        \
+            IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");                                   \
+            *out = h->impl.ntotal();                                                                              \
+        });                                                                                                       \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_reset(HT *h) { return guarded([&] { IXA_HANDLE(h); h->impl.reset(); }); }                \
+    IXA_EXPORT int PFX##_last_search_stats(const HT *h, flat_search_stats_t *out)                                 \
+    {                                                                                                             \
+        return guarded([&] { IXA_HANDLE(h); copy_stats(h->impl.stats(), out); });                                 \
+    }
+
+IXA_FLAT_COMMON(flat, flat_index_t, float)
+IXA_FLAT_COMMON(flat_i8, flat_i8_index_t, int8_t)
+
+IXA_EXPORT int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });
+}
+IXA_EXPORT int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+}
+IXA_EXPORT int flat_search_device(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances,
+                                  int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
+}
+IXA_EXPORT int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances,
+                              int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+}
+IXA_EXPORT int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances,
+                                     int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
 }
 
 }  // extern "C"

@@ -11,13 +11,24 @@ void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_
 void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
                         const float *cn, int metric, float *out, int64_t ldo, hipStream_t s);
 
-// Best `ksel` columns of every row of a score matrix; out_idx and/or out_keys may be null.
-// out_keys carry (ordered score << 32) | (col_base + column).
+// Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
+// indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
+// (ordered score << 32) | (col_base + column): its content takes part in the selection and is
+// replaced by the result, so calling this over successive column chunks keeps a streaming top-k.
+// Fill it with 0xff bytes before the first chunk.
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                        int64_t col_base, unsigned long long *out_keys, hipStream_t s);
+                        int64_t col_base, unsigned long long *running, hipStream_t s);
+void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
+                            int64_t col_base, unsigned long long *running, hipStream_t s);
 
-// Canonical re-evaluation of cand[nq][ncand] (-1 = absent) and selection of the best nout.
+// Canonical re-evaluation of cand[nq][ncand] (-1 = absent) and selection of the best nout.  Rows of
+// the outputs are out_stride (>= nout) wide; columns past nout are padded with (-1, +-FLT_MAX).
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,
-                   const int32_t *cand, int ncand, int nout, int32_t *out_ids, float *out_dist, hipStream_t s);
+                   const int32_t *cand, int ncand, int nout, int out_stride, int32_t *out_ids, float *out_dist,
+                   hipStream_t s);
+
+// Exact int32 L2 scores on the int8 matrix cores: out[row * ldo + col] = |q|^2 + |b|^2 - 2 q.b.
+void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s);
 
 }  // namespace ixa

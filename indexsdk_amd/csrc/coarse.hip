@@ -207,38 +207,53 @@ void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, 
 
 // ------------------------------------------------------------------------------------------------
 // Per-row selection of the ksel smallest scores of a materialised score row.  One workgroup per
-// row, four wavefront pools, block merge.  Output: ksel column indices per row (best first),
-// -1 where the row has fewer than ksel columns.
-__global__ __launch_bounds__(256) void select_rows_kernel(const float *__restrict__ scores, int64_t ld, int64_t nc,
+// row, four wavefront pools, block merge.  Optionally the row's running best keys (from earlier
+// column chunks) take part in the merge and provide the initial bound, which turns a sequence of
+// calls over column chunks into a streaming top-k.  Output: ksel column indices per row (best
+// first, -1 where the row has fewer than ksel columns) and/or the keys themselves.
+template <typename S>
+__global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
                                                           int ksel, int cap, int merge_n,
                                                           int32_t *__restrict__ out_idx, int64_t col_base,
-                                                          key_t *__restrict__ out_keys)
+                                                          key_t *__restrict__ running)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // 4 * cap
     key_t *merge = pools + 4 * cap;                                     // merge_n
-    float *bounds = reinterpret_cast<float *>(merge + merge_n);         // 4
+    S *bounds = reinterpret_cast<S *>(merge + merge_n);                 // 4
     int *counts = reinterpret_cast<int *>(bounds + 4);                  // 4
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const float *row = scores + (int64_t)blockIdx.x * ld;
+    const S *row = scores + (int64_t)blockIdx.x * ld;
+    key_t *run = running ? running + (int64_t)blockIdx.x * ksel : nullptr;
+    S start = ScoreOps<S>::worst();
+    if (run) {
+        const key_t last = run[ksel - 1];
+        if (last != kEmptyKey) {
+            start = key_score_as<S>(last);
+        }
+    }
     if (tid < 4) {
-        bounds[tid] = __builtin_inff();
+        bounds[tid] = start;
     }
     __syncthreads();
-    WavePool pool;
+    WavePool<S> pool;
     pool.init(pools + wave * cap, cap, ksel);
+    pool.bound = start;
     int iter = 0;
     for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
         int64_t c = base + lane;
-        float v = c < nc ? row[c] : __builtin_inff();
-        const bool compacted = pool.push(c < nc && v <= pool.bound, v, (uint32_t)c, lane);
+        S v = c < nc ? row[c] : ScoreOps<S>::worst();
+        const bool compacted = pool.push(c < nc && v <= pool.bound, v, (uint32_t)(c + col_base), lane);
         if (compacted || (iter & 7) == 7) {
             // after a compaction (or every 8th step) publish the bound and adopt the best one
             if (lane == 0) {
                 bounds[wave] = pool.bound;
             }
-            float b = fminf(fminf(bounds[0], bounds[1]), fminf(bounds[2], bounds[3]));
+            S b = bounds[0];
+            for (int i = 1; i < 4; i++) {
+                b = bounds[i] < b ? bounds[i] : b;
+            }
             pool.bound = b < pool.bound ? b : pool.bound;
         }
     }
@@ -249,7 +264,13 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const float *__restric
     __syncthreads();
     for (int i = tid; i < merge_n; i += 256) {
         int w = i / ksel, r = i - w * ksel;
-        merge[i] = (w < 4 && r < counts[w]) ? pools[w * cap + r] : kEmptyKey;
+        key_t kk = kEmptyKey;
+        if (w < 4) {
+            kk = r < counts[w] ? pools[w * cap + r] : kEmptyKey;
+        } else if (w == 4 && run) {
+            kk = run[r];
+        }
+        merge[i] = kk;
     }
     block_bitonic_sort(merge, merge_n, tid, 256);
     for (int i = tid; i < ksel; i += 256) {
@@ -257,30 +278,42 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const float *__restric
         if (out_idx) {
             out_idx[(int64_t)blockIdx.x * ksel + i] = kk == kEmptyKey ? -1 : (int32_t)key_index(kk);
         }
-        if (out_keys) {
-            out_keys[(int64_t)blockIdx.x * ksel + i] =
-                kk == kEmptyKey ? kEmptyKey : (kk & 0xffffffff00000000ull) | (key_index(kk) + (uint32_t)col_base);
+        if (run) {
+            run[i] = kk;
         }
     }
 }
 
-void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                        int64_t col_base, unsigned long long *out_keys, hipStream_t s)
+template <typename S>
+static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
+                                 int64_t col_base, unsigned long long *running, hipStream_t s)
 {
     if (nrows == 0) {
         return;
     }
     IXA_REQUIRE(ksel >= 1 && ksel <= 2048, kErrInvalidParam, "selection size %d out of range [1, 2048]", ksel);
     const int cap = wave_pool_capacity(ksel);
-    const int merge_n = pow2_ceil(4 * ksel);
+    const int merge_n = pow2_ceil((running ? 5 : 4) * ksel);
     const size_t smem = (size_t)(4 * cap + merge_n) * sizeof(key_t) + 32;
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "selection size %d needs %zu bytes of LDS", ksel, smem);
     if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel),
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel<S>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     }
-    hipLaunchKernelGGL(select_rows_kernel, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
-                       merge_n, out_idx, col_base, out_keys);
+    hipLaunchKernelGGL(select_rows_kernel<S>, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
+                       merge_n, out_idx, col_base, running);
+}
+
+void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
+                        int64_t col_base, unsigned long long *running, hipStream_t s)
+{
+    launch_select_rows_t<float>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, s);
+}
+
+void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
+                            int64_t col_base, unsigned long long *running, hipStream_t s)
+{
+    launch_select_rows_t<int32_t>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, s);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -294,7 +327,7 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
                                                      const float *__restrict__ C, int d,
                                                      const float *__restrict__ qn, const float *__restrict__ cn,
                                                      int metric, const int32_t *__restrict__ cand, int ncand, int P,
-                                                     int nout, int32_t *__restrict__ out_ids,
+                                                     int nout, int out_stride, int32_t *__restrict__ out_ids,
                                                      float *__restrict__ out_dist)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -356,30 +389,31 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
         }
     }
     __syncthreads();
-    for (int e = tid; e < rows_per_block * nout; e += 256) {
-        const int sub = e / nout, t = e - sub * nout;
+    for (int e = tid; e < rows_per_block * out_stride; e += 256) {
+        const int sub = e / out_stride, t = e - sub * out_stride;
         const int64_t row = (int64_t)blockIdx.x * rows_per_block + sub;
         if (row >= nq) {
             continue;
         }
-        key_t kk = keys[sub * P + t];
+        key_t kk = t < nout ? keys[sub * P + t] : kEmptyKey;
         const bool ok = kk != kEmptyKey;
-        out_ids[row * nout + t] = ok ? (int32_t)key_index(kk) : -1;
+        out_ids[row * out_stride + t] = ok ? (int32_t)key_index(kk) : -1;
         if (out_dist) {
             float v = key_score(kk);
             const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
-            out_dist[row * nout + t] = ok ? (metric == kMetricL2 ? v : -v) : pad;
+            out_dist[row * out_stride + t] = ok ? (metric == kMetricL2 ? v : -v) : pad;
         }
     }
 }
 
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,
-                   const int32_t *cand, int ncand, int nout, int32_t *out_ids, float *out_dist, hipStream_t s)
+                   const int32_t *cand, int ncand, int nout, int out_stride, int32_t *out_ids, float *out_dist,
+                   hipStream_t s)
 {
     if (nq == 0) {
         return;
     }
-    IXA_REQUIRE(ncand >= 1 && ncand <= 4096 && nout <= ncand, kErrInvalidParam,
+    IXA_REQUIRE(ncand >= 1 && ncand <= 4096 && nout <= ncand && out_stride >= nout, kErrInvalidParam,
                 "refine candidate count %d out of range [1, 4096]", ncand);
     const int P = pow2_ceil(ncand < 2 ? 2 : ncand);
     const int rows_per_block = P >= 256 ? 1 : 256 / P;
@@ -389,10 +423,10 @@ void launch_refine(const float *Q, int64_t nq, const float *C, int d, const floa
                       (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     if (vec4) {
         hipLaunchKernelGGL(refine_kernel<true>, dim3(grid), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, cand,
-                           ncand, P, nout, out_ids, out_dist);
+                           ncand, P, nout, out_stride, out_ids, out_dist);
     } else {
         hipLaunchKernelGGL(refine_kernel<false>, dim3(grid), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, cand,
-                           ncand, P, nout, out_ids, out_dist);
+                           ncand, P, nout, out_stride, out_ids, out_dist);
     }
 }
 

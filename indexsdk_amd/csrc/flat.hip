@@ -1,0 +1,534 @@
+// Brute-force Flat search: fp32 (scores on the fp32 matrix cores, exact refine) and int8 (exact
+// int32 L2 on the int8 matrix cores).  See flat_index.h for the reference counterparts.
+#include <algorithm>
+#include <cstring>
+
+#include "coarse.h"
+#include "flat_index.h"
+#include "topk.h"
+
+namespace ixa {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int64_t kMaxN = 1000000000;
+constexpr int64_t kMaxK = 2048;
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+// |row|^2 of int8 rows in int32 (FR/ascenddaemon/impl/IndexInt8Flat.cpp:938-967).  One wavefront
+// per row; integer sums are order-free.
+__global__ __launch_bounds__(256) void sqnorm_rows_i8_kernel(const int8_t *__restrict__ x, int64_t n, int d,
+                                                             int32_t *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n) {
+        return;
+    }
+    const int8_t *p = x + row * d;
+    int32_t s = 0;
+    for (int j = lane; j < d; j += 64) {
+        const int32_t v = p[j];
+        s += v * v;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        s += __shfl_down(s, o);
+    }
+    if (lane == 0) {
+        out[row] = s;
+    }
+}
+
+// Exact int32 L2 score tile: out[row][col] = |q|^2 + |b|^2 - 2 q.b   (integer part of
+// FR/ops/ascendc/op_kernel/ascendc_dist_int8_flat_l2.cpp:201-203, 485-500).
+// 128 x 128 tile per workgroup, 64 x 64 per wavefront as 2 x 2 blocks of v_mfma_i32_32x32x32_i8;
+// K-steps of 64 bytes staged in LDS with an 80-byte row stride (conflict-free 128-bit reads).
+constexpr int kTile = 128;
+constexpr int kKBytes = 64;
+constexpr int kRowStride = 80;
+
+template <bool VEC16>
+__device__ __forceinline__ uint4 load_k16(const int8_t *row, int k, int d)
+{
+    if (VEC16) {
+        if (k < d) {
+            return *reinterpret_cast<const uint4 *>(row + k);
+        }
+        return make_uint4(0, 0, 0, 0);
+    }
+    uint32_t w[4] = {0, 0, 0, 0};
+    for (int t = 0; t < 16; t++) {
+        if (k + t < d) {
+            w[t >> 2] |= (uint32_t)(uint8_t)row[k + t] << (8 * (t & 3));
+        }
+    }
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <bool VEC16>
+__global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__restrict__ Q, int64_t nq,
+                                                            const int8_t *__restrict__ B, int64_t nb, int d,
+                                                            const int32_t *__restrict__ qn,
+                                                            const int32_t *__restrict__ bn, int32_t *__restrict__ out,
+                                                            int64_t ldo, int tiles_n)
+{
+    __shared__ __align__(16) unsigned char As[2][kTile * kRowStride];
+    __shared__ __align__(16) unsigned char Bs[2][kTile * kRowStride];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const int64_t i0 = tile_m * kTile, j0 = tile_n * kTile;
+
+    const int lrow0 = tid >> 2, lrow1 = (tid + 256) >> 2, lk = (tid & 3) * 16;
+    const int64_t qa0 = i0 + lrow0 < nq ? i0 + lrow0 : nq - 1, qa1 = i0 + lrow1 < nq ? i0 + lrow1 : nq - 1;
+    const int64_t ba0 = j0 + lrow0 < nb ? j0 + lrow0 : nb - 1, ba1 = j0 + lrow1 < nb ? j0 + lrow1 : nb - 1;
+    const int8_t *qrow0 = Q + qa0 * d, *qrow1 = Q + qa1 * d;
+    const int8_t *brow0 = B + ba0 * d, *brow1 = B + ba1 * d;
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[a][b][r] = 0;
+            }
+        }
+    }
+    const int nk = (d + kKBytes - 1) / kKBytes;
+    uint4 ra0 = load_k16<VEC16>(qrow0, lk, d), ra1 = load_k16<VEC16>(qrow1, lk, d);
+    uint4 rb0 = load_k16<VEC16>(brow0, lk, d), rb1 = load_k16<VEC16>(brow1, lk, d);
+    *reinterpret_cast<uint4 *>(&As[0][lrow0 * kRowStride + lk]) = ra0;
+    *reinterpret_cast<uint4 *>(&As[0][lrow1 * kRowStride + lk]) = ra1;
+    *reinterpret_cast<uint4 *>(&Bs[0][lrow0 * kRowStride + lk]) = rb0;
+    *reinterpret_cast<uint4 *>(&Bs[0][lrow1 * kRowStride + lk]) = rb1;
+    __syncthreads();
+    for (int ks = 0; ks < nk; ks++) {
+        const int buf = ks & 1;
+        if (ks + 1 < nk) {
+            const int k = (ks + 1) * kKBytes + lk;
+            ra0 = load_k16<VEC16>(qrow0, k, d);
+            ra1 = load_k16<VEC16>(qrow1, k, d);
+            rb0 = load_k16<VEC16>(brow0, k, d);
+            rb1 = load_k16<VEC16>(brow1, k, d);
+        }
+        v4i a[2][2], b[2][2];
+#pragma unroll
+        for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                // the k index of an operand byte is a function of (lane half, byte position) that is
+                // the same for both operands, and integer sums are order-free, so any such
+                // assignment gives the exact dot product
+                a[blk][kk] = *reinterpret_cast<const v4i *>(
+                    &As[buf][(wr * 64 + blk * 32 + l32) * kRowStride + kk * 32 + half * 16]);
+                b[blk][kk] = *reinterpret_cast<const v4i *>(
+                    &Bs[buf][(wc * 64 + blk * 32 + l32) * kRowStride + kk * 32 + half * 16]);
+            }
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+            for (int ra = 0; ra < 2; ra++) {
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra][kk], b[rb][kk], acc[ra][rb], 0, 0, 0);
+                }
+            }
+        }
+        if (ks + 1 < nk) {
+            const int nbuf = buf ^ 1;
+            *reinterpret_cast<uint4 *>(&As[nbuf][lrow0 * kRowStride + lk]) = ra0;
+            *reinterpret_cast<uint4 *>(&As[nbuf][lrow1 * kRowStride + lk]) = ra1;
+            *reinterpret_cast<uint4 *>(&Bs[nbuf][lrow0 * kRowStride + lk]) = rb0;
+            *reinterpret_cast<uint4 *>(&Bs[nbuf][lrow1 * kRowStride + lk]) = rb1;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+        const int64_t col = j0 + wc * 64 + rb * 32 + l32;
+        const int32_t bnv = col < nb ? bn[col] : 0;
+#pragma unroll
+        for (int ra = 0; ra < 2; ra++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t row = i0 + wr * 64 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (row < nq && col < nb) {
+                    out[row * ldo + col] = qn[row] + bnv - 2 * acc[ra][rb][r];
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+
+void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s)
+{
+    if (nq == 0 || nb == 0) {
+        return;
+    }
+    const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nb + kTile - 1) / kTile;
+    IXA_REQUIRE(tiles_m * tiles_n < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
+    const bool vec = (d % 16 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                     (reinterpret_cast<uintptr_t>(B) % 16 == 0);
+    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    if (vec) {
+        hipLaunchKernelGGL(score_tile_i8_kernel<true>, grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
+                           (int)tiles_n);
+    } else {
+        hipLaunchKernelGGL(score_tile_i8_kernel<false>, grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
+                           (int)tiles_n);
+    }
+}
+
+namespace {
+
+// keys -> (distance, label); label = ids[position].
+template <typename S, typename OutT>
+__global__ __launch_bounds__(256) void finish_keys_kernel(const key_t *__restrict__ keys, int64_t n, int metric,
+                                                          const int64_t *__restrict__ ids, OutT pad,
+                                                          OutT *__restrict__ out_dist, int64_t *__restrict__ out_labels)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const key_t kk = keys[i];
+    if (kk == kEmptyKey) {
+        out_dist[i] = pad;
+        out_labels[i] = -1;
+        return;
+    }
+    const S v = key_score_as<S>(kk);
+    out_dist[i] = metric == kMetricL2 ? (OutT)v : (OutT)(-v);
+    out_labels[i] = ids[key_index(kk)];
+}
+
+__global__ __launch_bounds__(256) void keys_to_idx_kernel(const key_t *__restrict__ keys, int64_t n,
+                                                          int32_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        out[i] = keys[i] == kEmptyKey ? -1 : (int32_t)key_index(keys[i]);
+    }
+}
+
+__global__ __launch_bounds__(256) void map_labels_kernel(const int32_t *__restrict__ idx, int64_t n,
+                                                         const int64_t *__restrict__ ids, int64_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        out[i] = idx[i] < 0 ? -1 : ids[idx[i]];
+    }
+}
+
+__global__ __launch_bounds__(256) void iota_ids_kernel(int64_t *out, int64_t n, int64_t base)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        out[i] = base + i;
+    }
+}
+
+}  // namespace
+
+// -------------------------------------------------------------------------------------------------
+
+template <typename T>
+FlatBase<T>::FlatBase(int d, int metric, int64_t scratch_bytes) : d_(d), metric_(metric), scratch_bytes_(scratch_bytes)
+{
+    IXA_REQUIRE(metric == kMetricL2 || metric == kMetricInnerProduct, kErrInvalidParam, "Unsupported metric type");
+    IXA_REQUIRE(d >= 1 && d <= 4096, kErrInvalidParam, "Unsupported dims: %d\n", d);
+    IXA_REQUIRE(scratch_bytes >= (1 << 20), kErrInvalidParam, "scratch_bytes must be at least 1 MiB");
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    IXA_REQUIRE(e == hipSuccess && ndev > 0, kErrIndexNotInit,
+                "no HIP device available (%s): this library has no CPU path", hipGetErrorString(e));
+    IXA_HIP(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+    for (auto &ev : ev_) {
+        IXA_HIP(hipEventCreate(&ev));
+    }
+}
+
+template <typename T>
+FlatBase<T>::~FlatBase()
+{
+    if (stream_) {
+        (void)hipStreamSynchronize(stream_);
+    }
+    for (auto &ev : ev_) {
+        if (ev) {
+            (void)hipEventDestroy(ev);
+        }
+    }
+    if (stream_) {
+        (void)hipStreamDestroy(stream_);
+    }
+}
+
+// Grows the base / id arrays geometrically, keeping their content.
+template <typename T>
+void FlatBase<T>::reserve(int64_t n)
+{
+    if (n <= capacity_) {
+        return;
+    }
+    const int64_t cap = std::max<int64_t>(n, capacity_ + capacity_ / 2);
+    DeviceBuffer<T> nb((size_t)cap * d_);
+    DeviceBuffer<int64_t> ni((size_t)cap);
+    if (ntotal_ > 0) {
+        IXA_HIP(hipMemcpyAsync(nb.data(), base_.data(), (size_t)ntotal_ * d_ * sizeof(T), hipMemcpyDeviceToDevice,
+                               stream_));
+        IXA_HIP(hipMemcpyAsync(ni.data(), ids_.data(), (size_t)ntotal_ * 8, hipMemcpyDeviceToDevice, stream_));
+        IXA_HIP(hipStreamSynchronize(stream_));
+    }
+    base_ = std::move(nb);
+    ids_ = std::move(ni);
+    capacity_ = cap;
+}
+
+// add / add_with_ids (FR/ascend/AscendIndex.h:66-71); ids default to ntotal + i.
+template <typename T>
+void FlatBase<T>::add(int64_t n, const T *x, const int64_t *ids, bool on_device)
+{
+    IXA_REQUIRE(x, kErrInvalidParam, "x can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(ntotal_ + n < ((int64_t)1 << 32) - 1, kErrInvalidParam, "index would exceed the 32-bit row space");
+    reserve(ntotal_ + n);
+    const hipMemcpyKind kind = on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+    IXA_HIP(hipMemcpyAsync(base_.data() + ntotal_ * d_, x, (size_t)n * d_ * sizeof(T), kind, stream_));
+    if (ids) {
+        IXA_HIP(hipMemcpyAsync(ids_.data() + ntotal_, ids, (size_t)n * 8, kind, stream_));
+    } else {
+        hipLaunchKernelGGL(iota_ids_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, ids_.data() + ntotal_, n,
+                           ntotal_);
+    }
+    IXA_HIP(hipStreamSynchronize(stream_));
+    ntotal_ += n;
+}
+
+template <typename T>
+void FlatBase<T>::get_base(int64_t offset, int64_t n, T *out) const
+{
+    IXA_REQUIRE(offset >= 0 && n >= 0 && offset + n <= ntotal_ && (n == 0 || out), kErrInvalidParam,
+                "range [%ld, %ld) is outside the index (ntotal %ld)", (long)offset, (long)(offset + n), (long)ntotal_);
+    if (n) {
+        IXA_HIP(hipMemcpyAsync(out, base_.data() + offset * d_, (size_t)n * d_ * sizeof(T), hipMemcpyDeviceToHost,
+                               stream_));
+        IXA_HIP(hipStreamSynchronize(stream_));
+    }
+}
+
+template <typename T>
+void FlatBase<T>::get_ids(int64_t offset, int64_t n, int64_t *out) const
+{
+    IXA_REQUIRE(offset >= 0 && n >= 0 && offset + n <= ntotal_ && (n == 0 || out), kErrInvalidParam,
+                "range [%ld, %ld) is outside the index (ntotal %ld)", (long)offset, (long)(offset + n), (long)ntotal_);
+    if (n) {
+        IXA_HIP(hipMemcpyAsync(out, ids_.data() + offset, (size_t)n * 8, hipMemcpyDeviceToHost, stream_));
+        IXA_HIP(hipStreamSynchronize(stream_));
+    }
+}
+
+template <typename T>
+void FlatBase<T>::reset()
+{
+    IXA_HIP(hipStreamSynchronize(stream_));
+    base_.release();
+    ids_.release();
+    ntotal_ = capacity_ = 0;
+}
+
+template class FlatBase<float>;
+template class FlatBase<int8_t>;
+
+// ---- fp32 ---------------------------------------------------------------------------------------
+
+FlatIndex::FlatIndex(int d, int metric, int64_t scratch_bytes) : FlatBase<float>(d, metric, scratch_bytes) {}
+
+void FlatIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_device)
+{
+    const int64_t before = ntotal_;
+    FlatBase<float>::add(n, x, ids, on_device);
+    // norms of the whole base are kept in one array; recompute the tail (left-to-right fp32)
+    DeviceBuffer<float> nn((size_t)capacity_);
+    if (before > 0) {
+        IXA_HIP(hipMemcpyAsync(nn.data(), norms_.data(), (size_t)before * 4, hipMemcpyDeviceToDevice, stream_));
+    }
+    launch_sqnorm_rows(base_.data() + before * d_, n, d_, nn.data() + before, stream_);
+    IXA_HIP(hipStreamSynchronize(stream_));
+    norms_ = std::move(nn);
+}
+
+void FlatIndex::reset()
+{
+    FlatBase<float>::reset();
+    norms_.release();
+}
+
+// search (FR/ascendhost/src/index/IndexFlatL2Aicpu.cpp:157-306): the base is walked in row chunks;
+// every chunk's scores are selected into a running top-(k + slack) per query, and the survivors
+// are re-evaluated in the canonical scalar arithmetic before the final top-k is written.
+void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
+{
+    IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+    const float *xd = x;
+    if (!on_device) {
+        ws_x_.upload(x, (size_t)n * d_, stream_);
+        xd = ws_x_.data();
+    }
+    float *dd = dist;
+    int64_t *ld = labels;
+    if (!on_device) {
+        ws_dist_.resize((size_t)n * k);
+        ws_labels_.resize((size_t)n * k);
+        dd = ws_dist_.data();
+        ld = ws_labels_.data();
+    }
+    const int ncand = (int)std::min<int64_t>(std::max<int64_t>(ntotal_, 1), k + 8 + k / 8);
+    ws_qn_.resize((size_t)n);
+    ws_running_.resize((size_t)n * ncand);
+    ws_cand_.resize((size_t)n * ncand);
+    ws_idx_.resize((size_t)n * k);
+    IXA_HIP(hipEventRecord(ev_[0], stream_));
+    launch_sqnorm_rows(xd, n, d_, ws_qn_.data(), stream_);
+    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+    const int64_t qb = std::min<int64_t>(round_up(n, 128), 4096);
+    int64_t nb = scratch_bytes_ / (qb * 4);
+    nb = std::max<int64_t>(128, nb / 128 * 128);
+    nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
+    ws_scores_.resize((size_t)qb * nb);
+    int launches = 0;
+    for (int64_t q0 = 0; q0 < n; q0 += qb) {
+        const int64_t nq = std::min(qb, n - q0);
+        for (int64_t b0 = 0; b0 < ntotal_; b0 += nb) {
+            const int64_t nbc = std::min(nb, ntotal_ - b0);
+            launch_score_tiles(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
+                               norms_.data() + b0, metric_, ws_scores_.data(), nb, stream_);
+            launch_select_rows(ws_scores_.data(), nq, nb, nbc, ncand, nullptr, b0,
+                               ws_running_.data() + q0 * ncand, stream_);
+            launches++;
+        }
+    }
+    IXA_HIP(hipEventRecord(ev_[1], stream_));
+    hipLaunchKernelGGL(keys_to_idx_kernel, dim3(blocks_for(n * ncand)), dim3(256), 0, stream_, ws_running_.data(),
+                       n * ncand, ws_cand_.data());
+    launch_refine(xd, n, base_.data(), d_, ws_qn_.data(), norms_.data(), metric_, ws_cand_.data(), ncand,
+                  (int)std::min<int64_t>(k, ncand), (int)k, ws_idx_.data(), dd, stream_);
+    hipLaunchKernelGGL(map_labels_kernel, dim3(blocks_for(n * k)), dim3(256), 0, stream_, ws_idx_.data(), n * k,
+                       ids_.data(), ld);
+    IXA_HIP(hipEventRecord(ev_[2], stream_));
+    IXA_HIP(hipStreamSynchronize(stream_));
+    if (!on_device) {
+        ws_dist_.download(dist, (size_t)n * k, stream_);
+        ws_labels_.download(labels, (size_t)n * k, stream_);
+    }
+    float a = 0, b = 0;
+    IXA_HIP(hipEventElapsedTime(&a, ev_[0], ev_[1]));
+    IXA_HIP(hipEventElapsedTime(&b, ev_[1], ev_[2]));
+    stats_.ms_score = a;
+    stats_.ms_select = b;
+    stats_.ms_total = a + b;
+    stats_.score_launches = launches;
+}
+
+// ---- int8 ---------------------------------------------------------------------------------------
+
+FlatI8Index::FlatI8Index(int d, int metric, int64_t scratch_bytes) : FlatBase<int8_t>(d, metric, scratch_bytes)
+{
+    // the reference's Int8Flat serves L2 and cosine; only the exact-int32 L2 path is built here
+    IXA_REQUIRE(metric == kMetricL2, kErrInvalidParam, "Unsupported metric type");
+}
+
+void FlatI8Index::add(int64_t n, const int8_t *x, const int64_t *ids, bool on_device)
+{
+    const int64_t before = ntotal_;
+    FlatBase<int8_t>::add(n, x, ids, on_device);
+    DeviceBuffer<int32_t> nn((size_t)capacity_);
+    if (before > 0) {
+        IXA_HIP(hipMemcpyAsync(nn.data(), norms_.data(), (size_t)before * 4, hipMemcpyDeviceToDevice, stream_));
+    }
+    hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_,
+                       base_.data() + before * d_, n, d_, nn.data() + before);
+    IXA_HIP(hipStreamSynchronize(stream_));
+    norms_ = std::move(nn);
+}
+
+void FlatI8Index::reset()
+{
+    FlatBase<int8_t>::reset();
+    norms_.release();
+}
+
+void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device)
+{
+    IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+    const int8_t *xd = x;
+    if (!on_device) {
+        ws_x_.upload(x, (size_t)n * d_, stream_);
+        xd = ws_x_.data();
+    }
+    int32_t *dd = dist;
+    int64_t *ld = labels;
+    if (!on_device) {
+        ws_dist_.resize((size_t)n * k);
+        ws_labels_.resize((size_t)n * k);
+        dd = ws_dist_.data();
+        ld = ws_labels_.data();
+    }
+    ws_qn_.resize((size_t)n);
+    ws_running_.resize((size_t)n * k);
+    IXA_HIP(hipEventRecord(ev_[0], stream_));
+    hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_, xd, n, d_,
+                       ws_qn_.data());
+    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+    const int64_t qb = std::min<int64_t>(round_up(n, 128), 4096);
+    int64_t nb = scratch_bytes_ / (qb * 4);
+    nb = std::max<int64_t>(128, nb / 128 * 128);
+    nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
+    ws_scores_.resize((size_t)qb * nb);
+    int launches = 0;
+    float ms_score = 0;
+    for (int64_t q0 = 0; q0 < n; q0 += qb) {
+        const int64_t nq = std::min(qb, n - q0);
+        for (int64_t b0 = 0; b0 < ntotal_; b0 += nb) {
+            const int64_t nbc = std::min(nb, ntotal_ - b0);
+            launch_score_tiles_i8(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
+                                  norms_.data() + b0, ws_scores_.data(), nb, stream_);
+            launch_select_rows_i32(ws_scores_.data(), nq, nb, nbc, (int)k, nullptr, b0, ws_running_.data() + q0 * k,
+                                   stream_);
+            launches++;
+        }
+    }
+    hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,
+                       ws_running_.data(), n * k, kMetricL2, ids_.data(), (int32_t)0x7fffffff, dd, ld);
+    IXA_HIP(hipEventRecord(ev_[1], stream_));
+    IXA_HIP(hipStreamSynchronize(stream_));
+    if (!on_device) {
+        ws_dist_.download(dist, (size_t)n * k, stream_);
+        ws_labels_.download(labels, (size_t)n * k, stream_);
+    }
+    float a = 0;
+    IXA_HIP(hipEventElapsedTime(&a, ev_[0], ev_[1]));
+    (void)ms_score;
+    stats_.ms_score = 0;
+    stats_.ms_select = 0;
+    stats_.ms_total = a;
+    stats_.score_launches = launches;
+}
+
+}  // namespace ixa

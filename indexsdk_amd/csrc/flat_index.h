@@ -1,0 +1,78 @@
+// Brute-force Flat indexes on one MI355X ("the coarse stage in isolation"):
+//   FlatIndex    -- fp32 vectors, L2 or inner product; counterpart of AscendIndexFlat ->
+//                   IndexFlatL2Aicpu / IndexFlatIPAicpu (FR/ascendhost/src/index/IndexFlatL2Aicpu.cpp:157-306),
+//                   but with fp32 instead of fp16 distances.
+//   FlatI8Index  -- int8 vectors, exact int32 L2; counterpart of AscendIndexInt8Flat ->
+//                   IndexInt8FlatL2Aicpu (FR/ascendhost/src/index/IndexInt8FlatL2Aicpu.cpp:41-126), without the
+//                   reference's final scale-and-round-to-fp16 step.
+#pragma once
+#include <cstdint>
+
+#include "common.h"
+
+namespace ixa {
+
+struct FlatStats {
+    double ms_score = 0;        // all score-tile launches of the last search
+    double ms_select = 0;       // all selection launches (+ refine / finalisation)
+    double ms_total = 0;
+    double score_launches = 0;
+};
+
+template <typename T>
+class FlatBase {
+public:
+    FlatBase(int d, int metric, int64_t scratch_bytes);
+    ~FlatBase();
+    FlatBase(const FlatBase &) = delete;
+    FlatBase &operator=(const FlatBase &) = delete;
+
+    int d() const { return d_; }
+    int metric() const { return metric_; }
+    int64_t ntotal() const { return ntotal_; }
+    void add(int64_t n, const T *x, const int64_t *ids, bool on_device);
+    void get_base(int64_t offset, int64_t n, T *out) const;   // host output
+    void get_ids(int64_t offset, int64_t n, int64_t *out) const;
+    void reset();
+    const FlatStats &stats() const { return stats_; }
+
+protected:
+    void reserve(int64_t n);
+    int d_, metric_;
+    int64_t scratch_bytes_;
+    int64_t ntotal_ = 0, capacity_ = 0;
+    hipStream_t stream_ = nullptr;
+    hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
+    DeviceBuffer<T> base_;
+    DeviceBuffer<int64_t> ids_;
+    DeviceBuffer<unsigned long long> ws_running_;
+    DeviceBuffer<T> ws_x_;
+    FlatStats stats_;
+};
+
+class FlatIndex : public FlatBase<float> {
+public:
+    FlatIndex(int d, int metric, int64_t scratch_bytes);
+    void add(int64_t n, const float *x, const int64_t *ids, bool on_device);
+    void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
+    void reset();
+
+private:
+    DeviceBuffer<float> norms_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<int32_t> ws_cand_, ws_idx_;
+    DeviceBuffer<int64_t> ws_labels_;
+};
+
+class FlatI8Index : public FlatBase<int8_t> {
+public:
+    FlatI8Index(int d, int metric, int64_t scratch_bytes);
+    void add(int64_t n, const int8_t *x, const int64_t *ids, bool on_device);
+    void search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device);
+    void reset();
+
+private:
+    DeviceBuffer<int32_t> norms_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<int64_t> ws_labels_;
+};
+
+}  // namespace ixa

@@ -246,8 +246,8 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
                            select_metric, ws_scores_.data(), nlist_, stream_);
         launch_select_rows(ws_scores_.data(), nr, nlist_, nlist_, ncand, ws_cand_.data(), 0, nullptr, stream_);
         launch_refine(x_dev + r0 * d_, nr, centroids_.data(), d_, ws_qn_.data() + r0, cnorm_.data(), select_metric,
-                      ws_cand_.data(), ncand, nout, out_ids + r0 * nout, out_dist ? out_dist + r0 * nout : nullptr,
-                      stream_);
+                      ws_cand_.data(), ncand, nout, nout, out_ids + r0 * nout,
+                      out_dist ? out_dist + r0 * nout : nullptr, stream_);
     }
 }
 

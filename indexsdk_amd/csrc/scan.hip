@@ -130,7 +130,7 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
 
     // ---- stages 3 + 4: the probed lists form one sequence of 64-code groups; wavefront w takes
     // groups w, w + W, ... of that sequence, so the waves stay balanced whatever the list lengths.
-    WavePool pool;
+    WavePool<float> pool;
     pool.init(pools + wave * p.cap, p.cap, p.k);
     const int l32 = lane & 31;
     const int total = nlocal > 0 ? t_gend[nlocal - 1] : 0;

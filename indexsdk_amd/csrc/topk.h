@@ -32,11 +32,33 @@ __device__ __forceinline__ float unordered_bits(uint32_t o)
     return __uint_as_float(u);
 }
 
-__device__ __forceinline__ key_t make_key(float score, uint32_t idx)
+// int32 scores (exact integer distances) order by flipping the sign bit.
+__device__ __forceinline__ uint32_t ordered_bits(int32_t v) { return (uint32_t)v ^ 0x80000000u; }
+
+template <typename S>
+struct ScoreOps;
+template <>
+struct ScoreOps<float> {
+    static __device__ __forceinline__ float from_ordered(uint32_t o) { return unordered_bits(o); }
+    static __device__ __forceinline__ float worst() { return __builtin_inff(); }
+};
+template <>
+struct ScoreOps<int32_t> {
+    static __device__ __forceinline__ int32_t from_ordered(uint32_t o) { return (int32_t)(o ^ 0x80000000u); }
+    static __device__ __forceinline__ int32_t worst() { return 0x7fffffff; }
+};
+
+template <typename S>
+__device__ __forceinline__ key_t make_key(S score, uint32_t idx)
 {
     return ((key_t)ordered_bits(score) << 32) | idx;
 }
 __device__ __forceinline__ float key_score(key_t k) { return unordered_bits((uint32_t)(k >> 32)); }
+template <typename S>
+__device__ __forceinline__ S key_score_as(key_t k)
+{
+    return ScoreOps<S>::from_ordered((uint32_t)(k >> 32));
+}
 __device__ __forceinline__ uint32_t key_index(key_t k) { return (uint32_t)k; }
 
 // Orders LDS traffic of ONE wavefront (its lanes exchange data through LDS without s_barrier).
@@ -89,12 +111,13 @@ __device__ inline void block_bitonic_sort(key_t *buf, int n, int tid, int nthrea
     __syncthreads();
 }
 
+template <typename S = float>
 struct WavePool {
     key_t *buf;   // LDS, cap entries, private to this wave
     int cap;      // power of two, >= k + 2 * kWave
     int k;
     int count;    // wave-uniform
-    float bound;  // wave-uniform: a candidate enters iff score <= bound
+    S bound;      // wave-uniform: a candidate enters iff score <= bound
 
     __device__ __forceinline__ void init(key_t *b, int cap_, int k_)
     {
@@ -102,7 +125,7 @@ struct WavePool {
         cap = cap_;
         k = k_;
         count = 0;
-        bound = __builtin_inff();
+        bound = ScoreOps<S>::worst();
     }
 
     // Sort, keep the best k, tighten the bound.  All lanes of the wave must call it.
@@ -116,14 +139,14 @@ struct WavePool {
             count = k;
         }
         if (count == k) {
-            float b = key_score(buf[k - 1]);
+            S b = key_score_as<S>(buf[k - 1]);
             bound = b < bound ? b : bound;
         }
     }
 
     // All lanes call; lanes with pass == false contribute nothing.  Returns true when the
     // pool was compacted (the bound may have tightened).
-    __device__ __forceinline__ bool push(bool pass, float score, uint32_t idx, int lane)
+    __device__ __forceinline__ bool push(bool pass, S score, uint32_t idx, int lane)
     {
         unsigned long long mask = __ballot(pass);
         if (mask == 0) {

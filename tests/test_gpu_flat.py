@@ -1,0 +1,99 @@
+"""GPU parity tests of the Flat paths (through the C ABI) against the CPU oracle.
+
+int8: exact int32 distances and ids, bit for bit.  fp32: the final candidates are re-evaluated in
+the canonical scalar arithmetic, so distances and ids equal the oracle's bit for bit as well.
+"""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ivfpq_small.npz")
+
+
+@pytest.fixture(scope="module")
+def ix():
+    import indexsdk_amd
+    return indexsdk_amd
+
+
+@pytest.mark.parametrize("d,n,nq,k", [(64, 5000, 33, 10), (512, 20000, 130, 100), (96, 3000, 7, 128), (40, 1000, 5, 3)])
+def test_flat_i8_exact(ix, oracle, d, n, nq, k):
+    rng = np.random.default_rng(d + n)
+    base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    base[17] = base[5]                 # exact duplicates: ties resolve to the vector added first
+    q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    q[0] = base[5]
+    ids = (np.arange(n, dtype=np.int64) * 7 + 3)
+    # a small scratch forces several base chunks, exercising the streaming top-k
+    index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=4 << 20)
+    index.add_with_ids(base[: n // 2], ids[: n // 2])
+    index.add_with_ids(base[n // 2:], ids[n // 2:])
+    assert index.ntotal == n
+    assert np.array_equal(index.getBase(3, 10), base[3:13])
+    D, I = index.search_int32(q, k)
+    Dr, Ir = oracle.flat_i8(base, q, k, ids=ids)
+    assert np.array_equal(D, Dr)
+    assert np.array_equal(I, Ir)
+    assert D[0, 0] == 0 and I[0, 0] == ids[5] and I[0, 1] == ids[17]
+    Df, If = index.search(q, k)
+    assert np.array_equal(If, Ir) and np.array_equal(Df, Dr.astype(np.float32))
+
+
+def test_flat_i8_extremes_and_padding(ix, oracle):
+    base = np.full((3, 512), -127, dtype=np.int8)
+    base[1] = 127
+    q = np.full((2, 512), 127, dtype=np.int8)
+    index = ix.AscendIndexInt8Flat(512)
+    index.add(base)
+    D, I = index.search_int32(q, 5)
+    Dr, Ir = oracle.flat_i8(base, q, 5)
+    assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+    assert D[0].tolist() == [0, 512 * 254 * 254, 512 * 254 * 254, 2**31 - 1, 2**31 - 1]
+    assert I[0].tolist() == [1, 0, 2, -1, -1]
+    index.reset()
+    assert index.ntotal == 0
+    D, I = index.search_int32(q, 2)
+    assert np.all(I == -1)
+
+
+def test_flat_i8_golden(ix):
+    g = np.load(GOLDEN, allow_pickle=False)
+    index = ix.AscendIndexInt8Flat(64)
+    index.add(g["flat_i8_base"])
+    D, I = index.search_int32(g["flat_i8_queries"], 12)
+    assert np.array_equal(D, g["flat_i8_D"]) and np.array_equal(I, g["flat_i8_I"])
+
+
+@pytest.mark.parametrize("metric_name", ["L2", "IP"])
+@pytest.mark.parametrize("d,n,nq,k", [(128, 20000, 100, 10), (96, 7000, 40, 100), (30, 900, 9, 5)])
+def test_flat_f32_bit_exact(ix, oracle, metric_name, d, n, nq, k):
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    rng = np.random.default_rng(n + d)
+    centres = rng.standard_normal((20, d)).astype(np.float32)
+    base = (centres[rng.integers(0, 20, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 20, nq)] + 0.3 * rng.standard_normal((nq, d))).astype(np.float32)
+    index = ix.AscendIndexFlat(d, metric, scratch_bytes=2 << 20)
+    index.add(base[: n // 3])
+    index.add(base[n // 3:])
+    D, I = index.search(q, k)
+    Dr, Ir = oracle.flat_f32(base, q, k, metric)
+    assert np.array_equal(I, Ir)
+    assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+    assert np.array_equal(index.getBase(10, 5), base[10:15])
+
+
+def test_flat_f32_padding_and_golden(ix, oracle):
+    g = np.load(GOLDEN, allow_pickle=False)
+    x, q = g["base"].astype(np.float32), g["queries"].astype(np.float32)
+    index = ix.AscendIndexFlatL2(32)
+    index.add(x[:400])
+    D, I = index.search(q[:6], 12)
+    assert np.array_equal(D.view(np.uint32), g["flat_f32_D"].view(np.uint32)) and np.array_equal(I, g["flat_f32_I"])
+    small = ix.AscendIndexFlatL2(32)
+    small.add(x[:5])
+    D, I = small.search(q[:3], 9)
+    Dr, Ir = oracle.flat_f32(x[:5], q[:3], 9)
+    assert np.array_equal(I, Ir) and np.array_equal(D, Dr)
+    assert np.all(I[:, 5:] == -1) and np.all(D[:, 5:] == np.finfo(np.float32).max)
