@@ -53,6 +53,8 @@ def main():
     ap.add_argument("--layout", type=int, default=-1)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 1 GiB plain copy kernel (yardstick for rocprofv3 traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: this build has no multi-GPU path (one MI355X holds the whole index); "
@@ -120,6 +122,13 @@ def main():
     achieved = scan_bytes / (scan_ms_avg * 1e-3) / 1e9
     log(f"step {ms_per_step:.3f} ms (coarse {np.mean(coarse_ms):.3f} ms, scan {scan_ms_avg:.3f} ms), "
         f"{qps:.0f} QPS, scan {achieved:.0f} GB/s")
+
+    if args.copy_probe:
+        src = torch.zeros(1 << 28, device="cuda", dtype=torch.float32)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        _capi.check(lib.ixa_copy_probe(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), 1 << 30))
+        del src, dst
 
     result = {
         "metric": "queries/sec and ADC-scan GB/s (% HBM peak) at k=100 on 1 MI355X",

@@ -48,6 +48,11 @@ extern "C" {
 /* Message of the last failed call on this thread ("" if none). */
 const char *ixa_last_error(void);
 
+/* Copies bytes (a multiple of 16) between two DEVICE buffers with a plain copy kernel and waits for
+ * it.  No counterpart in the reference: it is the kernel of known size that hardware traffic
+ * counters (FETCH_SIZE / WRITE_SIZE) of the search kernels are scaled by. */
+int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes);
+
 /* ---------------------------------------------------------------------------------------------
  * IVFPQ
  * ------------------------------------------------------------------------------------------- */

@@ -260,6 +260,10 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
 IXA_FLAT_COMMON(flat, flat_index_t, float)
 IXA_FLAT_COMMON(flat_i8, flat_i8_index_t, int8_t)
 
+IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
+{
+    return guarded([&] { ixa::launch_copy_probe(src_dev, dst_dev, bytes); });
+}
 IXA_EXPORT int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });

@@ -242,6 +242,24 @@ __global__ __launch_bounds__(256) void iota_ids_kernel(int64_t *out, int64_t n, 
 
 }  // namespace
 
+// Plain 16-byte-per-lane copy of known size: the yardstick that HBM traffic counters of the other
+// kernels are scaled by.
+__global__ __launch_bounds__(256) void copy_probe_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                         int64_t n16)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) {
+        dst[i] = src[i];
+    }
+}
+
+void launch_copy_probe(const void *src, void *dst, int64_t bytes)
+{
+    IXA_REQUIRE(src && dst && bytes > 0 && bytes % 16 == 0, kErrInvalidParam, "copy probe needs a multiple of 16 bytes");
+    hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 16), dim3(256), 0, nullptr, static_cast<const uint4 *>(src),
+                       static_cast<uint4 *>(dst), bytes / 16);
+    IXA_HIP(hipDeviceSynchronize());
+}
+
 // -------------------------------------------------------------------------------------------------
 
 template <typename T>

@@ -75,4 +75,7 @@ private:
     DeviceBuffer<int64_t> ws_labels_;
 };
 
+// dst[0:bytes] = src[0:bytes] on the device with a plain copy kernel (traffic-counter yardstick).
+void launch_copy_probe(const void *src, void *dst, int64_t bytes);
+
 }  // namespace ixa

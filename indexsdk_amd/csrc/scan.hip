@@ -64,7 +64,10 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
     int *t_len = reinterpret_cast<int *>(t_off + p.table_n);                  // its length
     int *t_gend = t_len + p.table_n;                                          // groups up to and incl. list i
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wavefront index is uniform: keeping it (and everything derived from it) in scalar
+    // registers turns the group bookkeeping below into scalar code
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t q = blockIdx.x / p.nsplit;
     const int split = blockIdx.x % p.nsplit;
 
@@ -133,19 +136,21 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
     WavePool<float> pool;
     pool.init(pools + wave * p.cap, p.cap, p.k);
     const int l32 = lane & 31;
-    const int total = nlocal > 0 ? t_gend[nlocal - 1] : 0;
-    int li = 0;          // list the current group belongs to (monotone)
+    const int total = nlocal > 0 ? __builtin_amdgcn_readfirstlane(t_gend[nlocal - 1]) : 0;
+    int li = 0;          // list the current group belongs to (monotone, wave-uniform)
     int gstart = 0;      // first group of that list
+    int gend = nlocal > 0 ? __builtin_amdgcn_readfirstlane(t_gend[0]) : 0;
 
     auto locate = [&](int G) -> GroupRef {
-        while (G >= t_gend[li]) {
-            gstart = t_gend[li];
+        while (G >= gend) {
+            gstart = gend;
             li++;
+            gend = __builtin_amdgcn_readfirstlane(t_gend[li]);
         }
         const int pos = ((G - gstart) << 6) + lane;
         GroupRef r;
-        r.slot = t_off[li] + (uint32_t)pos;
-        r.valid = pos < t_len[li];
+        r.slot = (uint32_t)__builtin_amdgcn_readfirstlane((int)t_off[li]) + (uint32_t)pos;
+        r.valid = pos < __builtin_amdgcn_readfirstlane(t_len[li]);
         return r;
     };
 
@@ -218,37 +223,39 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
         return s;
     };
 
+    // One step: start the loads of the group after next, evaluate the current group, offer it to
+    // the pool.  Two register sets alternate so that no code registers are ever copied.
+    auto step = [&](int G, const GroupRef &cur, const uint32_t (&wcur)[NW], GroupRef &nxt, uint32_t (&wnxt)[NW]) {
+        if (G + W < total) {
+            nxt = locate(G + W);
+            load_codes(nxt.slot, wnxt);   // in flight while the current group is evaluated
+        }
+        const float s = adc(cur.slot, wcur);
+        const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane);
+        if (compacted) {
+            if (lane == 0) {
+                bounds[wave] = pool.bound;
+            }
+        }
+        if (compacted || (G & (16 * W - 1)) < W) {
+            // adopt the tightest bound any wavefront of this workgroup has published
+            float b = bounds[0];
+#pragma unroll
+            for (int i = 1; i < W; i++) {
+                b = fminf(b, bounds[i]);
+            }
+            b = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(b)));
+            pool.bound = b < pool.bound ? b : pool.bound;
+        }
+    };
     if (wave < total) {
-        uint32_t wc[NW], wn[NW];
-        GroupRef cur = locate(wave);
-        load_codes(cur.slot, wc);
-        for (int G = wave; G < total; G += W) {
-            GroupRef nxt = cur;
-            const bool more = G + W < total;
-            if (more) {
-                nxt = locate(G + W);
-                load_codes(nxt.slot, wn);   // in flight while the current group is evaluated
-            }
-            const float s = adc(cur.slot, wc);
-            const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane);
-            if (compacted) {
-                if (lane == 0) {
-                    bounds[wave] = pool.bound;
-                }
-            }
-            if (compacted || (G & (16 * W - 1)) < W) {
-                // adopt the tightest bound any wavefront of this workgroup has published
-                float b = bounds[0];
-#pragma unroll
-                for (int i = 1; i < W; i++) {
-                    b = fminf(b, bounds[i]);
-                }
-                pool.bound = b < pool.bound ? b : pool.bound;
-            }
-            cur = nxt;
-#pragma unroll
-            for (int v = 0; v < NW; v++) {
-                wc[v] = wn[v];
+        uint32_t wa[NW], wb[NW];
+        GroupRef ga = locate(wave), gb = ga;
+        load_codes(ga.slot, wa);
+        for (int G = wave; G < total; G += 2 * W) {
+            step(G, ga, wa, gb, wb);
+            if (G + W < total) {
+                step(G + W, gb, wb, ga, wa);
             }
         }
     }

@@ -48,6 +48,12 @@ struct ScoreOps<int32_t> {
     static __device__ __forceinline__ int32_t worst() { return 0x7fffffff; }
 };
 
+__device__ __forceinline__ float wave_uniform(float v)
+{
+    return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v)));
+}
+__device__ __forceinline__ int32_t wave_uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
 template <typename S>
 __device__ __forceinline__ key_t make_key(S score, uint32_t idx)
 {
@@ -139,7 +145,7 @@ struct WavePool {
             count = k;
         }
         if (count == k) {
-            S b = key_score_as<S>(buf[k - 1]);
+            S b = wave_uniform(key_score_as<S>(buf[k - 1]));
             bound = b < bound ? b : bound;
         }
     }

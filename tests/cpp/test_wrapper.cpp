@@ -1,0 +1,83 @@
+// Host-side check of the C++ wrappers: constructor validation messages as in
+// FR/ut/TestAscendIndexUTIVFPQ.cpp:77-184.  With a GPU present (argv[1] == "gpu") it also runs a
+// tiny train/add/search through the class interface.
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "ascend/AscendIndexFlat.h"
+#include "ascend/AscendIndexIVFPQ.h"
+
+using namespace faiss::ascend;
+
+static int failures = 0;
+#define EXPECT(cond)                                                   \
+    do {                                                               \
+        if (!(cond)) {                                                 \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+            failures++;                                                \
+        }                                                              \
+    } while (0)
+
+static std::string construct_msg(int dim, int nlist, int msub, int nbit)
+{
+    try {
+        AscendIndexIVFPQConfig conf({0});
+        AscendIndexIVFPQ index(dim, faiss::METRIC_L2, nlist, msub, nbit, conf);
+    } catch (std::exception &e) {
+        return e.what();
+    }
+    return "";
+}
+
+int main(int argc, char **argv)
+{
+    EXPECT(construct_msg(64, 1024, 4, 8).find("Unsupported dims") != std::string::npos);
+    EXPECT(construct_msg(128, 512, 4, 8).find("Unsupported nlists") != std::string::npos);
+    for (int nlist : {262144, 524288}) {
+        std::string m = construct_msg(128, nlist, 3, 8);
+        EXPECT(m.find("Unsupported nlists") == std::string::npos);
+        EXPECT(m.find("Unsupported msubs") != std::string::npos);
+    }
+    EXPECT(construct_msg(128, 1024, 4, 4).find("Unsupported nbits") != std::string::npos);
+    if (argc > 1 && std::strcmp(argv[1], "gpu") == 0) {
+        const int d = 128, nlist = 1024, M = 16, n = 40000, nq = 16, k = 5;
+        std::mt19937 gen(1);
+        std::normal_distribution<float> nd;
+        std::vector<float> x((size_t)n * d);
+        for (auto &v : x) {
+            v = nd(gen);
+        }
+        AscendIndexIVFPQConfig conf({0});
+        conf.niter = 3;
+        AscendIndexIVFPQ index(d, faiss::METRIC_L2, nlist, M, 8, conf);
+        EXPECT(!index.is_trained);
+        index.train(n, x.data());
+        index.add(n, x.data());
+        EXPECT(index.ntotal == n);
+        index.setNumProbes(32);
+        std::vector<float> D((size_t)nq * k);
+        std::vector<faiss::idx_t> I((size_t)nq * k);
+        index.search(nq, x.data(), k, D.data(), I.data());
+        int self = 0;
+        for (int i = 0; i < nq; i++) {
+            self += I[(size_t)i * k] == i;
+        }
+        EXPECT(self >= nq - 1);
+        size_t total = 0;
+        for (int l = 0; l < nlist; l++) {
+            total += index.getListLength(l);
+        }
+        EXPECT(total == (size_t)n);
+        AscendIndexFlatL2 flat(d);
+        flat.add(n, x.data());
+        flat.search(nq, x.data(), k, D.data(), I.data());
+        for (int i = 0; i < nq; i++) {
+            EXPECT(I[(size_t)i * k] == i);
+        }
+    }
+    std::printf(failures ? "wrapper test FAILED\n" : "wrapper test ok\n");
+    return failures ? 1 : 0;
+}
