@@ -213,17 +213,17 @@ void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, 
 // first, -1 where the row has fewer than ksel columns) and/or the keys themselves.
 template <typename S>
 __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
-                                                          int ksel, int cap, int merge_n,
-                                                          int32_t *__restrict__ out_idx, int64_t col_base,
-                                                          key_t *__restrict__ running)
+                                                          int ksel, int cap, int32_t *__restrict__ out_idx,
+                                                          int64_t col_base, key_t *__restrict__ running)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // 4 * cap
-    key_t *merge = pools + 4 * cap;                                     // merge_n
-    S *bounds = reinterpret_cast<S *>(merge + merge_n);                 // 4
-    int *counts = reinterpret_cast<int *>(bounds + 4);                  // 4
+    key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // pow2_ceil(4 * cap + ksel)
+    const int region = running ? 8 * cap : 4 * cap;
+    S *share = reinterpret_cast<S *>(pools + region);                   // 4
+    int *counts = reinterpret_cast<int *>(share + 4);                   // 4
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const S *row = scores + (int64_t)blockIdx.x * ld;
     key_t *run = running ? running + (int64_t)blockIdx.x * ksel : nullptr;
     S start = ScoreOps<S>::worst();
@@ -234,47 +234,40 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ 
         }
     }
     if (tid < 4) {
-        bounds[tid] = start;
+        share[tid] = ScoreOps<S>::worst();
     }
     __syncthreads();
     WavePool<S> pool;
     pool.init(pools + wave * cap, cap, ksel);
-    pool.bound = start;
+    pool.bound = wave_uniform(start);
+    const int share_rank = (ksel + 3) / 4;
+    auto adopt_shared = [&]() {
+        S b = share[0];
+        for (int i = 1; i < 4; i++) {
+            b = share[i] > b ? share[i] : b;
+        }
+        b = wave_uniform(b);
+        pool.bound = b < pool.bound ? b : pool.bound;
+    };
     int iter = 0;
     for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
         int64_t c = base + lane;
         S v = c < nc ? row[c] : ScoreOps<S>::worst();
-        const bool compacted = pool.push(c < nc && v <= pool.bound, v, (uint32_t)(c + col_base), lane);
+        const bool compacted =
+            pool.push(c < nc && v <= pool.bound, v, (uint32_t)(c + col_base), lane, &share[wave], share_rank);
         if (compacted || (iter & 7) == 7) {
-            // after a compaction (or every 8th step) publish the bound and adopt the best one
-            if (lane == 0) {
-                bounds[wave] = pool.bound;
-            }
-            S b = bounds[0];
-            for (int i = 1; i < 4; i++) {
-                b = bounds[i] < b ? bounds[i] : b;
-            }
-            pool.bound = b < pool.bound ? b : pool.bound;
+            adopt_shared();
         }
     }
-    pool.compact(lane);
+    __syncthreads();
+    adopt_shared();
+    pool.finish(lane);
     if (lane == 0) {
         counts[wave] = pool.count;
     }
-    __syncthreads();
-    for (int i = tid; i < merge_n; i += 256) {
-        int w = i / ksel, r = i - w * ksel;
-        key_t kk = kEmptyKey;
-        if (w < 4) {
-            kk = r < counts[w] ? pools[w * cap + r] : kEmptyKey;
-        } else if (w == 4 && run) {
-            kk = run[r];
-        }
-        merge[i] = kk;
-    }
-    block_bitonic_sort(merge, merge_n, tid, 256);
+    const int total = block_merge_pools<4>(pools, cap, counts, run, run ? ksel : 0, tid);
     for (int i = tid; i < ksel; i += 256) {
-        key_t kk = merge[i];
+        key_t kk = i < total ? pools[i] : kEmptyKey;
         if (out_idx) {
             out_idx[(int64_t)blockIdx.x * ksel + i] = kk == kEmptyKey ? -1 : (int32_t)key_index(kk);
         }
@@ -293,15 +286,14 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
     }
     IXA_REQUIRE(ksel >= 1 && ksel <= 2048, kErrInvalidParam, "selection size %d out of range [1, 2048]", ksel);
     const int cap = wave_pool_capacity(ksel);
-    const int merge_n = pow2_ceil((running ? 5 : 4) * ksel);
-    const size_t smem = (size_t)(4 * cap + merge_n) * sizeof(key_t) + 32;
+    const size_t smem = (size_t)(running ? 8 : 4) * cap * sizeof(key_t) + 64;
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "selection size %d needs %zu bytes of LDS", ksel, smem);
     if (smem > 48 * 1024) {
         IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel<S>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     }
     hipLaunchKernelGGL(select_rows_kernel<S>, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
-                       merge_n, out_idx, col_base, running);
+                       out_idx, col_base, running);
 }
 
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,

@@ -57,9 +57,8 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
     LutT *lut = reinterpret_cast<LutT *>(smem_raw);
     float *qs = reinterpret_cast<float *>(smem_raw + p.off_query);
     key_t *pools = reinterpret_cast<key_t *>(smem_raw + p.off_pools);
-    key_t *merge = reinterpret_cast<key_t *>(smem_raw + p.off_merge);
-    float *bounds = reinterpret_cast<float *>(smem_raw + p.off_misc);   // W
-    int *counts = reinterpret_cast<int *>(bounds + W);                  // W
+    float *share = reinterpret_cast<float *>(smem_raw + p.off_misc);    // W: score at rank ceil(k/W) per wave
+    int *counts = reinterpret_cast<int *>(share + W);                   // W
     uint32_t *t_off = reinterpret_cast<uint32_t *>(smem_raw + p.off_table);  // first slot of local list i
     int *t_len = reinterpret_cast<int *>(t_off + p.table_n);                  // its length
     int *t_gend = t_len + p.table_n;                                          // groups up to and incl. list i
@@ -77,7 +76,7 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
         qs[j] = p.queries[q * p.d + j];
     }
     if (tid < W) {
-        bounds[tid] = __builtin_inff();
+        share[tid] = __builtin_inff();
     }
     for (int i = tid; i < nlocal; i += NT) {
         const int l = p.probes[q * p.nprobe + split + i * p.nsplit];
@@ -223,6 +222,18 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
         return s;
     };
 
+    // The largest of the W published rank-ceil(k/W) scores has >= k candidates at or below it
+    // across the workgroup: a valid bound for every wave.
+    const int share_rank = (p.k + W - 1) / W;
+    auto adopt_shared = [&]() {
+        float b = share[0];
+#pragma unroll
+        for (int i = 1; i < W; i++) {
+            b = fmaxf(b, share[i]);
+        }
+        b = wave_uniform(b);
+        pool.bound = b < pool.bound ? b : pool.bound;
+    };
     // One step: start the loads of the group after next, evaluate the current group, offer it to
     // the pool.  Two register sets alternate so that no code registers are ever copied.
     auto step = [&](int G, const GroupRef &cur, const uint32_t (&wcur)[NW], GroupRef &nxt, uint32_t (&wnxt)[NW]) {
@@ -231,21 +242,9 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
             load_codes(nxt.slot, wnxt);   // in flight while the current group is evaluated
         }
         const float s = adc(cur.slot, wcur);
-        const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane);
-        if (compacted) {
-            if (lane == 0) {
-                bounds[wave] = pool.bound;
-            }
-        }
+        const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane, &share[wave], share_rank);
         if (compacted || (G & (16 * W - 1)) < W) {
-            // adopt the tightest bound any wavefront of this workgroup has published
-            float b = bounds[0];
-#pragma unroll
-            for (int i = 1; i < W; i++) {
-                b = fminf(b, bounds[i]);
-            }
-            b = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(b)));
-            pool.bound = b < pool.bound ? b : pool.bound;
+            adopt_shared();
         }
     };
     if (wave < total) {
@@ -259,27 +258,24 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
             }
         }
     }
-    pool.compact(lane);
+    __syncthreads();  // every wave has published its last value; the LUT is no longer needed
+    adopt_shared();
+    pool.finish(lane);
     if (lane == 0) {
         counts[wave] = pool.count;
     }
-    __syncthreads();  // everyone is done with the LUT: its space may now hold the merge array
-
-    for (int i = tid; i < p.merge_n; i += NT) {
-        int w = i / p.k, r = i - w * p.k;
-        merge[i] = (w < W && r < counts[w]) ? pools[w * p.cap + r] : kEmptyKey;
-    }
-    block_bitonic_sort(merge, p.merge_n, tid, NT);
+    const int total_keys = block_merge_pools<W>(pools, p.cap, counts, nullptr, 0, tid);
+    const key_t *merge = pools;
 
     if (p.nsplit > 1) {
         key_t *dst = p.partial + ((int64_t)q * p.nsplit + split) * p.k;
         for (int i = tid; i < p.k; i += NT) {
-            dst[i] = merge[i];
+            dst[i] = i < total_keys ? merge[i] : kEmptyKey;
         }
         return;
     }
     for (int i = tid; i < p.k; i += NT) {
-        const key_t kk = merge[i];
+        const key_t kk = i < total_keys ? merge[i] : kEmptyKey;
         const bool ok = kk != kEmptyKey;
         const float v = key_score(kk);
         const float pad = p.metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
@@ -390,20 +386,14 @@ static size_t plan_with_waves(ScanParams &p, int waves)
     const size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
     p.waves = waves;
     p.cap = wave_pool_capacity(p.k);
-    p.merge_n = pow2_ceil(waves * p.k);
+    p.merge_n = waves * p.cap;
     p.table_n = (p.nprobe + p.nsplit - 1) / p.nsplit;
     size_t off = round_up((int64_t)lut_bytes, 16);
     p.off_query = (int)off;
     off += round_up((int64_t)p.d * 4, 16);
     p.off_pools = (int)off;
-    off += (size_t)waves * p.cap * sizeof(key_t);
-    const size_t merge_bytes = (size_t)p.merge_n * sizeof(key_t);
-    if (merge_bytes <= (size_t)p.off_pools) {
-        p.off_merge = 0;  // reuse the LUT (+ query) space once the scan is over
-    } else {
-        p.off_merge = (int)off;
-        off += merge_bytes;
-    }
+    off += (size_t)waves * p.cap * sizeof(key_t);   // also the merge array of the epilogue
+    p.off_merge = p.off_pools;
     p.off_table = (int)off;
     off += round_up((int64_t)p.table_n * 12, 16);
     p.off_misc = (int)off;

@@ -1,14 +1,18 @@
 // Device-side top-k building blocks for 64-wide wavefronts (gfx950).
 //
 // Every candidate is a 64-bit key  (ordered(score) << 32) | index  where "score" is the quantity
-// to MINIMISE (the L2 distance, or the negated inner product) and index is a 32-bit position
-// (arena slot / centroid id / base row).  Smaller key == better candidate; exact score ties
-// resolve to the smaller index.  A key of all ones is the empty slot.
+// to MINIMISE (the L2 distance, the negated inner product, or an exact int32 distance) and index
+// is a 32-bit position (arena slot / centroid id / base row).  Smaller key == better candidate;
+// exact score ties resolve to the smaller index.  A key of all ones is the empty slot.
 //
-// WavePool: each wavefront keeps a private pool of candidates in LDS.  A candidate enters only
-// if its score is <= the wave's current bound; when the pool fills, the wave sorts it (bitonic,
-// in LDS, wave-synchronous: no workgroup barrier), keeps the best k and tightens the bound to
-// the k-th score.  Waves of a workgroup publish their bounds so that each can adopt the minimum.
+// WavePool: each wavefront keeps a private, UNSORTED pool of candidates in LDS.  A candidate
+// enters only if its score is <= the wave's current bound.  When the pool fills, the wave finds
+// (by a bitwise search over the top 20 bits of the ordered scores, one ballot per key and bit) the
+// smallest score bucket that still holds k candidates, drops everything above it and tightens its
+// bound to the top of that bucket -- no sorting, no workgroup barrier.  The same search at rank
+// ceil(k / W) gives a value every wave publishes; the maximum of the W published values has at
+// least k candidates below it across the workgroup, so every wave may adopt it as its bound.
+// Sorting happens once, at the end, on the few survivors of all pools.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -19,6 +23,7 @@ namespace ixa {
 using key_t = unsigned long long;
 constexpr key_t kEmptyKey = ~0ull;
 constexpr int kWave = 64;
+constexpr int kSelectBits = 20;  // resolution of the bucket search (sign + exponent + 11 mantissa bits)
 
 __device__ __forceinline__ uint32_t ordered_bits(float f)
 {
@@ -41,11 +46,18 @@ template <>
 struct ScoreOps<float> {
     static __device__ __forceinline__ float from_ordered(uint32_t o) { return unordered_bits(o); }
     static __device__ __forceinline__ float worst() { return __builtin_inff(); }
+    // largest score of the bucket with the given ordered prefix (never NaN)
+    static __device__ __forceinline__ float bucket_top(uint32_t o)
+    {
+        float v = unordered_bits(o);
+        return v == v ? v : __builtin_inff();
+    }
 };
 template <>
 struct ScoreOps<int32_t> {
     static __device__ __forceinline__ int32_t from_ordered(uint32_t o) { return (int32_t)(o ^ 0x80000000u); }
     static __device__ __forceinline__ int32_t worst() { return 0x7fffffff; }
+    static __device__ __forceinline__ int32_t bucket_top(uint32_t o) { return (int32_t)(o ^ 0x80000000u); }
 };
 
 __device__ __forceinline__ float wave_uniform(float v)
@@ -96,7 +108,7 @@ __device__ inline void wave_bitonic_sort(key_t *buf, int n, int lane)
     wave_lds_fence();
 }
 
-// Same sort, executed by a whole workgroup with barriers (used for the final merge).
+// Same sort, executed by a whole workgroup with barriers.
 __device__ inline void block_bitonic_sort(key_t *buf, int n, int tid, int nthreads)
 {
     for (int size = 2; size <= n; size <<= 1) {
@@ -119,7 +131,7 @@ __device__ inline void block_bitonic_sort(key_t *buf, int n, int tid, int nthrea
 
 template <typename S = float>
 struct WavePool {
-    key_t *buf;   // LDS, cap entries, private to this wave
+    key_t *buf;   // LDS, cap entries, private to this wave, unsorted
     int cap;      // power of two, >= k + 2 * kWave
     int k;
     int count;    // wave-uniform
@@ -134,25 +146,115 @@ struct WavePool {
         bound = ScoreOps<S>::worst();
     }
 
-    // Sort, keep the best k, tighten the bound.  All lanes of the wave must call it.
-    __device__ inline void compact(int lane)
+    // Smallest kSelectBits-bit prefix P such that at least `rank` pool entries have a score prefix
+    // <= P.  Requires 1 <= rank <= count.  Wave-uniform result.
+    __device__ inline uint32_t select_prefix(int rank, int lane) const
     {
-        for (int i = count + lane; i < cap; i += kWave) {
-            buf[i] = kEmptyKey;
+        constexpr int SH = 32 - kSelectBits;
+        uint32_t P = 0;
+        if (count <= 4 * kWave) {
+            // common case: up to four prefixes per lane live in registers
+            uint32_t pre[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = j * kWave + lane;
+                pre[j] = i < count ? (uint32_t)(buf[i] >> (32 + SH)) : 0xffffffffu;
+            }
+            for (int b = kSelectBits - 1; b >= 0; b--) {
+                const uint32_t c = P | ((1u << b) - 1u);
+                int cnt = 0;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    cnt += __popcll(__ballot(pre[j] <= c));
+                }
+                if (cnt < rank) {
+                    P |= 1u << b;
+                }
+            }
+            return P;
         }
-        wave_bitonic_sort(buf, cap, lane);
-        if (count > k) {
+        for (int b = kSelectBits - 1; b >= 0; b--) {
+            const uint32_t c = P | ((1u << b) - 1u);
+            int cnt = 0;
+            for (int i0 = 0; i0 < count; i0 += kWave) {
+                const int i = i0 + lane;
+                const uint32_t pre = i < count ? (uint32_t)(buf[i] >> (32 + SH)) : 0xffffffffu;
+                cnt += __popcll(__ballot(pre <= c));
+            }
+            if (cnt < rank) {
+                P |= 1u << b;
+            }
+        }
+        return P;
+    }
+
+    // Keeps the entries whose score is <= limit (in place, order preserved).
+    __device__ inline void keep_below(S limit, int lane)
+    {
+        int kept = 0;
+        for (int i0 = 0; i0 < count; i0 += kWave) {
+            const int i = i0 + lane;
+            key_t kk = i < count ? buf[i] : kEmptyKey;
+            const bool keep = i < count && key_score_as<S>(kk) <= limit;
+            const unsigned long long mask = __ballot(keep);
+            const int pre =
+                __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+            wave_lds_fence();  // all reads of this chunk are done before anything is overwritten
+            if (keep) {
+                buf[kept + pre] = kk;  // kept + pre <= i: never ahead of the read frontier
+            }
+            kept += __popcll(mask);
+        }
+        wave_lds_fence();
+        count = kept;
+    }
+
+    // Drops what cannot be among the k best and tightens the bound.  `share` (may be null) is
+    // this wave's slot for the value at rank share_rank.  All lanes of the wave must call it.
+    __device__ inline void compact(int lane, S *share, int share_rank)
+    {
+        constexpr int SH = 32 - kSelectBits;
+        wave_lds_fence();
+        if (share != nullptr && count >= share_rank) {
+            const uint32_t Ps = select_prefix(share_rank, lane);
+            const S top = ScoreOps<S>::bucket_top((Ps << SH) | ((1u << SH) - 1u));
+            if (lane == 0 && top < *share) {
+                *share = top;
+            }
+        }
+        if (count < k) {
+            return;
+        }
+        const uint32_t P = select_prefix(k, lane);
+        const S top = ScoreOps<S>::bucket_top((P << SH) | ((1u << SH) - 1u));
+        bound = top < bound ? top : bound;
+        keep_below(bound, lane);
+        if (count > cap - 2 * kWave) {
+            // degenerate score distribution (one bucket holds almost everything): exact path
+            for (int i = count + lane; i < cap; i += kWave) {
+                buf[i] = kEmptyKey;
+            }
+            wave_bitonic_sort(buf, cap, lane);
             count = k;
-        }
-        if (count == k) {
-            S b = wave_uniform(key_score_as<S>(buf[k - 1]));
+            const S b = wave_uniform(key_score_as<S>(buf[k - 1]));
             bound = b < bound ? b : bound;
+        }
+    }
+
+    // End of the stream: prune with the final bound so that the workgroup merge sees few keys.
+    __device__ inline void finish(int lane)
+    {
+        if (count >= k) {
+            compact(lane, nullptr, 0);
+        } else {
+            wave_lds_fence();
+            keep_below(bound, lane);
         }
     }
 
     // All lanes call; lanes with pass == false contribute nothing.  Returns true when the
     // pool was compacted (the bound may have tightened).
-    __device__ __forceinline__ bool push(bool pass, S score, uint32_t idx, int lane)
+    __device__ __forceinline__ bool push(bool pass, S score, uint32_t idx, int lane, S *share, int share_rank)
     {
         unsigned long long mask = __ballot(pass);
         if (mask == 0) {
@@ -164,12 +266,64 @@ struct WavePool {
         }
         count += __popcll(mask);
         if (count > cap - kWave) {
-            compact(lane);
+            compact(lane, share, share_rank);
             return true;
         }
         return false;
     }
 };
+
+// Workgroup epilogue: gathers the W pools (wave w owns pools[w*cap .. w*cap + counts[w])) to the
+// front of the pool region, appends `extra_n` further keys (may be 0), sorts ascending and
+// returns the number of valid keys; afterwards pools[0..result) is sorted.  The region must hold
+// pow2_ceil(W*cap + extra_n) keys.  Called by all threads of the workgroup.
+template <int W>
+__device__ inline int block_merge_pools(key_t *pools, int cap, const int *counts, const key_t *extra, int extra_n,
+                                        int tid)
+{
+    constexpr int NT = W * kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < W; w++) {
+        const int c = counts[w];
+        if (w < wave) {
+            before += c;
+        }
+        total += c;
+    }
+    // waves move their block to the left one after the other: the destination of wave w ends
+    // where its own source begins at the latest, and never reaches into a block not yet moved
+    for (int w = 1; w < W; w++) {
+        if (wave == w) {
+            const int c = counts[w];
+            const key_t *src = pools + w * cap;
+            for (int i0 = 0; i0 < c; i0 += kWave) {
+                const int i = i0 + lane;
+                key_t kk = i < c ? src[i] : kEmptyKey;
+                wave_lds_fence();
+                if (i < c) {
+                    pools[before + i] = kk;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < extra_n; i += NT) {
+        pools[total + i] = extra[i];
+    }
+    total += extra_n;
+    int n = 2;
+    while (n < total) {
+        n <<= 1;
+    }
+    for (int i = total + tid; i < n; i += NT) {
+        pools[i] = kEmptyKey;
+    }
+    block_bitonic_sort(pools, n, tid, NT);
+    return total;
+}
 
 inline int wave_pool_capacity(int k)
 {
