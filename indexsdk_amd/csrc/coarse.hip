@@ -249,14 +249,52 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ 
         b = wave_uniform(b);
         pool.bound = b < pool.bound ? b : pool.bound;
     };
+    const bool vec4 = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(scores) % 16 == 0);
     int iter = 0;
-    for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
-        int64_t c = base + lane;
-        S v = c < nc ? row[c] : ScoreOps<S>::worst();
-        const bool compacted =
-            pool.push(c < nc && v <= pool.bound, v, (uint32_t)(c + col_base), lane, &share[wave], share_rank);
-        if (compacted || (iter & 7) == 7) {
-            adopt_shared();
+    if (vec4) {
+        // 128-bit loads: a wavefront covers 256 consecutive columns per step
+        for (int64_t base = (int64_t)wave * 256; base < nc; base += 1024, iter++) {
+            const int64_t c = base + lane * 4;
+            S v[4];
+            if (c + 3 < nc) {
+                const uint4 u = *reinterpret_cast<const uint4 *>(row + c);
+                v[0] = __builtin_bit_cast(S, u.x);
+                v[1] = __builtin_bit_cast(S, u.y);
+                v[2] = __builtin_bit_cast(S, u.z);
+                v[3] = __builtin_bit_cast(S, u.w);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    v[t] = c + t < nc ? row[c + t] : ScoreOps<S>::worst();
+                }
+            }
+            bool pass[4];
+            bool any = false;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                pass[t] = c + t < nc && v[t] <= pool.bound;
+                any |= pass[t];
+            }
+            bool compacted = false;
+            if (__ballot(any)) {
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    compacted |= pool.push(pass[t], v[t], (uint32_t)(c + t + col_base), lane, &share[wave], share_rank);
+                }
+            }
+            if (compacted || (iter & 3) == 3) {
+                adopt_shared();
+            }
+        }
+    } else {
+        for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
+            int64_t c = base + lane;
+            S v = c < nc ? row[c] : ScoreOps<S>::worst();
+            const bool compacted =
+                pool.push(c < nc && v <= pool.bound, v, (uint32_t)(c + col_base), lane, &share[wave], share_rank);
+            if (compacted || (iter & 7) == 7) {
+                adopt_shared();
+            }
         }
     }
     __syncthreads();

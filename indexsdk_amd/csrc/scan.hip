@@ -21,6 +21,8 @@
 
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
+
 #include "topk.h"
 
 namespace ixa {
@@ -309,22 +311,27 @@ __global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restric
     }
 }
 
-// Sum of the lengths of all probed lists (the number of codes the scan visits).
+// Sum of the lengths of all probed lists (the number of codes the scan visits): grid-stride
+// partial sums, one atomic per workgroup.
 __global__ __launch_bounds__(256) void count_scanned_kernel(const int32_t *__restrict__ probes, int64_t n,
                                                             const int32_t *__restrict__ list_len,
                                                             unsigned long long *__restrict__ out)
 {
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    __shared__ unsigned long long part[4];
     unsigned long long v = 0;
-    if (i < n) {
-        int l = probes[i];
-        v = l >= 0 ? (unsigned long long)list_len[l] : 0ull;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int l = probes[i];
+        v += l >= 0 ? (unsigned long long)list_len[l] : 0ull;
     }
     for (int o = 32; o > 0; o >>= 1) {
         v += __shfl_down(v, o);
     }
-    if ((threadIdx.x & 63) == 0 && v) {
-        atomicAdd(out, v);
+    if ((threadIdx.x & 63) == 0) {
+        part[threadIdx.x >> 6] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        atomicAdd(out, part[0] + part[1] + part[2] + part[3]);
     }
 }
 
@@ -334,8 +341,8 @@ void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_
     if (n == 0) {
         return;
     }
-    hipLaunchKernelGGL(count_scanned_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, probes, n, list_len,
-                       out);
+    const unsigned grid = (unsigned)std::min<int64_t>(64, (n + 255) / 256);
+    hipLaunchKernelGGL(count_scanned_kernel, dim3(grid), dim3(256), 0, s, probes, n, list_len, out);
 }
 
 template <int MT, typename LutT, int LAYOUT>
