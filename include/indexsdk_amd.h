@@ -65,7 +65,8 @@ typedef struct ivfpq_index ivfpq_index_t;
 typedef struct ivfpq_config {
     int32_t niter;                  /* cp.niter of the coarse k-means; reference CPU mode uses 25 */
     int32_t pq_niter;               /* pqNiter; -1 = niter */
-    int32_t spherical;              /* cp.spherical; 0 = plain Lloyd (default here), 1 = reference default */
+    int32_t spherical;              /* cp.spherical for the COARSE quantizer; 0 = plain Lloyd (default here),
+                                       1 = centroids L2-normalised every iteration (reference default) */
     int32_t train_samples_per_list; /* trainSamplesPerList */
     int64_t max_train_samples;      /* maxTrainSamples */
     int32_t lut_fp16;               /* 1 = store the per-query LUT as IEEE half (accumulate in fp32) */

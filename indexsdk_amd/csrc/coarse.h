@@ -7,9 +7,32 @@ namespace ixa {
 // out[i] = |x_i|^2, accumulated left to right in fp32.
 void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_t s);
 
+// Filtered epilogue of the score kernels: instead of storing the scores, every score <= tau[row]
+// is appended as a key (ordered score << 32 | col_base + col) to cand[row * cap + cnt[row]++].
+// cnt may run past cap (the excess is dropped); the merge step reports that as an overflow.
+template <typename S>
+struct ScoreFilter {
+    const S *tau;              // [nq] admission bound per row
+    int32_t *cnt;              // [nq] number of appended keys
+    unsigned long long *cand;  // [nq][cap]
+    int cap;
+    int64_t col_base;
+};
+
 // out[row * ldo + col] = score(Q[row], C[col]) for row < nq, col < nc (fp32 MFMA).
 void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
                         const float *cn, int metric, float *out, int64_t ldo, hipStream_t s);
+
+void launch_score_tiles_filtered(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                                 const float *cn, int metric, ScoreFilter<float> flt, hipStream_t s);
+
+// Merges the filtered candidates of every row into its running best-k keys (sorted, kEmptyKey
+// padded), sets tau[row] to the k-th score (or leaves it when fewer than k keys exist), resets
+// cnt[row] and raises *overflow when a row had appended more than cap keys.
+void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<float> flt, float *tau, int64_t nq,
+                             int *overflow, hipStream_t s);
+void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter<int32_t> flt, int32_t *tau,
+                                 int64_t nq, int *overflow, hipStream_t s);
 
 // Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
 // indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
@@ -30,5 +53,7 @@ void launch_refine(const float *Q, int64_t nq, const float *C, int d, const floa
 // Exact int32 L2 scores on the int8 matrix cores: out[row * ldo + col] = |q|^2 + |b|^2 - 2 q.b.
 void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                            const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s);
+void launch_score_tiles_i8_filtered(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
+                                    const int32_t *qn, const int32_t *bn, ScoreFilter<int32_t> flt, hipStream_t s);
 
 }  // namespace ixa

@@ -71,12 +71,24 @@ __device__ __forceinline__ float4 load_k4(const float *row, int k, int d)
     return v;
 }
 
-template <bool VEC4>
+// Tile order: 8 consecutive workgroups (one per XCD) take 8 different column tiles, and each XCD
+// then walks all row tiles of its column tile, so a column tile is fetched from HBM once and
+// re-used out of that XCD's L2 while the (smaller) row operand stays L2-resident everywhere.
+__device__ __forceinline__ bool xcd_tile(int64_t b, int tiles_m, int tiles_n, int64_t &tile_m, int64_t &tile_n)
+{
+    const int64_t gs = (int64_t)8 * tiles_m;
+    const int64_t g = b / gs, r = b % gs;
+    tile_n = g * 8 + (r & 7);
+    tile_m = r >> 3;
+    return tile_n < tiles_n;
+}
+
+template <bool VEC4, bool FILTER>
 __global__ __launch_bounds__(256) void score_tile_kernel(const float *__restrict__ Q, int64_t nq,
                                                          const float *__restrict__ C, int64_t nc, int d,
                                                          const float *__restrict__ qn, const float *__restrict__ cn,
                                                          int metric, float *__restrict__ out, int64_t ldo,
-                                                         int tiles_n)
+                                                         int tiles_m, int tiles_n, ScoreFilter<float> flt)
 {
     __shared__ float As[2][kTile * kLdsStride];
     __shared__ float Bs[2][kTile * kLdsStride];
@@ -85,7 +97,10 @@ __global__ __launch_bounds__(256) void score_tile_kernel(const float *__restrict
     const int lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1;
     const int half = lane >> 5, l32 = lane & 31;
-    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    int64_t tile_m, tile_n;
+    if (!xcd_tile(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n)) {
+        return;
+    }
     const int64_t i0 = tile_m * kTile, j0 = tile_n * kTile;
 
     // global -> register mapping: a tile step is 128 rows x 4 float4; thread t moves float4 t, t+256
@@ -178,31 +193,125 @@ __global__ __launch_bounds__(256) void score_tile_kernel(const float *__restrict
                     } else {
                         v = -g;
                     }
-                    out[row * ldo + col] = v;
+                    if (FILTER) {
+                        if (v <= flt.tau[row]) {
+                            const int pos = atomicAdd(&flt.cnt[row], 1);
+                            if (pos < flt.cap) {
+                                flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
+                            }
+                        }
+                    } else {
+                        out[row * ldo + col] = v;
+                    }
                 }
             }
         }
     }
 }
 
-void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
-                        const float *cn, int metric, float *out, int64_t ldo, hipStream_t s)
+template <bool FILTER>
+static void launch_score_tiles_t(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                                 const float *cn, int metric, float *out, int64_t ldo, ScoreFilter<float> flt,
+                                 hipStream_t s)
 {
     if (nq == 0 || nc == 0) {
         return;
     }
     const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nc + kTile - 1) / kTile;
-    IXA_REQUIRE(tiles_m * tiles_n < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
+    const int64_t nblocks = (tiles_n + 7) / 8 * 8 * tiles_m;
+    IXA_REQUIRE(nblocks < (int64_t)1 << 31 && tiles_m < (1 << 28), kErrInvalidParam, "score tile grid too large");
     const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(C) % 16 == 0);
-    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    dim3 grid((unsigned)nblocks), block(256);
     if (vec4) {
-        hipLaunchKernelGGL(score_tile_kernel<true>, grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo,
-                           (int)tiles_n);
+        hipLaunchKernelGGL((score_tile_kernel<true, FILTER>), grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out,
+                           ldo, (int)tiles_m, (int)tiles_n, flt);
     } else {
-        hipLaunchKernelGGL(score_tile_kernel<false>, grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo,
-                           (int)tiles_n);
+        hipLaunchKernelGGL((score_tile_kernel<false, FILTER>), grid, block, 0, s, Q, nq, C, nc, d, qn, cn, metric, out,
+                           ldo, (int)tiles_m, (int)tiles_n, flt);
     }
+}
+
+void launch_score_tiles(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                        const float *cn, int metric, float *out, int64_t ldo, hipStream_t s)
+{
+    launch_score_tiles_t<false>(Q, nq, C, nc, d, qn, cn, metric, out, ldo, ScoreFilter<float>{}, s);
+}
+
+void launch_score_tiles_filtered(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                                 const float *cn, int metric, ScoreFilter<float> flt, hipStream_t s)
+{
+    launch_score_tiles_t<true>(Q, nq, C, nc, d, qn, cn, metric, nullptr, 0, flt, s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Merge of filtered candidates into the running best-k keys of each row (one workgroup per row).
+template <typename S>
+__global__ __launch_bounds__(256) void merge_candidates_kernel(key_t *__restrict__ running, int k, ScoreFilter<S> flt,
+                                                               S *__restrict__ tau, int *__restrict__ overflow)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    key_t *buf = reinterpret_cast<key_t *>(smem_raw);
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    int n = flt.cnt[row];
+    if (n == 0) {
+        return;  // nothing was admitted for this row in this chunk
+    }
+    if (n > flt.cap) {
+        if (tid == 0) {
+            *overflow = 1;
+        }
+        n = flt.cap;
+    }
+    key_t *run = running + row * k;
+    const int total = k + n;
+    int p2 = 2;
+    while (p2 < total) {
+        p2 <<= 1;
+    }
+    for (int i = tid; i < p2; i += 256) {
+        buf[i] = i < k ? run[i] : (i < total ? flt.cand[row * flt.cap + (i - k)] : kEmptyKey);
+    }
+    block_bitonic_sort(buf, p2, tid, 256);
+    for (int i = tid; i < k; i += 256) {
+        run[i] = buf[i];
+    }
+    if (tid == 0) {
+        flt.cnt[row] = 0;
+        if (buf[k - 1] != kEmptyKey) {
+            tau[row] = key_score_as<S>(buf[k - 1]);
+        }
+    }
+}
+
+template <typename S>
+static void launch_merge_candidates_t(key_t *running, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *overflow,
+                                      hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    const size_t smem = (size_t)pow2_ceil(k + flt.cap) * sizeof(key_t);
+    IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "candidate merge of %d + %d keys exceeds LDS", k, flt.cap);
+    if (smem > 48 * 1024) {
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(merge_candidates_kernel<S>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    }
+    hipLaunchKernelGGL(merge_candidates_kernel<S>, dim3((unsigned)nq), dim3(256), smem, s, running, k, flt, tau,
+                       overflow);
+}
+
+void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<float> flt, float *tau, int64_t nq,
+                             int *overflow, hipStream_t s)
+{
+    launch_merge_candidates_t<float>(running, k, flt, tau, nq, overflow, s);
+}
+
+void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter<int32_t> flt, int32_t *tau,
+                                 int64_t nq, int *overflow, hipStream_t s)
+{
+    launch_merge_candidates_t<int32_t>(running, k, flt, tau, nq, overflow, s);
 }
 
 // ------------------------------------------------------------------------------------------------

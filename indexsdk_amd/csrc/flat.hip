@@ -69,12 +69,13 @@ __device__ __forceinline__ uint4 load_k16(const int8_t *row, int k, int d)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <bool VEC16>
+template <bool VEC16, bool FILTER>
 __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__restrict__ Q, int64_t nq,
                                                             const int8_t *__restrict__ B, int64_t nb, int d,
                                                             const int32_t *__restrict__ qn,
                                                             const int32_t *__restrict__ bn, int32_t *__restrict__ out,
-                                                            int64_t ldo, int tiles_n)
+                                                            int64_t ldo, int tiles_m, int tiles_n,
+                                                            ScoreFilter<int32_t> flt)
 {
     __shared__ __align__(16) unsigned char As[2][kTile * kRowStride];
     __shared__ __align__(16) unsigned char Bs[2][kTile * kRowStride];
@@ -82,7 +83,14 @@ __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__rest
     const int lane = tid & 63, wave = tid >> 6;
     const int wr = wave >> 1, wc = wave & 1;
     const int half = lane >> 5, l32 = lane & 31;
-    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    // 8 consecutive workgroups (one per XCD) take 8 different base tiles; each XCD then walks all
+    // query tiles of its base tile, so a base tile is fetched from HBM once and re-used from L2
+    const int64_t gs = (int64_t)8 * tiles_m;
+    const int64_t grp = blockIdx.x / gs, rem = blockIdx.x % gs;
+    const int64_t tile_n = grp * 8 + (rem & 7), tile_m = rem >> 3;
+    if (tile_n >= tiles_n) {
+        return;
+    }
     const int64_t i0 = tile_m * kTile, j0 = tile_n * kTile;
 
     const int lrow0 = tid >> 2, lrow1 = (tid + 256) >> 2, lk = (tid & 3) * 16;
@@ -162,7 +170,17 @@ __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__rest
             for (int r = 0; r < 16; r++) {
                 const int64_t row = i0 + wr * 64 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                 if (row < nq && col < nb) {
-                    out[row * ldo + col] = qn[row] + bnv - 2 * acc[ra][rb][r];
+                    const int32_t v = qn[row] + bnv - 2 * acc[ra][rb][r];
+                    if (FILTER) {
+                        if (v <= flt.tau[row]) {
+                            const int pos = atomicAdd(&flt.cnt[row], 1);
+                            if (pos < flt.cap) {
+                                flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
+                            }
+                        }
+                    } else {
+                        out[row * ldo + col] = v;
+                    }
                 }
             }
         }
@@ -171,24 +189,39 @@ __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__rest
 
 }  // namespace
 
-void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
-                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s)
+template <bool FILTER>
+static void launch_score_tiles_i8_t(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
+                                    const int32_t *qn, const int32_t *bn, int32_t *out, int64_t ldo,
+                                    ScoreFilter<int32_t> flt, hipStream_t s)
 {
     if (nq == 0 || nb == 0) {
         return;
     }
     const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nb + kTile - 1) / kTile;
-    IXA_REQUIRE(tiles_m * tiles_n < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
+    const int64_t nblocks = (tiles_n + 7) / 8 * 8 * tiles_m;
+    IXA_REQUIRE(nblocks < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
     const bool vec = (d % 16 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(B) % 16 == 0);
-    dim3 grid((unsigned)(tiles_m * tiles_n)), block(256);
+    dim3 grid((unsigned)nblocks), block(256);
     if (vec) {
-        hipLaunchKernelGGL(score_tile_i8_kernel<true>, grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
-                           (int)tiles_n);
+        hipLaunchKernelGGL((score_tile_i8_kernel<true, FILTER>), grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
+                           (int)tiles_m, (int)tiles_n, flt);
     } else {
-        hipLaunchKernelGGL(score_tile_i8_kernel<false>, grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
-                           (int)tiles_n);
+        hipLaunchKernelGGL((score_tile_i8_kernel<false, FILTER>), grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
+                           (int)tiles_m, (int)tiles_n, flt);
     }
+}
+
+void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s)
+{
+    launch_score_tiles_i8_t<false>(Q, nq, B, nb, d, qn, bn, out, ldo, ScoreFilter<int32_t>{}, s);
+}
+
+void launch_score_tiles_i8_filtered(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
+                                    const int32_t *qn, const int32_t *bn, ScoreFilter<int32_t> flt, hipStream_t s)
+{
+    launch_score_tiles_i8_t<true>(Q, nq, B, nb, d, qn, bn, nullptr, 0, flt, s);
 }
 
 namespace {
@@ -229,6 +262,18 @@ __global__ __launch_bounds__(256) void map_labels_kernel(const int32_t *__restri
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) {
         out[i] = idx[i] < 0 ? -1 : ids[idx[i]];
+    }
+}
+
+// tau[row] = score of the last running key of the row, or the worst score while the row is not full.
+template <typename S>
+__global__ __launch_bounds__(256) void tau_from_running_kernel(const key_t *__restrict__ running, int k, int64_t n,
+                                                               S *__restrict__ tau)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const key_t last = running[i * k + (k - 1)];
+        tau[i] = last == kEmptyKey ? ScoreOps<S>::worst() : key_score_as<S>(last);
     }
 }
 
@@ -429,16 +474,58 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
     nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
     ws_scores_.resize((size_t)qb * nb);
     int launches = 0;
-    for (int64_t q0 = 0; q0 < n; q0 += qb) {
-        const int64_t nq = std::min(qb, n - q0);
-        for (int64_t b0 = 0; b0 < ntotal_; b0 += nb) {
-            const int64_t nbc = std::min(nb, ntotal_ - b0);
-            launch_score_tiles(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
-                               norms_.data() + b0, metric_, ws_scores_.data(), nb, stream_);
-            launch_select_rows(ws_scores_.data(), nq, nb, nbc, ncand, nullptr, b0,
-                               ws_running_.data() + q0 * ncand, stream_);
-            launches++;
+    // Pass 1 (streaming): a first stretch of the base goes through the score scratch and seeds the
+    // running keys; after that the score kernel itself drops everything above each query's current
+    // bound and only the few admitted candidates are merged -- no score ever reaches HBM again.
+    const int cap = pow2_ceil((int)std::max<int64_t>(1024, 8 * (int64_t)ncand));
+    const int64_t seed_rows = std::min<int64_t>(ntotal_, std::max<int64_t>(16384, 64 * (int64_t)ncand));
+    ws_tau_.resize((size_t)n);
+    ws_cnt_.resize((size_t)n + 1);
+    ws_filter_.resize((size_t)qb * cap);
+    IXA_HIP(hipMemsetAsync(ws_cnt_.data(), 0, ws_cnt_.bytes(), stream_));
+    int *overflow = ws_cnt_.data() + n;
+    bool fused = true;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        for (int64_t q0 = 0; q0 < n; q0 += qb) {
+            const int64_t nq = std::min(qb, n - q0);
+            const int64_t head = fused ? seed_rows : ntotal_;
+            for (int64_t b0 = 0; b0 < head; b0 += nb) {
+                const int64_t nbc = std::min(nb, head - b0);
+                launch_score_tiles(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
+                                   norms_.data() + b0, metric_, ws_scores_.data(), nb, stream_);
+                launch_select_rows(ws_scores_.data(), nq, nb, nbc, ncand, nullptr, b0,
+                                   ws_running_.data() + q0 * ncand, stream_);
+                launches++;
+            }
+            if (!fused || head >= ntotal_) {
+                continue;
+            }
+            hipLaunchKernelGGL(tau_from_running_kernel<float>, dim3(blocks_for(nq)), dim3(256), 0, stream_,
+                               ws_running_.data() + q0 * ncand, ncand, nq, ws_tau_.data() + q0);
+            int64_t seen = head;
+            while (seen < ntotal_) {
+                const int64_t nbc = std::min<int64_t>({ntotal_ - seen, seen, (int64_t)1 << 22});
+                ScoreFilter<float> flt{ws_tau_.data() + q0, ws_cnt_.data() + q0, ws_filter_.data(), cap, seen};
+                launch_score_tiles_filtered(xd + q0 * d_, nq, base_.data() + seen * d_, nbc, d_, ws_qn_.data() + q0,
+                                            norms_.data() + seen, metric_, flt, stream_);
+                launch_merge_candidates(ws_running_.data() + q0 * ncand, ncand, flt, ws_tau_.data() + q0, nq, overflow,
+                                        stream_);
+                launches++;
+                seen += nbc;
+            }
         }
+        int ovf = 0;
+        if (fused) {
+            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, stream_));
+            IXA_HIP(hipStreamSynchronize(stream_));
+        }
+        if (!ovf) {
+            break;
+        }
+        // a row admitted more candidates than its buffer holds (adversarial base order): redo the
+        // whole search through the score scratch, which has no such limit
+        fused = false;
+        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
     }
     IXA_HIP(hipEventRecord(ev_[1], stream_));
     hipLaunchKernelGGL(keys_to_idx_kernel, dim3(blocks_for(n * ncand)), dim3(256), 0, stream_, ws_running_.data(),
@@ -520,17 +607,55 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
     ws_scores_.resize((size_t)qb * nb);
     int launches = 0;
-    float ms_score = 0;
-    for (int64_t q0 = 0; q0 < n; q0 += qb) {
-        const int64_t nq = std::min(qb, n - q0);
-        for (int64_t b0 = 0; b0 < ntotal_; b0 += nb) {
-            const int64_t nbc = std::min(nb, ntotal_ - b0);
-            launch_score_tiles_i8(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
-                                  norms_.data() + b0, ws_scores_.data(), nb, stream_);
-            launch_select_rows_i32(ws_scores_.data(), nq, nb, nbc, (int)k, nullptr, b0, ws_running_.data() + q0 * k,
-                                   stream_);
-            launches++;
+    // same two-phase scheme as the fp32 Flat search: seed through the score scratch, then let the
+    // score kernel admit only what beats each query's current k-th distance
+    const int cap = pow2_ceil((int)std::max<int64_t>(1024, 8 * k));
+    const int64_t seed_rows = std::min<int64_t>(ntotal_, std::max<int64_t>(16384, 64 * k));
+    ws_tau_.resize((size_t)n);
+    ws_cnt_.resize((size_t)n + 1);
+    ws_filter_.resize((size_t)qb * cap);
+    IXA_HIP(hipMemsetAsync(ws_cnt_.data(), 0, ws_cnt_.bytes(), stream_));
+    int *overflow = ws_cnt_.data() + n;
+    bool fused = true;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        for (int64_t q0 = 0; q0 < n; q0 += qb) {
+            const int64_t nq = std::min(qb, n - q0);
+            const int64_t head = fused ? seed_rows : ntotal_;
+            for (int64_t b0 = 0; b0 < head; b0 += nb) {
+                const int64_t nbc = std::min(nb, head - b0);
+                launch_score_tiles_i8(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
+                                      norms_.data() + b0, ws_scores_.data(), nb, stream_);
+                launch_select_rows_i32(ws_scores_.data(), nq, nb, nbc, (int)k, nullptr, b0,
+                                       ws_running_.data() + q0 * k, stream_);
+                launches++;
+            }
+            if (!fused || head >= ntotal_) {
+                continue;
+            }
+            hipLaunchKernelGGL(tau_from_running_kernel<int32_t>, dim3(blocks_for(nq)), dim3(256), 0, stream_,
+                               ws_running_.data() + q0 * k, (int)k, nq, ws_tau_.data() + q0);
+            int64_t seen = head;
+            while (seen < ntotal_) {
+                const int64_t nbc = std::min<int64_t>({ntotal_ - seen, seen, (int64_t)1 << 22});
+                ScoreFilter<int32_t> flt{ws_tau_.data() + q0, ws_cnt_.data() + q0, ws_filter_.data(), cap, seen};
+                launch_score_tiles_i8_filtered(xd + q0 * d_, nq, base_.data() + seen * d_, nbc, d_, ws_qn_.data() + q0,
+                                               norms_.data() + seen, flt, stream_);
+                launch_merge_candidates_i32(ws_running_.data() + q0 * k, (int)k, flt, ws_tau_.data() + q0, nq,
+                                            overflow, stream_);
+                launches++;
+                seen += nbc;
+            }
         }
+        int ovf = 0;
+        if (fused) {
+            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, stream_));
+            IXA_HIP(hipStreamSynchronize(stream_));
+        }
+        if (!ovf) {
+            break;
+        }
+        fused = false;
+        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
     }
     hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,
                        ws_running_.data(), n * k, kMetricL2, ids_.data(), (int32_t)0x7fffffff, dd, ld);
@@ -542,7 +667,6 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     }
     float a = 0;
     IXA_HIP(hipEventElapsedTime(&a, ev_[0], ev_[1]));
-    (void)ms_score;
     stats_.ms_score = 0;
     stats_.ms_select = 0;
     stats_.ms_total = a;

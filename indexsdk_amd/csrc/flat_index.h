@@ -45,7 +45,8 @@ protected:
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
     DeviceBuffer<T> base_;
     DeviceBuffer<int64_t> ids_;
-    DeviceBuffer<unsigned long long> ws_running_;
+    DeviceBuffer<unsigned long long> ws_running_, ws_filter_;
+    DeviceBuffer<int32_t> ws_cnt_;   // per-query admitted-candidate counters + one overflow flag
     DeviceBuffer<T> ws_x_;
     FlatStats stats_;
 };
@@ -58,7 +59,7 @@ public:
     void reset();
 
 private:
-    DeviceBuffer<float> norms_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<float> norms_, ws_qn_, ws_scores_, ws_dist_, ws_tau_;
     DeviceBuffer<int32_t> ws_cand_, ws_idx_;
     DeviceBuffer<int64_t> ws_labels_;
 };
@@ -71,7 +72,7 @@ public:
     void reset();
 
 private:
-    DeviceBuffer<int32_t> norms_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<int32_t> norms_, ws_qn_, ws_scores_, ws_dist_, ws_tau_;
     DeviceBuffer<int64_t> ws_labels_;
 };
 

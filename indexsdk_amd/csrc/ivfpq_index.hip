@@ -766,9 +766,8 @@ void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
                 }
             }
             split_empty(sub, sc, 256, dsub_);
-            if (cfg_.spherical) {
-                normalise_rows(sub, 256, dsub_);
-            }
+            // cfg_.spherical is NOT applied to the sub-quantizers: the reference does normalise them
+            // (AscendIndexIVFPQImpl.cpp:1064-1067), which only makes sense for unit-norm sub-vectors
             std::copy(sub.begin(), sub.end(), cb.begin() + (size_t)m * 256 * dsub_);
         }
     }

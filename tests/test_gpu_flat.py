@@ -97,3 +97,42 @@ def test_flat_f32_padding_and_golden(ix, oracle):
     Dr, Ir = oracle.flat_f32(x[:5], q[:3], 9)
     assert np.array_equal(I, Ir) and np.array_equal(D, Dr)
     assert np.all(I[:, 5:] == -1) and np.all(D[:, 5:] == np.finfo(np.float32).max)
+
+
+def test_flat_i8_many_fused_chunks_and_overflow_fallback(ix, oracle):
+    # 150k rows: one seeded stretch through the score scratch, then several filtered chunks
+    rng = np.random.default_rng(77)
+    d, n, nq, k = 64, 150_000, 70, 50
+    base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=8 << 20)
+    index.add(base)
+    D, I = index.search_int32(q, k)
+    Dr, Ir = oracle.flat_i8(base, q, k)
+    assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+    # adversarial order: every later row is closer to the query than all earlier ones, so the
+    # filtered chunks admit everything and overflow their candidate buffers -> exact fallback path
+    n2 = 60_000
+    ramp = np.zeros((n2, d), dtype=np.int8)
+    steps = np.linspace(127, 0, n2).astype(np.int64)
+    ramp[:, 0] = steps.astype(np.int8)
+    ramp[:, 1] = (np.arange(n2) % 100).astype(np.int8)      # breaks ties between equal first coordinates
+    q2 = np.zeros((3, d), dtype=np.int8)
+    index2 = ix.AscendIndexInt8Flat(d, ix.METRIC_L2)
+    index2.add(ramp)
+    D, I = index2.search_int32(q2, 20)
+    Dr, Ir = oracle.flat_i8(ramp, q2, 20)
+    assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+
+
+def test_flat_f32_many_fused_chunks(ix, oracle):
+    rng = np.random.default_rng(78)
+    d, n, nq, k = 32, 120_000, 40, 20
+    base = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    for metric in (ix.METRIC_L2, ix.METRIC_INNER_PRODUCT):
+        index = ix.AscendIndexFlat(d, metric, scratch_bytes=8 << 20)
+        index.add(base)
+        D, I = index.search(q, k)
+        Dr, Ir = oracle.flat_f32(base, q, k, metric)
+        assert np.array_equal(I, Ir) and np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
