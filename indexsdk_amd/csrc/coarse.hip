@@ -485,6 +485,7 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
                 const float *cv = C + (int64_t)c * d;
                 float g = 0.f;
                 if (VEC4) {
+#pragma unroll 8
                     for (int j = 0; j < d; j += 4) {
                         float4 a = *reinterpret_cast<const float4 *>(q + j);
                         float4 b = *reinterpret_cast<const float4 *>(cv + j);

@@ -5,6 +5,7 @@
 
 #include "coarse.h"
 #include "flat_index.h"
+#include "stream_select.h"
 #include "topk.h"
 
 namespace ixa {
@@ -247,33 +248,12 @@ __global__ __launch_bounds__(256) void finish_keys_kernel(const key_t *__restric
     out_labels[i] = ids[key_index(kk)];
 }
 
-__global__ __launch_bounds__(256) void keys_to_idx_kernel(const key_t *__restrict__ keys, int64_t n,
-                                                          int32_t *__restrict__ out)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) {
-        out[i] = keys[i] == kEmptyKey ? -1 : (int32_t)key_index(keys[i]);
-    }
-}
-
 __global__ __launch_bounds__(256) void map_labels_kernel(const int32_t *__restrict__ idx, int64_t n,
                                                          const int64_t *__restrict__ ids, int64_t *__restrict__ out)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) {
         out[i] = idx[i] < 0 ? -1 : ids[idx[i]];
-    }
-}
-
-// tau[row] = score of the last running key of the row, or the worst score while the row is not full.
-template <typename S>
-__global__ __launch_bounds__(256) void tau_from_running_kernel(const key_t *__restrict__ running, int k, int64_t n,
-                                                               S *__restrict__ tau)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) {
-        const key_t last = running[i * k + (k - 1)];
-        tau[i] = last == kEmptyKey ? ScoreOps<S>::worst() : key_score_as<S>(last);
     }
 }
 
@@ -468,68 +448,10 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
     IXA_HIP(hipEventRecord(ev_[0], stream_));
     launch_sqnorm_rows(xd, n, d_, ws_qn_.data(), stream_);
     IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
-    const int64_t qb = std::min<int64_t>(round_up(n, 128), 4096);
-    int64_t nb = scratch_bytes_ / (qb * 4);
-    nb = std::max<int64_t>(128, nb / 128 * 128);
-    nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
-    ws_scores_.resize((size_t)qb * nb);
-    int launches = 0;
-    // Pass 1 (streaming): a first stretch of the base goes through the score scratch and seeds the
-    // running keys; after that the score kernel itself drops everything above each query's current
-    // bound and only the few admitted candidates are merged -- no score ever reaches HBM again.
-    const int cap = pow2_ceil((int)std::max<int64_t>(1024, 8 * (int64_t)ncand));
-    const int64_t seed_rows = std::min<int64_t>(ntotal_, std::max<int64_t>(16384, 64 * (int64_t)ncand));
-    ws_tau_.resize((size_t)n);
-    ws_cnt_.resize((size_t)n + 1);
-    ws_filter_.resize((size_t)qb * cap);
-    IXA_HIP(hipMemsetAsync(ws_cnt_.data(), 0, ws_cnt_.bytes(), stream_));
-    int *overflow = ws_cnt_.data() + n;
-    bool fused = true;
-    for (int attempt = 0; attempt < 2; attempt++) {
-        for (int64_t q0 = 0; q0 < n; q0 += qb) {
-            const int64_t nq = std::min(qb, n - q0);
-            const int64_t head = fused ? seed_rows : ntotal_;
-            for (int64_t b0 = 0; b0 < head; b0 += nb) {
-                const int64_t nbc = std::min(nb, head - b0);
-                launch_score_tiles(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
-                                   norms_.data() + b0, metric_, ws_scores_.data(), nb, stream_);
-                launch_select_rows(ws_scores_.data(), nq, nb, nbc, ncand, nullptr, b0,
-                                   ws_running_.data() + q0 * ncand, stream_);
-                launches++;
-            }
-            if (!fused || head >= ntotal_) {
-                continue;
-            }
-            hipLaunchKernelGGL(tau_from_running_kernel<float>, dim3(blocks_for(nq)), dim3(256), 0, stream_,
-                               ws_running_.data() + q0 * ncand, ncand, nq, ws_tau_.data() + q0);
-            int64_t seen = head;
-            while (seen < ntotal_) {
-                const int64_t nbc = std::min<int64_t>({ntotal_ - seen, seen, (int64_t)1 << 22});
-                ScoreFilter<float> flt{ws_tau_.data() + q0, ws_cnt_.data() + q0, ws_filter_.data(), cap, seen};
-                launch_score_tiles_filtered(xd + q0 * d_, nq, base_.data() + seen * d_, nbc, d_, ws_qn_.data() + q0,
-                                            norms_.data() + seen, metric_, flt, stream_);
-                launch_merge_candidates(ws_running_.data() + q0 * ncand, ncand, flt, ws_tau_.data() + q0, nq, overflow,
-                                        stream_);
-                launches++;
-                seen += nbc;
-            }
-        }
-        int ovf = 0;
-        if (fused) {
-            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, stream_));
-            IXA_HIP(hipStreamSynchronize(stream_));
-        }
-        if (!ovf) {
-            break;
-        }
-        // a row admitted more candidates than its buffer holds (adversarial base order): redo the
-        // whole search through the score scratch, which has no such limit
-        fused = false;
-        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
-    }
+    const int launches = stream_select_f32(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), metric_,
+                                           ncand, ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
-    hipLaunchKernelGGL(keys_to_idx_kernel, dim3(blocks_for(n * ncand)), dim3(256), 0, stream_, ws_running_.data(),
-                       n * ncand, ws_cand_.data());
+    launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
     launch_refine(xd, n, base_.data(), d_, ws_qn_.data(), norms_.data(), metric_, ws_cand_.data(), ncand,
                   (int)std::min<int64_t>(k, ncand), (int)k, ws_idx_.data(), dd, stream_);
     hipLaunchKernelGGL(map_labels_kernel, dim3(blocks_for(n * k)), dim3(256), 0, stream_, ws_idx_.data(), n * k,
@@ -601,62 +523,8 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_, xd, n, d_,
                        ws_qn_.data());
     IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
-    const int64_t qb = std::min<int64_t>(round_up(n, 128), 4096);
-    int64_t nb = scratch_bytes_ / (qb * 4);
-    nb = std::max<int64_t>(128, nb / 128 * 128);
-    nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(ntotal_, 1), 128));
-    ws_scores_.resize((size_t)qb * nb);
-    int launches = 0;
-    // same two-phase scheme as the fp32 Flat search: seed through the score scratch, then let the
-    // score kernel admit only what beats each query's current k-th distance
-    const int cap = pow2_ceil((int)std::max<int64_t>(1024, 8 * k));
-    const int64_t seed_rows = std::min<int64_t>(ntotal_, std::max<int64_t>(16384, 64 * k));
-    ws_tau_.resize((size_t)n);
-    ws_cnt_.resize((size_t)n + 1);
-    ws_filter_.resize((size_t)qb * cap);
-    IXA_HIP(hipMemsetAsync(ws_cnt_.data(), 0, ws_cnt_.bytes(), stream_));
-    int *overflow = ws_cnt_.data() + n;
-    bool fused = true;
-    for (int attempt = 0; attempt < 2; attempt++) {
-        for (int64_t q0 = 0; q0 < n; q0 += qb) {
-            const int64_t nq = std::min(qb, n - q0);
-            const int64_t head = fused ? seed_rows : ntotal_;
-            for (int64_t b0 = 0; b0 < head; b0 += nb) {
-                const int64_t nbc = std::min(nb, head - b0);
-                launch_score_tiles_i8(xd + q0 * d_, nq, base_.data() + b0 * d_, nbc, d_, ws_qn_.data() + q0,
-                                      norms_.data() + b0, ws_scores_.data(), nb, stream_);
-                launch_select_rows_i32(ws_scores_.data(), nq, nb, nbc, (int)k, nullptr, b0,
-                                       ws_running_.data() + q0 * k, stream_);
-                launches++;
-            }
-            if (!fused || head >= ntotal_) {
-                continue;
-            }
-            hipLaunchKernelGGL(tau_from_running_kernel<int32_t>, dim3(blocks_for(nq)), dim3(256), 0, stream_,
-                               ws_running_.data() + q0 * k, (int)k, nq, ws_tau_.data() + q0);
-            int64_t seen = head;
-            while (seen < ntotal_) {
-                const int64_t nbc = std::min<int64_t>({ntotal_ - seen, seen, (int64_t)1 << 22});
-                ScoreFilter<int32_t> flt{ws_tau_.data() + q0, ws_cnt_.data() + q0, ws_filter_.data(), cap, seen};
-                launch_score_tiles_i8_filtered(xd + q0 * d_, nq, base_.data() + seen * d_, nbc, d_, ws_qn_.data() + q0,
-                                               norms_.data() + seen, flt, stream_);
-                launch_merge_candidates_i32(ws_running_.data() + q0 * k, (int)k, flt, ws_tau_.data() + q0, nq,
-                                            overflow, stream_);
-                launches++;
-                seen += nbc;
-            }
-        }
-        int ovf = 0;
-        if (fused) {
-            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, stream_));
-            IXA_HIP(hipStreamSynchronize(stream_));
-        }
-        if (!ovf) {
-            break;
-        }
-        fused = false;
-        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
-    }
+    const int launches = stream_select_i8(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), (int)k,
+                                          ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
     hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,
                        ws_running_.data(), n * k, kMetricL2, ids_.data(), (int32_t)0x7fffffff, dd, ld);
     IXA_HIP(hipEventRecord(ev_[1], stream_));

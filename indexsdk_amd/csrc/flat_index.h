@@ -9,6 +9,7 @@
 #include <cstdint>
 
 #include "common.h"
+#include "stream_select.h"
 
 namespace ixa {
 
@@ -45,8 +46,7 @@ protected:
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
     DeviceBuffer<T> base_;
     DeviceBuffer<int64_t> ids_;
-    DeviceBuffer<unsigned long long> ws_running_, ws_filter_;
-    DeviceBuffer<int32_t> ws_cnt_;   // per-query admitted-candidate counters + one overflow flag
+    DeviceBuffer<unsigned long long> ws_running_;
     DeviceBuffer<T> ws_x_;
     FlatStats stats_;
 };
@@ -59,7 +59,8 @@ public:
     void reset();
 
 private:
-    DeviceBuffer<float> norms_, ws_qn_, ws_scores_, ws_dist_, ws_tau_;
+    DeviceBuffer<float> norms_, ws_qn_, ws_dist_;
+    StreamSelectWorkspace<float> ws_sel_;
     DeviceBuffer<int32_t> ws_cand_, ws_idx_;
     DeviceBuffer<int64_t> ws_labels_;
 };
@@ -72,7 +73,8 @@ public:
     void reset();
 
 private:
-    DeviceBuffer<int32_t> norms_, ws_qn_, ws_scores_, ws_dist_, ws_tau_;
+    DeviceBuffer<int32_t> norms_, ws_qn_, ws_dist_;
+    StreamSelectWorkspace<int32_t> ws_sel_;
     DeviceBuffer<int64_t> ws_labels_;
 };
 

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "stream_select.h"
 
 namespace ixa {
 
@@ -97,7 +98,9 @@ private:
     std::vector<int32_t> list_len_;
     int64_t total_slots_ = 0;
     // search workspaces (grown on demand, reused between calls)
-    DeviceBuffer<float> ws_x_, ws_qn_, ws_scores_, ws_dist_;
+    DeviceBuffer<float> ws_x_, ws_qn_, ws_dist_;
+    StreamSelectWorkspace<float> ws_sel_;
+    DeviceBuffer<unsigned long long> ws_running_;
     DeviceBuffer<int32_t> ws_cand_, ws_probes_;
     DeviceBuffer<int64_t> ws_labels_;
     DeviceBuffer<unsigned long long> ws_partial_, ws_counter_;

@@ -3,6 +3,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 #include <random>
@@ -11,6 +12,7 @@
 #include "coarse.h"
 #include "pq.h"
 #include "scan.h"
+#include "stream_select.h"
 
 namespace ixa {
 
@@ -235,20 +237,14 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     const int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
-    int64_t rows = cfg_.scratch_bytes / ((int64_t)nlist_ * 4);
-    rows = std::max<int64_t>(128, rows / 128 * 128);
-    rows = std::min<int64_t>(rows, round_up(n, 128));
-    ws_scores_.resize((size_t)rows * nlist_);
-    ws_cand_.resize((size_t)rows * ncand);
-    for (int64_t r0 = 0; r0 < n; r0 += rows) {
-        const int64_t nr = std::min(rows, n - r0);
-        launch_score_tiles(x_dev + r0 * d_, nr, centroids_.data(), nlist_, d_, ws_qn_.data() + r0, cnorm_.data(),
-                           select_metric, ws_scores_.data(), nlist_, stream_);
-        launch_select_rows(ws_scores_.data(), nr, nlist_, nlist_, ncand, ws_cand_.data(), 0, nullptr, stream_);
-        launch_refine(x_dev + r0 * d_, nr, centroids_.data(), d_, ws_qn_.data() + r0, cnorm_.data(), select_metric,
-                      ws_cand_.data(), ncand, nout, nout, out_ids + r0 * nout,
-                      out_dist ? out_dist + r0 * nout : nullptr, stream_);
-    }
+    ws_running_.resize((size_t)n * ncand);
+    ws_cand_.resize((size_t)n * ncand);
+    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+    stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric, ncand,
+                      ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
+    launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
+    launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric, ws_cand_.data(), ncand,
+                  nout, nout, out_ids, out_dist, stream_);
 }
 
 void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)
@@ -568,6 +564,8 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     }
     p.out_dist = dd;
     p.out_labels = ld;
+    p.order = nullptr;
+    p.xcd_chunks = (getenv("IXA_XCD_CHUNKS") && nsplit == 1) ? 1 : 0;
     launch_scan(p, n, stream_);
     IXA_HIP(hipEventRecord(ev_[2], stream_));
 

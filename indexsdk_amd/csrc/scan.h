@@ -26,6 +26,10 @@ struct ScanParams {
     unsigned long long *partial;  // [nq][nsplit][k] keys
     float *out_dist;           // [nq][k]
     int64_t *out_labels;       // [nq][k]
+    // scheduling
+    const int32_t *order;      // optional permutation of the queries (execution order), may be null
+    int xcd_chunks;            // 1: deal contiguous chunks of the execution order to the 8 XCDs
+    int64_t nq;                // filled by launch_scan()
     // filled by plan_scan()
     int waves, cap, merge_n, table_n, off_query, off_pools, off_merge, off_table, off_misc;
 };

@@ -69,7 +69,18 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
     // the wavefront index is uniform: keeping it (and everything derived from it) in scalar
     // registers turns the group bookkeeping below into scalar code
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int64_t q = blockIdx.x / p.nsplit;
+    // Workgroups are dealt to the 8 XCDs round-robin.  With xcd_chunks the query order is cut into 8
+    // contiguous chunks, one per XCD, so that neighbouring queries (which tend to probe the same
+    // lists when the caller orders them by locality) share one L2.
+    int64_t qslot = blockIdx.x / p.nsplit;
+    if (p.xcd_chunks) {
+        const int64_t per = (p.nq + 7) / 8;
+        qslot = (qslot & 7) * per + (qslot >> 3);
+        if (qslot >= p.nq) {
+            return;
+        }
+    }
+    const int64_t q = p.order ? p.order[qslot] : qslot;
     const int split = blockIdx.x % p.nsplit;
 
     // ---- list table of this workgroup: local list i = probe rank split + i * nsplit
@@ -348,20 +359,21 @@ void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_
 template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
+    const int64_t slots = p.xcd_chunks ? (nq + 7) / 8 * 8 : nq;
     if (p.waves == 8) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8>;
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         }
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(512), smem, s, p);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4>;
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         }
-        hipLaunchKernelGGL(kern, dim3((unsigned)(nq * p.nsplit)), dim3(256), smem, s, p);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(256), smem, s, p);
     }
 }
 
@@ -424,6 +436,7 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
     if (nq == 0) {
         return;
     }
+    p.nq = nq;
     const size_t smem = plan_scan(p);
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam,
                 "IVFPQ scan needs %zu bytes of LDS (M=%d, k=%d, %s LUT); the limit is 163840", smem, p.M, p.k,

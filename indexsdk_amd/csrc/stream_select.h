@@ -1,0 +1,32 @@
+// Streaming brute-force selection: the best `ncand` base rows for every query row, kept as sorted
+// keys, without ever materialising more than a bounded stretch of the score matrix.
+#pragma once
+#include "coarse.h"
+
+namespace ixa {
+
+template <typename S>
+struct StreamSelectWorkspace {
+    DeviceBuffer<S> scores, tau;
+    DeviceBuffer<int32_t> cnt;                    // per-query admitted-candidate counters + overflow flag
+    DeviceBuffer<unsigned long long> filter;
+};
+
+// running[nq][ncand] must be filled with 0xff bytes by the caller; on return (the stream has been
+// synchronised) it holds each query's best ncand keys (ordered score << 32 | base row), ascending.
+// A first stretch of the base goes through a score scratch of at most scratch_bytes and seeds
+// the running keys; afterwards the score kernel admits only what beats each query's current
+// ncand-th score and the admitted keys are merged.  If a query ever admits more keys than its
+// buffer holds (adversarial base order), the whole selection is redone through the scratch.
+// Returns the number of score launches.
+int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn, const float *bn,
+                      int metric, int ncand, unsigned long long *running, StreamSelectWorkspace<float> &ws,
+                      int64_t scratch_bytes, hipStream_t s);
+int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                     const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
+                     int64_t scratch_bytes, hipStream_t s);
+
+// idx[i] = row index of keys[i], or -1 for an empty key.
+void launch_keys_to_idx(const unsigned long long *keys, int64_t n, int32_t *idx, hipStream_t s);
+
+}  // namespace ixa

@@ -1,0 +1,182 @@
+// Host driver of the streaming brute-force selection (see stream_select.h).
+#include "stream_select.h"
+
+#include <algorithm>
+
+#include "topk.h"
+
+namespace ixa {
+
+namespace {
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+// tau[row] = score of the last running key of the row, or the worst score while the row is not full.
+template <typename S>
+__global__ __launch_bounds__(256) void tau_from_running_kernel(const key_t *__restrict__ running, int k, int64_t n,
+                                                               S *__restrict__ tau)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const key_t last = running[i * k + (k - 1)];
+        tau[i] = last == kEmptyKey ? ScoreOps<S>::worst() : key_score_as<S>(last);
+    }
+}
+
+__global__ __launch_bounds__(256) void keys_to_idx_kernel(const key_t *__restrict__ keys, int64_t n,
+                                                          int32_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        out[i] = keys[i] == kEmptyKey ? -1 : (int32_t)key_index(keys[i]);
+    }
+}
+
+struct F32Ops {
+    using T = float;
+    using S = float;
+    const float *qn, *bn;
+    int metric;
+    void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
+                hipStream_t s) const
+    {
+        launch_score_tiles(Q, nq, B, nb, d, qn + q0, bn + b0, metric, out, ldo, s);
+    }
+    void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
+                  hipStream_t s) const
+    {
+        launch_score_tiles_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, metric, flt, s);
+    }
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    {
+        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s);
+    }
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    {
+        launch_merge_candidates(run, k, flt, tau, nq, ovf, s);
+    }
+};
+
+struct I8Ops {
+    using T = int8_t;
+    using S = int32_t;
+    const int32_t *qn, *bn;
+    void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
+                hipStream_t s) const
+    {
+        launch_score_tiles_i8(Q, nq, B, nb, d, qn + q0, bn + b0, out, ldo, s);
+    }
+    void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
+                  hipStream_t s) const
+    {
+        launch_score_tiles_i8_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, flt, s);
+    }
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    {
+        launch_select_rows_i32(sc, nq, ld, nc, k, nullptr, base, run, s);
+    }
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    {
+        launch_merge_candidates_i32(run, k, flt, tau, nq, ovf, s);
+    }
+};
+
+template <typename Ops>
+int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, const typename Ops::T *B, int64_t nb_total,
+                  int d, int ncand, key_t *running, StreamSelectWorkspace<typename Ops::S> &ws, int64_t scratch_bytes,
+                  hipStream_t s)
+{
+    using S = typename Ops::S;
+    if (nq_total == 0) {
+        return 0;
+    }
+    const int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
+    int64_t nb = scratch_bytes / (qb * (int64_t)sizeof(S));
+    nb = std::max<int64_t>(128, nb / 128 * 128);
+    nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(nb_total, 1), 128));
+    const int cap = pow2_ceil((int)std::max<int64_t>(1024, 16 * (int64_t)ncand));
+    const int64_t seed_rows = std::min<int64_t>(nb_total, std::max<int64_t>(2048, 16 * (int64_t)ncand));
+    // when the whole score matrix of a query block fits the scratch, one materialised pass is the
+    // cheapest plan (this is the IVFPQ coarse stage); the filtered plan is for long bases
+    const bool can_fuse = nb_total > nb && seed_rows < nb_total && pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    // the scratch only has to hold the seeding stretch unless the fallback is taken
+    ws.scores.resize((size_t)qb * (can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb));
+    const int64_t ld = can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb;
+    ws.tau.resize((size_t)nq_total);
+    ws.cnt.resize((size_t)nq_total + 1);
+    if (can_fuse) {
+        ws.filter.resize((size_t)qb * cap);
+    }
+    IXA_HIP(hipMemsetAsync(ws.cnt.data(), 0, ws.cnt.bytes(), s));
+    int *overflow = ws.cnt.data() + nq_total;
+    int launches = 0;
+    bool fused = can_fuse;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        int64_t ldo = ld;
+        if (!fused && can_fuse) {
+            ws.scores.resize((size_t)qb * nb);  // fallback: the scratch walks the whole base
+            ldo = nb;
+        }
+        for (int64_t q0 = 0; q0 < nq_total; q0 += qb) {
+            const int64_t nq = std::min(qb, nq_total - q0);
+            const int64_t head = fused ? seed_rows : nb_total;
+            for (int64_t b0 = 0; b0 < head; b0 += ldo) {
+                const int64_t nbc = std::min(ldo, head - b0);
+                ops.scores(Q + q0 * d, nq, q0, B + b0 * d, nbc, b0, d, ws.scores.data(), ldo, s);
+                ops.select(ws.scores.data(), nq, ldo, nbc, ncand, b0, running + q0 * ncand, s);
+                launches++;
+            }
+            if (!fused) {
+                continue;
+            }
+            hipLaunchKernelGGL(tau_from_running_kernel<S>, dim3(blocks_for(nq)), dim3(256), 0, s,
+                               running + q0 * ncand, ncand, nq, ws.tau.data() + q0);
+            int64_t seen = head;
+            while (seen < nb_total) {
+                // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query
+                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * 2, (int64_t)1 << 22});
+                ScoreFilter<S> flt{ws.tau.data() + q0, ws.cnt.data() + q0, ws.filter.data(), cap, seen};
+                ops.filtered(Q + q0 * d, nq, q0, B + seen * d, nbc, seen, d, flt, s);
+                ops.merge(running + q0 * ncand, ncand, flt, ws.tau.data() + q0, nq, overflow, s);
+                launches++;
+                seen += nbc;
+            }
+        }
+        int ovf = 0;
+        if (fused) {
+            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, s));
+        }
+        IXA_HIP(hipStreamSynchronize(s));
+        if (!ovf) {
+            break;
+        }
+        fused = false;
+        IXA_HIP(hipMemsetAsync(running, 0xff, (size_t)nq_total * ncand * sizeof(key_t), s));
+    }
+    return launches;
+}
+
+}  // namespace
+
+int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn, const float *bn,
+                      int metric, int ncand, unsigned long long *running, StreamSelectWorkspace<float> &ws,
+                      int64_t scratch_bytes, hipStream_t s)
+{
+    return stream_select(F32Ops{qn, bn, metric}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s);
+}
+
+int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                     const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
+                     int64_t scratch_bytes, hipStream_t s)
+{
+    return stream_select(I8Ops{qn, bn}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s);
+}
+
+void launch_keys_to_idx(const unsigned long long *keys, int64_t n, int32_t *idx, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(keys_to_idx_kernel, dim3(blocks_for(n)), dim3(256), 0, s, keys, n, idx);
+    }
+}
+
+}  // namespace ixa
