@@ -13,6 +13,7 @@ void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_
 template <typename S>
 struct ScoreFilter {
     const S *tau;              // [nq] admission bound per row
+    const S *thr;              // [nq] tau - |q|^2 (exact integer scores only; may be null)
     int32_t *cnt;              // [nq] number of appended keys
     unsigned long long *cand;  // [nq][cap]
     int cap;

@@ -7,7 +7,7 @@ namespace ixa {
 
 template <typename S>
 struct StreamSelectWorkspace {
-    DeviceBuffer<S> scores, tau;
+    DeviceBuffer<S> scores, tau, thr;
     DeviceBuffer<int32_t> cnt;                    // per-query admitted-candidate counters + overflow flag
     DeviceBuffer<unsigned long long> filter;
 };

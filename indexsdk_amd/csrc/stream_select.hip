@@ -32,11 +32,23 @@ __global__ __launch_bounds__(256) void keys_to_idx_kernel(const key_t *__restric
     }
 }
 
+// thr[i] = tau[i] - qn[i]
+__global__ __launch_bounds__(256) void threshold_i32_kernel(const int32_t *__restrict__ tau,
+                                                            const int32_t *__restrict__ qn, int64_t n,
+                                                            int32_t *__restrict__ thr)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        thr[i] = tau[i] - qn[i];   // tau <= INT32_MAX and qn >= 0: no overflow
+    }
+}
+
 struct F32Ops {
     using T = float;
     using S = float;
     const float *qn, *bn;
     int metric;
+    const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
     void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
                 hipStream_t s) const
     {
@@ -61,6 +73,12 @@ struct I8Ops {
     using T = int8_t;
     using S = int32_t;
     const int32_t *qn, *bn;
+    const S *threshold(StreamSelectWorkspace<S> &ws, int64_t q0, int64_t nq, hipStream_t s) const
+    {
+        hipLaunchKernelGGL(threshold_i32_kernel, dim3(blocks_for(nq)), dim3(256), 0, s, ws.tau.data() + q0, qn + q0, nq,
+                           ws.thr.data() + q0);
+        return ws.thr.data() + q0;
+    }
     void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
                 hipStream_t s) const
     {
@@ -103,6 +121,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     ws.scores.resize((size_t)qb * (can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb));
     const int64_t ld = can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb;
     ws.tau.resize((size_t)nq_total);
+    ws.thr.resize((size_t)nq_total);
     ws.cnt.resize((size_t)nq_total + 1);
     if (can_fuse) {
         ws.filter.resize((size_t)qb * cap);
@@ -135,7 +154,8 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             while (seen < nb_total) {
                 // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query
                 const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * 2, (int64_t)1 << 22});
-                ScoreFilter<S> flt{ws.tau.data() + q0, ws.cnt.data() + q0, ws.filter.data(), cap, seen};
+                ScoreFilter<S> flt{ws.tau.data() + q0, ops.threshold(ws, q0, nq, s), ws.cnt.data() + q0, ws.filter.data(), cap,
+                                   seen};
                 ops.filtered(Q + q0 * d, nq, q0, B + seen * d, nbc, seen, d, flt, s);
                 ops.merge(running + q0 * ncand, ncand, flt, ws.tau.data() + q0, nq, overflow, s);
                 launches++;
