@@ -248,29 +248,33 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
         pool.bound = b < pool.bound ? b : pool.bound;
     };
     // One step: start the loads of the group after next, evaluate the current group, offer it to
-    // the pool.  Two register sets alternate so that no code registers are ever copied.
-    auto step = [&](int G, const GroupRef &cur, const uint32_t (&wcur)[NW], GroupRef &nxt, uint32_t (&wnxt)[NW]) {
-        if (G + W < total) {
-            nxt = locate(G + W);
-            load_codes(nxt.slot, wnxt);   // in flight while the current group is evaluated
-        }
-        const float s = adc(cur.slot, wcur);
-        const bool compacted = pool.push(cur.valid && s <= pool.bound, s, cur.slot, lane, &share[wave], share_rank);
-        if (compacted || (G & (16 * W - 1)) < W) {
-            adopt_shared();
-        }
-    };
+    // the pool.  Two register sets (a, b) alternate so that no code registers are ever copied; the
+    // step is a macro so that both sets stay in registers (no address of either is ever taken).
+#define IXA_SCAN_STEP(G, CUR, WCUR, NXT, WNXT)                                                        \
+    do {                                                                                              \
+        if ((G) + W < total) {                                                                        \
+            NXT = locate((G) + W);                                                                    \
+            load_codes(NXT.slot, WNXT); /* in flight while the current group is evaluated */          \
+        }                                                                                             \
+        const float s_ = adc(CUR.slot, WCUR);                                                         \
+        const bool compacted_ =                                                                       \
+            pool.push(CUR.valid && s_ <= pool.bound, s_, CUR.slot, lane, &share[wave], share_rank);   \
+        if (compacted_ || ((G) & (16 * W - 1)) < W) {                                                 \
+            adopt_shared();                                                                           \
+        }                                                                                             \
+    } while (0)
     if (wave < total) {
         uint32_t wa[NW], wb[NW];
         GroupRef ga = locate(wave), gb = ga;
         load_codes(ga.slot, wa);
         for (int G = wave; G < total; G += 2 * W) {
-            step(G, ga, wa, gb, wb);
+            IXA_SCAN_STEP(G, ga, wa, gb, wb);
             if (G + W < total) {
-                step(G + W, gb, wb, ga, wa);
+                IXA_SCAN_STEP(G + W, gb, wb, ga, wa);
             }
         }
     }
+#undef IXA_SCAN_STEP
     __syncthreads();  // every wave has published its last value; the LUT is no longer needed
     adopt_shared();
     pool.finish(lane);

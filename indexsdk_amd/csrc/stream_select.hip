@@ -153,7 +153,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             int64_t seen = head;
             while (seen < nb_total) {
                 // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query
-                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * 2, (int64_t)1 << 22});
+                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * 4, (int64_t)1 << 23});
                 ScoreFilter<S> flt{ws.tau.data() + q0, ops.threshold(ws, q0, nq, s), ws.cnt.data() + q0, ws.filter.data(), cap,
                                    seen};
                 ops.filtered(Q + q0 * d, nq, q0, B + seen * d, nbc, seen, d, flt, s);
