@@ -242,10 +242,10 @@ def main():
         del src, dst
 
     # HBM traffic of the scan kernel per launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by the
-    # copy probe (profiles/ivfpq_scan_kernel_c2_10M_traffic.md): 1.042 x the algorithmic bytes are fetched,
+    # copy probe (profiles/ivfpq_scan_kernel_c2_10M_traffic.md): 1.030 x the algorithmic bytes are fetched,
     # 12.2 MB are written.  Only quoted for the default workload it was measured on.
     default_c2 = args.workload == "C2" and not any(getattr(args, key) for key in ("n", "nq", "nlist", "nprobe", "k"))
-    traffic = 1.042 * scan_bytes + 12.2e6 if default_c2 else None
+    traffic = 1.030 * scan_bytes + 12.2e6 if default_c2 else None
     layout_name = "rot32" if (args.layout != 0 and M in (32, 64, 96)) else "row"
     result = {
         "metric": "queries/sec and ADC-scan GB/s (% HBM peak) at k=100 on 1 MI355X",
