@@ -35,6 +35,16 @@ void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<flo
 void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter<int32_t> flt, int32_t *tau,
                                  int64_t nq, int *overflow, hipStream_t s);
 
+// Persistent ring kernels (score_ring.hip): same results as the tile kernels, at a much higher
+// matrix-core rate.  Return false when the shape does not qualify (d not a multiple of one K-step,
+// fewer than 1024 base rows, unaligned operands); nothing has been launched then.
+bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                          const int32_t *bn, int32_t *out, int64_t ldo, bool filter, ScoreFilter<int32_t> flt,
+                          hipStream_t s);
+bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn,
+                           const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
+                           hipStream_t s);
+
 // Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
 // indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
 // (ordered score << 32) | (col_base + column): its content takes part in the selection and is

@@ -217,6 +217,9 @@ static void launch_score_tiles_t(const float *Q, int64_t nq, const float *C, int
     if (nq == 0 || nc == 0) {
         return;
     }
+    if (launch_score_ring_f32(Q, nq, C, nc, d, qn, cn, metric, out, ldo, FILTER, flt, s)) {
+        return;
+    }
     const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nc + kTile - 1) / kTile;
     const int64_t nblocks = (tiles_n + 7) / 8 * 8 * tiles_m;
     IXA_REQUIRE(nblocks < (int64_t)1 << 31 && tiles_m < (1 << 28), kErrInvalidParam, "score tile grid too large");

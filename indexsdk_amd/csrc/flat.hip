@@ -190,199 +190,6 @@ __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__rest
 
 }  // namespace
 
-// ---- persistent ring kernel ---------------------------------------------------------------------
-// The same exact int32 score tile, restructured for the int8 matrix rate (a 128-byte K-step of MFMAs
-// takes only a few hundred cycles, far less than a trip to L2/HBM):
-//   * a workgroup is persistent and walks a list of 256 x 128 tiles; the stream of K-steps runs
-//     continuously across tile boundaries;
-//   * operands go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
-//     into a ring of kStages buffers, kStages - 1 steps ahead of the MFMAs;
-//   * each wavefront owns 128 x 64 of the tile (4 x 2 blocks of v_mfma_i32_32x32x32_i8), so one
-//     operand fragment read from LDS feeds 1.33 MFMAs on average;
-//   * rows are stored unpadded (64 bytes per row and step); the 16-byte chunk index is XOR-swizzled
-//     with bits 2-3 of the row, which makes the 128-bit fragment reads of 16 consecutive rows hit
-//     16 different bank groups;
-//   * tiles are dealt so that all workgroups of an XCD work on the same base tile at the same time.
-constexpr int kRingTM = 256, kRingTN = 128, kRingRows = kRingTM + kRingTN;
-constexpr int kRingStageBytes = kRingRows * 64;
-constexpr int kRingStages = 3;
-constexpr int kRingLoadsPerWave = kRingRows / 16 / 4;  // wave-wide 1 KB loads per stage and wavefront
-
-template <bool FILTER>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void score_ring_i8_kernel(const int8_t *__restrict__ Q, int64_t nq,
-                                                            const int8_t *__restrict__ B, int64_t nb, int d,
-                                                            const int32_t *__restrict__ qn,
-                                                            const int32_t *__restrict__ bn, int32_t *__restrict__ out,
-                                                            int64_t ldo, int tiles_m, int tiles_n,
-                                                            ScoreFilter<int32_t> flt)
-{
-    extern __shared__ __align__(16) unsigned char ring[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave >> 1, wc = wave & 1;
-    const int half = lane >> 5, l32 = lane & 31;
-    const int nk = d / 64;
-
-    // work list: XCD x owns base tiles x, x + 8, ...; its workgroups take (base tile, query tile)
-    // pairs round-robin, query tile fastest
-    const int xcd = blockIdx.x & 7, wi = blockIdx.x >> 3, wpx = gridDim.x >> 3;
-    const int own_n = tiles_n > xcd ? (tiles_n - xcd + 7) / 8 : 0;
-    const int64_t items = (int64_t)own_n * tiles_m;
-    const int my_items = items > wi ? (int)((items - wi + wpx - 1) / wpx) : 0;   // host keeps this below 2^24
-    const int total = my_items * nk;
-    if (total == 0) {
-        return;
-    }
-    auto item_tile = [&](int it, int64_t &tm, int64_t &tn) {
-        const uint32_t t = (uint32_t)wi + (uint32_t)it * (uint32_t)wpx;
-        tn = xcd + 8 * (int64_t)(t / (uint32_t)tiles_m);
-        tm = t % (uint32_t)tiles_m;
-    };
-
-    // issue the loads of one K-step (item it, step ks) into ring buffer `slot`
-    auto issue = [&](int it, int ks, int slot) {
-        int64_t tm, tn;
-        item_tile(it, tm, tn);
-        unsigned char *stage = ring + slot * kRingStageBytes;
-#pragma unroll
-        for (int j = 0; j < kRingLoadsPerWave; j++) {
-            const int rg = wave * kRingLoadsPerWave + j;          // group of 16 stage rows
-            const int row = rg * 16 + (lane >> 2);                // stage row: 0..255 queries, 256..383 base
-            const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-            const int8_t *src;
-            if (rg < kRingTM / 16) {
-                int64_t r = tm * kRingTM + row;
-                r = r < nq ? r : nq - 1;
-                src = Q + r * d;
-            } else {
-                int64_t r = tn * kRingTN + (row - kRingTM);
-                r = r < nb ? r : nb - 1;
-                src = B + r * d;
-            }
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(src + ks * 64 + chunk * 16),
-                (__attribute__((address_space(3))) void *)(stage + rg * 1024), 16, 0, 0);
-        }
-    };
-
-    v16i acc[4][2];
-#pragma unroll
-    for (int a = 0; a < 4; a++) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[a][b][r] = 0;
-            }
-        }
-    }
-
-    // (item, step, ring slot) of the next K-step to issue and of the one being computed
-    int issued = 0, i_it = 0, i_ks = 0, i_slot = 0;
-    auto issue_next = [&]() {
-        issue(i_it, i_ks, i_slot);
-        issued++;
-        i_slot = i_slot + 1 == kRingStages ? 0 : i_slot + 1;
-        if (++i_ks == nk) {
-            i_ks = 0;
-            i_it++;
-        }
-    };
-    while (issued < kRingStages - 1 && issued < total) {
-        issue_next();
-    }
-    int c_it = 0, c_ks = 0, c_slot = 0;
-    for (int g = 0; g < total; g++) {
-        // the loads of step g must have landed; later steps may still be in flight
-        if (issued - g - 1 >= kRingStages - 2) {
-            __builtin_amdgcn_s_waitcnt(0x0f70 | ((kRingStages - 2) * kRingLoadsPerWave));
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0f70);
-        }
-        __builtin_amdgcn_s_barrier();
-        if (issued < total) {
-            issue_next();  // goes into the buffer that step g - 1 has just finished reading
-        }
-        const unsigned char *stage = ring + c_slot * kRingStageBytes;
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            const int c = kk * 2 + half;
-            v4i a[4], b[2];
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-                const int r = wr * 128 + ra * 32 + l32;
-                a[ra] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
-                const int r = kRingTM + wc * 64 + rb * 32 + l32;
-                b[rb] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-#pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
-                }
-            }
-        }
-        const bool last_step = c_ks == nk - 1;
-        const int done_it = c_it;
-        c_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
-        if (++c_ks == nk) {
-            c_ks = 0;
-            c_it++;
-        }
-        if (last_step) {
-            int64_t tm, tn;
-            item_tile(done_it, tm, tn);
-            const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
-            int32_t bnv[2];
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
-                const int64_t col = j0 + wc * 64 + rb * 32 + l32;
-                bnv[rb] = col < nb ? bn[col] : 0;
-            }
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-                // one 32-row block at a time keeps the per-row operands of only 16 rows live
-                asm volatile("" ::: "memory");
-                int32_t rowv[16];
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    // FILTER: thr = tau - |q|^2, so  |b|^2 - 2 q.b <= thr  <=>  distance <= tau
-                    rowv[r] = row < nq ? (FILTER ? flt.thr[row] : qn[row]) : (FILTER ? (int32_t)0x80000000 : 0);
-                }
-#pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-                    const int64_t col = j0 + wc * 64 + rb * 32 + l32;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int32_t part = bnv[rb] - 2 * acc[ra][rb][r];
-                        acc[ra][rb][r] = 0;
-                        if (FILTER) {
-                            if (part <= rowv[r] && col < nb) {
-                                const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                                const int32_t v = part + qn[row];
-                                const int pos = atomicAdd(&flt.cnt[row], 1);
-                                if (pos < flt.cap) {
-                                    flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
-                                }
-                            }
-                        } else {
-                            const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                            if (row < nq && col < nb) {
-                                out[row * ldo + col] = part + rowv[r];
-                            }
-                        }
-                    }
-                }
-            }
-        }
-    }
-}
-
 template <bool FILTER>
 static void launch_score_tiles_i8_t(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
                                     const int32_t *qn, const int32_t *bn, int32_t *out, int64_t ldo,
@@ -393,21 +200,7 @@ static void launch_score_tiles_i8_t(const int8_t *Q, int64_t nq, const int8_t *B
     }
     const bool vec = (d % 16 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(B) % 16 == 0);
-    if (vec && d % 64 == 0 && nb >= 8 * kRingTN) {
-        // persistent ring kernel: two workgroups per CU
-        const int64_t rt_m = (nq + kRingTM - 1) / kRingTM, rt_n = (nb + kRingTN - 1) / kRingTN;
-        IXA_REQUIRE(rt_m * rt_n < ((int64_t)1 << 31) && rt_m * ((rt_n + 7) / 8) * (d / 64) < ((int64_t)1 << 30),
-                    kErrInvalidParam, "score tile grid too large");
-        int dev = 0, cus = 256;
-        IXA_HIP(hipGetDevice(&dev));
-        IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        const unsigned grid = (unsigned)((2 * cus + 7) / 8 * 8);
-        const size_t smem = (size_t)kRingStages * kRingStageBytes;
-        auto kern = score_ring_i8_kernel<FILTER>;
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, Q, nq, B, nb, d, qn, bn, out, ldo, (int)rt_m,
-                           (int)rt_n, flt);
+    if (vec && launch_score_ring_i8(Q, nq, B, nb, d, qn, bn, out, ldo, FILTER, flt, s)) {
         return;
     }
     const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nb + kTile - 1) / kTile;

@@ -1,0 +1,344 @@
+// Persistent "ring" score kernels: query x base score tiles at matrix-core rate.
+//
+// A K-step of MFMAs lasts a few hundred (int8) to a few thousand (fp32) cycles, and a tile of the
+// headline shapes has only 8 K-steps, so a kernel that starts and drains a pipeline per tile spends
+// a large share of its time waiting for the first operands.  Here instead
+//   * a workgroup is persistent and walks a list of 256 x 128 tiles; the stream of K-steps (64 bytes
+//     of every operand row each) runs continuously across tile boundaries;
+//   * operands go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
+//     into a ring of kStages buffers, kStages - 1 steps ahead of the MFMAs; completion is tracked
+//     with s_waitcnt vmcnt + s_barrier, without the full memory fence of __syncthreads();
+//   * each wavefront owns 128 x 64 of the tile (4 x 2 blocks of 32 x 32), so one operand fragment
+//     read from LDS feeds 1.33 MFMA blocks on average;
+//   * rows are stored unpadded (64 bytes per row and step); the 16-byte chunk index is XOR-swizzled
+//     with bits 2-3 of the row, which makes the 128-bit fragment reads of 16 consecutive rows hit
+//     16 different bank groups;
+//   * tiles are dealt so that all workgroups of an XCD work on the same base tile at the same time
+//     (it is fetched from HBM once and re-used out of that XCD's L2);
+//   * two workgroups share a CU, so one's epilogue overlaps the other's MFMAs.
+// Scores: int8 -> exact int32 |q|^2 + |b|^2 - 2 q.b (v_mfma_i32_32x32x32_i8);
+//         fp32 -> (|q|^2 + |b|^2) - g - g or -g (v_mfma_f32_32x32x2_f32).
+// The sum over k is order-free for integers, and for fp32 any fixed k-assignment that is the same
+// for both operands is a valid accumulation order, so each lane half owns half of a K-step.
+#include "coarse.h"
+#include "topk.h"
+
+namespace ixa {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kRingTM = 256, kRingTN = 128, kRingRows = kRingTM + kRingTN;
+constexpr int kRingStageBytes = kRingRows * 64;
+constexpr int kRingStages = 3;
+constexpr int kRingLoadsPerWave = kRingRows / 16 / 4;  // wave-wide 1 KB loads per stage and wavefront
+
+struct I8Traits {
+    using T = int8_t;
+    using S = int32_t;
+    using Acc = v16i;
+    static constexpr int kElemsPerStep = 64;
+    // one K-step = 2 sub-steps of 32 bytes; a lane half owns 16 of them
+    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
+                                               Acc (&acc)[4][2])
+    {
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int c = kk * 2 + half;
+            v4i a[4], b[2];
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+                const int r = wr * 128 + ra * 32 + l32;
+                a[ra] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const int r = kRingTM + wc * 64 + rb * 32 + l32;
+                b[rb] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                }
+            }
+        }
+    }
+};
+
+struct F32Traits {
+    using T = float;
+    using S = float;
+    using Acc = v16f;
+    static constexpr int kElemsPerStep = 16;
+    // one K-step = 16 floats; a lane half owns 8 of them (two 16-byte chunks) and feeds them to 8
+    // consecutive 32x32x2 MFMAs
+    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
+                                               Acc (&acc)[4][2])
+    {
+        v4f a[4][2], b[2][2];
+#pragma unroll
+        for (int cc = 0; cc < 2; cc++) {
+            const int c = half * 2 + cc;
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+                const int r = wr * 128 + ra * 32 + l32;
+                a[ra][cc] = *reinterpret_cast<const v4f *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const int r = kRingTM + wc * 64 + rb * 32 + l32;
+                b[rb][cc] = *reinterpret_cast<const v4f *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    acc[ra][rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ra][t >> 2][t & 3], b[rb][t >> 2][t & 3],
+                                                                       acc[ra][rb], 0, 0, 0);
+                }
+            }
+        }
+    }
+};
+
+template <typename Tr, bool FILTER>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void score_ring_kernel(
+    const typename Tr::T *__restrict__ Q, int64_t nq, const typename Tr::T *__restrict__ B, int64_t nb, int d,
+    const typename Tr::S *__restrict__ qn, const typename Tr::S *__restrict__ bn, int metric,
+    typename Tr::S *__restrict__ out, int64_t ldo, int tiles_m, int tiles_n, ScoreFilter<typename Tr::S> flt)
+{
+    using T = typename Tr::T;
+    using S = typename Tr::S;
+    constexpr bool kInt = sizeof(T) == 1;
+    extern __shared__ __align__(16) unsigned char ring[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int nk = d / Tr::kElemsPerStep;
+    const int64_t row_bytes = (int64_t)d * sizeof(T);
+
+    // work list: XCD x owns base tiles x, x + 8, ...; its workgroups take (base tile, query tile)
+    // pairs round-robin, query tile fastest
+    const int xcd = blockIdx.x & 7, wi = blockIdx.x >> 3, wpx = gridDim.x >> 3;
+    const int own_n = tiles_n > xcd ? (tiles_n - xcd + 7) / 8 : 0;
+    const int64_t items = (int64_t)own_n * tiles_m;
+    const int my_items = items > wi ? (int)((items - wi + wpx - 1) / wpx) : 0;
+    const int total = my_items * nk;
+    if (total == 0) {
+        return;
+    }
+    auto item_tile = [&](int it, int64_t &tm, int64_t &tn) {
+        const uint32_t t = (uint32_t)wi + (uint32_t)it * (uint32_t)wpx;
+        tn = xcd + 8 * (int64_t)(t / (uint32_t)tiles_m);
+        tm = t % (uint32_t)tiles_m;
+    };
+    const unsigned char *Qb = reinterpret_cast<const unsigned char *>(Q);
+    const unsigned char *Bb = reinterpret_cast<const unsigned char *>(B);
+
+    // issue the loads of one K-step (item it, step ks) into ring buffer `slot`
+    auto issue = [&](int it, int ks, int slot) {
+        int64_t tm, tn;
+        item_tile(it, tm, tn);
+        unsigned char *stage = ring + slot * kRingStageBytes;
+#pragma unroll
+        for (int j = 0; j < kRingLoadsPerWave; j++) {
+            const int rg = wave * kRingLoadsPerWave + j;          // group of 16 stage rows
+            const int row = rg * 16 + (lane >> 2);                // stage row: 0..255 queries, 256..383 base
+            const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+            const unsigned char *src;
+            if (rg < kRingTM / 16) {
+                int64_t r = tm * kRingTM + row;
+                r = r < nq ? r : nq - 1;
+                src = Qb + r * row_bytes;
+            } else {
+                int64_t r = tn * kRingTN + (row - kRingTM);
+                r = r < nb ? r : nb - 1;
+                src = Bb + r * row_bytes;
+            }
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(src + ks * 64 + chunk * 16),
+                (__attribute__((address_space(3))) void *)(stage + rg * 1024), 16, 0, 0);
+        }
+    };
+
+    typename Tr::Acc acc[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[a][b][r] = 0;
+            }
+        }
+    }
+
+    // (item, step, ring slot) of the next K-step to issue and of the one being computed
+    int issued = 0, i_it = 0, i_ks = 0, i_slot = 0;
+    auto issue_next = [&]() {
+        issue(i_it, i_ks, i_slot);
+        issued++;
+        i_slot = i_slot + 1 == kRingStages ? 0 : i_slot + 1;
+        if (++i_ks == nk) {
+            i_ks = 0;
+            i_it++;
+        }
+    };
+    while (issued < kRingStages - 1 && issued < total) {
+        issue_next();
+    }
+    int c_it = 0, c_ks = 0, c_slot = 0;
+    for (int g = 0; g < total; g++) {
+        // the loads of step g must have landed; later steps may still be in flight
+        if (issued - g - 1 >= kRingStages - 2) {
+            __builtin_amdgcn_s_waitcnt(0x0f70 | ((kRingStages - 2) * kRingLoadsPerWave));
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+        }
+        __builtin_amdgcn_s_barrier();
+        if (issued < total) {
+            issue_next();  // goes into the buffer that step g - 1 has just finished reading
+        }
+        Tr::mma(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
+        const bool last_step = c_ks == nk - 1;
+        const int done_it = c_it;
+        c_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
+        if (++c_ks == nk) {
+            c_ks = 0;
+            c_it++;
+        }
+        if (last_step) {
+            int64_t tm, tn;
+            item_tile(done_it, tm, tn);
+            const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
+            S bnv[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const int64_t col = j0 + wc * 64 + rb * 32 + l32;
+                bnv[rb] = (col < nb && (kInt || metric == kMetricL2)) ? bn[col] : (S)0;
+            }
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+                // one 32-row block at a time keeps the per-row operands of only 16 rows live
+                asm volatile("" ::: "memory");
+                S rowv[16];   // int8 + FILTER: tau - |q|^2; otherwise |q|^2
+                S tauv[16];   // fp32 + FILTER: tau
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    if (kInt) {
+                        // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
+                        rowv[r] = row < nq ? (FILTER ? flt.thr[row] : qn[row]) : (FILTER ? (S)0x80000000 : (S)0);
+                    } else {
+                        rowv[r] = (row < nq && metric == kMetricL2) ? qn[row] : (S)0;
+                        tauv[r] = (FILTER && row < nq) ? flt.tau[row] : (S)(-__builtin_inff());
+                    }
+                }
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    const int64_t col = j0 + wc * 64 + rb * 32 + l32;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        S v;
+                        bool admit;
+                        if constexpr (kInt) {
+                            const S part = bnv[rb] - 2 * acc[ra][rb][r];
+                            admit = part <= rowv[r];
+                            v = FILTER ? part : part + rowv[r];
+                        } else {
+                            const float g = acc[ra][rb][r];
+                            if (metric == kMetricL2) {
+                                v = __fadd_rn(rowv[r], bnv[rb]);
+                                v = __fsub_rn(v, g);
+                                v = __fsub_rn(v, g);
+                            } else {
+                                v = -g;
+                            }
+                            admit = v <= tauv[r];
+                        }
+                        acc[ra][rb][r] = 0;
+                        if (FILTER) {
+                            if (admit && col < nb) {
+                                if constexpr (kInt) {
+                                    v += qn[row];
+                                }
+                                const int pos = atomicAdd(&flt.cnt[row], 1);
+                                if (pos < flt.cap) {
+                                    flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
+                                }
+                            }
+                        } else if (row < nq && col < nb) {
+                            out[row * ldo + col] = v;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename Tr>
+bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, int64_t nb, int d,
+                 const typename Tr::S *qn, const typename Tr::S *bn, int metric, typename Tr::S *out, int64_t ldo,
+                 bool filter, ScoreFilter<typename Tr::S> flt, hipStream_t s)
+{
+    if (d % Tr::kElemsPerStep != 0 || nb < 8 * kRingTN || reinterpret_cast<uintptr_t>(Q) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(B) % 16 != 0) {
+        return false;
+    }
+    const int64_t rt_m = (nq + kRingTM - 1) / kRingTM, rt_n = (nb + kRingTN - 1) / kRingTN;
+    if (rt_m * rt_n >= ((int64_t)1 << 31) || rt_m * ((rt_n + 7) / 8) * (d / Tr::kElemsPerStep) >= ((int64_t)1 << 30)) {
+        return false;
+    }
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        IXA_HIP(hipGetDevice(&dev));
+        IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+    const unsigned grid = (unsigned)((2 * cus + 7) / 8 * 8);   // two persistent workgroups per CU
+    const size_t smem = (size_t)kRingStages * kRingStageBytes;
+    if (filter) {
+        auto kern = score_ring_kernel<Tr, true>;
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo, (int)rt_m,
+                           (int)rt_n, flt);
+    } else {
+        auto kern = score_ring_kernel<Tr, false>;
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo, (int)rt_m,
+                           (int)rt_n, flt);
+    }
+    return true;
+}
+
+}  // namespace
+
+bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
+                          const int32_t *bn, int32_t *out, int64_t ldo, bool filter, ScoreFilter<int32_t> flt,
+                          hipStream_t s)
+{
+    return launch_ring<I8Traits>(Q, nq, B, nb, d, qn, bn, kMetricL2, out, ldo, filter, flt, s);
+}
+
+bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn,
+                           const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
+                           hipStream_t s)
+{
+    return launch_ring<F32Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter, flt, s);
+}
+
+}  // namespace ixa
