@@ -198,13 +198,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         issue_next();
     }
     int c_it = 0, c_ks = 0, c_slot = 0;
+    bool stored = false;  // the previous iteration ended with an epilogue that issued stores
     for (int g = 0; g < total; g++) {
-        // the loads of step g must have landed; later steps may still be in flight
-        if (issued - g - 1 >= kRingStages - 2) {
+        // The loads of step g must have landed; later steps may still be in flight.  vmcnt counts
+        // loads and stores in issue order, so right after a storing epilogue the usual count would
+        // also wait for all of its (much younger) stores; 63 is the largest expressible count and
+        // still covers the loads of step g, which are older than every store.
+        if (!FILTER && stored && issued - g - 1 >= kRingStages - 2) {
+            __builtin_amdgcn_s_waitcnt(0xcf7f);
+        } else if (issued - g - 1 >= kRingStages - 2) {
             __builtin_amdgcn_s_waitcnt(0x0f70 | ((kRingStages - 2) * kRingLoadsPerWave));
         } else {
             __builtin_amdgcn_s_waitcnt(0x0f70);
         }
+        stored = false;
         __builtin_amdgcn_s_barrier();
         if (issued < total) {
             issue_next();  // goes into the buffer that step g - 1 has just finished reading
@@ -218,6 +225,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             c_it++;
         }
         if (last_step) {
+            stored = true;
             int64_t tm, tn;
             item_tile(done_it, tm, tn);
             const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;

@@ -115,8 +115,13 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     const int cap = pow2_ceil((int)std::max<int64_t>(1024, 16 * (int64_t)ncand));
     const int64_t seed_rows = std::min<int64_t>(nb_total, std::max<int64_t>(2048, 16 * (int64_t)ncand));
     // when the whole score matrix of a query block fits the scratch, one materialised pass is the
-    // cheapest plan (this is the IVFPQ coarse stage); the filtered plan is for long bases
-    const bool can_fuse = nb_total > nb && seed_rows < nb_total && pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    // cheapest plan (measured on the IVFPQ coarse stage: 16384 centroids); the filtered plan is for
+    // long bases
+    const bool can_fuse = nb_total > nb && nb_total >= 4 * seed_rows &&
+                          pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query; keep
+    // that expectation below a quarter of the candidate buffer
+    const int64_t growth = std::max<int64_t>(2, cap / (4 * (int64_t)ncand));
     // the scratch only has to hold the seeding stretch unless the fallback is taken
     ws.scores.resize((size_t)qb * (can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb));
     const int64_t ld = can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb;
@@ -152,8 +157,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
                                running + q0 * ncand, ncand, nq, ws.tau.data() + q0);
             int64_t seen = head;
             while (seen < nb_total) {
-                // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query
-                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * 4, (int64_t)1 << 23});
+                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * growth, (int64_t)1 << 23});
                 ScoreFilter<S> flt{ws.tau.data() + q0, ops.threshold(ws, q0, nq, s), ws.cnt.data() + q0, ws.filter.data(), cap,
                                    seen};
                 ops.filtered(Q + q0 * d, nq, q0, B + seen * d, nbc, seen, d, flt, s);
