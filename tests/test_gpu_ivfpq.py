@@ -189,3 +189,72 @@ def test_train_on_gpu_then_parity_with_oracle_on_same_codebooks(ix, oracle):
     assert (I[:, 0] == np.arange(500)).mean() > 0.9
     lens = np.array([gpu.getListLength(l) for l in range(128)])
     assert lens.sum() == 30000 and (lens > 0).mean() > 0.9
+
+
+def _twin(ix, oracle, seed, n, nq, d, comp, sigma, nlist, M, metric, lut_fp16, nprobe, k, zipf=None, niter=4):
+    """Scaled-down twin of a benchmark configuration: trained and filled on the GPU, then the lists are
+    read back through the C ABI and handed to the oracle (same quantizers, same codes, same ids)."""
+    rng = np.random.default_rng(seed)
+    centres = rng.standard_normal((comp, d)).astype(np.float32)
+    w = None
+    if zipf:
+        w = 1.0 / np.arange(1, comp + 1) ** zipf
+        w /= w.sum()
+    unit = metric == ix.METRIC_INNER_PRODUCT
+    if unit:
+        centres /= np.linalg.norm(centres, axis=1, keepdims=True)
+
+    def draw(m):
+        x = centres[rng.choice(comp, m, p=w)] + sigma * rng.standard_normal((m, d)).astype(np.float32)
+        if unit:
+            x /= np.linalg.norm(x, axis=1, keepdims=True)
+        return x.astype(np.float32)
+
+    x, q = draw(n), draw(nq)
+    cfg = ix.AscendIndexIVFPQConfig(niter=niter, lut_fp16=lut_fp16, spherical=1 if unit else 0)
+    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, cfg)
+    gpu.train(x[: min(n, 64 * nlist)])
+    gpu.add(x)
+    cent, cb = gpu.get_trained()
+    lens = np.array([gpu.getListLength(l) for l in range(nlist)])
+    off = np.zeros(nlist + 1, dtype=np.int64)
+    np.cumsum(lens, out=off[1:])
+    codes = np.empty((n, M), dtype=np.uint8)
+    ids = np.empty(n, dtype=np.int64)
+    for l in range(nlist):
+        if lens[l]:
+            codes[off[l]:off[l + 1]], ids[off[l]:off[l + 1]] = gpu.getListCodesAndIds(l)
+    assert np.array_equal(np.sort(ids), np.arange(n))
+    # the codes the GPU stored are the reference encoder's codes of those vectors
+    probe = rng.choice(n, 2000, replace=False)
+    pos = np.empty(n, dtype=np.int64)
+    pos[ids] = np.arange(n)
+    assert np.array_equal(codes[pos[probe]], oracle.pq_encode(x[probe], cb))
+    ref = oracle.CsrIndex(d, M, metric, cent, cb, off, codes, ids)
+    gpu.setNumProbes(nprobe)
+    D, I = gpu.search(q, k)
+    Dr, Ir = ref.search(q, k, nprobe, lut_fp16=bool(lut_fp16))
+    pi, pd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, metric)
+    assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
+    exempt = assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP16 if lut_fp16 else TOL_FP32)
+    assert exempt <= 0.002 * I.size + 5
+    assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
+    return lens
+
+
+def test_twin_c2_l2_m32(ix, oracle):
+    _twin(ix, oracle, 31, 200_000, 400, 128, 256, 0.25, 1024, 32, ix.METRIC_L2, 0, 32, 100)
+
+
+def test_twin_c3_ip_m96_fp16_lut(ix, oracle):
+    _twin(ix, oracle, 32, 60_000, 150, 768, 128, 0.05, 256, 96, ix.METRIC_INNER_PRODUCT, 1, 16, 100, niter=3)
+
+
+def test_twin_c5_zipf_large_k(ix, oracle):
+    lens = _twin(ix, oracle, 33, 300_000, 64, 96, 64, 0.25, 1024, 48, ix.METRIC_L2, 0, 64, 1024, zipf=1.1)
+    assert lens.max() > 3 * np.median(lens[lens > 0])      # the lists really are imbalanced
+
+
+def test_twin_c1_small(ix, oracle):
+    _twin(ix, oracle, 34, 100_000, 300, 128, 64, 0.3, 256, 16, ix.METRIC_L2, 0, 16, 10, niter=6)
