@@ -106,6 +106,16 @@ public:
         syncTotal();
         return (size_t)removed;
     }
+    std::vector<idx_t> update(idx_t n, const float *x, const idx_t *ids)
+    {
+        std::vector<idx_t> missing((size_t)n);
+        int64_t nm = 0;
+        ixaThrowIfError(ivfpq_update(h_, n, x, reinterpret_cast<const int64_t *>(ids),
+                                     reinterpret_cast<int64_t *>(missing.data()), &nm));
+        missing.resize((size_t)nm);
+        syncTotal();
+        return missing;
+    }
     // AscendIndexIVF
     int getNumLists() const { return nlist_; }
     virtual void setNumProbes(int nprobes) { ixaThrowIfError(ivfpq_set_nprobe(h_, nprobes)); }

@@ -135,6 +135,11 @@ int ivfpq_get_list(const ivfpq_index_t *h, int64_t list, uint8_t *codes, int64_t
 
 /* AscendIndexIVFPQ::remove_ids(n, ids)  FR/ascend/AscendIndexIVFPQ.h:90; *removed may be NULL. */
 int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *removed);
+/* AscendIndexIVFPQ::update(n, x, ids)  FR/ascend/AscendIndexIVFPQ.h:92, AscendIndexIVFPQImpl.cpp:540-601:
+ * vectors whose id exists are replaced (delete + add); ids that do not exist are written to
+ * missing_ids (room for n entries, may be NULL) and counted in *n_missing (may be NULL). */
+int ivfpq_update(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids, int64_t *missing_ids,
+                 int64_t *n_missing);
 /* AscendIndexIVF::reset()  FR/ascend/AscendIndexIVF.h:93: drops the lists, keeps the quantizers. */
 int ivfpq_reset(ivfpq_index_t *h);
 int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out);

@@ -166,6 +166,16 @@ class AscendIndexIVFPQ:
         _capi.check(self._lib.ivfpq_remove_ids(self._h, ids.shape[0], _ptr(ids), ctypes.byref(out)))
         return out.value
 
+    def update(self, x, ids):
+        """Replaces the vectors of existing ids; returns the ids that were not found."""
+        x = _as(x, np.float32, 2, "x")
+        ids = _as(ids, np.int64, 1, "ids")
+        assert x.shape == (ids.shape[0], self.d)
+        missing = np.empty(ids.shape[0], dtype=np.int64)
+        nm = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_update(self._h, ids.shape[0], _ptr(x), _ptr(ids), _ptr(missing), ctypes.byref(nm)))
+        return missing[: nm.value].copy()
+
     def reset(self):
         _capi.check(self._lib.ivfpq_reset(self._h))
 

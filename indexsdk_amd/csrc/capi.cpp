@@ -2,6 +2,7 @@
 // catches C++ exceptions, stores the message for ixa_last_error() and returns the status code.
 #include "../../include/indexsdk_amd.h"
 
+#include <algorithm>
 #include <cstring>
 #include <new>
 #include <string>
@@ -184,6 +185,20 @@ IXA_EXPORT int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids,
         const int64_t r = h->impl.remove_ids(n, ids);
         if (removed) {
             *removed = r;
+        }
+    });
+}
+IXA_EXPORT int ivfpq_update(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids, int64_t *missing_ids,
+                            int64_t *n_missing)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        const std::vector<int64_t> m = h->impl.update(n, x, ids);
+        if (n_missing) {
+            *n_missing = (int64_t)m.size();
+        }
+        if (missing_ids) {
+            std::copy(m.begin(), m.end(), missing_ids);
         }
     });
 }

@@ -63,6 +63,8 @@ public:
     int64_t list_length(int64_t list) const;
     void get_list(int64_t list, uint8_t *codes, int64_t *ids) const;                    // host pointers
     int64_t remove_ids(int64_t n, const int64_t *ids);
+    // replaces the vectors of ids that exist; returns the ids that do not (host pointers)
+    std::vector<int64_t> update(int64_t n, const float *x, const int64_t *ids);
     void reset();
     const SearchStats &stats() const { return stats_; }
 

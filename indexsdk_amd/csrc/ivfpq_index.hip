@@ -491,6 +491,43 @@ int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
     return removed;
 }
 
+// update (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:540-601): ids that exist are deleted and re-added with
+// their new vectors (they move to the end of their new list); ids that do not exist are returned.
+std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t *ids)
+{
+    check_trained();
+    IXA_REQUIRE(x, kErrInvalidParam, "vector list is nullptr!");
+    IXA_REQUIRE(ids, kErrInvalidParam, "vector ID list is nullptr!");
+    IXA_REQUIRE(n > 0, kErrInvalidParam, "update vector number must be greater than 0!");
+    std::unordered_set<int64_t> present;
+    if (ntotal_ > 0) {
+        std::vector<int64_t> all_ids((size_t)total_slots_);
+        IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
+        IXA_HIP(hipStreamSynchronize(stream_));
+        for (int64_t l = 0; l < nlist_; l++) {
+            const int64_t off = list_off_[(size_t)l];
+            for (int64_t i = 0; i < list_len_[(size_t)l]; i++) {
+                present.insert(all_ids[(size_t)(off + i)]);
+            }
+        }
+    }
+    std::vector<int64_t> missing, exist_ids;
+    std::vector<float> exist_x;
+    for (int64_t i = 0; i < n; i++) {
+        if (present.count(ids[i])) {
+            exist_ids.push_back(ids[i]);
+            exist_x.insert(exist_x.end(), x + i * d_, x + (i + 1) * d_);
+        } else {
+            missing.push_back(ids[i]);
+        }
+    }
+    if (!exist_ids.empty()) {
+        remove_ids((int64_t)exist_ids.size(), exist_ids.data());
+        add((int64_t)exist_ids.size(), exist_x.data(), exist_ids.data(), false);
+    }
+    return missing;
+}
+
 // reset keeps the trained quantizers and drops every list (FR/ascend/AscendIndexIVF.h: reset()).
 void IvfpqIndex::reset()
 {

@@ -167,6 +167,26 @@ def test_add_in_two_calls_add_codes_and_remove(ix, oracle):
     assert not (set(I.ravel().tolist()) & vs)
 
 
+def test_update_replaces_existing_and_reports_missing(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 35, 4000, 20, 64, 16, 8, ix.METRIC_L2)
+    rng = np.random.default_rng(5)
+    new_x = (x[:50] + 0.5 * rng.standard_normal((50, 64))).astype(np.float32)
+    upd_ids = np.concatenate([ids[:40], np.array([10**9 + i for i in range(10)], dtype=np.int64)])
+    missing = gpu.update(new_x, upd_ids)
+    assert np.array_equal(missing, upd_ids[40:]) and gpu.ntotal == 4000
+    # the oracle index with the same replacement: old entries removed, new ones appended to their lists
+    keep = ~np.isin(ids, ids[:40])
+    x2 = np.concatenate([x[keep], new_x[:40]])
+    ids2 = np.concatenate([ids[keep], ids[:40]])
+    ref2 = oracle.CsrIndex.build(64, 8, ix.METRIC_L2, ref.cent, ref.codebook, x2, ids2)
+    for l in range(16):
+        codes, lid = gpu.getListCodesAndIds(l)
+        b, e = ref2.list_off[l], ref2.list_off[l + 1]
+        assert np.array_equal(lid, ref2.ids[b:e]) and np.array_equal(codes, ref2.codes[b:e])
+    D, I = gpu.search(new_x[:40], 1)
+    assert (I[:, 0] == ids[:40]).mean() > 0.9
+
+
 def test_train_on_gpu_then_parity_with_oracle_on_same_codebooks(ix, oracle):
     x, q = make_data(29, 30000, 100, 64)
     cfg = ix.AscendIndexIVFPQConfig(niter=6)
