@@ -75,7 +75,8 @@ typedef struct ivfpq_config {
     uint64_t seed;                  /* sampling / initialisation seed */
     int32_t strict_reference_params;/* 1 = enforce the reference whitelists d in {128}, nlist in
                                        {1024..16384, 262144, 524288}, M in {2,4,8,16,32} */
-    int32_t reserved;
+    int32_t coarse_fp32_only;       /* 0 = coarse candidates from bf16 x 3 matrix products, re-evaluated in fp32 and
+                                       verified (results identical to the fp32 plan); 1 = fp32 matrix products only */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */

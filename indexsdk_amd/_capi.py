@@ -29,7 +29,7 @@ class IvfpqConfig(ctypes.Structure):
         ("scratch_bytes", ctypes.c_int64),
         ("seed", ctypes.c_uint64),
         ("strict_reference_params", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("coarse_fp32_only", ctypes.c_int32),
     ]
 
 

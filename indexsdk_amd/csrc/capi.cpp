@@ -76,6 +76,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->scratch_bytes = d.scratch_bytes;
     cfg->seed = d.seed;
     cfg->strict_reference_params = d.strict_reference_params;
+    cfg->coarse_fp32_only = d.coarse_bf16 ? 0 : 1;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,
@@ -99,6 +100,7 @@ IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbi
             c.scratch_bytes = cfg->scratch_bytes;
             c.seed = cfg->seed;
             c.strict_reference_params = cfg->strict_reference_params;
+            c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
         }
         *out = new ivfpq_index(d, metric, nlist, msubs, nbits, c);
     });

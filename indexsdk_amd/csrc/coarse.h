@@ -45,6 +45,20 @@ bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t n
                            const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                            hipStream_t s);
 
+bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                            const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
+                            hipStream_t s);
+
+// out[row] = [hi | hi | lo] (query side) or [hi | lo | hi] (base side) of x[row], each segment
+// zero-padded from d to dp elements of bf16 (stored as uint16_t); out has n * 3 * dp elements.
+void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s);
+
+// Sets *flag = 1 if some query's approximate candidate list (running[nq][ncand], ascending keys) is
+// not provably a superset of its best nout centroids; see score_ring.hip.
+void launch_verify_superset(const unsigned long long *running, int ncand, const float *exact_dist, int nout,
+                            const float *qn, float cmax, float err_scale, int metric, int64_t nq, int *flag,
+                            hipStream_t s);
+
 // Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
 // indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
 // (ordered score << 32) | (col_base + column): its content takes part in the selection and is

@@ -21,6 +21,9 @@ struct IvfpqConfig {
     int64_t scratch_bytes = (int64_t)1 << 30;  // budget of the coarse score scratch
     uint64_t seed = 1234;
     int strict_reference_params = 0;  // 1 = enforce the reference's d / nlist / M whitelists
+    int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
+                                      // stay exact: candidates are re-evaluated in fp32 and the superset
+                                      // property is verified, with an fp32 rerun if it cannot be proven)
 };
 
 struct SearchStats {
@@ -91,6 +94,10 @@ private:
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
+    DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
+    DeviceBuffer<int32_t> ws_flag_;
+    float cmax_ = 0.f;                                      // largest centroid norm
+    int dp_ = 0;                                            // d rounded up to a multiple of 32
     // arena
     DeviceBuffer<uint8_t> codes_;
     DeviceBuffer<int64_t> ids_;
@@ -100,7 +107,7 @@ private:
     std::vector<int32_t> list_len_;
     int64_t total_slots_ = 0;
     // search workspaces (grown on demand, reused between calls)
-    DeviceBuffer<float> ws_x_, ws_qn_, ws_dist_;
+    DeviceBuffer<float> ws_x_, ws_qn_, ws_dist_, ws_exact_;
     StreamSelectWorkspace<float> ws_sel_;
     DeviceBuffer<unsigned long long> ws_running_;
     DeviceBuffer<int32_t> ws_cand_, ws_probes_;

@@ -197,6 +197,12 @@ void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
         centroids_.upload(centroids, (size_t)nlist_ * d_, stream_);
         cnorm_.resize((size_t)nlist_);
         launch_sqnorm_rows(centroids_.data(), nlist_, d_, cnorm_.data(), stream_);
+        dp_ = (int)round_up(d_, 32);
+        centroids_split_.resize((size_t)nlist_ * 3 * dp_);
+        launch_split_bf16x3(centroids_.data(), nlist_, d_, dp_, true, centroids_split_.data(), stream_);
+        std::vector<float> cn((size_t)nlist_);
+        cnorm_.download(cn.data(), cn.size(), stream_);
+        cmax_ = std::sqrt(*std::max_element(cn.begin(), cn.end()));
     }
     if (codebook) {
         codebook_.upload(codebook, (size_t)M_ * 256 * dsub_, stream_);
@@ -234,17 +240,55 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     if (n == 0) {
         return;
     }
-    const int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
-    ws_running_.resize((size_t)n * ncand);
-    ws_cand_.resize((size_t)n * ncand);
-    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
-    stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric, ncand,
-                      ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
-    launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
-    launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric, ws_cand_.data(), ncand,
-                  nout, nout, out_ids, out_dist, stream_);
+    // Candidate generation.  Fast plan: bf16 x 3 matrix products (|error| <= 3 * 2^-16 |q||c| on the
+    // dot product) with 16 spare candidates; the candidates are re-evaluated exactly, and a check
+    // proves that nothing outside them can reach the nout-th exact score.  If the check fails for
+    // any query (near-tied centroids), the fp32 plan below recomputes the whole call.
+    for (int attempt = cfg_.coarse_bf16 ? 0 : 1; attempt < 2; attempt++) {
+        const bool approx = attempt == 0;
+        const int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + (approx ? 16 : 8) + nout / 8);
+        ws_running_.resize((size_t)n * ncand);
+        ws_cand_.resize((size_t)n * ncand);
+        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+        float *dist = out_dist;
+        if (approx) {
+            ws_xsplit_.resize((size_t)n * 3 * dp_);
+            launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
+            const int rc = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_,
+                                                ws_qn_.data(), cnorm_.data(), select_metric, ncand, ws_running_.data(),
+                                                ws_sel_, cfg_.scratch_bytes, stream_);
+            if (rc < 0) {
+                continue;  // shape not served by the bf16 kernel
+            }
+            if (!dist) {
+                ws_exact_.resize((size_t)n * nout);
+                dist = ws_exact_.data();
+            }
+        } else {
+            stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
+                              ncand, ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
+        }
+        launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
+        launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric, ws_cand_.data(),
+                      ncand, nout, nout, out_ids, dist, stream_);
+        if (!approx) {
+            break;
+        }
+        // error of the approximate SCORE: 2 * (3 * 2^-16) |q||c| for L2 (score = norms - 2 dot), half of
+        // that for inner product; doubled again as a safety margin
+        const float err_scale = (select_metric == kMetricL2 ? 12.0f : 6.0f) / 65536.0f;
+        ws_flag_.resize(1);
+        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+        launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale, select_metric,
+                               n, ws_flag_.data(), stream_);
+        int32_t failed = 0;
+        ws_flag_.download(&failed, 1, stream_);
+        if (!failed) {
+            break;
+        }
+    }
 }
 
 void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)

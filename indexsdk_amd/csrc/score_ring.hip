@@ -30,6 +30,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kRingTM = 256, kRingTN = 128, kRingRows = kRingTM + kRingTN;
@@ -65,6 +66,40 @@ struct I8Traits {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
                     acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                }
+            }
+        }
+    }
+};
+
+// bf16 operands, fp32 accumulation (v_mfma_f32_32x32x16_bf16): same data movement as int8.
+struct Bf16Traits {
+    using T = uint16_t;
+    using S = float;
+    using Acc = v16f;
+    static constexpr int kElemsPerStep = 32;
+    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
+                                               Acc (&acc)[4][2])
+    {
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int c = kk * 2 + half;
+            bf16x8 a[4], b[2];
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+                const int r = wr * 128 + ra * 32 + l32;
+                a[ra] = *reinterpret_cast<const bf16x8 *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+                const int r = kRingTM + wc * 64 + rb * 32 + l32;
+                b[rb] = *reinterpret_cast<const bf16x8 *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
+            }
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+                    acc[ra][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
                 }
             }
         }
@@ -340,6 +375,87 @@ bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t 
                           hipStream_t s)
 {
     return launch_ring<I8Traits>(Q, nq, B, nb, d, qn, bn, kMetricL2, out, ldo, filter, flt, s);
+}
+
+bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                            const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
+                            hipStream_t s)
+{
+    return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter, flt, s);
+}
+
+// ---- bf16 x 3 split --------------------------------------------------------------------------------
+// x = hi + lo + rest with hi = bf16(x), lo = bf16(x - hi), |rest| <= 2^-16 |x|.  A dot product over
+// the concatenated rows  [hi | hi | lo] . [hi | lo | hi]  = hi.hi + hi.lo + lo.hi  differs from the
+// exact one by at most about 3 * 2^-16 * sum |x_i y_i|, at three bf16 MFMAs (16x the fp32 matrix
+// rate each) per fp32 product.  Rows are zero-padded to dp (a multiple of 32) per segment.
+__device__ __forceinline__ uint16_t bf16_rne(float v)
+{
+    uint32_t u = __float_as_uint(v);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__global__ __launch_bounds__(256) void split_bf16x3_kernel(const float *__restrict__ x, int64_t n, int d, int dp,
+                                                           int base_side, uint16_t *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * dp) {
+        return;
+    }
+    const int64_t row = e / dp;
+    const int j = (int)(e % dp);
+    const float v = j < d ? x[row * d + j] : 0.f;
+    const uint16_t hi = bf16_rne(v);
+    const float hif = __uint_as_float((uint32_t)hi << 16);
+    const uint16_t lo = bf16_rne(v - hif);
+    uint16_t *o = out + row * 3 * dp + j;
+    o[0] = hi;
+    o[dp] = base_side ? lo : hi;
+    o[2 * dp] = base_side ? hi : lo;
+}
+
+void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(split_bf16x3_kernel, dim3((unsigned)((n * dp + 255) / 256)), dim3(256), 0, s, x, n, d, dp,
+                           base_side ? 1 : 0, out);
+    }
+}
+
+// Raises *flag unless, for every query, no centroid outside its approximate candidate list can beat
+// its nout-th exact score: (approximate score of the last candidate) - err > (nout-th exact score),
+// err = err_scale * |q| * max|c|.  Rows whose candidate list is not full hold every centroid.
+__global__ __launch_bounds__(256) void verify_superset_kernel(const key_t *__restrict__ running, int ncand,
+                                                              const float *__restrict__ exact_dist, int nout,
+                                                              const float *__restrict__ qn, float cmax, float err_scale,
+                                                              int metric, int64_t nq, int *__restrict__ flag)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nq) {
+        return;
+    }
+    const key_t last = running[i * ncand + (ncand - 1)];
+    if (last == kEmptyKey) {
+        return;
+    }
+    const float a_last = key_score(last);
+    const float d_out = exact_dist[i * nout + (nout - 1)];
+    const float s_star = metric == kMetricL2 ? d_out : -d_out;
+    const float err = err_scale * sqrtf(qn[i]) * cmax;
+    if (!(a_last - err > s_star)) {
+        *flag = 1;
+    }
+}
+
+void launch_verify_superset(const unsigned long long *running, int ncand, const float *exact_dist, int nout,
+                            const float *qn, float cmax, float err_scale, int metric, int64_t nq, int *flag,
+                            hipStream_t s)
+{
+    if (nq > 0) {
+        hipLaunchKernelGGL(verify_superset_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, running, ncand,
+                           exact_dist, nout, qn, cmax, err_scale, metric, nq, flag);
+    }
 }
 
 bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn,

@@ -22,6 +22,12 @@ struct StreamSelectWorkspace {
 int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn, const float *bn,
                       int metric, int ncand, unsigned long long *running, StreamSelectWorkspace<float> &ws,
                       int64_t scratch_bytes, hipStream_t s);
+// Same selection with approximate scores: Qs / Bs are the bf16 x 3 splits of the operands (rows of d3
+// bf16 elements, see launch_split_bf16x3), qn / bn the exact fp32 norms.  Returns -1 without doing
+// anything when the shape does not qualify for the bf16 matrix-core kernel.
+int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3, const float *qn,
+                         const float *bn, int metric, int ncand, unsigned long long *running,
+                         StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, hipStream_t s);
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
                      int64_t scratch_bytes, hipStream_t s);

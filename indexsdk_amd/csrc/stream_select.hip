@@ -69,6 +69,35 @@ struct F32Ops {
     }
 };
 
+struct Bf16Ops {
+    using T = uint16_t;
+    using S = float;
+    const float *qn, *bn;
+    int metric;
+    const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
+    void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
+                hipStream_t s) const
+    {
+        const bool ok = launch_score_ring_bf16(Q, nq, B, nb, d, qn + q0, bn + b0, metric, out, ldo, false,
+                                               ScoreFilter<float>{}, s);
+        IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
+    }
+    void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
+                  hipStream_t s) const
+    {
+        const bool ok = launch_score_ring_bf16(Q, nq, B, nb, d, qn + q0, bn + b0, metric, nullptr, 0, true, flt, s);
+        IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
+    }
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    {
+        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s);
+    }
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    {
+        launch_merge_candidates(run, k, flt, tau, nq, ovf, s);
+    }
+};
+
 struct I8Ops {
     using T = int8_t;
     using S = int32_t;
@@ -187,6 +216,19 @@ int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, in
                       int64_t scratch_bytes, hipStream_t s)
 {
     return stream_select(F32Ops{qn, bn, metric}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s);
+}
+
+int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3, const float *qn,
+                         const float *bn, int metric, int ncand, unsigned long long *running,
+                         StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, hipStream_t s)
+{
+    // the ring kernel needs whole K-steps and at least 1024 base rows in every launch; the plan below
+    // only produces launches of the whole base or of >= 2048 rows
+    if (d3 % 32 != 0 || nb < 2048 || reinterpret_cast<uintptr_t>(Qs) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(Bs) % 16 != 0) {
+        return -1;
+    }
+    return stream_select(Bf16Ops{qn, bn, metric}, Qs, nq, Bs, nb, d3, ncand, running, ws, scratch_bytes, s);
 }
 
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
