@@ -44,6 +44,7 @@ struct I8Traits {
     using Acc = v16i;
     static constexpr int kElemsPerStep = 64;
     // one K-step = 2 sub-steps of 32 bytes; a lane half owns 16 of them
+    template <bool SWAP>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -65,7 +66,8 @@ struct I8Traits {
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[rb], a[ra], acc[ra][rb], 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
                 }
             }
         }
@@ -78,6 +80,7 @@ struct Bf16Traits {
     using S = float;
     using Acc = v16f;
     static constexpr int kElemsPerStep = 32;
+    template <bool SWAP>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -99,7 +102,8 @@ struct Bf16Traits {
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[rb], a[ra], acc[ra][rb], 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
                 }
             }
         }
@@ -113,6 +117,7 @@ struct F32Traits {
     static constexpr int kElemsPerStep = 16;
     // one K-step = 16 floats; a lane half owns 8 of them (two 16-byte chunks) and feeds them to 8
     // consecutive 32x32x2 MFMAs
+    template <bool SWAP>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -137,8 +142,9 @@ struct F32Traits {
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ra][t >> 2][t & 3], b[rb][t >> 2][t & 3],
-                                                                       acc[ra][rb], 0, 0, 0);
+                    const float av = a[ra][t >> 2][t & 3], bv = b[rb][t >> 2][t & 3];
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc[ra][rb], 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[ra][rb], 0, 0, 0);
                 }
             }
         }
@@ -240,7 +246,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // also wait for all of its (much younger) stores; 63 is the largest expressible count and
         // still covers the loads of step g, which are older than every store.
         if (!FILTER && stored && issued - g - 1 >= kRingStages - 2) {
-            __builtin_amdgcn_s_waitcnt(0xcf7f);
+            __builtin_amdgcn_s_waitcnt(0xcf7f);   // vmcnt(63): covers the <= 32 + 6 younger operations
         } else if (issued - g - 1 >= kRingStages - 2) {
             __builtin_amdgcn_s_waitcnt(0x0f70 | ((kRingStages - 2) * kRingLoadsPerWave));
         } else {
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (issued < total) {
             issue_next();  // goes into the buffer that step g - 1 has just finished reading
         }
-        Tr::mma(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
+        Tr::template mma<FILTER>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
         const bool last_step = c_ks == nk - 1;
         const int done_it = c_it;
         c_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
@@ -259,7 +265,121 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             c_ks = 0;
             c_it++;
         }
-        if (last_step) {
+        // Two epilogues.  Filtered launches make the BASE fragment the first MFMA operand, so a lane
+        // owns one query row per block (its bound is a per-lane scalar) -- cheapest test per score.
+        // Storing launches keep the query fragment first: a lane owns one base column and 32 lanes
+        // write 128 contiguous bytes of a score row, which is what the memory system wants.
+        if (FILTER && last_step) {
+            // The base fragment is the first MFMA operand, so in accumulator block (ra, rb) a lane
+            // owns ONE query row (ra * 32 + l32) and its 16 registers are base columns
+            // rb * 32 + 8 * (r / 4) + 4 * half + (r % 4): four runs of four consecutive columns.
+            // Per-query values are per-lane scalars and results leave as 128-bit stores.
+            int64_t tm, tn;
+            item_tile(done_it, tm, tn);
+            const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
+            const bool vec_out = !FILTER && (ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
+            // the base norms of this lane's 32 columns: eight 128-bit loads per tile
+            S bnq[2][4][4];
+            const bool use_bn = kInt || metric == kMetricL2;
+            const bool vec_bn = reinterpret_cast<uintptr_t>(bn) % 16 == 0;
+#pragma unroll
+            for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                for (int rq = 0; rq < 4; rq++) {
+                    const int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
+                    if (use_bn && vec_bn && col + 3 < nb) {
+                        const uint4 u = *reinterpret_cast<const uint4 *>(bn + col);
+                        bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
+                        bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
+                        bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
+                        bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            bnq[rb][rq][t] = (use_bn && col + t < nb) ? bn[col + t] : (S)0;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int ra = 0; ra < 4; ra++) {
+                asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
+                const int64_t row = i0 + wr * 128 + ra * 32 + l32;
+                const bool row_ok = row < nq;
+                S rowv, tauv;
+                if (kInt) {
+                    // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
+                    rowv = row_ok ? (FILTER ? flt.thr[row] : qn[row]) : (FILTER ? (S)0x80000000 : (S)0);
+                    tauv = 0;
+                } else {
+                    rowv = (row_ok && metric == kMetricL2) ? qn[row] : (S)0;
+                    tauv = (FILTER && row_ok) ? flt.tau[row] : (S)(-__builtin_inff());
+                }
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        const int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
+                        S v[4];
+                        bool admit[4];
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            const int r = rq * 4 + t;
+                            const S bnv = bnq[rb][rq][t];
+                            if constexpr (kInt) {
+                                const S part = bnv - 2 * acc[ra][rb][r];
+                                admit[t] = part <= rowv;
+                                v[t] = FILTER ? part : part + rowv;
+                            } else {
+                                const float g = acc[ra][rb][r];
+                                if (metric == kMetricL2) {
+                                    float w = __fadd_rn(rowv, bnv);
+                                    w = __fsub_rn(w, g);
+                                    v[t] = __fsub_rn(w, g);
+                                } else {
+                                    v[t] = -g;
+                                }
+                                admit[t] = v[t] <= tauv;
+                            }
+                            acc[ra][rb][r] = 0;
+                        }
+                        if (FILTER) {
+#pragma unroll
+                            for (int t = 0; t < 4; t++) {
+                                if (admit[t] && row_ok && col + t < nb) {
+                                    S val = v[t];
+                                    if constexpr (kInt) {
+                                        val += qn[row];
+                                    }
+                                    const int pos = atomicAdd(&flt.cnt[row], 1);
+                                    if (pos < flt.cap) {
+                                        flt.cand[row * flt.cap + pos] = make_key(val, (uint32_t)(col + t + flt.col_base));
+                                    }
+                                }
+                            }
+                        } else if (row_ok) {
+                            S *dst = out + row * ldo + col;
+                            if (vec_out && col + 3 < nb) {
+                                uint4 u;
+                                u.x = __builtin_bit_cast(uint32_t, v[0]);
+                                u.y = __builtin_bit_cast(uint32_t, v[1]);
+                                u.z = __builtin_bit_cast(uint32_t, v[2]);
+                                u.w = __builtin_bit_cast(uint32_t, v[3]);
+                                *reinterpret_cast<uint4 *>(dst) = u;
+                            } else {
+#pragma unroll
+                                for (int t = 0; t < 4; t++) {
+                                    if (col + t < nb) {
+                                        dst[t] = v[t];
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (!FILTER && last_step) {
             stored = true;
             int64_t tm, tn;
             item_tile(done_it, tm, tn);
