@@ -186,29 +186,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned char *Qb = reinterpret_cast<const unsigned char *>(Q);
     const unsigned char *Bb = reinterpret_cast<const unsigned char *>(B);
 
-    // issue the loads of one K-step (item it, step ks) into ring buffer `slot`
-    auto issue = [&](int it, int ks, int slot) {
+    // Per-lane source pointers of the tile whose K-steps are being issued (recomputed once per
+    // tile); a K-step then only adds ks * 64 bytes.
+    const unsigned char *src[kRingLoadsPerWave];
+    auto set_sources = [&](int it) {
         int64_t tm, tn;
         item_tile(it, tm, tn);
-        unsigned char *stage = ring + slot * kRingStageBytes;
 #pragma unroll
         for (int j = 0; j < kRingLoadsPerWave; j++) {
             const int rg = wave * kRingLoadsPerWave + j;          // group of 16 stage rows
             const int row = rg * 16 + (lane >> 2);                // stage row: 0..255 queries, 256..383 base
             const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-            const unsigned char *src;
             if (rg < kRingTM / 16) {
                 int64_t r = tm * kRingTM + row;
                 r = r < nq ? r : nq - 1;
-                src = Qb + r * row_bytes;
+                src[j] = Qb + r * row_bytes + chunk * 16;
             } else {
                 int64_t r = tn * kRingTN + (row - kRingTM);
                 r = r < nb ? r : nb - 1;
-                src = Bb + r * row_bytes;
+                src[j] = Bb + r * row_bytes + chunk * 16;
             }
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(src + ks * 64 + chunk * 16),
-                (__attribute__((address_space(3))) void *)(stage + rg * 1024), 16, 0, 0);
+        }
+    };
+    // issue the loads of one K-step (step ks of the current issue tile) into ring buffer `slot`
+    auto issue = [&](int ks, int slot) {
+        unsigned char *stage = ring + slot * kRingStageBytes;
+#pragma unroll
+        for (int j = 0; j < kRingLoadsPerWave; j++) {
+            const int rg = wave * kRingLoadsPerWave + j;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src[j] + ks * 64),
+                                             (__attribute__((address_space(3))) void *)(stage + rg * 1024), 16, 0, 0);
         }
     };
 
@@ -227,7 +234,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // (item, step, ring slot) of the next K-step to issue and of the one being computed
     int issued = 0, i_it = 0, i_ks = 0, i_slot = 0;
     auto issue_next = [&]() {
-        issue(i_it, i_ks, i_slot);
+        if (i_ks == 0) {
+            set_sources(i_it);
+        }
+        issue(i_ks, i_slot);
         issued++;
         i_slot = i_slot + 1 == kRingStages ? 0 : i_slot + 1;
         if (++i_ks == nk) {
