@@ -327,61 +327,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
+                    // all 16 scores of the block first, then ONE test of their minimum against the
+                    // lane's bound: admissions are rare, so the per-score path almost never runs
+                    S v[16];
+                    S best = ScoreOps<S>::worst();
 #pragma unroll
-                    for (int rq = 0; rq < 4; rq++) {
-                        const int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
-                        S v[4];
-                        bool admit[4];
-#pragma unroll
-                        for (int t = 0; t < 4; t++) {
-                            const int r = rq * 4 + t;
-                            const S bnv = bnq[rb][rq][t];
-                            if constexpr (kInt) {
-                                const S part = bnv - 2 * acc[ra][rb][r];
-                                admit[t] = part <= rowv;
-                                v[t] = FILTER ? part : part + rowv;
+                    for (int r = 0; r < 16; r++) {
+                        const S bnv = bnq[rb][r >> 2][r & 3];
+                        if constexpr (kInt) {
+                            v[r] = bnv - 2 * acc[ra][rb][r];          // compared with tau - |q|^2
+                        } else {
+                            const float g = acc[ra][rb][r];
+                            if (metric == kMetricL2) {
+                                float w = __fadd_rn(rowv, bnv);
+                                w = __fsub_rn(w, g);
+                                v[r] = __fsub_rn(w, g);
                             } else {
-                                const float g = acc[ra][rb][r];
-                                if (metric == kMetricL2) {
-                                    float w = __fadd_rn(rowv, bnv);
-                                    w = __fsub_rn(w, g);
-                                    v[t] = __fsub_rn(w, g);
-                                } else {
-                                    v[t] = -g;
-                                }
-                                admit[t] = v[t] <= tauv;
+                                v[r] = -g;
                             }
-                            acc[ra][rb][r] = 0;
                         }
-                        if (FILTER) {
+                        acc[ra][rb][r] = 0;
+                        best = v[r] < best ? v[r] : best;
+                    }
+                    const S lane_bound = kInt ? rowv : tauv;
+                    if (__ballot(row_ok && best <= lane_bound)) {
 #pragma unroll
-                            for (int t = 0; t < 4; t++) {
-                                if (admit[t] && row_ok && col + t < nb) {
-                                    S val = v[t];
-                                    if constexpr (kInt) {
-                                        val += qn[row];
-                                    }
-                                    const int pos = atomicAdd(&flt.cnt[row], 1);
-                                    if (pos < flt.cap) {
-                                        flt.cand[row * flt.cap + pos] = make_key(val, (uint32_t)(col + t + flt.col_base));
-                                    }
+                        for (int r = 0; r < 16; r++) {
+                            const int64_t col = j0 + wc * 64 + rb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                            if (row_ok && v[r] <= lane_bound && col < nb) {
+                                S val = v[r];
+                                if constexpr (kInt) {
+                                    val += qn[row];
                                 }
-                            }
-                        } else if (row_ok) {
-                            S *dst = out + row * ldo + col;
-                            if (vec_out && col + 3 < nb) {
-                                uint4 u;
-                                u.x = __builtin_bit_cast(uint32_t, v[0]);
-                                u.y = __builtin_bit_cast(uint32_t, v[1]);
-                                u.z = __builtin_bit_cast(uint32_t, v[2]);
-                                u.w = __builtin_bit_cast(uint32_t, v[3]);
-                                *reinterpret_cast<uint4 *>(dst) = u;
-                            } else {
-#pragma unroll
-                                for (int t = 0; t < 4; t++) {
-                                    if (col + t < nb) {
-                                        dst[t] = v[t];
-                                    }
+                                const int pos = atomicAdd(&flt.cnt[row], 1);
+                                if (pos < flt.cap) {
+                                    flt.cand[row * flt.cap + pos] = make_key(val, (uint32_t)(col + flt.col_base));
                                 }
                             }
                         }
