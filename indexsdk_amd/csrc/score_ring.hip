@@ -250,6 +250,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     int c_it = 0, c_ks = 0, c_slot = 0;
     bool stored = false;  // the previous iteration ended with an epilogue that issued stores
+
+    // Filtered launches fetch what the epilogue of a tile needs -- the base norms of the lane's 32
+    // columns and the bounds of its 4 query rows -- one K-step ahead, so the epilogue never waits
+    // for memory.  The fetch is a fixed number of loads (kPrefetchLoads) because the s_waitcnt
+    // immediates below count them.
+    constexpr int kPrefetchLoads = 8 + (kInt ? 4 : 8);
+    S bnq[2][4][4];
+    S rowq[4], tauq[4];
+    const bool prefetch = FILTER && nk >= 2 && nb % 4 == 0 && reinterpret_cast<uintptr_t>(bn) % 16 == 0 && bn != nullptr &&
+                          qn != nullptr;
+    bool fetched = false;   // the previous iteration issued the fetch
+    auto fetch_epilogue_operands = [&](int it) {
+        int64_t tm, tn;
+        item_tile(it, tm, tn);
+        const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
+#pragma unroll
+        for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
+                col = col + 3 < nb ? col : 0;     // out-of-range columns are rejected by index later
+                const uint4 u = *reinterpret_cast<const uint4 *>(bn + col);
+                bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
+                bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
+                bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
+                bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
+            }
+        }
+#pragma unroll
+        for (int ra = 0; ra < 4; ra++) {
+            int64_t row = i0 + wr * 128 + ra * 32 + l32;
+            row = row < nq ? row : 0;
+            if constexpr (kInt) {
+                rowq[ra] = flt.thr[row];
+            } else {
+                rowq[ra] = qn[row];
+                tauq[ra] = flt.tau[row];
+            }
+        }
+    };
     for (int g = 0; g < total; g++) {
         // The loads of step g must have landed; later steps may still be in flight.  vmcnt counts
         // loads and stores in issue order, so right after a storing epilogue the usual count would
@@ -258,14 +298,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (!FILTER && stored && issued - g - 1 >= kRingStages - 2) {
             __builtin_amdgcn_s_waitcnt(0xcf7f);   // vmcnt(63): covers the <= 32 + 6 younger operations
         } else if (issued - g - 1 >= kRingStages - 2) {
-            __builtin_amdgcn_s_waitcnt(0x0f70 | ((kRingStages - 2) * kRingLoadsPerWave));
+            constexpr int kInFlight = (kRingStages - 2) * kRingLoadsPerWave;
+            if (FILTER && fetched) {
+                // queue: [step g][step g + 1][epilogue fetch]; only step g has to be complete
+                constexpr int n = kInFlight + kPrefetchLoads;
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+            } else {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | kInFlight);
+            }
         } else {
             __builtin_amdgcn_s_waitcnt(0x0f70);
         }
         stored = false;
+        fetched = false;
         __builtin_amdgcn_s_barrier();
         if (issued < total) {
             issue_next();  // goes into the buffer that step g - 1 has just finished reading
+        }
+        if (FILTER && prefetch && c_ks == nk - 2) {
+            fetch_epilogue_operands(c_it);
+            fetched = true;
         }
         Tr::template mma<FILTER>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
         const bool last_step = c_ks == nk - 1;
@@ -288,12 +340,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             item_tile(done_it, tm, tn);
             const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
             const bool vec_out = !FILTER && (ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
-            // the base norms of this lane's 32 columns: eight 128-bit loads per tile
-            S bnq[2][4][4];
+            // without the early fetch: the base norms of this lane's 32 columns, loaded here
             const bool use_bn = kInt || metric == kMetricL2;
             const bool vec_bn = reinterpret_cast<uintptr_t>(bn) % 16 == 0;
 #pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
+            for (int rb = 0; rb < 2 && !prefetch; rb++) {
 #pragma unroll
                 for (int rq = 0; rq < 4; rq++) {
                     const int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
@@ -317,13 +368,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int64_t row = i0 + wr * 128 + ra * 32 + l32;
                 const bool row_ok = row < nq;
                 S rowv, tauv;
-                if (kInt) {
+                if (prefetch) {
+                    rowv = rowq[ra];
+                    tauv = kInt ? (S)0 : tauq[ra];
+                } else if (kInt) {
                     // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
-                    rowv = row_ok ? (FILTER ? flt.thr[row] : qn[row]) : (FILTER ? (S)0x80000000 : (S)0);
+                    rowv = row_ok ? flt.thr[row] : (S)0x80000000;
                     tauv = 0;
                 } else {
                     rowv = (row_ok && metric == kMetricL2) ? qn[row] : (S)0;
-                    tauv = (FILTER && row_ok) ? flt.tau[row] : (S)(-__builtin_inff());
+                    tauv = row_ok ? flt.tau[row] : (S)(-__builtin_inff());
                 }
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
