@@ -36,6 +36,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int kRingTM = 256, kRingTN = 128, kRingRows = kRingTM + kRingTN;
 constexpr int kRingStageBytes = kRingRows * 64;
 constexpr int kRingStages = 3;
+constexpr int kRingAuxBytes = 1280;   // per-wave staging of a filtered epilogue's operands
 constexpr int kRingLoadsPerWave = kRingRows / 16 / 4;  // wave-wide 1 KB loads per stage and wavefront
 
 struct I8Traits {
@@ -44,7 +45,7 @@ struct I8Traits {
     using Acc = v16i;
     static constexpr int kElemsPerStep = 64;
     // one K-step = 2 sub-steps of 32 bytes; a lane half owns 16 of them
-    template <bool SWAP>
+    template <bool SWAP, bool ZERO>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -66,8 +67,9 @@ struct I8Traits {
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[rb], a[ra], acc[ra][rb], 0, 0, 0)
-                                       : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                    const Acc c0 = (ZERO && kk == 0) ? Acc{} : acc[ra][rb];   // a tile's first product starts from zero
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[rb], a[ra], c0, 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], c0, 0, 0, 0);
                 }
             }
         }
@@ -80,7 +82,7 @@ struct Bf16Traits {
     using S = float;
     using Acc = v16f;
     static constexpr int kElemsPerStep = 32;
-    template <bool SWAP>
+    template <bool SWAP, bool ZERO>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -102,8 +104,9 @@ struct Bf16Traits {
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[rb], a[ra], acc[ra][rb], 0, 0, 0)
-                                       : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], acc[ra][rb], 0, 0, 0);
+                    const Acc c0 = (ZERO && kk == 0) ? Acc{} : acc[ra][rb];
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[rb], a[ra], c0, 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], c0, 0, 0, 0);
                 }
             }
         }
@@ -117,7 +120,7 @@ struct F32Traits {
     static constexpr int kElemsPerStep = 16;
     // one K-step = 16 floats; a lane half owns 8 of them (two 16-byte chunks) and feeds them to 8
     // consecutive 32x32x2 MFMAs
-    template <bool SWAP>
+    template <bool SWAP, bool ZERO>
     static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
                                                Acc (&acc)[4][2])
     {
@@ -143,8 +146,9 @@ struct F32Traits {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
                     const float av = a[ra][t >> 2][t & 3], bv = b[rb][t >> 2][t & 3];
-                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, acc[ra][rb], 0, 0, 0)
-                                       : __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[ra][rb], 0, 0, 0);
+                    const Acc c0 = (ZERO && t == 0) ? Acc{} : acc[ra][rb];
+                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, c0, 0, 0, 0)
+                                       : __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, c0, 0, 0, 0);
                 }
             }
         }
@@ -219,17 +223,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     };
 
-    typename Tr::Acc acc[4][2];
-#pragma unroll
-    for (int a = 0; a < 4; a++) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[a][b][r] = 0;
-            }
-        }
-    }
+    typename Tr::Acc acc[4][2];   // written from zero by the first K-step of every tile
 
     // (item, step, ring slot) of the next K-step to issue and of the one being computed
     int issued = 0, i_it = 0, i_ks = 0, i_slot = 0;
@@ -251,44 +245,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int c_it = 0, c_ks = 0, c_slot = 0;
     bool stored = false;  // the previous iteration ended with an epilogue that issued stores
 
-    // Filtered launches fetch what the epilogue of a tile needs -- the base norms of the lane's 32
-    // columns and the bounds of its 4 query rows -- one K-step ahead, so the epilogue never waits
-    // for memory.  The fetch is a fixed number of loads (kPrefetchLoads) because the s_waitcnt
-    // immediates below count them.
-    constexpr int kPrefetchLoads = 8 + (kInt ? 4 : 8);
-    S bnq[2][4][4];
-    S rowq[4], tauq[4];
-    const bool prefetch = FILTER && nk >= 2 && nb % 4 == 0 && reinterpret_cast<uintptr_t>(bn) % 16 == 0 && bn != nullptr &&
-                          qn != nullptr;
+    // Filtered launches stage what the epilogue of a tile needs -- the base norms of the wave's 64
+    // columns and the bounds (and norms) of its 128 query rows -- in a small per-wave LDS area, with
+    // the same global->LDS loads as the ring and one K-step ahead, so the epilogue never waits for
+    // memory and the main loop carries no registers for it.  The s_waitcnt immediates below count
+    // these loads (kPrefetchLoads per wave).
+    //   aux +   0: 64 base norms      (lanes 0..15, 16 bytes each)
+    //   aux + 256: 128 tau or thr     (lanes 16..47)
+    //   aux + 768: 128 query norms    (lanes 0..31 of a second load; fp32 scores only)
+    constexpr int kPrefetchLoads = kInt ? 1 : 2;
+    unsigned char *aux = ring + kRingStages * kRingStageBytes + wave * kRingAuxBytes;
+    const S *bound = kInt ? flt.thr : flt.tau;
+    const bool prefetch = FILTER && nk >= 2 && nb % 4 == 0 && nq % 4 == 0 && bn != nullptr && qn != nullptr &&
+                          bound != nullptr && reinterpret_cast<uintptr_t>(bn) % 16 == 0 &&
+                          reinterpret_cast<uintptr_t>(qn) % 16 == 0 && reinterpret_cast<uintptr_t>(bound) % 16 == 0;
     bool fetched = false;   // the previous iteration issued the fetch
     auto fetch_epilogue_operands = [&](int it) {
         int64_t tm, tn;
         item_tile(it, tm, tn);
         const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++) {
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
-                col = col + 3 < nb ? col : 0;     // out-of-range columns are rejected by index later
-                const uint4 u = *reinterpret_cast<const uint4 *>(bn + col);
-                bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
-                bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
-                bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
-                bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
-            }
-        }
-#pragma unroll
-        for (int ra = 0; ra < 4; ra++) {
-            int64_t row = i0 + wr * 128 + ra * 32 + l32;
-            row = row < nq ? row : 0;
-            if constexpr (kInt) {
-                rowq[ra] = flt.thr[row];
+        asm volatile("" ::: "memory");
+        if (lane < 48) {
+            // groups of four that start past the end read group 0 instead; their scores are rejected
+            // by index in the epilogue
+            const S *p;
+            if (lane < 16) {
+                const int64_t col = j0 + wc * 64 + lane * 4;
+                p = bn + (col < nb ? col : 0);
             } else {
-                rowq[ra] = qn[row];
-                tauq[ra] = flt.tau[row];
+                const int64_t row = i0 + wr * 128 + (lane - 16) * 4;
+                p = bound + (row < nq ? row : 0);
+            }
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
+                                             (__attribute__((address_space(3))) void *)aux, 16, 0, 0);
+        }
+        if constexpr (!kInt) {
+            if (lane < 32) {
+                const int64_t row = i0 + wr * 128 + lane * 4;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(qn + (row < nq ? row : 0)),
+                                                 (__attribute__((address_space(3))) void *)(aux + 768), 16, 0, 0);
             }
         }
+        asm volatile("" ::: "memory");
     };
     for (int g = 0; g < total; g++) {
         // The loads of step g must have landed; later steps may still be in flight.  vmcnt counts
@@ -312,14 +310,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         stored = false;
         fetched = false;
         __builtin_amdgcn_s_barrier();
-        if (issued < total) {
+        const bool issued_now = issued < total;
+        if (issued_now) {
             issue_next();  // goes into the buffer that step g - 1 has just finished reading
         }
         if (FILTER && prefetch && c_ks == nk - 2) {
             fetch_epilogue_operands(c_it);
             fetched = true;
         }
-        Tr::template mma<FILTER>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
+        if (c_ks == 0) {
+            Tr::template mma<FILTER, true>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
+        } else {
+            Tr::template mma<FILTER, false>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
+        }
         const bool last_step = c_ks == nk - 1;
         const int done_it = c_it;
         c_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
@@ -340,9 +343,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             item_tile(done_it, tm, tn);
             const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
             const bool vec_out = !FILTER && (ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
-            // without the early fetch: the base norms of this lane's 32 columns, loaded here
+            // the base norms of this lane's 32 columns: out of the staging area, or loaded here
+            S bnq[2][4][4];
             const bool use_bn = kInt || metric == kMetricL2;
             const bool vec_bn = reinterpret_cast<uintptr_t>(bn) % 16 == 0;
+            if (prefetch) {
+                // the staging loads are older than the K-step loads issued in this iteration
+                if (issued_now) {
+                    __builtin_amdgcn_s_waitcnt(0x0f70 | kRingLoadsPerWave);
+                } else {
+                    __builtin_amdgcn_s_waitcnt(0x0f70);
+                }
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
+                        bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
+                        bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
+                        bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
+                        bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
+                    }
+                }
+            }
 #pragma unroll
             for (int rb = 0; rb < 2 && !prefetch; rb++) {
 #pragma unroll
@@ -362,6 +386,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     }
                 }
             }
+            if constexpr (kInt) {
+                // -|b|^2, so that a score's test value is one shift-add: 2 q.b - |b|^2
+#pragma unroll
+                for (int t = 0; t < 32; t++) {
+                    bnq[t >> 4][(t >> 2) & 3][t & 3] = -bnq[t >> 4][(t >> 2) & 3][t & 3];
+                }
+            }
 #pragma unroll
             for (int ra = 0; ra < 4; ra++) {
                 asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
@@ -369,8 +400,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const bool row_ok = row < nq;
                 S rowv, tauv;
                 if (prefetch) {
-                    rowv = rowq[ra];
-                    tauv = kInt ? (S)0 : tauq[ra];
+                    const S bv = *reinterpret_cast<const S *>(aux + 256 + (ra * 32 + l32) * 4);
+                    rowv = kInt ? bv : *reinterpret_cast<const S *>(aux + 768 + (ra * 32 + l32) * 4);
+                    tauv = kInt ? (S)0 : bv;
                 } else if (kInt) {
                     // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
                     rowv = row_ok ? flt.thr[row] : (S)0x80000000;
@@ -389,7 +421,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     for (int r = 0; r < 16; r++) {
                         const S bnv = bnq[rb][r >> 2][r & 3];
                         if constexpr (kInt) {
-                            v[r] = bnv - 2 * acc[ra][rb][r];          // compared with tau - |q|^2
+                            // bnq holds -|b|^2: v = -(distance - |q|^2) in one shift-add, largest is best
+                            v[r] = (S)(((uint32_t)acc[ra][rb][r] << 1) + (uint32_t)bnv);
+                            best = (r == 0 || v[r] > best) ? v[r] : best;
+                            continue;
                         } else {
                             const float g = acc[ra][rb][r];
                             if (metric == kMetricL2) {
@@ -400,16 +435,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                 v[r] = -g;
                             }
                         }
-                        acc[ra][rb][r] = 0;
                         best = v[r] < best ? v[r] : best;
                     }
                     const S lane_bound = kInt ? rowv : tauv;
+                    if constexpr (kInt) {
+                        best = -best;
+                    }
                     if (__ballot(row_ok && best <= lane_bound)) {
+                        // opaque to the optimiser here, or it keeps all 32 column offsets of this rare
+                        // path in registers across the whole main loop
+                        int cb = wc * 64 + rb * 32 + 4 * half;
+                        asm volatile("" : "+v"(cb));
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
-                            const int64_t col = j0 + wc * 64 + rb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                            if (row_ok && v[r] <= lane_bound && col < nb) {
-                                S val = v[r];
+                            const int64_t col = j0 + cb + 8 * (r >> 2) + (r & 3);
+                            const S part = kInt ? -v[r] : v[r];
+                            if (row_ok && part <= lane_bound && col < nb) {
+                                S val = part;
                                 if constexpr (kInt) {
                                     val += qn[row];
                                 }
@@ -474,7 +516,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             }
                             admit = v <= tauv[r];
                         }
-                        acc[ra][rb][r] = 0;
                         if (FILTER) {
                             if (admit && col < nb) {
                                 if constexpr (kInt) {
@@ -515,7 +556,7 @@ bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, i
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     }
     const unsigned grid = (unsigned)((2 * cus + 7) / 8 * 8);   // two persistent workgroups per CU
-    const size_t smem = (size_t)kRingStages * kRingStageBytes;
+    const size_t smem = (size_t)kRingStages * kRingStageBytes + (filter ? 4 * kRingAuxBytes : 0);
     if (filter) {
         auto kern = score_ring_kernel<Tr, true>;
         IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
