@@ -154,6 +154,8 @@ typedef struct ivfpq_search_stats {
     double ms_total;
     double scan_launches; /* kernel launches covered by ms_scan */
     double nsplit;        /* workgroups per query in the scan */
+    double scan_waves;    /* wavefronts per scan workgroup */
+    double shared_pool;   /* 1: one workgroup-wide candidate pool (large k), 0: one pool per wavefront */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 

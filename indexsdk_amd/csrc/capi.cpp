@@ -224,6 +224,8 @@ IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stat
         out->ms_total = s.ms_total;
         out->scan_launches = s.scan_launches;
         out->nsplit = s.nsplit;
+        out->scan_waves = s.scan_waves;
+        out->shared_pool = s.shared_pool;
     });
 }
 

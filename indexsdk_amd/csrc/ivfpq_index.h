@@ -33,6 +33,8 @@ struct SearchStats {
     double ms_total = 0;        // device time of the whole search
     double scan_launches = 0;   // kernel launches the ms_scan figure covers
     double nsplit = 0;
+    double scan_waves = 0;
+    double shared_pool = 0;
 };
 
 class IvfpqIndex {

@@ -648,6 +648,12 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     p.order = nullptr;
     p.xcd_chunks = (getenv("IXA_XCD_CHUNKS") && nsplit == 1) ? 1 : 0;
     launch_scan(p, n, stream_);
+    {
+        ScanParams planned = p;
+        plan_scan(planned);
+        stats_.scan_waves = planned.waves;
+        stats_.shared_pool = planned.shared_pool;
+    }
     IXA_HIP(hipEventRecord(ev_[2], stream_));
 
     IXA_HIP(hipMemsetAsync(ws_counter_.data(), 0, 8, stream_));

@@ -31,7 +31,7 @@ struct ScanParams {
     int xcd_chunks;            // 1: deal contiguous chunks of the execution order to the 8 XCDs
     int64_t nq;                // filled by launch_scan()
     // filled by plan_scan()
-    int waves, cap, merge_n, table_n, off_query, off_pools, off_merge, off_table, off_misc;
+    int waves, shared_pool, cap, merge_n, table_n, off_query, off_pools, off_merge, off_table, off_hist, off_misc;
 };
 
 // Computes the LDS plan of a launch; returns the dynamic LDS bytes it needs.

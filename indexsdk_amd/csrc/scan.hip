@@ -50,7 +50,9 @@ struct GroupRef {
 
 // MT > 0: compile-time number of sub-quantizers; MT == 0: run-time p.M with byte loads.
 // W: wavefronts per workgroup (the workgroup serves one query, or one split of a query).
-template <int MT, typename LutT, int LAYOUT, int W>
+// SHARED: one workgroup-wide candidate pool (BlockPool) instead of W private ones (WavePool); the
+// choice for k so large that private pools would leave room for only a few waves per CU.
+template <int MT, typename LutT, int LAYOUT, int W, bool SHARED>
 __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -146,7 +148,14 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
     // ---- stages 3 + 4: the probed lists form one sequence of 64-code groups; wavefront w takes
     // groups w, w + W, ... of that sequence, so the waves stay balanced whatever the list lengths.
     WavePool<float> pool;
-    pool.init(pools + wave * p.cap, p.cap, p.k);
+    BlockPool<W> bpool;
+    if constexpr (SHARED) {
+        bpool.init(pools, p.cap, p.k, reinterpret_cast<int *>(smem_raw + p.off_hist),
+                   reinterpret_cast<BlockPoolCtl *>(counts + W), tid);
+        __syncthreads();
+    } else {
+        pool.init(pools + wave * p.cap, p.cap, p.k);
+    }
     const int l32 = lane & 31;
     const int total = nlocal > 0 ? __builtin_amdgcn_readfirstlane(t_gend[nlocal - 1]) : 0;
     int li = 0;          // list the current group belongs to (monotone, wave-uniform)
@@ -263,25 +272,61 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
             adopt_shared();                                                                           \
         }                                                                                             \
     } while (0)
-    if (wave < total) {
-        uint32_t wa[NW], wb[NW];
-        GroupRef ga = locate(wave), gb = ga;
-        load_codes(ga.slot, wa);
-        for (int G = wave; G < total; G += 2 * W) {
-            IXA_SCAN_STEP(G, ga, wa, gb, wb);
-            if (G + W < total) {
-                IXA_SCAN_STEP(G + W, gb, wb, ga, wa);
+    // The same step for the shared pool: poll for a pending prune, evaluate, reserve-and-append;
+    // a failed reservation is retried after the workgroup has pruned the pool.
+#define IXA_SCAN_STEP_SHARED(G, CUR, WCUR, NXT, WNXT)                                                 \
+    do {                                                                                              \
+        if ((G) + W < total) {                                                                        \
+            NXT = locate((G) + W);                                                                    \
+            load_codes(NXT.slot, WNXT);                                                               \
+        }                                                                                             \
+        if (bpool.poll()) {                                                                           \
+            bpool.rendezvous(tid);                                                                    \
+        }                                                                                             \
+        const float s_ = adc(CUR.slot, WCUR);                                                         \
+        while (!bpool.try_push(CUR.valid && s_ <= bpool.bound, s_, CUR.slot, lane)) {                 \
+            bpool.rendezvous(tid);                                                                    \
+        }                                                                                             \
+    } while (0)
+    int total_keys;
+    if constexpr (SHARED) {
+        if (wave < total) {
+            uint32_t wa[NW], wb[NW];
+            GroupRef ga = locate(wave), gb = ga;
+            load_codes(ga.slot, wa);
+            for (int G = wave; G < total; G += 2 * W) {
+                IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb);
+                if (G + W < total) {
+                    IXA_SCAN_STEP_SHARED(G + W, gb, wb, ga, wa);
+                }
             }
         }
+        bpool.finish_wave(lane);
+        while (!bpool.rendezvous(tid)) {
+        }
+        total_keys = bpool.sort_all(tid);
+    } else {
+        if (wave < total) {
+            uint32_t wa[NW], wb[NW];
+            GroupRef ga = locate(wave), gb = ga;
+            load_codes(ga.slot, wa);
+            for (int G = wave; G < total; G += 2 * W) {
+                IXA_SCAN_STEP(G, ga, wa, gb, wb);
+                if (G + W < total) {
+                    IXA_SCAN_STEP(G + W, gb, wb, ga, wa);
+                }
+            }
+        }
+        __syncthreads();  // every wave has published its last value; the LUT is no longer needed
+        adopt_shared();
+        pool.finish(lane);
+        if (lane == 0) {
+            counts[wave] = pool.count;
+        }
+        total_keys = block_merge_pools<W>(pools, p.cap, counts, nullptr, 0, tid);
     }
 #undef IXA_SCAN_STEP
-    __syncthreads();  // every wave has published its last value; the LUT is no longer needed
-    adopt_shared();
-    pool.finish(lane);
-    if (lane == 0) {
-        counts[wave] = pool.count;
-    }
-    const int total_keys = block_merge_pools<W>(pools, p.cap, counts, nullptr, 0, tid);
+#undef IXA_SCAN_STEP_SHARED
     const key_t *merge = pools;
 
     if (p.nsplit > 1) {
@@ -364,15 +409,22 @@ template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
     const int64_t slots = p.xcd_chunks ? (nq + 7) / 8 * 8 : nq;
-    if (p.waves == 8) {
-        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8>;
+    if (p.shared_pool) {
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, true>;
+        if (smem > 48 * 1024) {
+            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
+    } else if (p.waves == 8) {
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, false>;
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         }
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else {
-        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4>;
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4, false>;
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -404,35 +456,63 @@ static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
     }
 }
 
-static size_t plan_with_waves(ScanParams &p, int waves)
+static size_t plan_with_waves(ScanParams &p, int waves, bool shared)
 {
     const size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
     p.waves = waves;
-    p.cap = wave_pool_capacity(p.k);
-    p.merge_n = waves * p.cap;
+    p.shared_pool = shared ? 1 : 0;
+    p.cap = shared ? block_pool_capacity(p.k, waves) : wave_pool_capacity(p.k);
+    p.merge_n = shared ? p.cap : waves * p.cap;
     p.table_n = (p.nprobe + p.nsplit - 1) / p.nsplit;
     size_t off = round_up((int64_t)lut_bytes, 16);
     p.off_query = (int)off;
     off += round_up((int64_t)p.d * 4, 16);
     p.off_pools = (int)off;
-    off += (size_t)waves * p.cap * sizeof(key_t);   // also the merge array of the epilogue
+    off += (size_t)p.merge_n * sizeof(key_t);   // also the merge array of the epilogue
     p.off_merge = p.off_pools;
     p.off_table = (int)off;
     off += round_up((int64_t)p.table_n * 12, 16);
+    p.off_hist = (int)off;
+    off += shared ? 4096 : 0;
     p.off_misc = (int)off;
-    off += 128;
+    off += 128;   // share[W], counts[W], BlockPoolCtl
     return off;
 }
 
-// Eight wavefronts per workgroup when three such workgroups still fit the 160 KB of a CU,
-// otherwise four.
+// Wavefronts one CU can hold with this plan (LDS- and thread-limited; 160 KB, 2048 threads).
+static int resident_waves(size_t smem, int waves)
+{
+    const int by_lds = (int)(160 * 1024 / smem), by_threads = 2048 / (waves * 64);
+    return std::min(by_lds, by_threads) * waves;
+}
+
+// Private pools with eight wavefronts per workgroup when three such workgroups fit the 160 KB of
+// a CU; otherwise whichever of {private x 8, private x 4, shared x 8} keeps most wavefronts resident.
 size_t plan_scan(ScanParams &p)
 {
-    size_t smem = plan_with_waves(p, 8);
-    if (smem * 3 > 160 * 1024) {
-        smem = plan_with_waves(p, 4);
+    ScanParams best = p;
+    size_t best_smem = plan_with_waves(best, 8, false);
+    if (best_smem * 3 <= 160 * 1024) {
+        p = best;
+        return best_smem;
     }
-    return smem;
+    int best_waves = best_smem <= 160 * 1024 ? resident_waves(best_smem, 8) : 0;
+    const bool shared_ok = block_pool_capacity(p.k, 8) <= 8 * 8 * kWave;
+    for (int alt = 0; alt < 2; alt++) {
+        if (alt == 1 && !shared_ok) {
+            continue;
+        }
+        ScanParams q = p;
+        const size_t smem = alt == 0 ? plan_with_waves(q, 4, false) : plan_with_waves(q, 8, true);
+        const int rw = smem <= 160 * 1024 ? resident_waves(smem, alt == 0 ? 4 : 8) : 0;
+        if (rw > best_waves) {
+            best = q;
+            best_smem = smem;
+            best_waves = rw;
+        }
+    }
+    p = best;
+    return best_smem;
 }
 
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s)

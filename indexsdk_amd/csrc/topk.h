@@ -325,6 +325,261 @@ __device__ inline int block_merge_pools(key_t *pools, int cap, const int *counts
     return total;
 }
 
+// BlockPool: ONE unsorted candidate pool shared by the W wavefronts of a workgroup, for k too large
+// for W private pools.  A wave reserves room with one LDS atomic per push.  When a reservation does
+// not fit, the wave raises `flag` and waits at a rendezvous; every other wave joins at its next
+// checkpoint (it polls `flag` once per group) or when it has run out of work, and the whole
+// workgroup prunes the pool together: two 1024-bin histogram passes over the top 20 bits of the
+// ordered scores find the smallest bucket with k candidates at or below it, everything above is
+// dropped and the bound tightens to the top of that bucket.
+//
+// Protocol (each wave executes the same number of barriers):
+//   scanning wave:  if (poll()) rendezvous();  ...  while (!try_push(...)) rendezvous();
+//   finished wave:  finish_wave();  while (!rendezvous()) {}
+// rendezvous() returns true once every wave has called finish_wave().
+struct BlockPoolCtl {
+    int count;      // reserved entries (may run past cap once a reservation failed)
+    int valid_end;  // entries [0, min(count, valid_end)) are written
+    int flag;       // a reservation failed: prune at the next rendezvous
+    int done;       // waves that have finished their work
+    int kept;
+    int bin;        // histogram search result
+    int below;      // candidates in bins before `bin`
+    float bound;
+};
+
+template <int W>
+struct BlockPool {
+    static constexpr int NT = W * kWave;
+    static constexpr int kMaxPerThread = 8;   // cap <= 8 * NT
+    key_t *buf;
+    int *hist;                 // 1024 ints
+    volatile BlockPoolCtl *ctl;
+    int cap, k;
+    float bound;               // wave-uniform copy of ctl->bound
+
+    // All threads call; a __syncthreads() must follow before the first push.
+    __device__ __forceinline__ void init(key_t *b, int cap_, int k_, int *hist_, BlockPoolCtl *c, int tid)
+    {
+        buf = b;
+        cap = cap_;
+        k = k_;
+        hist = hist_;
+        ctl = c;
+        bound = __builtin_inff();
+        if (tid == 0) {
+            c->count = 0;
+            c->valid_end = cap_;
+            c->flag = 0;
+            c->done = 0;
+            c->kept = 0;
+            c->bound = __builtin_inff();
+        }
+    }
+
+    __device__ __forceinline__ bool poll() const { return __builtin_amdgcn_readfirstlane(ctl->flag) != 0; }
+
+    // All lanes of the wave call.  False: the pool is full -- call rendezvous(), re-test the
+    // candidates against the new bound and try again.
+    __device__ __forceinline__ bool try_push(bool pass, float score, uint32_t idx, int lane)
+    {
+        const unsigned long long mask = __ballot(pass);
+        if (mask == 0) {
+            return true;
+        }
+        const int n = __popcll(mask);
+        const int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+        int base = 0;
+        if (lane == 0) {
+            base = atomicAdd(const_cast<int *>(&ctl->count), n);
+        }
+        base = __builtin_amdgcn_readfirstlane(base);
+        if (base + n <= cap) {
+            if (pass) {
+                buf[base + pre] = make_key(score, idx);
+            }
+            return true;
+        }
+        if (lane == 0) {
+            if (base < cap) {
+                ctl->valid_end = base;   // the one reservation that straddles the end
+            }
+            ctl->flag = 1;
+        }
+        return false;
+    }
+
+    __device__ __forceinline__ void finish_wave(int lane)
+    {
+        if (lane == 0) {
+            atomicAdd(const_cast<int *>(&ctl->done), 1);
+        }
+    }
+
+    __device__ __forceinline__ int size() const
+    {
+        const int c = ctl->count, v = ctl->valid_end;
+        return c < v ? c : v;
+    }
+
+    // Wave 0: first bin whose inclusive prefix count reaches `rank` (1 <= rank <= total).
+    __device__ inline void find_bin(int rank, int tid)
+    {
+        if (tid < kWave) {
+            int part = 0;
+            for (int j = 0; j < 16; j++) {
+                part += hist[tid * 16 + j];
+            }
+            int incl = part;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const int up = __shfl_up(incl, o);
+                if (tid >= o) {
+                    incl += up;
+                }
+            }
+            const unsigned long long reach = __ballot(incl >= rank);
+            const int owner = reach ? __builtin_ctzll(reach) : kWave - 1;
+            if (tid == owner) {
+                int run = incl - part, bin = tid * 16 + 15;
+                for (int j = 0; j < 16; j++) {
+                    if (run + hist[tid * 16 + j] >= rank) {
+                        bin = tid * 16 + j;
+                        break;
+                    }
+                    run += hist[tid * 16 + j];
+                }
+                ctl->bin = bin;
+                ctl->below = run;
+            }
+        }
+    }
+
+    // All NT threads: drop what cannot be among the k best, tighten the bound, reopen the pool.
+    __device__ inline void prune(int tid)
+    {
+        constexpr int SH = 32 - kSelectBits;
+        const int lane = tid & 63;
+        const int n = size();
+        key_t e[kMaxPerThread];
+#pragma unroll
+        for (int j = 0; j < kMaxPerThread; j++) {
+            const int i = j * NT + tid;
+            e[j] = i < n ? buf[i] : kEmptyKey;
+        }
+        uint32_t P = 0xffffffffu >> SH;   // keep everything unless k candidates exist
+        if (n >= k) {
+            for (int i = tid; i < 1024; i += NT) {
+                hist[i] = 0;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < kMaxPerThread; j++) {
+                if (e[j] != kEmptyKey) {
+                    atomicAdd(&hist[(uint32_t)(e[j] >> (32 + SH + 10))], 1);
+                }
+            }
+            __syncthreads();
+            find_bin(k, tid);
+            __syncthreads();
+            const uint32_t b1 = (uint32_t)ctl->bin;
+            const int rank2 = k - ctl->below;
+            __syncthreads();
+            for (int i = tid; i < 1024; i += NT) {
+                hist[i] = 0;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < kMaxPerThread; j++) {
+                const uint32_t pre = (uint32_t)(e[j] >> (32 + SH));
+                if (e[j] != kEmptyKey && (pre >> 10) == b1) {
+                    atomicAdd(&hist[pre & 1023u], 1);
+                }
+            }
+            __syncthreads();
+            find_bin(rank2, tid);
+            __syncthreads();
+            P = (b1 << 10) | (uint32_t)ctl->bin;
+        }
+        if (tid == 0) {
+            ctl->kept = 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kMaxPerThread; j++) {
+            const bool keep = e[j] != kEmptyKey && (uint32_t)(e[j] >> (32 + SH)) <= P;
+            const unsigned long long mask = __ballot(keep);
+            if (mask) {
+                const int pre =
+                    __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+                int base = 0;
+                if (lane == 0) {
+                    base = atomicAdd(const_cast<int *>(&ctl->kept), __popcll(mask));
+                }
+                base = __builtin_amdgcn_readfirstlane(base);
+                if (keep) {
+                    buf[base + pre] = e[j];
+                }
+            }
+        }
+        __syncthreads();
+        int kept = ctl->kept;
+        float top = ScoreOps<float>::bucket_top((P << SH) | ((1u << SH) - 1u));
+        if (kept > cap - NT) {
+            // one bucket holds almost everything: exact selection by sorting
+            for (int i = kept + tid; i < cap; i += NT) {
+                buf[i] = kEmptyKey;
+            }
+            block_bitonic_sort(buf, cap, tid, NT);
+            kept = k;
+            top = key_score(buf[k - 1]);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            const float b = ctl->bound;
+            ctl->bound = (n >= k && top < b) ? top : b;
+            ctl->count = kept;
+            ctl->valid_end = cap;
+            ctl->flag = 0;
+        }
+        __syncthreads();
+    }
+
+    // All waves of the workgroup meet here.  True once every wave has finished its work.
+    __device__ inline bool rendezvous(int tid)
+    {
+        __syncthreads();
+        const int f = ctl->flag, d = ctl->done;
+        __syncthreads();
+        if (f) {
+            prune(tid);
+        }
+        bound = wave_uniform(ctl->bound);
+        return d == W;
+    }
+
+    // After the last rendezvous: sorts the pool ascending in place, returns the number of keys.
+    __device__ inline int sort_all(int tid)
+    {
+        const int n = size();
+        __syncthreads();
+        for (int i = n + tid; i < cap; i += NT) {
+            buf[i] = kEmptyKey;
+        }
+        block_bitonic_sort(buf, cap, tid, NT);
+        return n;
+    }
+};
+
+inline int block_pool_capacity(int k, int waves)
+{
+    int cap = 1024;
+    while (cap < k + 2 * waves * kWave) {
+        cap <<= 1;
+    }
+    return cap;
+}
+
 inline int wave_pool_capacity(int k)
 {
     int cap = 256;

@@ -278,3 +278,37 @@ def test_twin_c5_zipf_large_k(ix, oracle):
 
 def test_twin_c1_small(ix, oracle):
     _twin(ix, oracle, 34, 100_000, 300, 128, 64, 0.3, 256, 16, ix.METRIC_L2, 0, 16, 10, niter=6)
+
+
+def test_large_k_shared_pool_one_workgroup_per_query(ix, oracle):
+    """k = 1024 with enough queries that each gets a single workgroup: the workgroup-wide candidate
+    pool must prune many times per query and still return exactly the oracle's top-k."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 41, 40000, 2100, 96, 16, 48, ix.METRIC_L2)
+    gpu.setNumProbes(8)
+    D, I = gpu.search(q, 1024)
+    st = gpu.last_search_stats()
+    assert st["shared_pool"] == 1 and st["nsplit"] == 1
+    Dr, Ir = ref.search(q, 1024, 8)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+
+
+def test_large_k_shared_pool_all_scores_tie(ix, oracle):
+    """A base of few distinct vectors: whole lists share one distance, so the bucket search cannot
+    separate candidates and the pool falls back to exact selection by sorting."""
+    rng = np.random.default_rng(43)
+    d, M, nlist = 96, 48, 8
+    protos = rng.standard_normal((6, d)).astype(np.float32)
+    x = protos[rng.integers(0, 6, 20000)]
+    q = (protos[rng.integers(0, 6, 50)] + 0.1 * rng.standard_normal((50, d))).astype(np.float32)
+    cent, _ = oracle.kmeans(x + 0.01 * rng.standard_normal(x.shape).astype(np.float32), nlist, niter=3, seed=1)
+    cb = oracle.train_pq((x + 0.3 * rng.standard_normal(x.shape)).astype(np.float32)[:4000], M, niter=3, seed=1)
+    ids = np.arange(20000, dtype=np.int64)
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, ids)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add_with_ids(x, ids)
+    gpu.setNumProbes(nlist)
+    D, I = gpu.search(q, 1024)
+    assert gpu.last_search_stats()["shared_pool"] == 1
+    Dr, Ir = ref.search(q, 1024, nlist)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
