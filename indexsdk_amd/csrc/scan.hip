@@ -42,6 +42,25 @@ __device__ __forceinline__ __half to_lut<__half>(float v)
 __device__ __forceinline__ float from_lut(float v) { return v; }
 __device__ __forceinline__ float from_lut(__half v) { return __half2float(v); }
 
+// Half-precision LUT under the rot32 code layout.  Two halves share one 32-bit LDS word, so "32
+// lanes read 32 different sub-quantizers" only means 32 different banks if the two halves of a word
+// never belong to different sub-quantizer offsets of a 32-block.  Blocks of 32 sub-quantizers are
+// therefore paired: block pair p owns 32 KB, codeword kk a row of 32 words in it, word r holds
+// sub-quantizer r of the even block (low half) and of the odd block (high half).  A last unpaired
+// block pairs codewords instead: row kk / 2, half kk % 2.  Either way a lane's word index is
+// (row * 32 + r) and r is distinct across the 32 lanes: no bank conflicts for any code values.
+__host__ __device__ __forceinline__ int rot32_half_slot(int nblocks, int m, int kk)
+{
+    const int b = m >> 5, r = m & 31;
+    int byte;
+    if (b < (nblocks & ~1)) {
+        byte = (b >> 1) * 32768 + kk * 128 + r * 4 + 2 * (b & 1);
+    } else {
+        byte = (nblocks >> 1) * 32768 + (kk >> 1) * 128 + r * 4 + 2 * (kk & 1);
+    }
+    return byte >> 1;
+}
+
 // One 64-code group of a probed list, as a wavefront sees it.
 struct GroupRef {
     uint32_t slot;  // arena slot of this lane's code
@@ -52,8 +71,11 @@ struct GroupRef {
 // W: wavefronts per workgroup (the workgroup serves one query, or one split of a query).
 // SHARED: one workgroup-wide candidate pool (BlockPool) instead of W private ones (WavePool); the
 // choice for k so large that private pools would leave room for only a few waves per CU.
+// The half-LUT rot32 variants are held to 128 registers (4 waves per SIMD): their LDS plan admits
+// two 8-wave workgroups per CU and the register allocator would otherwise trade that away.
 template <int MT, typename LutT, int LAYOUT, int W, bool SHARED>
-__global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
+__global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARED) ? 4 : 1) void ivfpq_scan_kernel(
+    ScanParams p)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     constexpr int NT = W * 64;
@@ -139,7 +161,10 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
             } else {
                 v = -ip;  // minimise the negated inner product
             }
-            const int slot = LAYOUT == 1 ? kk * M + m : m * 256 + kk;
+            int slot = LAYOUT == 1 ? kk * M + m : m * 256 + kk;
+            if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
+                slot = rot32_half_slot(M / 32, m, kk);
+            }
             lut[slot] = to_lut<LutT>(v);
         }
     }
@@ -214,6 +239,16 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
         }
     };
 
+    // byte offset of this lane's word in a 32-word LUT row at each of the 32 rotation steps; kept
+    // in registers (opaque to the optimiser, which would otherwise recompute them per lookup)
+    uint32_t rot4[32];
+    if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
+#pragma unroll
+        for (int j = 0; j < 32; j++) {
+            rot4[j] = (uint32_t)((j + l32) & 31) << 2;
+            asm volatile("" : "+v"(rot4[j]));
+        }
+    }
     auto adc = [&](uint32_t slot, const uint32_t (&w)[NW]) -> float {
         if (MT == 0) {
             const uint8_t *cp = p.codes + (int64_t)slot * M;
@@ -223,7 +258,30 @@ __global__ __launch_bounds__(W * 64) void ivfpq_scan_kernel(ScanParams p)
             }
             return s;
         }
-        if (LAYOUT == 1) {
+        if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
+            // paired-block half LUT (rot32_half_slot); the conversion to fp32 and the addition are
+            // one v_fma_mix_f32 (half * 1.0 + fp32 accumulator: the same value as convert-then-add)
+            constexpr int NB = MT / 32;
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            const unsigned char *lb = reinterpret_cast<const unsigned char *>(lut);
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const uint32_t ww = w[(m >> 2) % NW];
+                const int b = m >> 5;
+                const uint32_t r4 = rot4[m & 31];
+                uint32_t off;
+                if (b < (NB & ~1)) {
+                    const uint32_t code = (ww >> (8 * (m & 3))) & 0xffu;
+                    off = ((code << 7) | r4) + (uint32_t)((b >> 1) * 32768 + 2 * (b & 1));
+                } else {
+                    const uint32_t c1 = (ww >> (8 * (m & 3) + 1)) & 0x7fu, c0 = (ww >> (8 * (m & 3))) & 1u;
+                    off = (((c1 << 7) | r4) | (c0 << 1)) + (uint32_t)((NB >> 1) * 32768);
+                }
+                const uint32_t raw = *reinterpret_cast<const uint16_t *>(lb + off);
+                asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(acc[m & 3]) : "v"(raw));
+            }
+            return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        } else if (LAYOUT == 1) {
             // any association is within tolerance: four independent partial sums
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
