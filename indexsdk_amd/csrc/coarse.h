@@ -69,6 +69,13 @@ void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t 
 void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
                             int64_t col_base, unsigned long long *running, hipStream_t s);
 
+// Exact best-nout SET from approximately scored, sorted candidates (see refine_boundary_kernel):
+// re-evaluates only the candidates within 2 * err of the rank-nout score; raises *flag when the
+// list cannot be proven to contain every winner.  out_ids: [nq][nout], unordered.
+void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
+                            int metric, const unsigned long long *running, int ncand, int nout, float cmax,
+                            float err_scale, int32_t *out_ids, int *flag, hipStream_t s);
+
 // Canonical re-evaluation of cand[nq][ncand] (-1 = absent) and selection of the best nout.  Rows of
 // the outputs are out_stride (>= nout) wide; columns past nout are padded with (-1, +-FLT_MAX).
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,

@@ -549,6 +549,139 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
     }
 }
 
+// Exact selection of the best `nout` candidates as a SET, touching only the candidates that the
+// approximate scores cannot decide.  `running` holds, per query, ncand keys sorted by approximate
+// score s, each within err = err_scale * |q| * cmax of the canonical score e.  With T = s at rank
+// nout: a candidate with s < T - 2 err is certainly among the nout best (fewer than nout others have
+// s < T, and only those can have e below its e < T - err); one with s > T + 2 err certainly is not
+// (the nout candidates with s <= T all have e <= T + err).  Only the candidates in between are
+// re-evaluated in the canonical scalar arithmetic and ranked by (e, id); the best
+// nout - |certain| of them complete the set.  Centroids outside the list have s >= s_last, so the
+// set is proven complete when s_last > T + 2 err; otherwise *flag is raised and the caller must use
+// another plan.  One wavefront per query; out_ids gets nout ids in no particular order.
+template <bool VEC4>
+__global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__restrict__ Q, int64_t nq,
+                                                              const float *__restrict__ C, int d,
+                                                              const float *__restrict__ qn,
+                                                              const float *__restrict__ cn, int metric,
+                                                              const key_t *__restrict__ running, int ncand, int nout,
+                                                              float cmax, float err_scale,
+                                                              int32_t *__restrict__ out_ids, int *__restrict__ flag)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= nq) {
+        return;
+    }
+    key_t *ekeys = reinterpret_cast<key_t *>(smem_raw) + (size_t)wave * ncand;          // exact keys of the undecided
+    int32_t *amb = reinterpret_cast<int32_t *>(smem_raw + (size_t)4 * ncand * sizeof(key_t)) + (size_t)wave * ncand;
+    const key_t *run = running + row * ncand;
+    int32_t *out = out_ids + row * nout;
+    const key_t at_rank = run[nout - 1];
+    if (at_rank == kEmptyKey) {
+        // fewer than nout candidates exist at all: every one of them is in
+        for (int i = lane; i < nout; i += kWave) {
+            const key_t kk = run[i];
+            out[i] = kk == kEmptyKey ? -1 : (int32_t)key_index(kk);
+        }
+        return;
+    }
+    const float T = key_score(at_rank);
+    const float err = err_scale * sqrtf(qn[row]) * cmax;
+    const float lo = T - 2.0f * err, hi = T + 2.0f * err;
+    const key_t last = run[ncand - 1];
+    if (lane == 0 && last != kEmptyKey && !(key_score(last) > hi)) {
+        *flag = 1;
+    }
+    int n_in = 0, n_amb = 0;
+    for (int base = 0; base < ncand; base += kWave) {
+        const int i = base + lane;
+        const key_t kk = i < ncand ? run[i] : kEmptyKey;
+        const float sc = key_score(kk);
+        const bool valid = kk != kEmptyKey;
+        const bool in = valid && sc < lo;
+        const bool und = valid && !in && sc <= hi;
+        const unsigned long long m_in = __ballot(in), m_und = __ballot(und);
+        const int p_in = __builtin_amdgcn_mbcnt_hi((uint32_t)(m_in >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m_in, 0));
+        const int p_und =
+            __builtin_amdgcn_mbcnt_hi((uint32_t)(m_und >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m_und, 0));
+        if (in) {
+            out[n_in + p_in] = (int32_t)key_index(kk);
+        }
+        if (und) {
+            amb[n_amb + p_und] = (int32_t)key_index(kk);
+        }
+        n_in += __popcll(m_in);
+        n_amb += __popcll(m_und);
+    }
+    wave_lds_fence();
+    const float *q = Q + row * d;
+    for (int j = lane; j < n_amb; j += kWave) {
+        const int32_t c = amb[j];
+        const float *cv = C + (int64_t)c * d;
+        float g = 0.f;
+        if (VEC4) {
+#pragma unroll 8
+            for (int t = 0; t < d; t += 4) {
+                const float4 a = *reinterpret_cast<const float4 *>(q + t);
+                const float4 b = *reinterpret_cast<const float4 *>(cv + t);
+                g = __fadd_rn(g, __fmul_rn(a.x, b.x));
+                g = __fadd_rn(g, __fmul_rn(a.y, b.y));
+                g = __fadd_rn(g, __fmul_rn(a.z, b.z));
+                g = __fadd_rn(g, __fmul_rn(a.w, b.w));
+            }
+        } else {
+            for (int t = 0; t < d; t++) {
+                g = __fadd_rn(g, __fmul_rn(q[t], cv[t]));
+            }
+        }
+        float v;
+        if (metric == kMetricL2) {
+            v = __fadd_rn(qn[row], cn[c]);
+            v = __fsub_rn(v, g);
+            v = __fsub_rn(v, g);
+        } else {
+            v = -g;
+        }
+        ekeys[j] = make_key(v, (uint32_t)c);
+    }
+    wave_lds_fence();
+    const int need = nout - n_in;   // >= 1: the candidate at rank nout is itself undecided
+    for (int j = lane; j < n_amb; j += kWave) {
+        const key_t mine = ekeys[j];
+        int rank = 0;
+        for (int t = 0; t < n_amb; t++) {
+            rank += ekeys[t] < mine ? 1 : 0;
+        }
+        if (rank < need) {
+            out[n_in + rank] = (int32_t)key_index(mine);
+        }
+    }
+}
+
+void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
+                            int metric, const unsigned long long *running, int ncand, int nout, float cmax,
+                            float err_scale, int32_t *out_ids, int *flag, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    IXA_REQUIRE(ncand >= 1 && ncand <= 3072 && nout >= 1 && nout <= ncand, kErrInvalidParam,
+                "refine candidate count %d out of range [1, 3072]", ncand);
+    const size_t smem = (size_t)4 * ncand * (sizeof(key_t) + sizeof(int32_t));
+    const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    auto kern = vec4 ? refine_boundary_kernel<true> : refine_boundary_kernel<false>;
+    if (smem > 48 * 1024) {
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
+                       ncand, nout, cmax, err_scale, out_ids, flag);
+}
+
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,
                    const int32_t *cand, int ncand, int nout, int out_stride, int32_t *out_ids, float *out_dist,
                    hipStream_t s)

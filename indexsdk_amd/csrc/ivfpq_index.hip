@@ -235,7 +235,7 @@ void IvfpqIndex::get_trained(float *centroids, float *codebook) const
 // Stage 1 driver: MFMA scores into a bounded scratch, per-row selection of nout + slack candidates,
 // exact refine.  Never materialises more than scratch_bytes of the n x nlist score matrix.
 void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
-                               float *out_dist)
+                               float *out_dist, bool set_only)
 {
     if (n == 0) {
         return;
@@ -262,32 +262,46 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
             if (rc < 0) {
                 continue;  // shape not served by the bf16 kernel
             }
-            if (!dist) {
-                ws_exact_.resize((size_t)n * nout);
-                dist = ws_exact_.data();
+            // error of the approximate SCORE against the canonical one: 2 * (3 * 2^-16) |q||c| from the
+            // split for L2 (score = norms - 2 dot; half of that for inner product), doubled as a safety
+            // margin, plus the rounding of the canonical left-to-right sum itself, (d + 4) 2^-24 |q||c|
+            // per dot product
+            const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
+            const float err_scale = dots * (6.0f / 65536.0f + (float)(d_ + 4) * 5.9604645e-8f);
+            ws_flag_.resize(1);
+            IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+            if (set_only && !out_dist && ncand > nout) {
+                // search: only the SET of probed lists matters, so only the candidates the approximate
+                // scores cannot decide are re-evaluated
+                launch_refine_boundary(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
+                                       ws_running_.data(), ncand, nout, cmax_, err_scale, out_ids, ws_flag_.data(),
+                                       stream_);
+            } else {
+                if (!dist) {
+                    ws_exact_.resize((size_t)n * nout);
+                    dist = ws_exact_.data();
+                }
+                launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
+                launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
+                              ws_cand_.data(), ncand, nout, nout, out_ids, dist, stream_);
+                launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale,
+                                       select_metric, n, ws_flag_.data(), stream_);
             }
+            int32_t failed = 0;
+            ws_flag_.download(&failed, 1, stream_);
+            if (!failed) {
+                break;
+            }
+            continue;
         } else {
             stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
                               ncand, ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
         }
+        // fp32 plan: every candidate re-evaluated
         launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
         launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric, ws_cand_.data(),
                       ncand, nout, nout, out_ids, dist, stream_);
-        if (!approx) {
-            break;
-        }
-        // error of the approximate SCORE: 2 * (3 * 2^-16) |q||c| for L2 (score = norms - 2 dot), half of
-        // that for inner product; doubled again as a safety margin
-        const float err_scale = (select_metric == kMetricL2 ? 12.0f : 6.0f) / 65536.0f;
-        ws_flag_.resize(1);
-        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
-        launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale, select_metric,
-                               n, ws_flag_.data(), stream_);
-        int32_t failed = 0;
-        ws_flag_.download(&failed, 1, stream_);
-        if (!failed) {
-            break;
-        }
+        break;
     }
 }
 
@@ -612,7 +626,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     ws_counter_.resize(1);
 
     IXA_HIP(hipEventRecord(ev_[0], stream_));
-    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr);
+    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
 
     ScanParams p{};

@@ -312,3 +312,33 @@ def test_large_k_shared_pool_all_scores_tie(ix, oracle):
     assert gpu.last_search_stats()["shared_pool"] == 1
     Dr, Ir = ref.search(q, 1024, nlist)
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+
+
+@pytest.mark.parametrize("metric_name", ["L2", "IP"])
+def test_search_with_tied_and_nearly_tied_centroids(ix, oracle, metric_name):
+    """Half of the centroids are exact or 1e-6-perturbed copies of the other half, so the approximate
+    coarse scores cannot decide the rank-nprobe boundary: the probed SET must still be the oracle's
+    (equal scanned-code counts, equal results) and the probe lists bit-identical."""
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    rng = np.random.default_rng(51)
+    d, M, nlist, nprobe = 64, 16, 256, 16
+    base_c = rng.standard_normal((nlist // 2, d)).astype(np.float32)
+    twin = base_c.copy()
+    twin[::2] += (1e-6 * rng.standard_normal((nlist // 4, d))).astype(np.float32)     # odd rows stay exact copies
+    cent = np.ascontiguousarray(np.concatenate([base_c, twin])[rng.permutation(nlist)])
+    x = (cent[rng.integers(0, nlist, 30000)] + 0.3 * rng.standard_normal((30000, d))).astype(np.float32)
+    q = (cent[rng.integers(0, nlist, 300)] + 0.3 * rng.standard_normal((300, d))).astype(np.float32)
+    cb = oracle.train_pq(x[:4000], M, niter=3, seed=2)
+    ids = np.arange(30000, dtype=np.int64)
+    ref = oracle.CsrIndex.build(d, M, metric, cent, cb, x, ids)
+    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add_with_ids(x, ids)
+    gpu.setNumProbes(nprobe)
+    pi, pd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, metric)
+    assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
+    D, I = gpu.search(q, 20)
+    Dr, Ir = ref.search(q, 20, nprobe)
+    assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
