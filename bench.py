@@ -103,8 +103,8 @@ def run_flat_i8(args, torch, ix, _capi, lib):
         "config": {"workload": f"C4 Flat int8 {n}x{d} uniform[-127,127], nq={nq}, k={k}, exact int32 L2"},
         "roofline": {"bound": "mfma", "achieved": ops / (ms * 1e-3) / 1e12, "peak": 5000.0, "unit": "TOP/s",
                      "frac": ops / (ms * 1e-3) / 1e12 / 5000.0, "traffic": None,
-                     "kernel": "score_tile_i8_kernel + select_rows_kernel<int> (whole search; the score kernel's "
-                               "own share is in profiles/)", "device_ms": stats["ms_total"]},
+                     "kernel": "score_ring_kernel<int8> (unfiltered seed + bound-filtered launches) + selection kernels: "
+                               "the whole search; the ring kernel's own share is in profiles/", "device_ms": stats["ms_total"]},
     }
     if not args.no_cpu:
         from oracle import oracle as orc
@@ -232,7 +232,7 @@ def main():
     scan_ms_avg = float(np.mean(scan_ms))
     achieved = scan_bytes / (scan_ms_avg * 1e-3) / 1e9
     log(f"step {ms_per_step:.3f} ms (coarse {np.mean(coarse_ms):.3f} ms, scan {scan_ms_avg:.3f} ms), "
-        f"{qps:.0f} QPS, scan {achieved:.0f} GB/s")
+        f"{qps:.0f} QPS, scan {achieved:.0f} GB/s, coarse fp32 rerun {int(stats.get('coarse_reruns', 0))}")
 
     if args.copy_probe:
         src = torch.zeros(1 << 28, device="cuda", dtype=torch.float32)

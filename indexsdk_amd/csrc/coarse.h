@@ -56,7 +56,8 @@ void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_sid
 // Sets *flag = 1 if some query's approximate candidate list (running[nq][ncand], ascending keys) is
 // not provably a superset of its best nout centroids; see score_ring.hip.
 void launch_verify_superset(const unsigned long long *running, int ncand, const float *exact_dist, int nout,
-                            const float *qn, float cmax, float err_scale, int metric, int64_t nq, int *flag,
+                            const float *qn, float cmax, float err_scale, float round_scale, int metric, int64_t nq,
+                            int *flag,
                             hipStream_t s);
 
 // Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
@@ -74,7 +75,7 @@ void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, in
 // list cannot be proven to contain every winner.  out_ids: [nq][nout], unordered.
 void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                             int metric, const unsigned long long *running, int ncand, int nout, float cmax,
-                            float err_scale, int32_t *out_ids, int *flag, hipStream_t s);
+                            float err_scale, float round_scale, int32_t *out_ids, int *flag, hipStream_t s);
 
 // Canonical re-evaluation of cand[nq][ncand] (-1 = absent) and selection of the best nout.  Rows of
 // the outputs are out_stride (>= nout) wide; columns past nout are padded with (-1, +-FLT_MAX).

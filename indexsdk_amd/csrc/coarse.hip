@@ -551,7 +551,7 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
 
 // Exact selection of the best `nout` candidates as a SET, touching only the candidates that the
 // approximate scores cannot decide.  `running` holds, per query, ncand keys sorted by approximate
-// score s, each within err = err_scale * |q| * cmax of the canonical score e.  With T = s at rank
+// score s, each within err = err_scale * |q| * cmax + round_scale * (|q| + cmax)^2 of the canonical score e.  With T = s at rank
 // nout: a candidate with s < T - 2 err is certainly among the nout best (fewer than nout others have
 // s < T, and only those can have e below its e < T - err); one with s > T + 2 err certainly is not
 // (the nout candidates with s <= T all have e <= T + err).  Only the candidates in between are
@@ -565,7 +565,7 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
                                                               const float *__restrict__ qn,
                                                               const float *__restrict__ cn, int metric,
                                                               const key_t *__restrict__ running, int ncand, int nout,
-                                                              float cmax, float err_scale,
+                                                              float cmax, float err_scale, float round_scale,
                                                               int32_t *__restrict__ out_ids, int *__restrict__ flag)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -589,7 +589,8 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
         return;
     }
     const float T = key_score(at_rank);
-    const float err = err_scale * sqrtf(qn[row]) * cmax;
+    const float qlen = sqrtf(qn[row]);
+    const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
     const float lo = T - 2.0f * err, hi = T + 2.0f * err;
     const key_t last = run[ncand - 1];
     if (lane == 0 && last != kEmptyKey && !(key_score(last) > hi)) {
@@ -663,7 +664,7 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
 
 void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                             int metric, const unsigned long long *running, int ncand, int nout, float cmax,
-                            float err_scale, int32_t *out_ids, int *flag, hipStream_t s)
+                            float err_scale, float round_scale, int32_t *out_ids, int *flag, hipStream_t s)
 {
     if (nq == 0) {
         return;
@@ -679,7 +680,7 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
                                     (int)smem));
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
-                       ncand, nout, cmax, err_scale, out_ids, flag);
+                       ncand, nout, cmax, err_scale, round_scale, out_ids, flag);
 }
 
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,

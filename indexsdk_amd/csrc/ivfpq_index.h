@@ -35,6 +35,7 @@ struct SearchStats {
     double nsplit = 0;
     double scan_waves = 0;
     double shared_pool = 0;
+    double coarse_reruns = 0;
 };
 
 class IvfpqIndex {
@@ -98,6 +99,7 @@ private:
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
     DeviceBuffer<int32_t> ws_flag_;
+    int last_coarse_reruns_ = 0;
     float cmax_ = 0.f;                                      // largest centroid norm
     int dp_ = 0;                                            // d rounded up to a multiple of 32
     // arena

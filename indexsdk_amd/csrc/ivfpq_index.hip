@@ -242,8 +242,7 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     }
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
-    // Candidate generation.  Fast plan: bf16 x 3 matrix products (|error| <= 3 * 2^-16 |q||c| on the
-    // dot product) with 16 spare candidates; the candidates are re-evaluated exactly, and a check
+    // Candidate generation.  Fast plan: bf16 x 3 matrix products (error bound below) with 16 spare candidates; the candidates are re-evaluated exactly, and a check
     // proves that nothing outside them can reach the nout-th exact score.  If the check fails for
     // any query (near-tied centroids), the fp32 plan below recomputes the whole call.
     for (int attempt = cfg_.coarse_bf16 ? 0 : 1; attempt < 2; attempt++) {
@@ -262,19 +261,26 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
             if (rc < 0) {
                 continue;  // shape not served by the bf16 kernel
             }
-            // error of the approximate SCORE against the canonical one: 2 * (3 * 2^-16) |q||c| from the
-            // split for L2 (score = norms - 2 dot; half of that for inner product), doubled as a safety
-            // margin, plus the rounding of the canonical left-to-right sum itself, (d + 4) 2^-24 |q||c|
-            // per dot product
+            // Bound on |approximate score - canonical score|, per unit of |q||c|, for one dot product:
+            //   split: x = hi + lo + r with |lo| <= 2^-9 |x|, |r| <= 2^-18 |x|, so the three products kept
+            //          miss lo.lo + r.y + x.r, at most 3 * 2^-18 sum |x_i y_i| <= 3 * 2^-18 |q||c|;
+            //   sums:  bf16 x bf16 products are exact in fp32; accumulating K = 3 dp of them in any order
+            //          errs by at most K 2^-24 sum |terms|, the canonical left-to-right sum by d 2^-24
+            //          sum |x_i y_i| (a few units added for the second-order terms).
+            // L2 scores hold two dot products and three further roundings of numbers no larger than
+            // (|q| + |c|)^2, the same on both sides up to one unit each.
             const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
-            const float err_scale = dots * (6.0f / 65536.0f + (float)(d_ + 4) * 5.9604645e-8f);
+            const float u = 5.9604645e-8f;
+            const float err_scale = dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * u);
+            const float round_scale = select_metric == kMetricL2 ? 4.0f * u : 0.0f;
             ws_flag_.resize(1);
             IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
             if (set_only && !out_dist && ncand > nout) {
                 // search: only the SET of probed lists matters, so only the candidates the approximate
                 // scores cannot decide are re-evaluated
                 launch_refine_boundary(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
-                                       ws_running_.data(), ncand, nout, cmax_, err_scale, out_ids, ws_flag_.data(),
+                                       ws_running_.data(), ncand, nout, cmax_, err_scale, round_scale, out_ids,
+                                       ws_flag_.data(),
                                        stream_);
             } else {
                 if (!dist) {
@@ -285,13 +291,14 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
                 launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
                               ws_cand_.data(), ncand, nout, nout, out_ids, dist, stream_);
                 launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale,
-                                       select_metric, n, ws_flag_.data(), stream_);
+                                       round_scale, select_metric, n, ws_flag_.data(), stream_);
             }
             int32_t failed = 0;
             ws_flag_.download(&failed, 1, stream_);
             if (!failed) {
                 break;
             }
+            last_coarse_reruns_ = 1;
             continue;
         } else {
             stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
@@ -626,7 +633,9 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     ws_counter_.resize(1);
 
     IXA_HIP(hipEventRecord(ev_[0], stream_));
+    last_coarse_reruns_ = 0;
     coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true);
+    stats_.coarse_reruns = last_coarse_reruns_;
     IXA_HIP(hipEventRecord(ev_[1], stream_));
 
     ScanParams p{};

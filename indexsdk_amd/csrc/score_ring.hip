@@ -590,10 +590,11 @@ bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, in
 }
 
 // ---- bf16 x 3 split --------------------------------------------------------------------------------
-// x = hi + lo + rest with hi = bf16(x), lo = bf16(x - hi), |rest| <= 2^-16 |x|.  A dot product over
-// the concatenated rows  [hi | hi | lo] . [hi | lo | hi]  = hi.hi + hi.lo + lo.hi  differs from the
-// exact one by at most about 3 * 2^-16 * sum |x_i y_i|, at three bf16 MFMAs (16x the fp32 matrix
-// rate each) per fp32 product.  Rows are zero-padded to dp (a multiple of 32) per segment.
+// x = hi + lo + rest with hi = bf16(x), lo = bf16(x - hi) (both round-to-nearest-even), so
+// |lo| <= 2^-9 |x| and |rest| <= 2^-18 |x|.  A dot product over the concatenated rows
+// [hi | hi | lo] . [hi | lo | hi]  = hi.hi + hi.lo + lo.hi  misses lo.lo + rest.y + x.rest, at most
+// 3 * 2^-18 * sum |x_i y_i|, at three bf16 MFMAs (16x the fp32 matrix rate each) per fp32 product.
+// Rows are zero-padded to dp (a multiple of 32) per segment.
 __device__ __forceinline__ uint16_t bf16_rne(float v)
 {
     uint32_t u = __float_as_uint(v);
@@ -630,11 +631,12 @@ void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_sid
 
 // Raises *flag unless, for every query, no centroid outside its approximate candidate list can beat
 // its nout-th exact score: (approximate score of the last candidate) - err > (nout-th exact score),
-// err = err_scale * |q| * max|c|.  Rows whose candidate list is not full hold every centroid.
+// err = err_scale * |q| * max|c| + round_scale * (|q| + max|c|)^2.  Rows whose candidate list is not full hold every centroid.
 __global__ __launch_bounds__(256) void verify_superset_kernel(const key_t *__restrict__ running, int ncand,
                                                               const float *__restrict__ exact_dist, int nout,
                                                               const float *__restrict__ qn, float cmax, float err_scale,
-                                                              int metric, int64_t nq, int *__restrict__ flag)
+                                                              float round_scale, int metric, int64_t nq,
+                                                              int *__restrict__ flag)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= nq) {
@@ -647,19 +649,20 @@ __global__ __launch_bounds__(256) void verify_superset_kernel(const key_t *__res
     const float a_last = key_score(last);
     const float d_out = exact_dist[i * nout + (nout - 1)];
     const float s_star = metric == kMetricL2 ? d_out : -d_out;
-    const float err = err_scale * sqrtf(qn[i]) * cmax;
+    const float qlen = sqrtf(qn[i]);
+    const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
     if (!(a_last - err > s_star)) {
         *flag = 1;
     }
 }
 
 void launch_verify_superset(const unsigned long long *running, int ncand, const float *exact_dist, int nout,
-                            const float *qn, float cmax, float err_scale, int metric, int64_t nq, int *flag,
-                            hipStream_t s)
+                            const float *qn, float cmax, float err_scale, float round_scale, int metric, int64_t nq,
+                            int *flag, hipStream_t s)
 {
     if (nq > 0) {
         hipLaunchKernelGGL(verify_superset_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, running, ncand,
-                           exact_dist, nout, qn, cmax, err_scale, metric, nq, flag);
+                           exact_dist, nout, qn, cmax, err_scale, round_scale, metric, nq, flag);
     }
 }
 
