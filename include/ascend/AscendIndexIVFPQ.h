@@ -154,6 +154,26 @@ public:
         ixaThrowIfError(ivfpq_add_codes(h_, listId, (int64_t)n, codes, reinterpret_cast<const int64_t *>(ids)));
         syncTotal();
     }
+    // File form of copyTo / copyFrom(faiss::IndexIVFPQ *): the byte layout of faiss::write_index for an
+    // IndexIVFPQ with by_residual = false.  readFaiss replaces this object's index; the file must have the
+    // dims, metric, nlist and msubs this object was constructed with.
+    void writeFaiss(const char *path) const { ixaThrowIfError(ivfpq_write_faiss(h_, path)); }
+    void readFaiss(const char *path)
+    {
+        ivfpq_index_t *loaded = nullptr;
+        ixaThrowIfError(ivfpq_read_faiss(path, nullptr, &loaded));
+        int fd = 0, fm = 0, fM = 0;
+        int64_t fl = 0;
+        ivfpq_get_shape(loaded, &fd, &fm, &fl, &fM);
+        if (fd != d || fm != (int)metric_type || fl != nlist_ || fM != msubs_) {
+            ivfpq_destroy(loaded);
+            throw FaissException("the file's dims / metric / nlist / msubs differ from this index");
+        }
+        ivfpq_destroy(h_);
+        h_ = loaded;
+        is_trained = true;
+        syncTotal();
+    }
     ivfpq_index_t *handle() const { return h_; }
 
 protected:

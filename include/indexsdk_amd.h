@@ -102,6 +102,17 @@ int ivfpq_set_trained(ivfpq_index_t *h, const float *centroids, const float *cod
 int ivfpq_get_trained(const ivfpq_index_t *h, float *centroids, float *codebook);
 int ivfpq_is_trained(const ivfpq_index_t *h, int *out);
 
+/* File form of copyTo / copyFrom(faiss::IndexIVFPQ*) (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:392-508): the
+ * index is written / read in the byte layout of faiss::write_index for an IndexIVFPQ with an IndexFlat
+ * coarse quantizer, by_residual = false and ArrayInvertedLists (fourcc "IwPQ"), so that faiss::read_index
+ * on the CPU side opens the file and files written by faiss::write_index load here.  Reading rejects
+ * by_residual = true (the reference accepts it silently and returns wrong distances).  cfg may be NULL. */
+int ivfpq_write_faiss(const ivfpq_index_t *h, const char *path);
+int ivfpq_read_faiss(const char *path, const ivfpq_config_t *cfg, ivfpq_index_t **out);
+/* Shape of an index (the public members d, metric_type, nlist and pq.M of the reference class); any output
+ * may be NULL. */
+int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int64_t *nlist, int *msubs);
+
 /* AscendIndex::add / add_with_ids  FR/ascend/AscendIndex.h:66-71, AscendIndexIVFPQImpl.cpp:694-864.
  * ids == NULL numbers the vectors ntotal, ntotal+1, ... */
 int ivfpq_add_with_ids(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids);

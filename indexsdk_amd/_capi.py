@@ -68,6 +68,10 @@ _SIGNATURES = {
                                            ctypes.c_void_p]),
     "ivfpq_assign": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_coarse_probe": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_write_faiss": (ctypes.c_int, [_H, ctypes.c_char_p]),
+    "ivfpq_read_faiss": (ctypes.c_int, [ctypes.c_char_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]),
+    "ivfpq_get_shape": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                       ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int)]),
     "ivfpq_encode": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_list_length": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
     "ivfpq_get_list": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),

@@ -59,6 +59,25 @@ class AscendIndexIVFPQ:
             self._lib.ivfpq_destroy(h)
             self._h = None
 
+    # ---- interchange with faiss (file form of copyTo / copyFrom, AscendIndexIVFPQImpl.cpp:392-508) --
+    def write_faiss(self, path):
+        """Writes the index in faiss.write_index's layout for an IndexIVFPQ (by_residual = False)."""
+        _capi.check(self._lib.ivfpq_write_faiss(self._h, str(path).encode()))
+
+    @classmethod
+    def read_faiss(cls, path, config=None):
+        """Loads a file written by write_faiss or by faiss.write_index(IndexIVFPQ with by_residual = False)."""
+        self = cls.__new__(cls)
+        self._lib = _capi.load()
+        self._h = ctypes.c_void_p()
+        cfg = ctypes.byref(config._c) if config is not None else None
+        _capi.check(self._lib.ivfpq_read_faiss(str(path).encode(), cfg, ctypes.byref(self._h)))
+        d, metric, nlist, m = ctypes.c_int(), ctypes.c_int(), ctypes.c_int64(), ctypes.c_int()
+        _capi.check(self._lib.ivfpq_get_shape(self._h, ctypes.byref(d), ctypes.byref(metric), ctypes.byref(nlist),
+                                              ctypes.byref(m)))
+        self.d, self.metric_type, self.nlist, self.msubs, self.nbits = d.value, metric.value, nlist.value, m.value, 8
+        return self
+
     # ---- training -----------------------------------------------------------------------------
     @property
     def is_trained(self):

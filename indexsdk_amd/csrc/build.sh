@@ -13,8 +13,10 @@ for src in coarse.hip score_ring.hip pq.hip scan.hip flat.hip stream_select.hip 
   ( /opt/rocm/bin/hipcc "${FLAGS[@]}" -c "${HERE}/${src}" -o "${OBJ}/${src%.hip}.o" 2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) ) &
   pids+=($!)
 done
-( /opt/rocm/bin/hipcc "${FLAGS[@]}" -x hip -c "${HERE}/capi.cpp" -o "${OBJ}/capi.o" 2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) ) &
-pids+=($!)
+for src in capi.cpp faiss_io.cpp; do
+  ( /opt/rocm/bin/hipcc "${FLAGS[@]}" -x hip -c "${HERE}/${src}" -o "${OBJ}/${src%.cpp}.o" 2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) ) &
+  pids+=($!)
+done
 for p in "${pids[@]}"; do wait "$p"; done
 /opt/rocm/bin/hipcc --offload-arch=gfx950 -shared -fPIC -o "${OUT}" "${OBJ}"/*.o
 echo "built ${OUT}"

@@ -4,18 +4,27 @@
 
 #include <algorithm>
 #include <cstring>
+#include <memory>
 #include <new>
 #include <string>
 
 #include "flat_index.h"
 #include "ivfpq_index.h"
 
+namespace ixa {
+void write_faiss_ivfpq(const IvfpqIndex &idx, const char *path);
+std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig &cfg);
+}  // namespace ixa
+
+// The handle owns the index through a pointer so that a loader can hand over a finished one.
 struct ivfpq_index {
-    ixa::IvfpqIndex impl;
+    std::unique_ptr<ixa::IvfpqIndex> owned;
+    ixa::IvfpqIndex &impl;
     ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
-        : impl(d, metric, nlist, M, nbits, c)
+        : owned(new ixa::IvfpqIndex(d, metric, nlist, M, nbits, c)), impl(*owned)
     {
     }
+    explicit ivfpq_index(std::unique_ptr<ixa::IvfpqIndex> p) : owned(std::move(p)), impl(*owned) {}
 };
 
 struct flat_index {
@@ -51,6 +60,28 @@ int guarded(F &&f)
 
 #define IXA_HANDLE(h) IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.")
 
+ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
+{
+    ixa::IvfpqConfig c;
+    if (cfg) {
+        IXA_REQUIRE(cfg->niter >= 0 && cfg->train_samples_per_list >= 1 && cfg->max_train_samples >= 1 &&
+                        cfg->scratch_bytes >= (1 << 20) && cfg->code_layout >= -1 && cfg->code_layout <= 1,
+                    ixa::kErrInvalidParam, "invalid ivfpq_config_t field");
+        c.niter = cfg->niter;
+        c.pq_niter = cfg->pq_niter;
+        c.spherical = cfg->spherical;
+        c.train_samples_per_list = cfg->train_samples_per_list;
+        c.max_train_samples = cfg->max_train_samples;
+        c.lut_fp16 = cfg->lut_fp16;
+        c.code_layout = cfg->code_layout;
+        c.scratch_bytes = cfg->scratch_bytes;
+        c.seed = cfg->seed;
+        c.strict_reference_params = cfg->strict_reference_params;
+        c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
+    }
+    return c;
+}
+
 }  // namespace
 
 extern "C" {
@@ -85,24 +116,43 @@ IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbi
     return guarded([&] {
         IXA_REQUIRE(out != nullptr, ixa::kErrInvalidParam, "out can not be nullptr.");
         *out = nullptr;
-        ixa::IvfpqConfig c;
-        if (cfg) {
-            IXA_REQUIRE(cfg->niter >= 0 && cfg->train_samples_per_list >= 1 && cfg->max_train_samples >= 1 &&
-                            cfg->scratch_bytes >= (1 << 20) && cfg->code_layout >= -1 && cfg->code_layout <= 1,
-                        ixa::kErrInvalidParam, "invalid ivfpq_config_t field");
-            c.niter = cfg->niter;
-            c.pq_niter = cfg->pq_niter;
-            c.spherical = cfg->spherical;
-            c.train_samples_per_list = cfg->train_samples_per_list;
-            c.max_train_samples = cfg->max_train_samples;
-            c.lut_fp16 = cfg->lut_fp16;
-            c.code_layout = cfg->code_layout;
-            c.scratch_bytes = cfg->scratch_bytes;
-            c.seed = cfg->seed;
-            c.strict_reference_params = cfg->strict_reference_params;
-            c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
-        }
+        const ixa::IvfpqConfig c = to_config(cfg);
         *out = new ivfpq_index(d, metric, nlist, msubs, nbits, c);
+    });
+}
+
+IXA_EXPORT int ivfpq_write_faiss(const ivfpq_index_t *h, const char *path)
+{
+    return guarded([&] { IXA_HANDLE(h); ixa::write_faiss_ivfpq(h->impl, path); });
+}
+
+IXA_EXPORT int ivfpq_read_faiss(const char *path, const ivfpq_config_t *cfg, ivfpq_index_t **out)
+{
+    return guarded([&] {
+        IXA_REQUIRE(out != nullptr, ixa::kErrInvalidParam, "out can not be nullptr.");
+        *out = nullptr;
+        ixa::IvfpqConfig c = to_config(cfg);
+        c.strict_reference_params = 0;   // the file decides the shape
+        *out = new ivfpq_index(ixa::read_faiss_ivfpq(path, c));
+    });
+}
+
+IXA_EXPORT int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int64_t *nlist, int *msubs)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        if (d) {
+            *d = h->impl.d();
+        }
+        if (metric) {
+            *metric = h->impl.metric();
+        }
+        if (nlist) {
+            *nlist = h->impl.nlist();
+        }
+        if (msubs) {
+            *msubs = h->impl.M();
+        }
     });
 }
 

@@ -62,6 +62,8 @@ public:
     void get_trained(float *centroids, float *codebook) const;          // host pointers, either may be null
     void add(int64_t n, const float *x, const int64_t *ids, bool on_device);
     void add_codes(int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids);  // host pointers
+    // n codes for arbitrary lists in one arena rebuild; list order inside a list = input order (host pointers)
+    void add_codes_bulk(int64_t n, const int32_t *list_no, const uint8_t *codes, const int64_t *ids);
     void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
     void assign(int64_t n, const float *x, int64_t *out, bool on_device);               // out: host
     void coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device);  // out: host

@@ -432,6 +432,22 @@ void IvfpqIndex::add_codes(int64_t list, int64_t n, const uint8_t *codes, const 
     append(n, list_no.data(), cd.data(), idd.data());
 }
 
+void IvfpqIndex::add_codes_bulk(int64_t n, const int32_t *list_no, const uint8_t *codes, const int64_t *ids)
+{
+    check_trained();
+    IXA_REQUIRE(n >= 0 && (n == 0 || (list_no && codes && ids)), kErrInvalidParam, "codes and ids can not be nullptr.");
+    if (n == 0) {
+        return;
+    }
+    DeviceBuffer<int32_t> ln;
+    DeviceBuffer<uint8_t> cd;
+    DeviceBuffer<int64_t> idd;
+    ln.upload(list_no, (size_t)n, stream_);
+    cd.upload(codes, (size_t)n * M_, stream_);
+    idd.upload(ids, (size_t)n, stream_);
+    append(n, ln.data(), cd.data(), idd.data());
+}
+
 void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev)
 {
     std::vector<int32_t> list_no((size_t)n), pos((size_t)n);

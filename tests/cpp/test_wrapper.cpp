@@ -71,6 +71,27 @@ int main(int argc, char **argv)
             total += index.getListLength(l);
         }
         EXPECT(total == (size_t)n);
+        // file form of copyTo / copyFrom: a second object loads what the first wrote
+        const std::string path = std::string(argc > 2 ? argv[2] : "/tmp") + "/wrapper_test.faissindex";
+        index.writeFaiss(path.c_str());
+        AscendIndexIVFPQ other(d, faiss::METRIC_L2, nlist, M, 8, conf);
+        other.readFaiss(path.c_str());
+        EXPECT(other.is_trained && other.ntotal == n && other.getNumProbes() == 32);
+        std::vector<float> D2((size_t)nq * k);
+        std::vector<faiss::idx_t> I2((size_t)nq * k);
+        other.search(nq, x.data(), k, D2.data(), I2.data());
+        EXPECT(I2 == I && D2 == D);
+        std::remove(path.c_str());
+        AscendIndexIVFPQ wrong(d, faiss::METRIC_L2, 2048, M, 8, conf);
+        bool threw = false;
+        try {
+            index.writeFaiss(path.c_str());
+            wrong.readFaiss(path.c_str());
+        } catch (const faiss::FaissException &) {
+            threw = true;
+        }
+        EXPECT(threw);
+        std::remove(path.c_str());
         AscendIndexFlatL2 flat(d);
         flat.add(n, x.data());
         flat.search(nq, x.data(), k, D.data(), I.data());

@@ -22,9 +22,9 @@ def test_wrapper_constructor_messages_host_only():
 
 
 @pytest.mark.gpu
-def test_wrapper_train_add_search_on_gpu():
+def test_wrapper_train_add_search_on_gpu(tmp_path):
     if not os.path.exists(BIN):
         pytest.skip("tests/cpp/test_wrapper has not been built (run __graft_entry__.build())")
-    out = subprocess.run([BIN, "gpu"], capture_output=True, text=True, timeout=300)
+    out = subprocess.run([BIN, "gpu", str(tmp_path)], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "wrapper test ok" in out.stdout
