@@ -3,23 +3,29 @@
 // A K-step of MFMAs lasts a few hundred (int8) to a few thousand (fp32) cycles, and a tile of the
 // headline shapes has only 8 K-steps, so a kernel that starts and drains a pipeline per tile spends
 // a large share of its time waiting for the first operands.  Here instead
-//   * a workgroup is persistent and walks a list of 256 x 128 tiles; the stream of K-steps (64 bytes
-//     of every operand row each) runs continuously across tile boundaries;
+//   * a workgroup of 8 wavefronts is persistent (one per CU) and walks a list of 256 x 256 tiles; the
+//     stream of K-steps (64 bytes of every operand row each) runs continuously across tile
+//     boundaries.  The square tile stages 512 rows for 65536 products per K-element: the L2 -> LDS
+//     traffic, which bounds the int8 and bf16 variants, is 2/3 of what a 256 x 128 tile needs;
 //   * operands go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
-//     into a ring of kStages buffers, kStages - 1 steps ahead of the MFMAs; completion is tracked
-//     with s_waitcnt vmcnt + s_barrier, without the full memory fence of __syncthreads();
+//     into a ring of kRingStages buffers, two to three steps ahead of the MFMAs; completion is
+//     tracked with s_waitcnt vmcnt + s_barrier, without the full memory fence of __syncthreads();
 //   * each wavefront owns 128 x 64 of the tile (4 x 2 blocks of 32 x 32), so one operand fragment
 //     read from LDS feeds 1.33 MFMA blocks on average;
+//   * a K-step is consumed as two half-steps with two fragment register sets: the LDS reads of the
+//     next half-step are issued before the MFMAs of the current one, and the once-per-step barrier
+//     sits between the two half-steps of a stage, so no wave ever waits for LDS in front of idle
+//     matrix cores;
 //   * rows are stored unpadded (64 bytes per row and step); the 16-byte chunk index is XOR-swizzled
 //     with bits 2-3 of the row, which makes the 128-bit fragment reads of 16 consecutive rows hit
 //     16 different bank groups;
 //   * tiles are dealt so that all workgroups of an XCD work on the same base tile at the same time
-//     (it is fetched from HBM once and re-used out of that XCD's L2);
-//   * two workgroups share a CU, so one's epilogue overlaps the other's MFMAs.
+//     (it is fetched from HBM once and re-used out of that XCD's L2).
 // Scores: int8 -> exact int32 |q|^2 + |b|^2 - 2 q.b (v_mfma_i32_32x32x32_i8);
+//         bf16 -> fp32 accumulation (v_mfma_f32_32x32x16_bf16);
 //         fp32 -> (|q|^2 + |b|^2) - g - g or -g (v_mfma_f32_32x32x2_f32).
-// The sum over k is order-free for integers, and for fp32 any fixed k-assignment that is the same
-// for both operands is a valid accumulation order, so each lane half owns half of a K-step.
+// The sum over k is order-free for integers, and for floating point any fixed k-assignment that is
+// the same for both operands is a valid accumulation order, so each lane half owns half of a K-step.
 #include "coarse.h"
 #include "topk.h"
 
@@ -33,44 +39,64 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kRingTM = 256, kRingTN = 128, kRingRows = kRingTM + kRingTN;
+constexpr int kRingWaves = 8;
+constexpr int kRingTM = 256, kRingTN = 256, kRingRows = kRingTM + kRingTN;
 constexpr int kRingStageBytes = kRingRows * 64;
 constexpr int kRingStages = 3;
 constexpr int kRingAuxBytes = 1280;   // per-wave staging of a filtered epilogue's operands
-constexpr int kRingLoadsPerWave = kRingRows / 16 / 4;  // wave-wide 1 KB loads per stage and wavefront
+constexpr int kRingLoadsPerWave = kRingRows / 16 / kRingWaves;  // wave-wide 1 KB loads per stage and wavefront
+
+// Operand fragments of one half-step: 4 query blocks and 2 base blocks of 32 rows, 16 bytes per lane.
+template <typename V>
+struct RingFrag {
+    V a[4], b[2];
+};
+
+// The fragment reads and the waits for them are written as inline assembly: the compiler would wait
+// for ALL outstanding LDS reads before the first MFMA of a half-step (it merges the counter states
+// of the loop's paths conservatively), which serialises the reads of the next half-step with the
+// MFMAs of the current one.  LDS reads complete in order, so "at most 6 outstanding" after issuing
+// the 6 reads of the next fragment set means the previous set has arrived.  Scalar loads share the
+// counter but can only make the wait stricter than needed, never weaker.
+// a_addr / b_addr: LDS byte address of this lane's chunk in the first query / base block of the stage.
+template <typename V>
+__device__ __forceinline__ void ring_read_frag(uint32_t a_addr, uint32_t b_addr, RingFrag<V> &f)
+{
+    asm volatile("ds_read_b128 %0, %1" : "=v"(f.a[0]) : "v"(a_addr));
+    asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(f.a[1]) : "v"(a_addr));
+    asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(f.a[2]) : "v"(a_addr));
+    asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(f.a[3]) : "v"(a_addr));
+    asm volatile("ds_read_b128 %0, %1" : "=v"(f.b[0]) : "v"(b_addr));
+    asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(f.b[1]) : "v"(b_addr));
+}
+// Waits until at most N LDS operations are outstanding; the fragment registers pass through the
+// statement so that no use of them can be scheduled ahead of it.
+template <int N, typename V>
+__device__ __forceinline__ void ring_wait_frag(RingFrag<V> &f)
+{
+    asm volatile("s_waitcnt lgkmcnt(%6)"
+                 : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1])
+                 : "n"(N));
+}
 
 struct I8Traits {
     using T = int8_t;
     using S = int32_t;
     using Acc = v16i;
+    using Frag = RingFrag<v4i>;
     static constexpr int kElemsPerStep = 64;
-    // one K-step = 2 sub-steps of 32 bytes; a lane half owns 16 of them
+    // half-step hs = 32 bytes of the K-step; a lane half owns 16 of them
+    static __device__ __forceinline__ int chunk(int hs, int half) { return hs * 2 + half; }
     template <bool SWAP, bool ZERO>
-    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
-                                               Acc (&acc)[4][2])
+    static __device__ __forceinline__ void mma(const Frag &f, Acc (&acc)[4][2])
     {
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            const int c = kk * 2 + half;
-            v4i a[4], b[2];
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-                const int r = wr * 128 + ra * 32 + l32;
-                a[ra] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
+        for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
-                const int r = kRingTM + wc * 64 + rb * 32 + l32;
-                b[rb] = *reinterpret_cast<const v4i *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-#pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-                    const Acc c0 = (ZERO && kk == 0) ? Acc{} : acc[ra][rb];   // a tile's first product starts from zero
-                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[rb], a[ra], c0, 0, 0, 0)
-                                       : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra], b[rb], c0, 0, 0, 0);
-                }
+                const Acc c0 = ZERO ? Acc{} : acc[ra][rb];   // a tile's first product starts from zero
+                acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[rb], f.a[ra], c0, 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[ra], f.b[rb], c0, 0, 0, 0);
             }
         }
     }
@@ -81,33 +107,19 @@ struct Bf16Traits {
     using T = uint16_t;
     using S = float;
     using Acc = v16f;
+    using Frag = RingFrag<bf16x8>;
     static constexpr int kElemsPerStep = 32;
+    static __device__ __forceinline__ int chunk(int hs, int half) { return hs * 2 + half; }
     template <bool SWAP, bool ZERO>
-    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
-                                               Acc (&acc)[4][2])
+    static __device__ __forceinline__ void mma(const Frag &f, Acc (&acc)[4][2])
     {
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-            const int c = kk * 2 + half;
-            bf16x8 a[4], b[2];
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-                const int r = wr * 128 + ra * 32 + l32;
-                a[ra] = *reinterpret_cast<const bf16x8 *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
+        for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
-                const int r = kRingTM + wc * 64 + rb * 32 + l32;
-                b[rb] = *reinterpret_cast<const bf16x8 *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-#pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-                    const Acc c0 = (ZERO && kk == 0) ? Acc{} : acc[ra][rb];
-                    acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[rb], a[ra], c0, 0, 0, 0)
-                                       : __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ra], b[rb], c0, 0, 0, 0);
-                }
+                const Acc c0 = ZERO ? Acc{} : acc[ra][rb];
+                acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[rb], f.a[ra], c0, 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ra], f.b[rb], c0, 0, 0, 0);
             }
         }
     }
@@ -117,35 +129,21 @@ struct F32Traits {
     using T = float;
     using S = float;
     using Acc = v16f;
+    using Frag = RingFrag<v4f>;
     static constexpr int kElemsPerStep = 16;
-    // one K-step = 16 floats; a lane half owns 8 of them (two 16-byte chunks) and feeds them to 8
-    // consecutive 32x32x2 MFMAs
+    // one K-step = 16 floats; a lane half owns 8 of them (two 16-byte chunks), one chunk per half-step,
+    // fed to 4 consecutive 32x32x2 MFMAs
+    static __device__ __forceinline__ int chunk(int hs, int half) { return half * 2 + hs; }
     template <bool SWAP, bool ZERO>
-    static __device__ __forceinline__ void mma(const unsigned char *stage, int wr, int wc, int l32, int half,
-                                               Acc (&acc)[4][2])
+    static __device__ __forceinline__ void mma(const Frag &f, Acc (&acc)[4][2])
     {
-        v4f a[4][2], b[2][2];
 #pragma unroll
-        for (int cc = 0; cc < 2; cc++) {
-            const int c = half * 2 + cc;
-#pragma unroll
-            for (int ra = 0; ra < 4; ra++) {
-                const int r = wr * 128 + ra * 32 + l32;
-                a[ra][cc] = *reinterpret_cast<const v4f *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
-                const int r = kRingTM + wc * 64 + rb * 32 + l32;
-                b[rb][cc] = *reinterpret_cast<const v4f *>(stage + r * 64 + ((c ^ ((r >> 2) & 3)) << 4));
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
+        for (int t = 0; t < 4; t++) {
 #pragma unroll
             for (int ra = 0; ra < 4; ra++) {
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
-                    const float av = a[ra][t >> 2][t & 3], bv = b[rb][t >> 2][t & 3];
+                    const float av = f.a[ra][t], bv = f.b[rb][t];
                     const Acc c0 = (ZERO && t == 0) ? Acc{} : acc[ra][rb];
                     acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_f32_32x32x2f32(bv, av, c0, 0, 0, 0)
                                        : __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, c0, 0, 0, 0);
@@ -155,8 +153,15 @@ struct F32Traits {
     }
 };
 
+// s_waitcnt immediate that waits until at most n vector-memory operations are outstanding and
+// leaves the other counters alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+__host__ __device__ constexpr int ring_vmcnt(int n)
+{
+    return 0x0f70 | ((n > 63 ? 63 : n) & 15) | (((n > 63 ? 63 : n) >> 4) << 14);
+}
+
 template <typename Tr, bool FILTER>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void score_ring_kernel(
+__global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void score_ring_kernel(
     const typename Tr::T *__restrict__ Q, int64_t nq, const typename Tr::T *__restrict__ B, int64_t nb, int d,
     const typename Tr::S *__restrict__ qn, const typename Tr::S *__restrict__ bn, int metric,
     typename Tr::S *__restrict__ out, int64_t ldo, int tiles_m, int tiles_n, ScoreFilter<typename Tr::S> flt)
@@ -167,7 +172,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     extern __shared__ __align__(16) unsigned char ring[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wr = wave >> 1, wc = wave & 1;
+    const int wr = wave >> 2, wc = wave & 3;
     const int half = lane >> 5, l32 = lane & 31;
     const int nk = d / Tr::kElemsPerStep;
     const int64_t row_bytes = (int64_t)d * sizeof(T);
@@ -190,40 +195,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const unsigned char *Qb = reinterpret_cast<const unsigned char *>(Q);
     const unsigned char *Bb = reinterpret_cast<const unsigned char *>(B);
 
-    // Per-lane source pointers of the tile whose K-steps are being issued (recomputed once per
-    // tile); a K-step then only adds ks * 64 bytes.
-    const unsigned char *src[kRingLoadsPerWave];
+    // Sources of the tile whose K-steps are being issued.  Waves 0..3 load the query rows, waves 4..7
+    // the base rows: a wave-uniform tile base plus a 32-bit per-lane byte offset per load (recomputed
+    // once per tile; rows past the end of the operand re-read its last row); a K-step then only
+    // advances the uniform base by ks * 64 bytes.
+    const bool loads_q = wave < kRingTM / 16 / kRingLoadsPerWave;
+    const unsigned char *tile_base = nullptr;
+    uint32_t src_off[kRingLoadsPerWave];
     auto set_sources = [&](int it) {
         int64_t tm, tn;
         item_tile(it, tm, tn);
+        const int64_t row0 = loads_q ? tm * kRingTM : tn * kRingTN;
+        const int64_t last = (loads_q ? nq : nb) - 1 - row0;     // >= 0: the tile exists
+        const int limit = (int)(last < kRingTM - 1 ? last : kRingTM - 1);
+        tile_base = (loads_q ? Qb : Bb) + row0 * row_bytes;
 #pragma unroll
         for (int j = 0; j < kRingLoadsPerWave; j++) {
             const int rg = wave * kRingLoadsPerWave + j;          // group of 16 stage rows
-            const int row = rg * 16 + (lane >> 2);                // stage row: 0..255 queries, 256..383 base
+            const int row = rg * 16 + (lane >> 2);                // stage row: 0..255 queries, 256..511 base
             const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-            if (rg < kRingTM / 16) {
-                int64_t r = tm * kRingTM + row;
-                r = r < nq ? r : nq - 1;
-                src[j] = Qb + r * row_bytes + chunk * 16;
-            } else {
-                int64_t r = tn * kRingTN + (row - kRingTM);
-                r = r < nb ? r : nb - 1;
-                src[j] = Bb + r * row_bytes + chunk * 16;
-            }
+            const int local = row & (kRingTM - 1);                // row inside the operand tile
+            src_off[j] = (uint32_t)(local < limit ? local : limit) * (uint32_t)row_bytes + (uint32_t)chunk * 16u;
         }
     };
     // issue the loads of one K-step (step ks of the current issue tile) into ring buffer `slot`
     auto issue = [&](int ks, int slot) {
         unsigned char *stage = ring + slot * kRingStageBytes;
+        const unsigned char *base = tile_base + ks * 64;
 #pragma unroll
         for (int j = 0; j < kRingLoadsPerWave; j++) {
             const int rg = wave * kRingLoadsPerWave + j;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src[j] + ks * 64),
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + src_off[j]),
                                              (__attribute__((address_space(3))) void *)(stage + rg * 1024), 16, 0, 0);
         }
     };
 
-    typename Tr::Acc acc[4][2];   // written from zero by the first K-step of every tile
+    typename Tr::Acc acc[4][2];   // written from zero by the first half-step of every tile
 
     // (item, step, ring slot) of the next K-step to issue and of the one being computed
     int issued = 0, i_it = 0, i_ks = 0, i_slot = 0;
@@ -239,11 +246,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             i_it++;
         }
     };
-    while (issued < kRingStages - 1 && issued < total) {
+    // The two wavefronts of a SIMD (waves w and w + 4) do their per-step bookkeeping (address updates
+    // and load issue: a few hundred cycles without an MFMA) at different points between the
+    // once-per-step barriers, so that one wave's bookkeeping coincides with the other's MFMAs:
+    // "early" waves (0..3) right after the barrier, "late" waves (4..7) after the second half-step.
+    const bool late = wave >= 4;
+    while (issued < kRingStages && issued < total) {
         issue_next();
     }
     int c_it = 0, c_ks = 0, c_slot = 0;
-    bool stored = false;  // the previous iteration ended with an epilogue that issued stores
+    bool stored = false;  // the previous K-step ended with an epilogue that issued stores
 
     // Filtered launches stage what the epilogue of a tile needs -- the base norms of the wave's 64
     // columns and the bounds (and norms) of its 128 query rows -- in a small per-wave LDS area, with
@@ -259,77 +271,113 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool prefetch = FILTER && nk >= 2 && nb % 4 == 0 && nq % 4 == 0 && bn != nullptr && qn != nullptr &&
                           bound != nullptr && reinterpret_cast<uintptr_t>(bn) % 16 == 0 &&
                           reinterpret_cast<uintptr_t>(qn) % 16 == 0 && reinterpret_cast<uintptr_t>(bound) % 16 == 0;
-    bool fetched = false;   // the previous iteration issued the fetch
+    bool fetched = false;   // the staging loads were issued during the previous K-step
     auto fetch_epilogue_operands = [&](int it) {
         int64_t tm, tn;
         item_tile(it, tm, tn);
         const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
         asm volatile("" ::: "memory");
+        // (the lane number is made opaque here so that nothing derived from it in this once-per-tile
+        // code is kept in registers across the main loop)
+        int lane = tid & 63;
+        asm volatile("" : "+v"(lane));
+        // groups of four values; a group that starts past the end of its array reads the array's
+        // first group instead (its scores are rejected by index in the epilogue)
         if (lane < 48) {
-            // groups of four that start past the end read group 0 instead; their scores are rejected
-            // by index in the epilogue
-            const S *p;
-            if (lane < 16) {
-                const int64_t col = j0 + wc * 64 + lane * 4;
-                p = bn + (col < nb ? col : 0);
-            } else {
-                const int64_t row = i0 + wr * 128 + (lane - 16) * 4;
-                p = bound + (row < nq ? row : 0);
-            }
+            const bool is_bn = lane < 16;
+            const int group = is_bn ? lane : lane - 16;
+            const int64_t first = is_bn ? j0 + wc * 64 : i0 + wr * 128;
+            const int64_t left = ((is_bn ? nb : nq) - first) >> 2;      // whole groups from `first` on
+            const S *arr = is_bn ? bn : bound;
+            const S *p = group < left ? arr + first + group * 4 : arr;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
                                              (__attribute__((address_space(3))) void *)aux, 16, 0, 0);
         }
         if constexpr (!kInt) {
             if (lane < 32) {
-                const int64_t row = i0 + wr * 128 + lane * 4;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(qn + (row < nq ? row : 0)),
+                const int64_t first = i0 + wr * 128;
+                const S *p = lane < ((nq - first) >> 2) ? qn + first + lane * 4 : qn;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
                                                  (__attribute__((address_space(3))) void *)(aux + 768), 16, 0, 0);
             }
         }
         asm volatile("" ::: "memory");
     };
+
+    // K-step 0 must have landed before its first fragments are read
+    if (issued >= 3) {
+        __builtin_amdgcn_s_waitcnt(ring_vmcnt(2 * kRingLoadsPerWave));
+    } else if (issued == 2) {
+        __builtin_amdgcn_s_waitcnt(ring_vmcnt(kRingLoadsPerWave));
+    } else {
+        __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+    }
+    __builtin_amdgcn_s_barrier();
+    // LDS addresses of this lane's fragment chunks: row blocks are 2048 bytes apart (immediate
+    // offsets); the swizzle term (row >> 2) & 3 only depends on the lane
+    const uint32_t ring_base = (uint32_t)reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)ring);
+    const int swz = (l32 >> 2) & 3;
+    const uint32_t a_row = ring_base + (uint32_t)(wr * 128 + l32) * 64, b_row = ring_base + (uint32_t)(kRingTM + wc * 64 + l32) * 64;
+    const uint32_t coff0 = (uint32_t)((Tr::chunk(0, half) ^ swz) << 4), coff1 = (uint32_t)((Tr::chunk(1, half) ^ swz) << 4);
+    typename Tr::Frag fa, fb;
+    ring_read_frag(a_row + coff0, b_row + coff0, fa);
+
     for (int g = 0; g < total; g++) {
-        // The loads of step g must have landed; later steps may still be in flight.  vmcnt counts
-        // loads and stores in issue order, so right after a storing epilogue the usual count would
-        // also wait for all of its (much younger) stores; 63 is the largest expressible count and
-        // still covers the loads of step g, which are older than every store.
-        if (!FILTER && stored && issued - g - 1 >= kRingStages - 2) {
-            __builtin_amdgcn_s_waitcnt(0xcf7f);   // vmcnt(63): covers the <= 32 + 6 younger operations
-        } else if (issued - g - 1 >= kRingStages - 2) {
-            constexpr int kInFlight = (kRingStages - 2) * kRingLoadsPerWave;
-            if (FILTER && fetched) {
-                // queue: [step g][step g + 1][epilogue fetch]; only step g has to be complete
-                constexpr int n = kInFlight + kPrefetchLoads;
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (n & 15) | ((n >> 4) << 14));
+        const uint32_t stage_off = (uint32_t)(c_slot * kRingStageBytes);
+        const int next_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
+        bool issued_now = false;
+        // the wait a wave does before barrier g: K-step g + 1 (its own part) must have landed.  vmcnt
+        // counts loads and stores in issue order; younger than the loads of K-step g + 1 are the loads
+        // of K-step g + 2 and the staging loads of a filtered epilogue, when those were issued.  A
+        // storing epilogue does this wait itself, before it issues its stores.
+        auto wait_next_step = [&]() {
+            if (g + 2 >= total) {
+                __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+            } else if (!FILTER && stored) {
+            } else if (FILTER && fetched) {
+                __builtin_amdgcn_s_waitcnt(ring_vmcnt(kRingLoadsPerWave + kPrefetchLoads));
             } else {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | kInFlight);
+                __builtin_amdgcn_s_waitcnt(ring_vmcnt(kRingLoadsPerWave));
             }
+        };
+        auto issue_and_fetch = [&]() {
+            if (issued < total) {
+                issue_next();  // into the buffer of K-step g
+                issued_now = true;
+            }
+            if (FILTER && prefetch && c_ks == nk - 2) {
+                fetch_epilogue_operands(c_it);
+                fetched = true;
+            } else {
+                fetched = false;
+            }
+        };
+        // ---- first half-step: its fragments (fa) were read during the previous half-step
+        ring_read_frag(a_row + stage_off + coff1, b_row + stage_off + coff1, fb);
+        ring_wait_frag<6>(fa);
+        if (c_ks == 0) {
+            Tr::template mma<FILTER, true>(fa, acc);
         } else {
-            __builtin_amdgcn_s_waitcnt(0x0f70);
+            Tr::template mma<FILTER, false>(fa, acc);
+        }
+        // ---- between the half-steps: barrier g.  Before it K-step g + 1 (this wave's part) must have
+        // landed and this wave must be done reading the buffer of K-step g (its second fragments are
+        // in registers once lgkmcnt is 0); after it K-step g + 3 may overwrite that buffer.
+        ring_wait_frag<0>(fb);
+        if (g + 1 < total) {
+            wait_next_step();
+            __builtin_amdgcn_s_barrier();
+            if (!late) {
+                issue_and_fetch();
+            }
+            const uint32_t next_off = (uint32_t)(next_slot * kRingStageBytes);
+            ring_read_frag(a_row + next_off + coff0, b_row + next_off + coff0, fa);
         }
         stored = false;
-        fetched = false;
-        __builtin_amdgcn_s_barrier();
-        const bool issued_now = issued < total;
-        if (issued_now) {
-            issue_next();  // goes into the buffer that step g - 1 has just finished reading
-        }
-        if (FILTER && prefetch && c_ks == nk - 2) {
-            fetch_epilogue_operands(c_it);
-            fetched = true;
-        }
-        if (c_ks == 0) {
-            Tr::template mma<FILTER, true>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
-        } else {
-            Tr::template mma<FILTER, false>(ring + c_slot * kRingStageBytes, wr, wc, l32, half, acc);
-        }
+        // ---- second half-step
+        Tr::template mma<FILTER, false>(fb, acc);
         const bool last_step = c_ks == nk - 1;
         const int done_it = c_it;
-        c_slot = c_slot + 1 == kRingStages ? 0 : c_slot + 1;
-        if (++c_ks == nk) {
-            c_ks = 0;
-            c_it++;
-        }
         // Two epilogues.  Filtered launches make the BASE fragment the first MFMA operand, so a lane
         // owns one query row per block (its bound is a per-lane scalar) -- cheapest test per score.
         // Storing launches keep the query fragment first: a lane owns one base column and 32 lanes
@@ -342,84 +390,69 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             int64_t tm, tn;
             item_tile(done_it, tm, tn);
             const int64_t i0 = tm * kRingTM, j0 = tn * kRingTN;
-            const bool vec_out = !FILTER && (ldo % 4 == 0) && (reinterpret_cast<uintptr_t>(out) % 16 == 0);
-            // the base norms of this lane's 32 columns: out of the staging area, or loaded here
-            S bnq[2][4][4];
-            const bool use_bn = kInt || metric == kMetricL2;
-            const bool vec_bn = reinterpret_cast<uintptr_t>(bn) % 16 == 0;
+            // lane-derived values of this once-per-tile code must not occupy registers in the main loop
+            int lane = tid & 63;
+            asm volatile("" : "+v"(lane));
+            const int half = lane >> 5, l32 = lane & 31;
+            // The epilogue's operands come out of the wave's staging area: put there one K-step ahead
+            // by fetch_epilogue_operands(), or (shapes the staging loads do not serve) filled here.
+            // int8: the norms are negated in place, so that a score's test value is one shift-add.
             if (prefetch) {
-                // the staging loads are older than the K-step loads issued in this iteration
+                // the staging loads are older than the K-step loads issued during this K-step
                 if (issued_now) {
-                    __builtin_amdgcn_s_waitcnt(0x0f70 | kRingLoadsPerWave);
+                    __builtin_amdgcn_s_waitcnt(ring_vmcnt(kRingLoadsPerWave));
                 } else {
-                    __builtin_amdgcn_s_waitcnt(0x0f70);
+                    __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
                 }
                 asm volatile("" ::: "memory");
+                if constexpr (kInt) {
+                    S *p = reinterpret_cast<S *>(aux) + lane;
+                    *p = -*p;
+                }
+            } else {
+                const int64_t col = j0 + wc * 64 + lane;
+                const bool use_bn = kInt || metric == kMetricL2;
+                const S bv = (use_bn && col < nb) ? bn[col] : (S)0;
+                reinterpret_cast<S *>(aux)[lane] = kInt ? -bv : bv;
 #pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-#pragma unroll
-                    for (int rq = 0; rq < 4; rq++) {
-                        const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
-                        bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
-                        bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
-                        bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
-                        bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
+                for (int t = 0; t < 2; t++) {
+                    const int64_t row = i0 + wr * 128 + t * 64 + lane;
+                    const bool ok = row < nq;
+                    reinterpret_cast<S *>(aux + 256)[t * 64 + lane] = ok ? bound[row] : (S)0;
+                    if constexpr (!kInt) {
+                        reinterpret_cast<S *>(aux + 768)[t * 64 + lane] = (ok && metric == kMetricL2) ? qn[row] : (S)0;
                     }
                 }
             }
-#pragma unroll
-            for (int rb = 0; rb < 2 && !prefetch; rb++) {
-#pragma unroll
-                for (int rq = 0; rq < 4; rq++) {
-                    const int64_t col = j0 + wc * 64 + rb * 32 + 8 * rq + 4 * half;
-                    if (use_bn && vec_bn && col + 3 < nb) {
-                        const uint4 u = *reinterpret_cast<const uint4 *>(bn + col);
-                        bnq[rb][rq][0] = __builtin_bit_cast(S, u.x);
-                        bnq[rb][rq][1] = __builtin_bit_cast(S, u.y);
-                        bnq[rb][rq][2] = __builtin_bit_cast(S, u.z);
-                        bnq[rb][rq][3] = __builtin_bit_cast(S, u.w);
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 4; t++) {
-                            bnq[rb][rq][t] = (use_bn && col + t < nb) ? bn[col + t] : (S)0;
-                        }
-                    }
-                }
-            }
-            if constexpr (kInt) {
-                // -|b|^2, so that a score's test value is one shift-add: 2 q.b - |b|^2
-#pragma unroll
-                for (int t = 0; t < 32; t++) {
-                    bnq[t >> 4][(t >> 2) & 3][t & 3] = -bnq[t >> 4][(t >> 2) & 3][t & 3];
-                }
-            }
+            wave_lds_fence();
 #pragma unroll
             for (int ra = 0; ra < 4; ra++) {
                 asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
-                const int64_t row = i0 + wr * 128 + ra * 32 + l32;
+                const int64_t row = i0 + (wr * 128 + ra * 32 + l32);
                 const bool row_ok = row < nq;
-                S rowv, tauv;
-                if (prefetch) {
-                    const S bv = *reinterpret_cast<const S *>(aux + 256 + (ra * 32 + l32) * 4);
-                    rowv = kInt ? bv : *reinterpret_cast<const S *>(aux + 768 + (ra * 32 + l32) * 4);
-                    tauv = kInt ? (S)0 : bv;
-                } else if (kInt) {
-                    // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
-                    rowv = row_ok ? flt.thr[row] : (S)0x80000000;
-                    tauv = 0;
-                } else {
-                    rowv = (row_ok && metric == kMetricL2) ? qn[row] : (S)0;
-                    tauv = row_ok ? flt.tau[row] : (S)(-__builtin_inff());
-                }
+                // int8: rowv = tau - |q|^2 (|b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau, exact in
+                // integers); fp32: rowv = |q|^2, tauv = tau
+                const S bv = *reinterpret_cast<const S *>(aux + 256 + (ra * 32 + l32) * 4);
+                const S rowv = kInt ? bv : *reinterpret_cast<const S *>(aux + 768 + (ra * 32 + l32) * 4);
+                const S tauv = kInt ? (S)0 : bv;
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
                     // all 16 scores of the block first, then ONE test of their minimum against the
                     // lane's bound: admissions are rare, so the per-score path almost never runs
                     S v[16];
                     S best = ScoreOps<S>::worst();
+                    S bnq[4][4];   // (minus, for int8) the base norms of this lane's 16 columns of the block
+#pragma unroll
+                    for (int rq = 0; rq < 4; rq++) {
+                        const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
+                        bnq[rq][0] = __builtin_bit_cast(S, u.x);
+                        bnq[rq][1] = __builtin_bit_cast(S, u.y);
+                        bnq[rq][2] = __builtin_bit_cast(S, u.z);
+                        bnq[rq][3] = __builtin_bit_cast(S, u.w);
+                    }
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const S bnv = bnq[rb][r >> 2][r & 3];
+                        const S bnv = bnq[r >> 2][r & 3];
                         if constexpr (kInt) {
                             // bnq holds -|b|^2: v = -(distance - |q|^2) in one shift-add, largest is best
                             v[r] = (S)(((uint32_t)acc[ra][rb][r] << 1) + (uint32_t)bnv);
@@ -466,6 +499,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         }
         if (!FILTER && last_step) {
+            // The stores below queue up behind the loads in flight, and how many of them a wave issues
+            // depends on the tile's position: the wait for the next K-step that the coming barrier
+            // needs happens here, while the loads are still the youngest operations.
+            if (issued_now) {
+                __builtin_amdgcn_s_waitcnt(ring_vmcnt(kRingLoadsPerWave));
+            } else {
+                __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
+            }
             stored = true;
             int64_t tm, tn;
             item_tile(done_it, tm, tn);
@@ -533,6 +574,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
             }
         }
+        if (late && g + 1 < total) {
+            issue_and_fetch();
+        }
+        c_slot = next_slot;
+        if (++c_ks == nk) {
+            c_ks = 0;
+            c_it++;
+        }
     }
 }
 
@@ -555,20 +604,20 @@ bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, i
         IXA_HIP(hipGetDevice(&dev));
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     }
-    const unsigned grid = (unsigned)((2 * cus + 7) / 8 * 8);   // two persistent workgroups per CU
-    const size_t smem = (size_t)kRingStages * kRingStageBytes + (filter ? 4 * kRingAuxBytes : 0);
+    const unsigned grid = (unsigned)((cus + 7) / 8 * 8);   // one persistent workgroup per CU
+    const size_t smem = (size_t)kRingStages * kRingStageBytes + (filter ? kRingWaves * kRingAuxBytes : 0);
     if (filter) {
         auto kern = score_ring_kernel<Tr, true>;
         IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)smem));
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo, (int)rt_m,
-                           (int)rt_n, flt);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
+                           (int)rt_m, (int)rt_n, flt);
     } else {
         auto kern = score_ring_kernel<Tr, false>;
         IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)smem));
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo, (int)rt_m,
-                           (int)rt_n, flt);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
+                           (int)rt_m, (int)rt_n, flt);
     }
     return true;
 }

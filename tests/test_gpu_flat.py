@@ -18,7 +18,10 @@ def ix():
     return indexsdk_amd
 
 
-@pytest.mark.parametrize("d,n,nq,k", [(64, 5000, 33, 10), (512, 20000, 130, 100), (96, 3000, 7, 128), (40, 1000, 5, 3)])
+@pytest.mark.parametrize("d,n,nq,k", [(64, 5000, 33, 10), (512, 20000, 130, 100), (96, 3000, 7, 128), (40, 1000, 5, 3),
+                                      # query rows in every 128-row block of several 256-row tiles, with and
+                                      # without the staged epilogue operands (nq % 4)
+                                      (128, 9000, 516, 20), (256, 6000, 301, 7)])
 def test_flat_i8_exact(ix, oracle, d, n, nq, k):
     rng = np.random.default_rng(d + n)
     base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
@@ -67,7 +70,7 @@ def test_flat_i8_golden(ix):
 
 
 @pytest.mark.parametrize("metric_name", ["L2", "IP"])
-@pytest.mark.parametrize("d,n,nq,k", [(128, 20000, 100, 10), (96, 7000, 40, 100), (30, 900, 9, 5)])
+@pytest.mark.parametrize("d,n,nq,k", [(128, 20000, 100, 10), (96, 7000, 40, 100), (30, 900, 9, 5), (64, 9000, 300, 10)])
 def test_flat_f32_bit_exact(ix, oracle, metric_name, d, n, nq, k):
     metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
     rng = np.random.default_rng(n + d)
