@@ -167,7 +167,8 @@ typedef struct ivfpq_search_stats {
     double nsplit;        /* workgroups per query in the scan */
     double scan_waves;    /* wavefronts per scan workgroup */
     double shared_pool;   /* 1: one workgroup-wide candidate pool (large k), 0: one pool per wavefront */
-    double coarse_reruns; /* 1: the bf16x3 coarse pass could not be proven complete and fp32 reran it */
+    double coarse_reruns; /* queries whose matrix-core coarse result could not be proven complete and that were
+                             redone from canonical scores of all centroids */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 

@@ -71,11 +71,18 @@ void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, in
                             int64_t col_base, unsigned long long *running, hipStream_t s);
 
 // Exact best-nout SET from approximately scored, sorted candidates (see refine_boundary_kernel):
-// re-evaluates only the candidates within 2 * err of the rank-nout score; raises *flag when the
-// list cannot be proven to contain every winner.  out_ids: [nq][nout], unordered.
+// re-evaluates only the candidates within 2 * err of the rank-nout score; a query whose list
+// cannot be proven to contain every winner is appended to flag[1 + flag[0]++] (flag: 1 + nq ints).  out_ids: [nq][nout], unordered.
 void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                             int metric, const unsigned long long *running, int ncand, int nout, float cmax,
                             float err_scale, float round_scale, int32_t *out_ids, int *flag, hipStream_t s);
+
+// Canonical scores of all nc centroids for every row (one lane per score; the exact plan of last resort).
+void launch_canonical_scores(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                             const float *cn, int metric, float *out, int64_t ldo, hipStream_t s);
+// dist[n][k] = public distances of the columns idx[n][k] of a score matrix (-1 -> +-FLT_MAX).
+void launch_gather_scores(const float *scores, int64_t ld, const int32_t *idx, int64_t n, int k, int metric, float *dist,
+                          hipStream_t s);
 
 // Canonical re-evaluation of cand[nq][ncand] (-1 = absent) and selection of the best nout.  Rows of
 // the outputs are out_stride (>= nout) wide; columns past nout are padded with (-1, +-FLT_MAX).

@@ -557,8 +557,8 @@ __global__ __launch_bounds__(256) void refine_kernel(const float *__restrict__ Q
 // (the nout candidates with s <= T all have e <= T + err).  Only the candidates in between are
 // re-evaluated in the canonical scalar arithmetic and ranked by (e, id); the best
 // nout - |certain| of them complete the set.  Centroids outside the list have s >= s_last, so the
-// set is proven complete when s_last > T + 2 err; otherwise *flag is raised and the caller must use
-// another plan.  One wavefront per query; out_ids gets nout ids in no particular order.
+// set is proven complete when s_last > T + 2 err; otherwise the query is appended to the list
+// flag[1 + flag[0]++] and the caller must use another plan for it.  One wavefront per query; out_ids gets nout ids in no particular order.
 template <bool VEC4>
 __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__restrict__ Q, int64_t nq,
                                                               const float *__restrict__ C, int d,
@@ -594,7 +594,7 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
     const float lo = T - 2.0f * err, hi = T + 2.0f * err;
     const key_t last = run[ncand - 1];
     if (lane == 0 && last != kEmptyKey && !(key_score(last) > hi)) {
-        *flag = 1;
+        flag[1 + atomicAdd(flag, 1)] = (int)row;   // the list of queries that need another plan
     }
     int n_in = 0, n_amb = 0;
     for (int base = 0; base < ncand; base += kWave) {
@@ -681,6 +681,91 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
                        ncand, nout, cmax, err_scale, round_scale, out_ids, flag);
+}
+
+// Canonical scores of whole rows: out[row * ldo + col] for every centroid, one lane per score, in the
+// arithmetic of the refinement kernels (dot product left to right, no FMA).  The plan of last resort
+// for queries whose approximate candidate lists cannot be proven complete: slow, exact by construction.
+template <bool VEC4>
+__global__ __launch_bounds__(256) void canonical_scores_kernel(const float *__restrict__ Q, int64_t nq,
+                                                               const float *__restrict__ C, int64_t nc, int d,
+                                                               const float *__restrict__ qn,
+                                                               const float *__restrict__ cn, int metric,
+                                                               float *__restrict__ out, int64_t ldo)
+{
+    const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (col >= nc) {
+        return;
+    }
+    const float *q = Q + row * d;
+    const float *cv = C + col * d;
+    float g = 0.f;
+    if (VEC4) {
+#pragma unroll 4
+        for (int t = 0; t < d; t += 4) {
+            const float4 a = *reinterpret_cast<const float4 *>(q + t);
+            const float4 b = *reinterpret_cast<const float4 *>(cv + t);
+            g = __fadd_rn(g, __fmul_rn(a.x, b.x));
+            g = __fadd_rn(g, __fmul_rn(a.y, b.y));
+            g = __fadd_rn(g, __fmul_rn(a.z, b.z));
+            g = __fadd_rn(g, __fmul_rn(a.w, b.w));
+        }
+    } else {
+        for (int t = 0; t < d; t++) {
+            g = __fadd_rn(g, __fmul_rn(q[t], cv[t]));
+        }
+    }
+    float v;
+    if (metric == kMetricL2) {
+        v = __fadd_rn(qn[row], cn[col]);
+        v = __fsub_rn(v, g);
+        v = __fsub_rn(v, g);
+    } else {
+        v = -g;
+    }
+    out[row * ldo + col] = v;
+}
+
+void launch_canonical_scores(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,
+                             const float *cn, int metric, float *out, int64_t ldo, hipStream_t s)
+{
+    if (nq == 0 || nc == 0) {
+        return;
+    }
+    IXA_REQUIRE(nq <= 65535, kErrInner, "canonical score launch of %ld rows", (long)nq);
+    const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    const dim3 grid((unsigned)((nc + 255) / 256), (unsigned)nq);
+    if (vec4) {
+        hipLaunchKernelGGL(canonical_scores_kernel<true>, grid, dim3(256), 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo);
+    } else {
+        hipLaunchKernelGGL(canonical_scores_kernel<false>, grid, dim3(256), 0, s, Q, nq, C, nc, d, qn, cn, metric, out, ldo);
+    }
+}
+
+// dist[row * k + t] = the score at column idx[row * k + t], as the public distance (inner products are
+// stored negated in the score matrix); (+-FLT_MAX where idx is -1).
+__global__ __launch_bounds__(256) void gather_scores_kernel(const float *__restrict__ scores, int64_t ld,
+                                                            const int32_t *__restrict__ idx, int64_t n, int k, int metric,
+                                                            float *__restrict__ dist)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * k) {
+        return;
+    }
+    const int32_t c = idx[e];
+    const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+    const float v = c >= 0 ? scores[(e / k) * ld + c] : 0.f;
+    dist[e] = c >= 0 ? (metric == kMetricL2 ? v : -v) : pad;
+}
+
+void launch_gather_scores(const float *scores, int64_t ld, const int32_t *idx, int64_t n, int k, int metric, float *dist,
+                          hipStream_t s)
+{
+    if (n * k > 0) {
+        hipLaunchKernelGGL(gather_scores_kernel, dim3((unsigned)((n * k + 255) / 256)), dim3(256), 0, s, scores, ld, idx,
+                           n, k, metric, dist);
+    }
 }
 
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,

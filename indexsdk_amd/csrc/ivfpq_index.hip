@@ -106,6 +106,22 @@ __global__ __launch_bounds__(256) void gather_list_kernel(const uint8_t *__restr
     out[e] = codes[(off + p) * M + j];
 }
 
+// out rows idx[i] <- rows i of the compact results (ids, and distances when given)
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const int32_t *__restrict__ ids, const float *__restrict__ dist,
+                                                           const int64_t *__restrict__ idx, int64_t n, int width,
+                                                           int32_t *__restrict__ out_ids, float *__restrict__ out_dist)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * width) {
+        return;
+    }
+    const int64_t i = e / width, t = e - i * width;
+    out_ids[idx[i] * width + t] = ids[e];
+    if (dist) {
+        out_dist[idx[i] * width + t] = dist[e];
+    }
+}
+
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ x, const int64_t *__restrict__ idx,
                                                           int64_t n, int d, float *__restrict__ out)
 {
@@ -234,6 +250,44 @@ void IvfpqIndex::get_trained(float *centroids, float *codebook) const
 // -------------------------------------------------------------------------------------------------
 // Stage 1 driver: MFMA scores into a bounded scratch, per-row selection of nout + slack candidates,
 // exact refine.  Never materialises more than scratch_bytes of the n x nlist score matrix.
+// Exact plan of last resort for the listed rows: canonical scores of every centroid, exact selection.
+void IvfpqIndex::coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
+                                   int32_t *out_ids, float *out_dist)
+{
+    const int64_t m = (int64_t)rows.size();
+    const int64_t per_launch = std::max<int64_t>(1, std::min<int64_t>(32768, cfg_.scratch_bytes / (4 * nlist_)));
+    DeviceBuffer<int64_t> rows_dev;
+    rows_dev.upload(rows.data(), rows.size(), stream_);
+    DeviceBuffer<float> xsub, qn, scores, dist;
+    DeviceBuffer<int32_t> idx;
+    for (int64_t r0 = 0; r0 < m; r0 += per_launch) {
+        const int64_t mr = std::min(per_launch, m - r0);
+        xsub.resize((size_t)mr * d_);
+        qn.resize((size_t)mr);
+        scores.resize((size_t)mr * nlist_);
+        idx.resize((size_t)mr * nout);
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for(mr * d_)), dim3(256), 0, stream_, x_dev,
+                           rows_dev.data() + r0, mr, d_, xsub.data());
+        launch_sqnorm_rows(xsub.data(), mr, d_, qn.data(), stream_);
+        launch_canonical_scores(xsub.data(), mr, centroids_.data(), nlist_, d_, qn.data(), cnorm_.data(), select_metric,
+                                scores.data(), nlist_, stream_);
+        launch_select_rows(scores.data(), mr, nlist_, nlist_, nout, idx.data(), 0, nullptr, stream_);
+        if (out_dist) {
+            dist.resize((size_t)mr * nout);
+            launch_gather_scores(scores.data(), nlist_, idx.data(), mr, nout, select_metric, dist.data(), stream_);
+        }
+        hipLaunchKernelGGL(scatter_rows_kernel, dim3(blocks_for(mr * nout)), dim3(256), 0, stream_, idx.data(),
+                           out_dist ? dist.data() : nullptr, rows_dev.data() + r0, mr, nout, out_ids, out_dist);
+    }
+    IXA_HIP(hipStreamSynchronize(stream_));   // the temporaries above are freed on return
+}
+
+// Candidate generation with matrix-core products -- bf16 x 3 (error bound below, 16 spare candidates)
+// or, where that kernel does not serve the shape or is switched off, fp32 (8 spare candidates) -- then
+// either the canonical re-evaluation of every candidate plus a proof that nothing outside the list can
+// reach the nout-th exact score, or (set_only, bf16 x 3) the boundary-only refinement with the same
+// proof.  Queries whose proof fails (near-tied centroids) are redone exactly from canonical scores of
+// all centroids.
 void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
                                float *out_dist, bool set_only)
 {
@@ -242,74 +296,73 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     }
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
-    // Candidate generation.  Fast plan: bf16 x 3 matrix products (error bound below) with 16 spare candidates; the candidates are re-evaluated exactly, and a check
-    // proves that nothing outside them can reach the nout-th exact score.  If the check fails for
-    // any query (near-tied centroids), the fp32 plan below recomputes the whole call.
-    for (int attempt = cfg_.coarse_bf16 ? 0 : 1; attempt < 2; attempt++) {
-        const bool approx = attempt == 0;
-        const int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + (approx ? 16 : 8) + nout / 8);
+    int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 16 + nout / 8);
+    bool approx = false;
+    if (cfg_.coarse_bf16) {
         ws_running_.resize((size_t)n * ncand);
-        ws_cand_.resize((size_t)n * ncand);
         IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+        ws_xsplit_.resize((size_t)n * 3 * dp_);
+        launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
+        approx = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
+                                      cnorm_.data(), select_metric, ncand, ws_running_.data(), ws_sel_,
+                                      cfg_.scratch_bytes, stream_) >= 0;   // < 0: shape not served
+    }
+    if (!approx) {
+        ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
+        ws_running_.resize((size_t)n * ncand);
+        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
+        stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric, ncand,
+                          ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
+    }
+    // Bound on |approximate score - canonical score|, per unit of |q||c|, for one dot product.
+    //   bf16 x 3: x = hi + lo + r with |lo| <= 2^-9 |x|, |r| <= 2^-18 |x|, so the three products kept miss
+    //          lo.lo + r.y + x.r, at most 3 * 2^-18 sum |x_i y_i| <= 3 * 2^-18 |q||c|; bf16 x bf16 products
+    //          are exact in fp32 and accumulating K = 3 dp of them in any order errs by at most
+    //          K 2^-24 sum |terms|;
+    //   fp32:  d rounded products summed in some order: at most (d + 1) 2^-24 sum |x_i y_i|;
+    //   both:  the canonical left-to-right sum itself errs by at most (d + 1) 2^-24 sum |x_i y_i|
+    //          (a few units added for the second-order terms).
+    // L2 scores hold two dot products and three further roundings of numbers no larger than
+    // (|q| + |c|)^2, the same on both sides up to one unit each.
+    const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
+    const float u = 5.9604645e-8f;
+    const float err_scale = approx ? dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * u)
+                                   : dots * (float)(2 * d_ + 8) * u;
+    const float round_scale = select_metric == kMetricL2 ? 4.0f * u : 0.0f;
+    ws_flag_.resize((size_t)n + 1);
+    IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+    if (approx && set_only && !out_dist && ncand > nout) {
+        // search: only the SET of probed lists matters, so only the candidates the approximate scores
+        // cannot decide are re-evaluated
+        launch_refine_boundary(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
+                               ws_running_.data(), ncand, nout, cmax_, err_scale, round_scale, out_ids,
+                               ws_flag_.data(), stream_);
+    } else {
         float *dist = out_dist;
-        if (approx) {
-            ws_xsplit_.resize((size_t)n * 3 * dp_);
-            launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
-            const int rc = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_,
-                                                ws_qn_.data(), cnorm_.data(), select_metric, ncand, ws_running_.data(),
-                                                ws_sel_, cfg_.scratch_bytes, stream_);
-            if (rc < 0) {
-                continue;  // shape not served by the bf16 kernel
-            }
-            // Bound on |approximate score - canonical score|, per unit of |q||c|, for one dot product:
-            //   split: x = hi + lo + r with |lo| <= 2^-9 |x|, |r| <= 2^-18 |x|, so the three products kept
-            //          miss lo.lo + r.y + x.r, at most 3 * 2^-18 sum |x_i y_i| <= 3 * 2^-18 |q||c|;
-            //   sums:  bf16 x bf16 products are exact in fp32; accumulating K = 3 dp of them in any order
-            //          errs by at most K 2^-24 sum |terms|, the canonical left-to-right sum by d 2^-24
-            //          sum |x_i y_i| (a few units added for the second-order terms).
-            // L2 scores hold two dot products and three further roundings of numbers no larger than
-            // (|q| + |c|)^2, the same on both sides up to one unit each.
-            const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
-            const float u = 5.9604645e-8f;
-            const float err_scale = dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * u);
-            const float round_scale = select_metric == kMetricL2 ? 4.0f * u : 0.0f;
-            ws_flag_.resize(1);
-            IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
-            if (set_only && !out_dist && ncand > nout) {
-                // search: only the SET of probed lists matters, so only the candidates the approximate
-                // scores cannot decide are re-evaluated
-                launch_refine_boundary(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
-                                       ws_running_.data(), ncand, nout, cmax_, err_scale, round_scale, out_ids,
-                                       ws_flag_.data(),
-                                       stream_);
-            } else {
-                if (!dist) {
-                    ws_exact_.resize((size_t)n * nout);
-                    dist = ws_exact_.data();
-                }
-                launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
-                launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
-                              ws_cand_.data(), ncand, nout, nout, out_ids, dist, stream_);
-                launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale,
-                                       round_scale, select_metric, n, ws_flag_.data(), stream_);
-            }
-            int32_t failed = 0;
-            ws_flag_.download(&failed, 1, stream_);
-            if (!failed) {
-                break;
-            }
-            last_coarse_reruns_ = 1;
-            continue;
-        } else {
-            stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
-                              ncand, ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
+        if (!dist) {
+            ws_exact_.resize((size_t)n * nout);
+            dist = ws_exact_.data();
         }
-        // fp32 plan: every candidate re-evaluated
+        ws_cand_.resize((size_t)n * ncand);
         launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
         launch_refine(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric, ws_cand_.data(),
                       ncand, nout, nout, out_ids, dist, stream_);
-        break;
+        if (ncand < nlist_) {   // a list that holds every centroid needs no proof
+            launch_verify_superset(ws_running_.data(), ncand, dist, nout, ws_qn_.data(), cmax_, err_scale, round_scale,
+                                   select_metric, n, ws_flag_.data(), stream_);
+        }
     }
+    int32_t nfail = 0;
+    ws_flag_.download(&nfail, 1, stream_);
+    if (nfail == 0) {
+        return;
+    }
+    last_coarse_reruns_ += nfail;
+    std::vector<int32_t> rows32((size_t)nfail);
+    IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
+    IXA_HIP(hipStreamSynchronize(stream_));
+    std::sort(rows32.begin(), rows32.end());   // the order of the appends is not deterministic
+    coarse_exact_rows(x_dev, std::vector<int64_t>(rows32.begin(), rows32.end()), nout, select_metric, out_ids, out_dist);
 }
 
 void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)

@@ -678,7 +678,7 @@ void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_sid
     }
 }
 
-// Raises *flag unless, for every query, no centroid outside its approximate candidate list can beat
+// Appends a query to the list flag[1 + flag[0]++] unless, for that query, no centroid outside its approximate candidate list can beat
 // its nout-th exact score: (approximate score of the last candidate) - err > (nout-th exact score),
 // err = err_scale * |q| * max|c| + round_scale * (|q| + max|c|)^2.  Rows whose candidate list is not full hold every centroid.
 __global__ __launch_bounds__(256) void verify_superset_kernel(const key_t *__restrict__ running, int ncand,
@@ -701,7 +701,7 @@ __global__ __launch_bounds__(256) void verify_superset_kernel(const key_t *__res
     const float qlen = sqrtf(qn[i]);
     const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
     if (!(a_last - err > s_star)) {
-        *flag = 1;
+        flag[1 + atomicAdd(flag, 1)] = (int)i;   // the list of queries that need another plan
     }
 }
 

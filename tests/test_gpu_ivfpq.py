@@ -342,3 +342,33 @@ def test_search_with_tied_and_nearly_tied_centroids(ix, oracle, metric_name):
     Dr, Ir = ref.search(q, 20, nprobe)
     assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+
+
+def test_search_redoes_only_the_queries_whose_coarse_proof_fails(ix, oracle):
+    """300 centroids within 1e-6 of each other: for queries near them the approximate coarse scores can
+    neither rank them nor prove the candidate list complete, so those queries (and only those) are
+    redone by the fp32 plan; results and probe lists must equal the oracle's for all queries."""
+    rng = np.random.default_rng(61)
+    d, M, nlist, nprobe = 64, 16, 2048, 16          # 2048 lists: enough for the bf16 x 3 plan to be used
+    cent = rng.standard_normal((nlist, d)).astype(np.float32)
+    cent[:300] = cent[0] + (1e-6 * rng.standard_normal((300, d))).astype(np.float32)
+    x = (cent[rng.integers(0, nlist, 40000)] + 0.3 * rng.standard_normal((40000, d))).astype(np.float32)
+    near = (cent[0] + 0.3 * rng.standard_normal((40, d))).astype(np.float32)
+    far = (cent[rng.integers(300, nlist, 360)] + 0.3 * rng.standard_normal((360, d))).astype(np.float32)
+    q = np.ascontiguousarray(np.concatenate([near, far])[rng.permutation(400)])
+    cb = oracle.train_pq(x[:4000], M, niter=3, seed=3)
+    ids = np.arange(40000, dtype=np.int64)
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, ids)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add_with_ids(x, ids)
+    gpu.setNumProbes(nprobe)
+    D, I = gpu.search(q, 20)
+    reruns = gpu.last_search_stats()["coarse_reruns"]
+    assert 1 <= reruns <= 100, reruns
+    Dr, Ir = ref.search(q, 20, nprobe)
+    assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    pi, pd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
+    assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
