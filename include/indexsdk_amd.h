@@ -184,6 +184,8 @@ typedef struct flat_search_stats {
     double ms_select;      /* fp32: exact refine + label mapping */
     double ms_total;
     double score_launches; /* number of (query block, base chunk) score launches */
+    double exact_reruns;   /* fp32: queries whose candidate list could not be proven complete and that were
+                              redone from canonical scores of the whole base */
 } flat_search_stats_t;
 
 /* AscendIndexFlat(dims, metric, config)  FR/ascend/AscendIndexFlat.h:48-90.  scratch_bytes bounds the

@@ -40,7 +40,8 @@ class IvfpqSearchStats(ctypes.Structure):
 
 
 class FlatSearchStats(ctypes.Structure):
-    _fields_ = [(n, ctypes.c_double) for n in ("ms_score", "ms_select", "ms_total", "score_launches")]
+    _fields_ = [(n, ctypes.c_double) for n in ("ms_score", "ms_select", "ms_total", "score_launches",
+                                                     "exact_reruns")]
 
 
 # every exported symbol of include/indexsdk_amd.h: name -> (restype, argtypes)

@@ -289,6 +289,7 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
     out->ms_select = s.ms_select;
     out->ms_total = s.ms_total;
     out->score_launches = s.score_launches;
+    out->exact_reruns = s.exact_reruns;
 }
 
 #define IXA_FLAT_COMMON(PFX, HT, ET)                                                                              \

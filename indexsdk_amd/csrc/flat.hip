@@ -1,7 +1,9 @@
 // Brute-force Flat search: fp32 (scores on the fp32 matrix cores, exact refine) and int8 (exact
 // int32 L2 on the int8 matrix cores).  See flat_index.h for the reference counterparts.
 #include <algorithm>
+#include <cmath>
 #include <cstring>
+#include <vector>
 
 #include "coarse.h"
 #include "flat_index.h"
@@ -251,6 +253,47 @@ __global__ __launch_bounds__(256) void finish_keys_kernel(const key_t *__restric
     out_labels[i] = ids[key_index(kk)];
 }
 
+// largest value of a non-negative float array: the bit patterns order like the values
+__global__ __launch_bounds__(256) void max_bits_kernel(const float *__restrict__ v, int64_t n, uint32_t *__restrict__ out)
+{
+    uint32_t m = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const uint32_t b = __float_as_uint(v[i]);
+        m = b > m ? b : m;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t t = __shfl_down(m, o);
+        m = t > m ? t : m;
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicMax(out, m);
+    }
+}
+
+__global__ __launch_bounds__(256) void gather_rows_f32_kernel(const float *__restrict__ x, const int64_t *__restrict__ idx,
+                                                              int64_t n, int d, float *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e < n * d) {
+        out[e] = x[idx[e / d] * d + e % d];
+    }
+}
+
+// result rows idx[i] <- rows i of the compact results
+__global__ __launch_bounds__(256) void scatter_result_rows_kernel(const float *__restrict__ dist,
+                                                                  const int64_t *__restrict__ labels,
+                                                                  const int64_t *__restrict__ idx, int64_t n, int k,
+                                                                  float *__restrict__ out_dist,
+                                                                  int64_t *__restrict__ out_labels)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e < n * k) {
+        const int64_t o = idx[e / k] * k + e % k;
+        out_dist[o] = dist[e];
+        out_labels[o] = labels[e];
+    }
+}
+
 __global__ __launch_bounds__(256) void map_labels_kernel(const int32_t *__restrict__ idx, int64_t n,
                                                          const int64_t *__restrict__ ids, int64_t *__restrict__ out)
 {
@@ -412,8 +455,56 @@ void FlatIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_devic
         IXA_HIP(hipMemcpyAsync(nn.data(), norms_.data(), (size_t)before * 4, hipMemcpyDeviceToDevice, stream_));
     }
     launch_sqnorm_rows(base_.data() + before * d_, n, d_, nn.data() + before, stream_);
-    IXA_HIP(hipStreamSynchronize(stream_));
+    // largest norm of the base (the error bound of the approximate scores is proportional to it)
+    DeviceBuffer<uint32_t> mx(1);
+    IXA_HIP(hipMemsetAsync(mx.data(), 0, 4, stream_));
+    hipLaunchKernelGGL(max_bits_kernel, dim3((unsigned)std::min<int64_t>(1024, (n + 255) / 256)), dim3(256), 0, stream_,
+                       nn.data() + before, n, mx.data());
+    uint32_t bits = 0;
+    mx.download(&bits, 1, stream_);
+    float sq;
+    std::memcpy(&sq, &bits, 4);
+    bmax_ = std::max(bmax_, std::sqrt(sq));
     norms_ = std::move(nn);
+}
+
+// Exact plan of last resort (queries whose candidate list cannot be proven complete): canonical scores
+// of the whole base, chunk by chunk, with an exact running selection.
+void FlatIndex::exact_rows(const float *xd, const std::vector<int64_t> &rows, int64_t k, float *dist_dev,
+                           int64_t *labels_dev)
+{
+    const int64_t total_rows = (int64_t)rows.size();
+    DeviceBuffer<int64_t> rows_dev;
+    rows_dev.upload(rows.data(), rows.size(), stream_);
+    DeviceBuffer<float> xsub, qn, scores, dsub;
+    DeviceBuffer<unsigned long long> running;
+    DeviceBuffer<int64_t> lsub;
+    for (int64_t r0 = 0; r0 < total_rows; r0 += 4096) {
+        const int64_t m = std::min<int64_t>(4096, total_rows - r0);
+        const int64_t cols = std::max<int64_t>(4096, std::min<int64_t>(ntotal_, scratch_bytes_ / (4 * m)));
+        xsub.resize((size_t)m * d_);
+        qn.resize((size_t)m);
+        scores.resize((size_t)m * cols);
+        running.resize((size_t)m * k);
+        dsub.resize((size_t)m * k);
+        lsub.resize((size_t)m * k);
+        hipLaunchKernelGGL(gather_rows_f32_kernel, dim3(blocks_for(m * d_)), dim3(256), 0, stream_, xd, rows_dev.data() + r0,
+                           m, d_, xsub.data());
+        launch_sqnorm_rows(xsub.data(), m, d_, qn.data(), stream_);
+        IXA_HIP(hipMemsetAsync(running.data(), 0xff, running.bytes(), stream_));
+        for (int64_t c0 = 0; c0 < ntotal_; c0 += cols) {
+            const int64_t nc = std::min(cols, ntotal_ - c0);
+            launch_canonical_scores(xsub.data(), m, base_.data() + c0 * d_, nc, d_, qn.data(), norms_.data() + c0, metric_,
+                                    scores.data(), nc, stream_);
+            launch_select_rows(scores.data(), m, nc, nc, (int)k, nullptr, c0, running.data(), stream_);
+        }
+        const float pad = metric_ == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+        hipLaunchKernelGGL((finish_keys_kernel<float, float>), dim3(blocks_for(m * k)), dim3(256), 0, stream_,
+                           running.data(), m * k, metric_, ids_.data(), pad, dsub.data(), lsub.data());
+        hipLaunchKernelGGL(scatter_result_rows_kernel, dim3(blocks_for(m * k)), dim3(256), 0, stream_, dsub.data(),
+                           lsub.data(), rows_dev.data() + r0, m, (int)k, dist_dev, labels_dev);
+    }
+    IXA_HIP(hipStreamSynchronize(stream_));   // the temporaries above are freed on return
 }
 
 void FlatIndex::reset()
@@ -459,6 +550,31 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
                   (int)std::min<int64_t>(k, ncand), (int)k, ws_idx_.data(), dd, stream_);
     hipLaunchKernelGGL(map_labels_kernel, dim3(blocks_for(n * k)), dim3(256), 0, stream_, ws_idx_.data(), n * k,
                        ids_.data(), ld);
+    // Proof that no base vector outside a query's candidate list can reach its k-th exact score; the
+    // approximate scores are fp32 matrix-core sums: they and the canonical left-to-right sums are each
+    // within (d + 1) 2^-24 sum |x_i y_i| of the exact dot product (a few units added for second-order
+    // terms); an L2 score holds two dot products and three further roundings of numbers no larger
+    // than (|q| + |b|)^2.  Queries without proof are redone exactly.
+    stats_.exact_reruns = 0;
+    if (ncand < ntotal_) {
+        const float u = 5.9604645e-8f;
+        const float err_scale = (metric_ == kMetricL2 ? 2.0f : 1.0f) * (float)(2 * d_ + 8) * u;
+        const float round_scale = metric_ == kMetricL2 ? 4.0f * u : 0.0f;
+        ws_flag_.resize((size_t)n + 1);
+        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+        launch_verify_superset(ws_running_.data(), ncand, dd, (int)k, ws_qn_.data(), bmax_, err_scale, round_scale, metric_,
+                               n, ws_flag_.data(), stream_);
+        int32_t nfail = 0;
+        ws_flag_.download(&nfail, 1, stream_);
+        if (nfail > 0) {
+            std::vector<int32_t> rows32((size_t)nfail);
+            IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
+            IXA_HIP(hipStreamSynchronize(stream_));
+            std::sort(rows32.begin(), rows32.end());
+            exact_rows(xd, std::vector<int64_t>(rows32.begin(), rows32.end()), k, dd, ld);
+            stats_.exact_reruns = nfail;
+        }
+    }
     IXA_HIP(hipEventRecord(ev_[2], stream_));
     IXA_HIP(hipStreamSynchronize(stream_));
     if (!on_device) {

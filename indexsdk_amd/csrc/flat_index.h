@@ -7,6 +7,7 @@
 //                   reference's final scale-and-round-to-fp16 step.
 #pragma once
 #include <cstdint>
+#include <vector>
 
 #include "common.h"
 #include "stream_select.h"
@@ -18,6 +19,7 @@ struct FlatStats {
     double ms_select = 0;       // all selection launches (+ refine / finalisation)
     double ms_total = 0;
     double score_launches = 0;
+    double exact_reruns = 0;    // fp32: queries redone from canonical scores of the whole base
 };
 
 template <typename T>
@@ -59,10 +61,13 @@ public:
     void reset();
 
 private:
+    // exact results for the listed query rows, from canonical scores of the whole base
+    void exact_rows(const float *xd, const std::vector<int64_t> &rows, int64_t k, float *dist_dev, int64_t *labels_dev);
     DeviceBuffer<float> norms_, ws_qn_, ws_dist_;
     StreamSelectWorkspace<float> ws_sel_;
-    DeviceBuffer<int32_t> ws_cand_, ws_idx_;
+    DeviceBuffer<int32_t> ws_cand_, ws_idx_, ws_flag_;
     DeviceBuffer<int64_t> ws_labels_;
+    float bmax_ = 0.f;   // largest base vector norm
 };
 
 class FlatI8Index : public FlatBase<int8_t> {

@@ -139,3 +139,27 @@ def test_flat_f32_many_fused_chunks(ix, oracle):
         D, I = index.search(q, k)
         Dr, Ir = oracle.flat_f32(base, q, k, metric)
         assert np.array_equal(I, Ir) and np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+
+
+@pytest.mark.parametrize("metric_name", ["L2", "IP"])
+def test_flat_f32_near_duplicates_are_redone_exactly(ix, oracle, metric_name):
+    """3000 base vectors within 1e-6 of each other: for queries near them the matrix-core scores can
+    neither rank them nor prove a candidate list complete; those queries are redone from canonical
+    scores of the whole base and every result still equals the oracle's bit for bit."""
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    rng = np.random.default_rng(71)
+    d, n, nq, k = 64, 12000, 60, 20
+    base = rng.standard_normal((n, d)).astype(np.float32)
+    base[:3000] = base[0] + (1e-6 * rng.standard_normal((3000, d))).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    q[:10] = base[0] + (0.05 * rng.standard_normal((10, d))).astype(np.float32)
+    if metric == ix.METRIC_INNER_PRODUCT:
+        q[:10] = 3.0 * base[0] + (0.05 * rng.standard_normal((10, d))).astype(np.float32)
+    index = ix.AscendIndexFlat(d, metric)
+    index.add(base)
+    D, I = index.search(q, k)
+    reruns = index.last_search_stats()["exact_reruns"]
+    assert 10 <= reruns < nq, reruns
+    Dr, Ir = oracle.flat_f32(base, q, k, metric)
+    assert np.array_equal(I, Ir)
+    assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
