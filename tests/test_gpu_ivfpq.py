@@ -372,3 +372,22 @@ def test_search_redoes_only_the_queries_whose_coarse_proof_fails(ix, oracle):
     pi, pd = gpu.coarse_probe(q)
     oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
     assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
+
+
+def test_reset_keeps_quantizers_and_readd_reproduces_codes(ix, oracle):
+    """Reference ST invariant (FR/test/ascend/TestAscendIndexIVFPQ.cpp, case All): add / reset / add gives
+    byte-identical lists; reset empties every list and leaves the index trained."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 81, 9000, 20, 64, 64, 16, ix.METRIC_L2)
+    before = [gpu.getListCodesAndIds(l) for l in range(64) if gpu.getListLength(l)]
+    D0, I0 = gpu.search(q, 7)
+    gpu.reset()
+    assert gpu.ntotal == 0 and gpu.is_trained and all(gpu.getListLength(l) == 0 for l in range(64))
+    D, I = gpu.search(q, 7)
+    assert np.all(I == -1) and np.all(D == FLT_MAX)
+    gpu.add_with_ids(x, ids)
+    after = [gpu.getListCodesAndIds(l) for l in range(64) if gpu.getListLength(l)]
+    assert len(before) == len(after)
+    for (c0, i0), (c1, i1) in zip(before, after):
+        assert np.array_equal(c0, c1) and np.array_equal(i0, i1)
+    D1, I1 = gpu.search(q, 7)
+    assert np.array_equal(I0, I1) and np.array_equal(D0.view(np.uint32), D1.view(np.uint32))
