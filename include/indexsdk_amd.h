@@ -171,6 +171,11 @@ typedef struct ivfpq_search_stats {
                              redone from canonical scores of all centroids */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
+/* Device times of the last search only (HIP events on the index's stream, in ms); either output may be NULL.
+ * Unlike ivfpq_last_search_stats, which counts the scanned codes with a kernel launch and a host
+ * synchronisation the first time it is called after a search, this call does no device work, so it can sit
+ * inside a timed loop.  No counterpart in the reference: a measurement aid. */
+int ivfpq_last_search_timings(const ivfpq_index_t *h, double *ms_coarse, double *ms_scan);
 
 /* ---------------------------------------------------------------------------------------------
  * Flat (brute force): the coarse stage in isolation

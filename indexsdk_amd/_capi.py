@@ -82,6 +82,7 @@ _SIGNATURES = {
     "ivfpq_reset": (ctypes.c_int, [_H]),
     "ivfpq_ntotal": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int64)]),
     "ivfpq_last_search_stats": (ctypes.c_int, [_H, ctypes.POINTER(IvfpqSearchStats)]),
+    "ivfpq_last_search_timings": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
 }
 
 for _pfx, _dist in (("flat", ctypes.c_void_p), ("flat_i8", ctypes.c_void_p)):

@@ -198,6 +198,12 @@ class AscendIndexIVFPQ:
     def reset(self):
         _capi.check(self._lib.ivfpq_reset(self._h))
 
+    def last_search_timings(self):
+        """(ms_coarse, ms_scan) of the last search; no device work, usable inside a timed loop."""
+        a, b = ctypes.c_double(), ctypes.c_double()
+        _capi.check(self._lib.ivfpq_last_search_timings(self._h, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
     def last_search_stats(self):
         s = _capi.IvfpqSearchStats()
         _capi.check(self._lib.ivfpq_last_search_stats(self._h, ctypes.byref(s)))

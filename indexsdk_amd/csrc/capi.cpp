@@ -121,6 +121,11 @@ IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbi
     });
 }
 
+IXA_EXPORT int ivfpq_last_search_timings(const ivfpq_index_t *h, double *ms_coarse, double *ms_scan)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.last_timings(ms_coarse, ms_scan); });
+}
+
 IXA_EXPORT int ivfpq_write_faiss(const ivfpq_index_t *h, const char *path)
 {
     return guarded([&] { IXA_HANDLE(h); ixa::write_faiss_ivfpq(h->impl, path); });

@@ -74,7 +74,8 @@ public:
     // replaces the vectors of ids that exist; returns the ids that do not (host pointers)
     std::vector<int64_t> update(int64_t n, const float *x, const int64_t *ids);
     void reset();
-    const SearchStats &stats() const { return stats_; }
+    const SearchStats &stats();   // of the last search; evaluates timings and the scanned-code count on demand
+    void last_timings(double *ms_coarse, double *ms_scan);   // device times of the last search only (no device work)
 
 private:
     void check_trained() const;
@@ -104,6 +105,16 @@ private:
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
     DeviceBuffer<int32_t> ws_flag_;
     int last_coarse_reruns_ = 0;
+    bool stats_pending_ = false;
+    int64_t stats_rows_ = 0;
+    int stats_nprobe_ = 0;
+    // the probe lists and list lengths the pending statistics refer to are about to change
+    void flush_stats()
+    {
+        if (stats_pending_) {
+            stats();
+        }
+    }
     float cmax_ = 0.f;                                      // largest centroid norm
     int dp_ = 0;                                            // d rounded up to a multiple of 32
     // arena

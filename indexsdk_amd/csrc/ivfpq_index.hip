@@ -189,6 +189,7 @@ IvfpqIndex::~IvfpqIndex()
 
 void IvfpqIndex::set_nprobe(int nprobe)
 {
+    flush_stats();
     IXA_REQUIRE(nprobe >= 1, kErrInvalidParam, "nprobe must be >= 1, got %d", nprobe);
     nprobe_ = (int)std::min<int64_t>(nprobe, nlist_);
 }
@@ -230,6 +231,7 @@ void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
 
 void IvfpqIndex::set_trained(const float *centroids, const float *codebook)
 {
+    flush_stats();
     IXA_REQUIRE(centroids && codebook, kErrInvalidParam, "centroids and codebook can not be nullptr.");
     IXA_REQUIRE(ntotal_ == 0, kErrIllegalOperation, "set_trained on a non-empty index; call reset first");
     upload_trained(centroids, codebook);
@@ -367,6 +369,7 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
 
 void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(x && out, kErrInvalidParam, "x can not be nullptr.");
     IXA_REQUIRE(n >= 0 && n < kMaxN, kErrInvalidParam, "n must be >= 0 and < %ld", (long)kMaxN);
@@ -390,6 +393,7 @@ void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)
 
 void IvfpqIndex::coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(x && out_ids, kErrInvalidParam, "x can not be nullptr.");
     const float *xd = x;
@@ -434,6 +438,7 @@ void IvfpqIndex::encode(int64_t n, const float *x, uint8_t *codes, bool on_devic
 // (:715-805; ids default to ntotal + i, FR/ascend/impl/AscendIndexImpl.h:59-83).
 void IvfpqIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_device)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(x, kErrInvalidParam, "x can not be nullptr.");
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
@@ -468,6 +473,7 @@ void IvfpqIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_devi
 
 void IvfpqIndex::add_codes(int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(list >= 0 && list < nlist_, kErrInvalidParam, "the listId is %ld, out of numLists(%ld)", (long)list,
                 (long)nlist_);
@@ -487,6 +493,7 @@ void IvfpqIndex::add_codes(int64_t list, int64_t n, const uint8_t *codes, const 
 
 void IvfpqIndex::add_codes_bulk(int64_t n, const int32_t *list_no, const uint8_t *codes, const int64_t *ids)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(n >= 0 && (n == 0 || (list_no && codes && ids)), kErrInvalidParam, "codes and ids can not be nullptr.");
     if (n == 0) {
@@ -575,6 +582,7 @@ void IvfpqIndex::get_list(int64_t list, uint8_t *codes, int64_t *ids) const
 // and re-appended list by list.
 int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
 {
+    flush_stats();
     IXA_REQUIRE(n >= 0 && (n == 0 || ids), kErrInvalidParam, "ids can not be nullptr.");
     if (n == 0 || ntotal_ == 0) {
         return 0;
@@ -629,6 +637,7 @@ int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
 // their new vectors (they move to the end of their new list); ids that do not exist are returned.
 std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t *ids)
 {
+    flush_stats();
     check_trained();
     IXA_REQUIRE(x, kErrInvalidParam, "vector list is nullptr!");
     IXA_REQUIRE(ids, kErrInvalidParam, "vector ID list is nullptr!");
@@ -665,6 +674,7 @@ std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t
 // reset keeps the trained quantizers and drops every list (FR/ascend/AscendIndexIVF.h: reset()).
 void IvfpqIndex::reset()
 {
+    flush_stats();
     IXA_HIP(hipStreamSynchronize(stream_));
     codes_.release();
     ids_.release();
@@ -748,23 +758,58 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     }
     IXA_HIP(hipEventRecord(ev_[2], stream_));
 
-    IXA_HIP(hipMemsetAsync(ws_counter_.data(), 0, 8, stream_));
-    launch_count_scanned(ws_probes_.data(), n * nprobe_, list_len_dev_.data(), ws_counter_.data(), stream_);
-    unsigned long long scanned = 0;
-    ws_counter_.download(&scanned, 1, stream_);
     if (!on_device) {
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);
+    } else {
+        IXA_HIP(hipStreamSynchronize(stream_));
     }
-    float ms01 = 0, ms12 = 0;
-    IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
-    IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
-    stats_.scanned_codes = (double)scanned;
-    stats_.ms_coarse = ms01;
-    stats_.ms_scan = ms12;
-    stats_.ms_total = ms01 + ms12;
     stats_.scan_launches = nsplit > 1 ? 2 : 1;
     stats_.nsplit = nsplit;
+    stats_pending_ = true;   // timings and the scanned-code count are worked out when somebody asks
+    stats_rows_ = n;
+    stats_nprobe_ = nprobe_;
+}
+
+// Statistics of the last search.  The event timings and the number of scanned codes (a kernel over
+// the probe lists, which stay in the workspace until the next search) are evaluated here, not in
+// search(): they cost a launch and a host synchronisation that the search path does not need.
+void IvfpqIndex::last_timings(double *ms_coarse, double *ms_scan)
+{
+    float ms01 = 0, ms12 = 0;
+    if (stats_pending_) {   // the events of the last search have completed: search() synchronises its stream
+        IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
+        IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+    } else {
+        ms01 = (float)stats_.ms_coarse;
+        ms12 = (float)stats_.ms_scan;
+    }
+    if (ms_coarse) {
+        *ms_coarse = ms01;
+    }
+    if (ms_scan) {
+        *ms_scan = ms12;
+    }
+}
+
+const SearchStats &IvfpqIndex::stats()
+{
+    if (stats_pending_) {
+        ws_counter_.resize(1);
+        IXA_HIP(hipMemsetAsync(ws_counter_.data(), 0, 8, stream_));
+        launch_count_scanned(ws_probes_.data(), stats_rows_ * stats_nprobe_, list_len_dev_.data(), ws_counter_.data(), stream_);
+        unsigned long long scanned = 0;
+        ws_counter_.download(&scanned, 1, stream_);
+        float ms01 = 0, ms12 = 0;
+        IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
+        IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+        stats_.scanned_codes = (double)scanned;
+        stats_.ms_coarse = ms01;
+        stats_.ms_scan = ms12;
+        stats_.ms_total = ms01 + ms12;
+        stats_pending_ = false;
+    }
+    return stats_;
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -776,6 +821,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
 
 void IvfpqIndex::train(int64_t n, const float *x, bool on_device)
 {
+    flush_stats();
     IXA_REQUIRE(x, kErrInvalidParam, "x can not be nullptr.");
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     if (trained_) {
