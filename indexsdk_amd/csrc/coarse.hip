@@ -35,12 +35,72 @@ __global__ __launch_bounds__(256) void sqnorm_rows_kernel(const float *__restric
     out[i] = s;
 }
 
+// The same sums with coalesced loads.  A wavefront serves 16 rows: its 64 lanes fetch 64 columns of
+// them at a time (four 128-bit loads per lane, 256 contiguous bytes per row), transpose the chunk
+// through LDS, and lanes 0..15 each add their own row's 64 squares in column order; the next chunk's
+// loads are in flight meanwhile.  The order of additions per row is unchanged.
+__global__ __launch_bounds__(256) void sqnorm_rows_tiled_kernel(const float *__restrict__ x, int64_t n, int d,
+                                                                float *__restrict__ out)
+{
+    __shared__ float tile[4][16][65];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 16;
+    if (row0 >= n) {
+        return;
+    }
+    const int cg = lane & 15, rsub = lane >> 4;   // column group of 4, row within a group of 4 rows
+    auto fetch = [&](int c0, float4 (&v)[4]) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const int64_t r = row0 + rsub + 4 * t;
+            const int c = c0 + 4 * cg;
+            v[t] = (r < n && c < d) ? *reinterpret_cast<const float4 *>(x + r * d + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    float4 cur[4], nxt[4];
+    fetch(0, cur);
+    float s = 0.0f;
+    for (int c0 = 0; c0 < d; c0 += 64) {
+        if (c0 + 64 < d) {
+            fetch(c0 + 64, nxt);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            float *p = &tile[wave][rsub + 4 * t][4 * cg];
+            p[0] = cur[t].x;
+            p[1] = cur[t].y;
+            p[2] = cur[t].z;
+            p[3] = cur[t].w;
+        }
+        wave_lds_fence();
+        if (lane < 16) {
+            const int cols = d - c0 < 64 ? d - c0 : 64;
+            for (int j = 0; j < cols; j++) {
+                const float v = tile[wave][lane][j];
+                s = __fadd_rn(s, __fmul_rn(v, v));
+            }
+        }
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            cur[t] = nxt[t];
+        }
+    }
+    if (lane < 16 && row0 + lane < n) {
+        out[row0 + lane] = s;
+    }
+}
+
 void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_t s)
 {
     if (n == 0) {
         return;
     }
-    hipLaunchKernelGGL(sqnorm_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, d, out);
+    if (d % 4 == 0 && d >= 32 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        hipLaunchKernelGGL(sqnorm_rows_tiled_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, s, x, n, d, out);
+    } else {
+        hipLaunchKernelGGL(sqnorm_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, d, out);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
