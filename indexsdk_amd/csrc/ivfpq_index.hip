@@ -107,6 +107,25 @@ __global__ __launch_bounds__(256) void gather_list_kernel(const uint8_t *__restr
 }
 
 // out rows idx[i] <- rows i of the compact results (ids, and distances when given)
+// out[c][t] = float( sum in float64, in list order, of x[order[i]][t] over the members i of segment c
+// / their number ); segments without members keep old[c][t].  One workgroup per segment, one thread
+// per component: the additions of a component happen in one fixed order.
+__global__ __launch_bounds__(256) void segment_mean_kernel(const float *__restrict__ x, int d,
+                                                           const int64_t *__restrict__ order,
+                                                           const int64_t *__restrict__ seg,
+                                                           const float *__restrict__ old, float *__restrict__ out)
+{
+    const int64_t c = blockIdx.x;
+    const int64_t b = seg[c], e = seg[c + 1];
+    for (int t = threadIdx.x; t < d; t += blockDim.x) {
+        double acc = 0.0;
+        for (int64_t i = b; i < e; i++) {
+            acc += (double)x[order[i] * d + t];
+        }
+        out[c * d + t] = e > b ? (float)(acc / (double)(e - b)) : old[c * d + t];
+    }
+}
+
 __global__ __launch_bounds__(256) void scatter_rows_kernel(const int32_t *__restrict__ ids, const float *__restrict__ dist,
                                                            const int64_t *__restrict__ idx, int64_t n, int width,
                                                            int32_t *__restrict__ out_ids, float *__restrict__ out_dist)
@@ -815,9 +834,11 @@ const SearchStats &IvfpqIndex::stats()
 // -------------------------------------------------------------------------------------------------
 // Training.  The reference delegates to faiss::Clustering (CPU mode) or runs device assignment with
 // a host centroid update (NPU mode: FR/ascendhost/src/impl/AscendClusteringImpl.cpp:686-762); this
-// build does the latter: assignment on the GPU (stage-1 kernels, PQ encode kernel), centroid update
-// on the host in float64.  Sampling follows computeTrainTotalSize / sampleTrainData
-// (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:51-112).  Plain Lloyd unless cfg.spherical.
+// build does the latter: assignment on the GPU (stage-1 kernels, PQ encode kernel); the coarse centroid
+// update also runs on the GPU (float64 sums in sample order, so the result does not depend on the
+// hardware's scheduling), the sub-quantizer update on the host in float64.  Sampling follows
+// computeTrainTotalSize / sampleTrainData (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:51-112).  Plain Lloyd
+// unless cfg.spherical.
 
 void IvfpqIndex::train(int64_t n, const float *x, bool on_device)
 {
@@ -910,30 +931,32 @@ void IvfpqIndex::kmeans_coarse(const std::vector<float> &sample, int64_t ns)
     xs.upload(sample.data(), sample.size(), stream_);
     DeviceBuffer<int32_t> asg((size_t)ns);
     std::vector<int32_t> h_asg((size_t)ns);
-    std::vector<double> acc((size_t)nlist_ * d_);
-    std::vector<int64_t> cnt((size_t)nlist_);
+    std::vector<int64_t> cnt((size_t)nlist_), seg((size_t)nlist_ + 1), order((size_t)ns);
+    DeviceBuffer<int64_t> order_dev, seg_dev;
+    DeviceBuffer<float> mean_dev((size_t)nlist_ * d_);
     for (int it = 0; it < cfg_.niter; it++) {
         upload_trained(cent.data(), nullptr);
         coarse_select(xs.data(), ns, 1, kMetricL2, asg.data(), nullptr);
         asg.download(h_asg.data(), (size_t)ns, stream_);
-        std::fill(acc.begin(), acc.end(), 0.0);
+        // members of every cluster in sample order (stable counting sort on the host); the means are
+        // then float64 sums in exactly that order, one workgroup per centroid on the device
         std::fill(cnt.begin(), cnt.end(), 0);
         for (int64_t i = 0; i < ns; i++) {
-            const int64_t a = h_asg[(size_t)i];
-            cnt[(size_t)a]++;
-            double *dst = &acc[(size_t)a * d_];
-            const float *src = &sample[(size_t)i * d_];
-            for (int t = 0; t < d_; t++) {
-                dst[t] += src[t];
-            }
+            cnt[(size_t)h_asg[(size_t)i]]++;
         }
+        seg[0] = 0;
         for (int64_t c = 0; c < nlist_; c++) {
-            if (cnt[(size_t)c] > 0) {
-                for (int t = 0; t < d_; t++) {
-                    cent[(size_t)c * d_ + t] = (float)(acc[(size_t)c * d_ + t] / (double)cnt[(size_t)c]);
-                }
-            }
+            seg[(size_t)c + 1] = seg[(size_t)c] + cnt[(size_t)c];
         }
+        std::vector<int64_t> fill(seg.begin(), seg.end() - 1);
+        for (int64_t i = 0; i < ns; i++) {
+            order[(size_t)fill[(size_t)h_asg[(size_t)i]]++] = i;
+        }
+        order_dev.upload(order.data(), order.size(), stream_);
+        seg_dev.upload(seg.data(), seg.size(), stream_);
+        hipLaunchKernelGGL(segment_mean_kernel, dim3((unsigned)nlist_), dim3(d_ <= 64 ? 64 : (d_ <= 128 ? 128 : 256)), 0,
+                           stream_, xs.data(), d_, order_dev.data(), seg_dev.data(), centroids_.data(), mean_dev.data());
+        mean_dev.download(cent.data(), cent.size(), stream_);
         split_empty(cent, cnt, nlist_, d_);
         if (cfg_.spherical) {
             normalise_rows(cent, nlist_, d_);
