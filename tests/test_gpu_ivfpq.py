@@ -391,3 +391,15 @@ def test_reset_keeps_quantizers_and_readd_reproduces_codes(ix, oracle):
         assert np.array_equal(c0, c1) and np.array_equal(i0, i1)
     D1, I1 = gpu.search(q, 7)
     assert np.array_equal(I0, I1) and np.array_equal(D0.view(np.uint32), D1.view(np.uint32))
+
+
+def test_maximum_k_and_every_list_probed(ix, oracle):
+    """k at the library's limit (2048) with nprobe = nlist: every vector is a candidate for every query."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 91, 6000, 12, 64, 32, 16, ix.METRIC_L2)
+    gpu.setNumProbes(32)
+    D, I = gpu.search(q, 2048)
+    Dr, Ir = ref.search(q, 2048, 32)
+    assert gpu.last_search_stats()["scanned_codes"] == 12 * 6000
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    with pytest.raises(ix.IndexSdkError):
+        gpu.search(q, 2049)
