@@ -246,7 +246,12 @@ def main():
     # 12.2 MB are written.  Only quoted for the default workload it was measured on.
     default_c2 = args.workload == "C2" and not any(getattr(args, key) for key in ("n", "nq", "nlist", "nprobe", "k"))
     traffic = 1.030 * scan_bytes + 12.2e6 if default_c2 else None
-    layout_name = "rot32" if (args.layout != 0 and M in (32, 64, 96)) else "row"
+    if args.layout in (-1, 1) and M in (32, 64, 96):
+        layout_name = "rot32"
+    elif args.layout in (-1, 2) and M == 48 and not w["lut_fp16"]:
+        layout_name = "xor48"
+    else:
+        layout_name = "row"
     result = {
         "metric": "queries/sec and ADC-scan GB/s (% HBM peak) at k=100 on 1 MI355X",
         "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

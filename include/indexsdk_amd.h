@@ -70,7 +70,8 @@ typedef struct ivfpq_config {
     int32_t train_samples_per_list; /* trainSamplesPerList */
     int64_t max_train_samples;      /* maxTrainSamples */
     int32_t lut_fp16;               /* 1 = store the per-query LUT as IEEE half (accumulate in fp32) */
-    int32_t code_layout;            /* -1 = choose, 0 = row-major codes, 1 = bank-rotated (M in {32,64,96}) */
+    int32_t code_layout;            /* -1 = choose, 0 = row-major codes, 1 = bank-rotated (M in {32,64,96}),
+                                       2 = xor-rotated (M = 48, fp32 LUT) */
     int64_t scratch_bytes;          /* resourceSize: bound of the coarse-score scratch in HBM */
     uint64_t seed;                  /* sampling / initialisation seed */
     int32_t strict_reference_params;/* 1 = enforce the reference whitelists d in {128}, nlist in

@@ -17,7 +17,7 @@ struct IvfpqConfig {
     int train_samples_per_list = 256; // rows sampled per coarse centroid (trainSamplesPerList)
     int64_t max_train_samples = 10000000;  // maxTrainSamples
     int lut_fp16 = 0;                 // LUT entries stored as IEEE half
-    int code_layout = -1;             // -1 = pick (rot32 when M % 32 == 0), 0 = row, 1 = rot32
+    int code_layout = -1;             // -1 = pick, 0 = row, 1 = rot32 (M in {32, 64, 96}), 2 = xor48 (M = 48)
     int64_t scratch_bytes = (int64_t)1 << 30;  // budget of the coarse score scratch
     uint64_t seed = 1234;
     int strict_reference_params = 0;  // 1 = enforce the reference's d / nlist / M whitelists

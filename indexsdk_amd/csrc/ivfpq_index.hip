@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void scatter_new_kernel(int64_t n, const int32
     const uint8_t *src = codes_in + i * M;
     uint8_t *dst = codes + slot * M;
     for (int j = 0; j < M; j++) {
-        const int m = layout == 1 ? ((j & ~31) | ((j + p) & 31)) : j;
+        const int m = layout == 1 ? ((j & ~31) | ((j + p) & 31)) : (layout == 2 ? xor48_sq_of_byte(j, p) : j);
         dst[j] = src[m];
     }
     ids[slot] = ids_in ? ids_in[i] : id_base + i;
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void gather_list_kernel(const uint8_t *__restr
     }
     const int p = (int)(e / M), m = (int)(e % M);
     // sub-quantizer m of position p is stored at byte j with (j + p) % 32 == m % 32 inside its 32-block
-    const int j = layout == 1 ? ((m & ~31) | ((m - p) & 31)) : m;
+    const int j = layout == 1 ? ((m & ~31) | ((m - p) & 31)) : (layout == 2 ? xor48_byte_of_sq(m, p) : m);
     out[e] = codes[(off + p) * M + j];
 }
 
@@ -176,7 +176,11 @@ IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const
         IXA_REQUIRE(M == 32 || M == 64 || M == 96, kErrInvalidParam,
                     "code layout rot32 needs msubs in {32, 64, 96}, got %d", M);
     }
-    layout_ = cfg.code_layout >= 0 ? cfg.code_layout : ((M == 32 || M == 64 || M == 96) ? 1 : 0);
+    if (cfg.code_layout == 2) {
+        IXA_REQUIRE(M == 48 && !cfg.lut_fp16, kErrInvalidParam, "code layout xor48 needs msubs = 48 and an fp32 LUT");
+    }
+    layout_ = cfg.code_layout >= 0 ? cfg.code_layout
+                                   : ((M == 32 || M == 64 || M == 96) ? 1 : ((M == 48 && !cfg.lut_fp16) ? 2 : 0));
     nprobe_ = (int)std::min<int64_t>(64, nlist);
     int ndev = 0;
     hipError_t e = hipGetDeviceCount(&ndev);

@@ -4,6 +4,15 @@
 
 namespace ixa {
 
+// Code layout 2 ("xor48", M = 48, fp32 LUT): byte j of the slot at list position p holds sub-quantizer
+//   j < 32:  (j ^ p) & 31              (the 32 lanes of a half wavefront read 32 different ones)
+//   j >= 32: 32 + ((j ^ p) & 15)       (16 different ones; lanes 0..15 and 16..31 read two LUT copies)
+// The LUT row of a codeword is 64 words: sub-quantizers 0..31, then 32..47 twice.  A lane's word in
+// the row is then (c ^ (p & 31)) + block offset with a per-step constant c, whatever the code value:
+// conflict-free, and no table of rotation offsets has to live in registers.
+__host__ __device__ inline int xor48_sq_of_byte(int j, int p) { return j < 32 ? ((j ^ p) & 31) : 32 + ((j ^ p) & 15); }
+__host__ __device__ inline int xor48_byte_of_sq(int m, int p) { return m < 32 ? ((m ^ p) & 31) : 32 + ((m ^ p) & 15); }
+
 struct ScanParams {
     // query side
     const float *queries;      // [nq][d]
@@ -19,7 +28,7 @@ struct ScanParams {
     const int64_t *ids;
     const int64_t *list_off;   // first slot of each list
     const int32_t *list_len;   // valid entries of each list
-    int code_layout;           // 0 = row, 1 = rot32
+    int code_layout;           // 0 = row, 1 = rot32, 2 = xor48
     // selection
     int k;
     int nsplit;                // workgroups per query; > 1 needs `partial`

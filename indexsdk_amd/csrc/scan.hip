@@ -49,6 +49,8 @@ __device__ __forceinline__ float from_lut(__half v) { return __half2float(v); }
 // sub-quantizer r of the even block (low half) and of the odd block (high half).  A last unpaired
 // block pairs codewords instead: row kk / 2, half kk % 2.  Either way a lane's word index is
 // (row * 32 + r) and r is distinct across the 32 lanes: no bank conflicts for any code values.
+// (Giving the unpaired block 32 KB of its own with fp32 words makes every address one shift-add,
+// but the larger LUT costs a resident workgroup at M = 96: measured slower.)
 __host__ __device__ __forceinline__ int rot32_half_slot(int nblocks, int m, int kk)
 {
     const int b = m >> 5, r = m & 31;
@@ -161,11 +163,19 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             } else {
                 v = -ip;  // minimise the negated inner product
             }
-            int slot = LAYOUT == 1 ? kk * M + m : m * 256 + kk;
-            if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
-                slot = rot32_half_slot(M / 32, m, kk);
+            if constexpr (LAYOUT == 2) {
+                // xor48: rows of 64 words per codeword; sub-quantizers 32..47 are stored twice
+                lut[kk * 64 + m] = to_lut<LutT>(v);
+                if (m >= 32) {
+                    lut[kk * 64 + m + 16] = to_lut<LutT>(v);
+                }
+            } else {
+                int slot = LAYOUT == 1 ? kk * M + m : m * 256 + kk;
+                if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
+                    slot = rot32_half_slot(M / 32, m, kk);
+                }
+                lut[slot] = to_lut<LutT>(v);
             }
-            lut[slot] = to_lut<LutT>(v);
         }
     }
     __syncthreads();
@@ -239,13 +249,17 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
         }
     };
 
-    // byte offset of this lane's word in a 32-word LUT row at each of the 32 rotation steps; kept
-    // in registers (opaque to the optimiser, which would otherwise recompute them per lookup)
+    // LDS address of this lane's word in the first 32-word LUT row at each of the 32 rotation steps;
+    // kept in registers (opaque to the optimiser, which would otherwise recompute them per lookup),
+    // so that a lookup's address is one shift-add of the code
+    typedef __attribute__((address_space(3))) const uint16_t lds_half_t;
     uint32_t rot4[32];
     if constexpr (LAYOUT == 1 && sizeof(LutT) == 2) {
+        const uint32_t lut_base =
+            (uint32_t) reinterpret_cast<size_t>((__attribute__((address_space(3))) const unsigned char *)lut);
 #pragma unroll
         for (int j = 0; j < 32; j++) {
-            rot4[j] = (uint32_t)((j + l32) & 31) << 2;
+            rot4[j] = lut_base + ((uint32_t)((j + l32) & 31) << 2);
             asm volatile("" : "+v"(rot4[j]));
         }
     }
@@ -263,7 +277,6 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             // one v_fma_mix_f32 (half * 1.0 + fp32 accumulator: the same value as convert-then-add)
             constexpr int NB = MT / 32;
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
-            const unsigned char *lb = reinterpret_cast<const unsigned char *>(lut);
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 const uint32_t ww = w[(m >> 2) % NW];
@@ -271,14 +284,30 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
                 const uint32_t r4 = rot4[m & 31];
                 uint32_t off;
                 if (b < (NB & ~1)) {
-                    const uint32_t code = (ww >> (8 * (m & 3))) & 0xffu;
-                    off = ((code << 7) | r4) + (uint32_t)((b >> 1) * 32768 + 2 * (b & 1));
+                    uint32_t code = (ww >> (8 * (m & 3))) & 0xffu;
+                    asm("" : "+v"(code));   // keep extract-then-shift-add (two instructions for every byte)
+                    off = ((code << 7) + r4) + (uint32_t)((b >> 1) * 32768 + 2 * (b & 1));
                 } else {
                     const uint32_t c1 = (ww >> (8 * (m & 3) + 1)) & 0x7fu, c0 = (ww >> (8 * (m & 3))) & 1u;
-                    off = (((c1 << 7) | r4) | (c0 << 1)) + (uint32_t)((NB >> 1) * 32768);
+                    off = (((c1 << 7) + r4) + (c0 << 1)) + (uint32_t)((NB >> 1) * 32768);
                 }
-                const uint32_t raw = *reinterpret_cast<const uint16_t *>(lb + off);
+                const uint32_t raw = *(lds_half_t *)off;
                 asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(acc[m & 3]) : "v"(raw));
+            }
+            return (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        } else if constexpr (LAYOUT == 2) {
+            // xor48: byte address = (code << 8) + ((4 * l32) ^ (4 * c)) + block offset, c the step's
+            // constant: one byte permute (code into bits 8..15), one xor-add, one fp add per lookup
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            const unsigned char *lb = reinterpret_cast<const unsigned char *>(lut);
+            const uint32_t x4 = (uint32_t)l32 << 2;
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const uint32_t ww = w[(m >> 2) % NW];
+                const uint32_t code8 = __builtin_amdgcn_perm(0u, ww, 0x0c0c000cu | ((uint32_t)(m & 3) << 8));
+                const uint32_t c4 = (uint32_t)(m < 32 ? m : (m & 15)) << 2;
+                const uint32_t off = (x4 ^ c4) + code8 + (m < 32 ? 0u : 128u);
+                acc[m & 3] += *reinterpret_cast<const float *>(lb + off);
             }
             return (acc[0] + acc[1]) + (acc[2] + acc[3]);
         } else if (LAYOUT == 1) {
@@ -286,7 +315,8 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int m = 0; m < MT; m++) {
-                const uint32_t code = (w[(m >> 2) % NW] >> (8 * (m & 3))) & 0xffu;
+                uint32_t code = (w[(m >> 2) % NW] >> (8 * (m & 3))) & 0xffu;
+                asm("" : "+v"(code));   // keep extract-then-shift-add (two instructions for every byte)
                 const int mm = (m & ~31) | ((m + l32) & 31);
                 acc[m & 3] += from_lut(lut[code * MT + mm]);
             }
@@ -467,7 +497,14 @@ template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
     const int64_t slots = p.xcd_chunks ? (nq + 7) / 8 * 8 : nq;
-    if (p.shared_pool) {
+    if (p.shared_pool && p.waves == 16) {
+        auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 16, true>;
+        if (smem > 48 * 1024) {
+            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(1024), smem, s, p);
+    } else if (p.shared_pool) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, true>;
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -494,6 +531,14 @@ static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
 template <typename LutT>
 static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
+    if (p.code_layout == 2) {
+        if constexpr (sizeof(LutT) == 4) {
+            if (p.M == 48) {
+                return launch_one<48, LutT, 2>(p, nq, smem, s);
+            }
+        }
+        fail(kErrInner, "xor48 code layout needs M = 48 and an fp32 LUT");
+    }
     if (p.code_layout == 1) {
         switch (p.M) {
             case 32: return launch_one<32, LutT, 1>(p, nq, smem, s);
@@ -516,7 +561,10 @@ static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
 
 static size_t plan_with_waves(ScanParams &p, int waves, bool shared)
 {
-    const size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
+    size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
+    if (p.code_layout == 2) {
+        lut_bytes = (size_t)64 * 256 * 4;
+    }
     p.waves = waves;
     p.shared_pool = shared ? 1 : 0;
     p.cap = shared ? block_pool_capacity(p.k, waves) : wave_pool_capacity(p.k);
@@ -545,7 +593,8 @@ static int resident_waves(size_t smem, int waves)
 }
 
 // Private pools with eight wavefronts per workgroup when three such workgroups fit the 160 KB of
-// a CU; otherwise whichever of {private x 8, private x 4, shared x 8} keeps most wavefronts resident.
+// a CU; otherwise whichever of {private x 8, private x 4, shared x 8, shared x 16} keeps most
+// wavefronts resident (earlier in that list on ties).
 size_t plan_scan(ScanParams &p)
 {
     ScanParams best = p;
@@ -555,14 +604,19 @@ size_t plan_scan(ScanParams &p)
         return best_smem;
     }
     int best_waves = best_smem <= 160 * 1024 ? resident_waves(best_smem, 8) : 0;
-    const bool shared_ok = block_pool_capacity(p.k, 8) <= 8 * 8 * kWave;
-    for (int alt = 0; alt < 2; alt++) {
-        if (alt == 1 && !shared_ok) {
+    const struct {
+        int waves;
+        bool shared;
+    } alts[] = {{4, false}, {8, true}, {16, true}};
+    for (const auto &alt : alts) {
+        if (alt.shared && block_pool_capacity(p.k, alt.waves) > (alt.waves >= 16 ? 4 : 8) * alt.waves * kWave) {
             continue;
         }
         ScanParams q = p;
-        const size_t smem = alt == 0 ? plan_with_waves(q, 4, false) : plan_with_waves(q, 8, true);
-        const int rw = smem <= 160 * 1024 ? resident_waves(smem, alt == 0 ? 4 : 8) : 0;
+        const size_t smem = plan_with_waves(q, alt.waves, alt.shared);
+        // a shared-pool workgroup keeps its CU to itself: those kernels need more than the 64
+        // registers per lane that a second resident workgroup would leave them
+        const int rw = smem <= 160 * 1024 ? (alt.shared ? alt.waves : resident_waves(smem, alt.waves)) : 0;
         if (rw > best_waves) {
             best = q;
             best_smem = smem;

@@ -351,7 +351,7 @@ struct BlockPoolCtl {
 template <int W>
 struct BlockPool {
     static constexpr int NT = W * kWave;
-    static constexpr int kMaxPerThread = 8;   // cap <= 8 * NT
+    static constexpr int kMaxPerThread = W >= 16 ? 4 : 8;   // cap <= kMaxPerThread * NT
     key_t *buf;
     int *hist;                 // 1024 ints
     volatile BlockPoolCtl *ctl;

@@ -292,6 +292,50 @@ def test_large_k_shared_pool_one_workgroup_per_query(ix, oracle):
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
 
 
+@pytest.mark.parametrize("d,M,layout,waves", [(96, 48, 2, 16), (96, 48, 0, 16), (128, 64, 1, 16), (128, 64, 0, 16),
+                                              (64, 32, 1, 16), (128, 128, 0, 8)])
+def test_large_k_shared_pool_layouts_and_workgroup_sizes(ix, oracle, d, M, layout, waves):
+    """The workgroup-wide pool under every code layout, with the workgroup size the LDS plan picks for
+    it (sixteen wavefronts unless the LUT leaves no room for their larger pool)."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 45 + M + layout, 30000, 2100, d, 16, M, ix.METRIC_L2, layout=layout)
+    gpu.setNumProbes(8)
+    D, I = gpu.search(q, 1024)
+    st = gpu.last_search_stats()
+    assert st["shared_pool"] == 1 and st["nsplit"] == 1 and st["scan_waves"] == waves
+    sub = slice(0, 2100, 7)
+    Dr, Ir = ref.search(q[sub], 1024, 8)
+    assert_topk_parity(oracle, ref, q[sub], D[sub], I[sub], Dr, Ir, TOL_FP32)
+
+
+def test_xor48_layout_is_the_default_for_m48_and_lists_read_back_in_row_order(ix, oracle):
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 47, 20000, 64, 96, 32, 48, ix.METRIC_L2)
+    row, _, _, _, _ = build_pair(ix, oracle, 47, 20000, 64, 96, 32, 48, ix.METRIC_L2, layout=0)
+    for l in range(32):
+        c_a, i_a = gpu.getListCodesAndIds(l)
+        c_b, i_b = row.getListCodesAndIds(l)
+        assert np.array_equal(c_a, c_b) and np.array_equal(i_a, i_b)
+    gpu.setNumProbes(8)
+    row.setNumProbes(8)
+    D, I = gpu.search(q, 50)
+    D0, I0 = row.search(q, 50)
+    Dr, Ir = ref.search(q, 50, 8)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    assert_topk_parity(oracle, ref, q, D0, I0, Dr, Ir, TOL_FP32)
+    # removal and a second add keep the position-dependent byte order consistent
+    gone = ids[::3]
+    assert gpu.remove_ids(gone) == len(gone) and row.remove_ids(gone) == len(gone)
+    extra = np.arange(10 ** 7, 10 ** 7 + 500, dtype=np.int64)
+    gpu.add_with_ids(x[:500], extra)
+    row.add_with_ids(x[:500], extra)
+    for l in range(32):
+        c_a, i_a = gpu.getListCodesAndIds(l)
+        c_b, i_b = row.getListCodesAndIds(l)
+        assert np.array_equal(c_a, c_b) and np.array_equal(i_a, i_b)
+    D, I = gpu.search(q, 50)
+    D0, I0 = row.search(q, 50)
+    assert (I == I0).mean() > 0.99 and np.allclose(D, D0, rtol=TOL_FP32, atol=0)
+
+
 def test_large_k_shared_pool_all_scores_tie(ix, oracle):
     """A base of few distinct vectors: whole lists share one distance, so the bucket search cannot
     separate candidates and the pool falls back to exact selection by sorting."""
