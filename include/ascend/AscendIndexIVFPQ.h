@@ -187,5 +187,21 @@ protected:
     int nlist_, msubs_;
 };
 
+// AscendIndexImpl::mergeSearchResult (FR/ascend/impl/AscendIndexImpl.cpp:587-640) for callers that
+// shard an index over several devices themselves: dist[j] / label[j] hold the [n][k] results of shard j.
+inline void mergeSearchResult(const std::vector<std::vector<float>> &dist,
+                              const std::vector<std::vector<idx_t>> &label, idx_t n, idx_t k, MetricType metric,
+                              float *distances, idx_t *labels)
+{
+    std::vector<const float *> dp;
+    std::vector<const int64_t *> lp;
+    for (size_t j = 0; j < dist.size(); j++) {
+        dp.push_back(dist[j].data());
+        lp.push_back(reinterpret_cast<const int64_t *>(label[j].data()));
+    }
+    ixaThrowIfError(ixa_merge_search_results((int)dist.size(), n, k, (int)metric, dp.data(), lp.data(), distances,
+                                             reinterpret_cast<int64_t *>(labels)));
+}
+
 }  // namespace ascend
 }  // namespace faiss

@@ -53,6 +53,14 @@ const char *ixa_last_error(void);
  * counters (FETCH_SIZE / WRITE_SIZE) of the search kernels are scaled by. */
 int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes);
 
+/* AscendIndexImpl::mergeSearchResult  FR/ascend/impl/AscendIndexImpl.cpp:587-640: merges the result
+ * lists that `ndev` devices (or index shards) returned for the same n queries into one list of k per
+ * query.  dist[j] / labels[j]: HOST arrays [n][k] of device j, best first.  Entries with label -1 are
+ * skipped wherever they stand, equal distances go to the lower j, and lists that run out are padded
+ * with (FLT_MAX, -1).  Host code, as in the reference; touches no GPU. */
+int ixa_merge_search_results(int ndev, int64_t n, int64_t k, int metric, const float *const *dist,
+                             const int64_t *const *labels, float *distances, int64_t *out_labels);
+
 /* ---------------------------------------------------------------------------------------------
  * IVFPQ
  * ------------------------------------------------------------------------------------------- */

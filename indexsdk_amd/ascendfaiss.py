@@ -210,6 +210,21 @@ class AscendIndexIVFPQ:
         return {n: getattr(s, n) for n, _ in s._fields_}
 
 
+def merge_search_results(distances, labels, metric=METRIC_L2):
+    """AscendIndexImpl::mergeSearchResult (FR/ascend/impl/AscendIndexImpl.cpp:587-640): merges the
+    [n, k] result lists of several devices or shards (sequences of arrays, best first) into one."""
+    dist = [_as(a, np.float32, 2, "distances") for a in distances]
+    lab = [_as(a, np.int64, 2, "labels") for a in labels]
+    assert len(dist) == len(lab) >= 1 and all(a.shape == dist[0].shape for a in dist + lab)
+    n, k = dist[0].shape
+    out_d = np.empty((n, k), dtype=np.float32)
+    out_l = np.empty((n, k), dtype=np.int64)
+    dp = (ctypes.c_void_p * len(dist))(*[a.ctypes.data for a in dist])
+    lp = (ctypes.c_void_p * len(lab))(*[a.ctypes.data for a in lab])
+    _capi.check(_capi.load().ixa_merge_search_results(len(dist), n, k, metric, dp, lp, _ptr(out_d), _ptr(out_l)))
+    return out_d, out_l
+
+
 class _FlatCommon:
     _pfx = None
     _dtype = None

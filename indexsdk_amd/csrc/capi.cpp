@@ -336,6 +336,54 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
 IXA_FLAT_COMMON(flat, flat_index_t, float)
 IXA_FLAT_COMMON(flat_i8, flat_i8_index_t, int8_t)
 
+IXA_EXPORT int ixa_merge_search_results(int ndev, int64_t n, int64_t k, int metric, const float *const *dist,
+                                        const int64_t *const *labels, float *distances, int64_t *out_labels)
+{
+    return guarded([&] {
+        IXA_REQUIRE(ndev >= 1 && n >= 0 && k >= 1, ixa::kErrInvalidParam, "ndev and k must be >= 1 and n >= 0");
+        IXA_REQUIRE(metric == ixa::kMetricL2 || metric == ixa::kMetricInnerProduct, ixa::kErrInvalidParam, "Unsupported metric type");
+        IXA_REQUIRE(dist && labels && distances && out_labels, ixa::kErrInvalidParam, "result arrays can not be nullptr.");
+        for (int j = 0; j < ndev; j++) {
+            IXA_REQUIRE(dist[j] && labels[j], ixa::kErrInvalidParam, "result arrays can not be nullptr.");
+        }
+        const bool smaller_wins = metric == ixa::kMetricL2;
+        std::vector<int64_t> cursor((size_t)ndev);
+        for (int64_t q = 0; q < n; q++) {
+            const int64_t row = q * k;
+            // a cursor always rests on a valid entry of its list, or on k
+            auto settle = [&](int j) {
+                while (cursor[j] < k && labels[j][row + cursor[j]] == -1) {
+                    cursor[j]++;
+                }
+            };
+            for (int j = 0; j < ndev; j++) {
+                cursor[j] = 0;
+                settle(j);
+            }
+            for (int64_t out = 0; out < k; out++) {
+                int from = -1;
+                for (int j = 0; j < ndev; j++) {
+                    if (cursor[j] >= k) {
+                        continue;
+                    }
+                    const float v = dist[j][row + cursor[j]];
+                    if (from < 0 || (smaller_wins ? v < dist[from][row + cursor[from]] : v > dist[from][row + cursor[from]])) {
+                        from = j;
+                    }
+                }
+                if (from < 0) {
+                    distances[row + out] = 3.402823466e+38f;
+                    out_labels[row + out] = -1;
+                    continue;
+                }
+                distances[row + out] = dist[from][row + cursor[from]];
+                out_labels[row + out] = labels[from][row + cursor[from]];
+                cursor[from]++;
+                settle(from);
+            }
+        }
+    });
+}
 IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
 {
     return guarded([&] { ixa::launch_copy_probe(src_dev, dst_dev, bytes); });

@@ -23,6 +23,9 @@
  *                                       (FR/test/aicpu/test_topk_flat.cc:52-187)
  *   orc_flat_i8 ....................... exact integer closed form vs int64 numpy
  *   orc_flat_f32 ...................... closed form vs float64 numpy + full sort
+ *   orc_merge_results ................. stable sort of the device-major concatenation (what a k-way
+ *                                       merge with a strict comparison must equal), hand-made case
+ *                                       with invalid labels in the middle of a list
  *   orc_kmeans ........................ PARITY UNPINNED against faiss::Clustering (faiss is absent);
  *                                       only Lloyd invariants (objective non-increasing) are checked.
  *                                       Search parity is judged on shared, injected codebooks.
@@ -617,6 +620,53 @@ ORC_API double orc_kmeans(const float *x, int64_t n, int d, int64_t kc, int nite
     free(acc);
     free(cnt);
     return obj;
+}
+
+/* Merge of the per-device result lists of one search: FR/ascend/impl/AscendIndexImpl.cpp:587-640.
+ * dist/labels: [ndev][n][k], every list best first.  Entries whose label is -1 (or all ones) are
+ * skipped wherever they stand; a strict comparison picks the winner, so equal distances go to the
+ * lower device; exhausted lists pad with (FLT_MAX, -1) for both metrics. */
+ORC_API void orc_merge_results(int ndev, const float *dist, const int64_t *labels, int64_t n, int64_t k, int metric,
+                               float *out_dist, int64_t *out_labels)
+{
+    int64_t *posit = (int64_t *)malloc((size_t)ndev * sizeof(int64_t));
+    for (int64_t i = 0; i < n; i++) {
+        const int64_t offset = i * k;
+        for (int j = 0; j < ndev; j++) {
+            posit[j] = 0;
+        }
+        for (int64_t num = 0; num < k; num++) {
+            int id = ndev;
+            float best = FLT_MAX;
+            int64_t best_label = -1;
+            for (int j = 0; j < ndev; j++) {
+                const float *dj = dist + (int64_t)j * n * k;
+                const int64_t *lj = labels + (int64_t)j * n * k;
+                while (posit[j] < k && lj[offset + posit[j]] == -1) {
+                    posit[j]++;
+                }
+                if (posit[j] >= k) {
+                    continue;
+                }
+                const float v = dj[offset + posit[j]];
+                const int wins = metric == ORC_METRIC_L2 ? (v < best) : (v > best);
+                if (id == ndev || wins) {
+                    best = v;
+                    best_label = lj[offset + posit[j]];
+                    id = j;
+                }
+            }
+            if (id == ndev) {
+                out_dist[offset + num] = FLT_MAX;
+                out_labels[offset + num] = -1;
+            } else {
+                out_dist[offset + num] = best;
+                out_labels[offset + num] = best_label;
+                posit[id]++;
+            }
+        }
+    }
+    free(posit);
 }
 
 ORC_API int orc_num_threads(void)

@@ -203,6 +203,18 @@ def flat_i8(base, q, k, ids=None):
     return dist, labels
 
 
+def merge_results(dist, labels, metric=METRIC_L2):
+    """dist/labels: [ndev][n][k] per-device result lists -> merged ([n][k], [n][k])."""
+    dist = _f32(dist)
+    labels = np.ascontiguousarray(labels, dtype=np.int64)
+    ndev, n, k = dist.shape
+    out_d = np.empty((n, k), dtype=np.float32)
+    out_l = np.empty((n, k), dtype=np.int64)
+    lib().orc_merge_results(ctypes.c_int(ndev), _p(dist, _c_f32p), _p(labels, _c_i64p), ctypes.c_int64(n),
+                            ctypes.c_int64(k), ctypes.c_int(metric), _p(out_d, _c_f32p), _p(out_l, _c_i64p))
+    return out_d, out_l
+
+
 def kmeans(x, k, niter=25, spherical=False, seed=1234):
     x = _f32(x)
     cent = np.empty((k, x.shape[1]), dtype=np.float32)

@@ -42,6 +42,17 @@ int main(int argc, char **argv)
         EXPECT(m.find("Unsupported msubs") != std::string::npos);
     }
     EXPECT(construct_msg(128, 1024, 4, 4).find("Unsupported nbits") != std::string::npos);
+    {
+        // merge of two shards' results (FR/ascend/impl/AscendIndexImpl.cpp:587-640): invalid labels are
+        // skipped, equal distances go to the lower shard, short results are padded
+        std::vector<std::vector<float>> dist = {{1.f, 2.f, 5.f}, {2.f, 3.f, 4.f}};
+        std::vector<std::vector<faiss::idx_t>> label = {{7, -1, 9}, {20, 21, -1}};
+        float out_d[3];
+        faiss::idx_t out_l[3];
+        mergeSearchResult(dist, label, 1, 3, faiss::METRIC_L2, out_d, out_l);
+        EXPECT(out_l[0] == 7 && out_l[1] == 20 && out_l[2] == 21);
+        EXPECT(out_d[0] == 1.f && out_d[1] == 2.f && out_d[2] == 3.f);
+    }
     if (argc > 1 && std::strcmp(argv[1], "gpu") == 0) {
         const int d = 128, nlist = 1024, M = 16, n = 40000, nq = 16, k = 5;
         std::mt19937 gen(1);

@@ -1,6 +1,7 @@
 """Host-only checks of the C ABI: the library loads, exports every symbol the header declares,
 validates constructor parameters with the reference's messages, and refuses to run without a GPU
-(no CPU fallback).  No compute entry point is called here."""
+(no CPU fallback).  No search/add/train entry point is called here; the merge of per-device result
+lists is host code in the reference too and is checked against the oracle."""
 import ctypes
 import os
 import re
@@ -100,3 +101,28 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".h", ".hip", ".cpp", ".sh")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+# FR/ascend/impl/AscendIndexImpl.cpp:587-640: the merge of per-device results is host code in the
+# reference and here; it is the one entry point that computes without a GPU.
+@pytest.mark.parametrize("metric_l2,ndev,holes", [(True, 1, 0.0), (True, 4, 0.3), (False, 3, 0.2), (True, 2, 1.0)])
+def test_merge_search_results_matches_the_oracle(capi, oracle, metric_l2, ndev, holes):
+    import numpy as np
+    import indexsdk_amd as ix
+    rng = np.random.default_rng(11 + ndev)
+    n, k = 300, 33
+    d = np.sort(np.round(rng.standard_normal((ndev, n, k)) * 4).astype(np.float32) / 4, axis=2)
+    if not metric_l2:
+        d = d[:, :, ::-1].copy()
+    lab = rng.permutation(ndev * n * k).reshape(ndev, n, k).astype(np.int64)
+    lab[rng.random(lab.shape) < holes] = -1
+    metric = ix.METRIC_L2 if metric_l2 else ix.METRIC_INNER_PRODUCT
+    got_d, got_l = ix.merge_search_results(list(d), list(lab), metric)
+    want_d, want_l = oracle.merge_results(d, lab, metric)
+    assert np.array_equal(got_l, want_l) and np.array_equal(got_d.view(np.uint32), want_d.view(np.uint32))
+
+
+def test_merge_search_results_rejects_bad_arguments(capi):
+    lib = capi.load()
+    rc = lib.ixa_merge_search_results(0, 1, 1, 1, None, None, None, None)
+    assert rc != 0 and "ndev" in lib.ixa_last_error().decode()

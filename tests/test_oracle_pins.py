@@ -287,3 +287,45 @@ def test_kmeans_objective_decreases(oracle):
     assert all(b <= a * (1 + 1e-6) for a, b in zip(objs, objs[1:]))
     cent, _ = oracle.kmeans(x, 16, niter=3, spherical=True, seed=5)
     assert np.allclose(np.linalg.norm(cent, axis=1), 1.0, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------------------------
+def _device_lists(rng, ndev, n, k, metric_l2, ties=False, holes=0.0):
+    """ndev sorted result lists per query, optionally with repeated distances and invalid labels."""
+    d = rng.standard_normal((ndev, n, k)).astype(np.float32)
+    if ties:
+        d = np.round(d * 2) / 2
+    d = np.sort(d, axis=2)
+    if not metric_l2:
+        d = d[:, :, ::-1].copy()
+    lab = rng.permutation(ndev * n * k).reshape(ndev, n, k).astype(np.int64)
+    if holes:
+        lab[rng.random(lab.shape) < holes] = -1
+    return d, lab
+
+
+@pytest.mark.parametrize("metric_l2", [True, False])
+def test_merge_results_equals_stable_sort_of_the_concatenation(oracle, metric_l2):
+    """A k-way merge of sorted lists with a strict comparison, scanning the devices in order, is the
+    stable sort of the device-major concatenation (FR/ascend/impl/AscendIndexImpl.cpp:587-640)."""
+    rng = np.random.default_rng(7)
+    d, lab = _device_lists(rng, 3, 40, 17, metric_l2, ties=True)
+    metric = oracle.METRIC_L2 if metric_l2 else oracle.METRIC_INNER_PRODUCT
+    got_d, got_l = oracle.merge_results(d, lab, metric)
+    cat_d = np.concatenate(list(d), axis=1)
+    cat_l = np.concatenate(list(lab), axis=1)
+    order = np.argsort(cat_d if metric_l2 else -cat_d, axis=1, kind="stable")[:, :17]
+    assert np.array_equal(got_d, np.take_along_axis(cat_d, order, 1))
+    assert np.array_equal(got_l, np.take_along_axis(cat_l, order, 1))
+
+
+def test_merge_results_skips_invalid_labels_anywhere_and_pads(oracle):
+    d = np.array([[[1.0, 2.0, 3.0, 9.0]], [[0.5, 2.0, 2.5, 4.0]]], dtype=np.float32)
+    lab = np.array([[[10, -1, 12, -1]], [[-1, 21, -1, -1]]], dtype=np.int64)
+    got_d, got_l = oracle.merge_results(d, lab, oracle.METRIC_L2)
+    assert got_l.tolist() == [[10, 21, 12, -1]]
+    assert got_d.tolist() == [[1.0, 2.0, 3.0, float(FLT_MAX)]]
+    # inner product: larger first, padding is still (FLT_MAX, -1)
+    got_d, got_l = oracle.merge_results(d[:, :, ::-1].copy(), lab[:, :, ::-1].copy(), oracle.METRIC_INNER_PRODUCT)
+    assert got_l.tolist() == [[12, 21, 10, -1]]
+    assert got_d.tolist() == [[3.0, 2.0, 1.0, float(FLT_MAX)]]
