@@ -384,11 +384,10 @@ void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter
 // calls over column chunks into a streaming top-k.  Output: ksel column indices per row (best
 // first, -1 where the row has fewer than ksel columns) and/or the keys themselves.
 template <typename S>
-__global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
-                                                          int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                          int64_t col_base, key_t *__restrict__ running)
+__device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, const S *__restrict__ scores, int64_t ld,
+                                                     int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
+                                                     int64_t col_base, key_t *__restrict__ running)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
     key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // pow2_ceil(4 * cap + ksel)
     const int region = running ? 8 * cap : 4 * cap;
     S *share = reinterpret_cast<S *>(pools + region);                   // 4
@@ -488,6 +487,273 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ 
 }
 
 template <typename S>
+__global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
+                                                          int ksel, int cap, int32_t *__restrict__ out_idx,
+                                                          int64_t col_base, key_t *__restrict__ running)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same selection for rows of >= 4096 columns and ksel <= 384, built around registers instead of
+// pools.  The workgroup loads a segment of 16384 columns at once (64 values per lane, all loads in
+// flight together), and needs a bound B with at least ksel values at or below it before it can
+// discard anything.  The first segment gets B from group minima: every lane reduces its values to G
+// group minima, every wave finds the ceil(ksel / 4)-th smallest of its 64 G minima (that many values
+// of the wave lie at or below it), and B is the largest of the four: with the rank near a third of
+// the group count only about 1.3 ksel values of the segment pass.  Passing values are appended to a
+// candidate list in LDS (ballot compaction per wave), and after every segment that added something
+// the list is reduced to its ksel smallest keys in order, by counting ranks (keys are distinct):
+// that list is the running result, and its last score is the next segment's B.  Rows with so many
+// equal scores that the list overflows are redone by the streaming selection above; the result is
+// the same set of keys in either case: the ksel smallest (score, column) keys of the row and of
+// `running`.
+#ifndef IXA_SELREG_WAVES
+#define IXA_SELREG_WAVES 4
+#endif
+constexpr int kSelRegSeg = 16384;     // columns per segment: 64 per lane
+constexpr int kSelRegStage = 160;     // new candidates per wave and segment
+constexpr int kSelRegMaxK = 384;
+constexpr int kSelRegCap = kSelRegMaxK + 4 * kSelRegStage;   // 1024
+
+// dst[0 .. min(n, keep)) = the smallest keys of src[0 .. n) in ascending order.  n <= 1024, src is
+// 16-byte aligned with src[n] writable; all 256 threads call it; barriers inside.
+__device__ __forceinline__ void rank_select_256(key_t *src, int n, key_t *dst, int keep, int tid)
+{
+    if (tid == 0 && (n & 1)) {
+        src[n] = kEmptyKey;   // never below a key
+    }
+    __syncthreads();
+    key_t mine[4];
+    int rank[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        mine[e] = tid + 256 * e < n ? src[tid + 256 * e] : 0;   // 0: rank stays 0 and is not used
+        rank[e] = 0;
+    }
+    const int owned = (n + 255 - tid) >> 8;   // entries tid, tid + 256, ... below n
+    const ulonglong2 *pairs = reinterpret_cast<const ulonglong2 *>(src);
+    if (n <= 256) {
+        for (int f = 0; f < (n + 1) >> 1; f++) {
+            const ulonglong2 pr = pairs[f];   // same address in every lane: one broadcast read
+            rank[0] += (pr.x < mine[0]) + (pr.y < mine[0]);
+        }
+    } else {
+        for (int f = 0; f < (n + 1) >> 1; f++) {
+            const ulonglong2 pr = pairs[f];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                rank[e] += (pr.x < mine[e]) + (pr.y < mine[e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        if (e < owned && rank[e] < keep) {
+            dst[rank[e]] = mine[e];
+        }
+    }
+    __syncthreads();
+}
+
+template <typename S, int G>
+__global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
+    const S *__restrict__ scores, int64_t ld, int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
+    int64_t col_base, key_t *__restrict__ running)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    key_t *cand = reinterpret_cast<key_t *>(smem_raw);            // kSelRegCap + 2
+    key_t *best = cand + kSelRegCap + 2;                          // kSelRegMaxK
+    key_t *stage = best + kSelRegMaxK;                            // 4 x kSelRegStage
+    S *gm = reinterpret_cast<S *>(stage + 4 * kSelRegStage);      // 4 x 64 G group minima
+    S *wb = gm + 4 * 64 * G;                                      // 4 wave bounds
+    int *ctl = reinterpret_cast<int *>(wb + 4);                   // [0..3] new candidates per wave, [4] overflow
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const S *row = scores + (int64_t)blockIdx.x * ld;
+    key_t *run = running ? running + (int64_t)blockIdx.x * ksel : nullptr;
+
+    // the running result so far (sorted, kEmptyKey-padded) opens the candidate list
+    int have = 0;   // workgroup-uniform: keys in cand[] before this segment, sorted
+    if (run) {
+        for (int i = tid; i < ksel; i += 256) {
+            cand[i] = run[i];
+        }
+        __syncthreads();
+        int lo = 0, hi = ksel;   // valid keys form a prefix
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (cand[mid] != kEmptyKey) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        have = lo;
+    }
+    bool bounded = have >= ksel;
+    S B = bounded ? key_score_as<S>(cand[ksel - 1]) : ScoreOps<S>::worst();
+    if (tid == 0) {
+        ctl[4] = 0;
+    }
+    __syncthreads();
+
+    for (int64_t seg0 = 0; seg0 < nc; seg0 += kSelRegSeg) {
+        S v[16][4];
+        const S *seg = row + seg0;
+        const int lim = (int)(nc - seg0 < kSelRegSeg ? nc - seg0 : kSelRegSeg);   // valid columns of the segment
+        if (lim == kSelRegSeg) {
+            // whole segment: sixteen 128-bit loads per lane, all in flight together
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const uint4 u = *reinterpret_cast<const uint4 *>(seg + (i * 256 + tid) * 4);
+                v[i][0] = __builtin_bit_cast(S, u.x);
+                v[i][1] = __builtin_bit_cast(S, u.y);
+                v[i][2] = __builtin_bit_cast(S, u.z);
+                v[i][3] = __builtin_bit_cast(S, u.w);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int c = (i * 256 + tid) * 4;
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    v[i][t] = c + t < lim ? seg[c + t] : ScoreOps<S>::worst();
+                }
+            }
+        }
+        if (!bounded) {
+            // group j of this lane: its loads i with i % G == j
+            S mine[G];
+#pragma unroll
+            for (int j = 0; j < G; j++) {
+                S m = ScoreOps<S>::worst();
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    if ((i & (G - 1)) == j) {
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            m = v[i][t] < m ? v[i][t] : m;
+                        }
+                    }
+                }
+                mine[j] = m;
+                gm[wave * 64 * G + j * 64 + lane] = m;
+            }
+            wave_lds_fence();
+            // how many of the wave's minima lie at or below each of mine
+            int below[G];
+#pragma unroll
+            for (int j = 0; j < G; j++) {
+                below[j] = 0;
+            }
+            const uint4 *quads = reinterpret_cast<const uint4 *>(gm + wave * 64 * G);
+            for (int f = 0; f < 16 * G; f++) {
+                const uint4 u = quads[f];   // same address in every lane: one broadcast read
+                const S x0 = __builtin_bit_cast(S, u.x), x1 = __builtin_bit_cast(S, u.y);
+                const S x2 = __builtin_bit_cast(S, u.z), x3 = __builtin_bit_cast(S, u.w);
+#pragma unroll
+                for (int j = 0; j < G; j++) {
+                    below[j] += (x0 <= mine[j]) + (x1 <= mine[j]) + (x2 <= mine[j]) + (x3 <= mine[j]);
+                }
+            }
+            // the smallest of the wave's minima with at least ceil(ksel / 4) minima at or below it
+            const int need = (ksel + 3) >> 2;
+            S wbound = ScoreOps<S>::worst();
+#pragma unroll
+            for (int j = 0; j < G; j++) {
+                if (below[j] >= need && mine[j] < wbound) {
+                    wbound = mine[j];
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const S o = __shfl_xor(wbound, off);
+                wbound = o < wbound ? o : wbound;
+            }
+            if (lane == 0) {
+                wb[wave] = wbound;
+            }
+            __syncthreads();
+            B = wb[0];
+#pragma unroll
+            for (int w = 1; w < 4; w++) {
+                B = wb[w] > B ? wb[w] : B;
+            }
+        }
+        // ballot compaction of the passing values into this wave's staging area
+        int added = 0;   // wave-uniform
+        {
+            const uint32_t first_col = (uint32_t)(seg0 + col_base);
+            key_t *mystage = stage + wave * kSelRegStage;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int c = (i * 256 + tid) * 4;
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const bool pass = v[i][t] <= B && c + t < lim;
+                    const unsigned long long mask = __ballot(pass);
+                    if (mask) {
+                        const int pos = added + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                                               __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+                        if (pass && pos < kSelRegStage) {
+                            mystage[pos] = make_key(v[i][t], first_col + (uint32_t)(c + t));
+                        }
+                        added += __builtin_popcountll(mask);
+                    }
+                }
+            }
+        }
+        if (lane == 0) {
+            ctl[wave] = added;
+            if (added > kSelRegStage) {
+                ctl[4] = 1;
+            }
+        }
+        __syncthreads();
+        if (ctl[4]) {
+            // too many equal scores for the list: the streaming selection redoes the row
+            __syncthreads();
+            select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running);
+            return;
+        }
+        int before = have, total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const int cw = ctl[w];
+            before += w < wave ? cw : 0;
+            total += cw;
+        }
+        if (total > 0) {
+            for (int i = lane; i < added; i += 64) {
+                cand[before + i] = stage[wave * kSelRegStage + i];
+            }
+            const int n = have + total;
+            rank_select_256(cand, n, best, ksel, tid);
+            have = n < ksel ? n : ksel;
+            for (int i = tid; i < have; i += 256) {
+                cand[i] = best[i];
+            }
+            bounded = have >= ksel;
+            if (bounded) {
+                B = key_score_as<S>(best[ksel - 1]);
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < ksel; i += 256) {
+        const key_t kk = i < have ? cand[i] : kEmptyKey;
+        if (out_idx) {
+            out_idx[(int64_t)blockIdx.x * ksel + i] = kk == kEmptyKey ? -1 : (int32_t)key_index(kk);
+        }
+        if (run) {
+            run[i] = kk;
+        }
+    }
+}
+
+template <typename S>
 static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
                                  int64_t col_base, unsigned long long *running, hipStream_t s)
 {
@@ -496,8 +762,20 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
     }
     IXA_REQUIRE(ksel >= 1 && ksel <= 2048, kErrInvalidParam, "selection size %d out of range [1, 2048]", ksel);
     const int cap = wave_pool_capacity(ksel);
-    const size_t smem = (size_t)(running ? 8 : 4) * cap * sizeof(key_t) + 64;
+    size_t smem = (size_t)(running ? 8 : 4) * cap * sizeof(key_t) + 64;
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "selection size %d needs %zu bytes of LDS", ksel, smem);
+    const bool vec4 = ld % 4 == 0 && reinterpret_cast<uintptr_t>(scores) % 16 == 0;
+    // measured: the register kernel wins on rows of up to a few segments (16384 columns: 0.17 ms against
+    // 0.27 ms for 10000 rows, ksel 88), the streaming kernel on rows of hundreds of thousands of columns
+    if (vec4 && ksel <= kSelRegMaxK && nc >= 4096 && nc <= 6 * kSelRegSeg) {
+        smem = std::max(smem, (size_t)(kSelRegCap + 2 + kSelRegMaxK + 4 * kSelRegStage) * sizeof(key_t) + 4 * 64 * 4 * 4 + 64);
+        // groups per lane: ksel / (256 G) stays near 1/3
+        auto kern = ksel <= 96 ? select_rows_reg_kernel<S, 1>
+                               : (ksel <= 192 ? select_rows_reg_kernel<S, 2> : select_rows_reg_kernel<S, 4>);
+        hipLaunchKernelGGL(kern, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap, out_idx,
+                           col_base, running);
+        return;
+    }
     if (smem > 48 * 1024) {
         IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel<S>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
