@@ -163,3 +163,54 @@ def test_flat_f32_near_duplicates_are_redone_exactly(ix, oracle, metric_name):
     Dr, Ir = oracle.flat_f32(base, q, k, metric)
     assert np.array_equal(I, Ir)
     assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+
+
+# Score rows of 4096 .. 98304 columns with k <= 384 are selected from registers (bound from group
+# minima); the cases below hold a ragged last segment, every group count, running keys from an
+# earlier chunk, and rows of many equal scores, which overflow the candidate list and are redone by
+# the streaming selection.
+@pytest.mark.parametrize("n,k,scratch", [(20003, 100, 0), (20003, 300, 0), (33000, 150, 0), (40000, 60, 6 << 20)])
+def test_flat_f32_rows_selected_from_registers(ix, oracle, n, k, scratch):
+    d, nq = 64, 50
+    rng = np.random.default_rng(n + k)
+    centres = rng.standard_normal((30, d)).astype(np.float32)
+    base = (centres[rng.integers(0, 30, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 30, nq)] + 0.3 * rng.standard_normal((nq, d))).astype(np.float32)
+    index = ix.AscendIndexFlat(d, ix.METRIC_L2, scratch_bytes=scratch)
+    index.add(base)
+    D, I = index.search(q, k)
+    Dr, Ir = oracle.flat_f32(base, q, k, ix.METRIC_L2)
+    assert np.array_equal(I, Ir)
+    assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+
+
+def test_flat_rows_of_equal_scores_overflow_the_register_selection(ix, oracle):
+    d, n, nq, k = 64, 24000, 20, 100
+    rng = np.random.default_rng(5)
+    protos = rng.standard_normal((5, d)).astype(np.float32)
+    base = protos[rng.integers(0, 5, n)]
+    q = (protos[rng.integers(0, 5, nq)] + 0.05 * rng.standard_normal((nq, d))).astype(np.float32)
+    index = ix.AscendIndexFlat(d, ix.METRIC_L2)
+    index.add(base)
+    D, I = index.search(q, k)
+    Dr, Ir = oracle.flat_f32(base, q, k, ix.METRIC_L2)
+    assert np.array_equal(I, Ir) and np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+    b8 = rng.integers(-127, 128, size=(4, d), dtype=np.int8)[rng.integers(0, 4, n)]
+    q8 = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    i8 = ix.AscendIndexInt8Flat(d)
+    i8.add(b8)
+    D, I = i8.search_int32(q8, k)
+    Dr, Ir = oracle.flat_i8(b8, q8, k)
+    assert np.array_equal(I, Ir) and np.array_equal(D, Dr)
+
+
+def test_flat_i8_rows_selected_from_registers(ix, oracle):
+    d, n, nq, k = 64, 30001, 40, 200
+    rng = np.random.default_rng(6)
+    base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    index = ix.AscendIndexInt8Flat(d)
+    index.add(base)
+    D, I = index.search_int32(q, k)
+    Dr, Ir = oracle.flat_i8(base, q, k)
+    assert np.array_equal(I, Ir) and np.array_equal(D, Dr)

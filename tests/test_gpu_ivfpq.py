@@ -74,6 +74,40 @@ def test_coarse_probe_bit_exact(ix, oracle, metric_name, nprobe):
     assert np.array_equal(gd.view(np.uint32), od.view(np.uint32))
 
 
+@pytest.mark.parametrize("metric_name", ["L2", "IP"])
+@pytest.mark.parametrize("nlist,nprobe", [(5003, 64), (5003, 150), (4096, 300), (20000, 32)])
+def test_coarse_probe_bit_exact_with_thousands_of_lists(ix, oracle, metric_name, nlist, nprobe):
+    """Probe selection over score rows long enough for the register-based row selection (every group
+    count, a ragged last segment, two segments)."""
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    d, M, nq = 64, 8, 200
+    rng = np.random.default_rng(nlist + nprobe)
+    centres = rng.standard_normal((40, d)).astype(np.float32)
+    cent = (centres[rng.integers(0, 40, nlist)] + 0.4 * rng.standard_normal((nlist, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 40, nq)] + 0.4 * rng.standard_normal((nq, d))).astype(np.float32)
+    if metric == ix.METRIC_INNER_PRODUCT:
+        cent /= np.linalg.norm(cent, axis=1, keepdims=True)
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    cb = rng.standard_normal((M, 256, d // M)).astype(np.float32)
+    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.setNumProbes(nprobe)
+    gi, gd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, metric)
+    assert np.array_equal(gi, oi)
+    assert np.array_equal(gd.view(np.uint32), od.view(np.uint32))
+    # the search path refines only the boundary of the probe set: same set of lists
+    x = (centres[rng.integers(0, 40, 30000)] + 0.4 * rng.standard_normal((30000, d))).astype(np.float32)
+    if metric == ix.METRIC_INNER_PRODUCT:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    gpu.add(x)
+    ref = oracle.CsrIndex.build(d, M, metric, cent, cb, x, np.arange(30000, dtype=np.int64))
+    D, I = gpu.search(q, 20)
+    Dr, Ir = ref.search(q, 20, nprobe)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
+
+
 @pytest.mark.parametrize("d,M,nlist,layout", [(128, 16, 64, 0), (128, 32, 64, 0), (128, 32, 64, 1), (96, 48, 32, 0),
                                               (64, 8, 16, 0), (60, 12, 16, 0), (192, 96, 16, 1), (128, 64, 16, 1)])
 def test_search_l2_fp32(ix, oracle, d, M, nlist, layout):
