@@ -64,11 +64,12 @@ void launch_verify_superset(const unsigned long long *running, int ncand, const 
 // indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
 // (ordered score << 32) | (col_base + column): its content takes part in the selection and is
 // replaced by the result, so calling this over successive column chunks keeps a streaming top-k.
-// Fill it with 0xff bytes before the first chunk.
+// Before the first chunk fill it with 0xff bytes, or pass fresh = true for that chunk (`running` is then
+// only written).
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                        int64_t col_base, unsigned long long *running, hipStream_t s);
+                        int64_t col_base, unsigned long long *running, hipStream_t s, bool fresh = false);
 void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                            int64_t col_base, unsigned long long *running, hipStream_t s);
+                            int64_t col_base, unsigned long long *running, hipStream_t s, bool fresh = false);
 
 // Exact best-nout SET from approximately scored, sorted candidates (see refine_boundary_kernel):
 // re-evaluates only the candidates within 2 * err of the rank-nout score; a query whose list

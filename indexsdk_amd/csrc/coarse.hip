@@ -386,10 +386,11 @@ void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter
 template <typename S>
 __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, const S *__restrict__ scores, int64_t ld,
                                                      int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                     int64_t col_base, key_t *__restrict__ running)
+                                                     int64_t col_base, key_t *__restrict__ running, bool fresh)
 {
     key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // pow2_ceil(4 * cap + ksel)
     const int region = running ? 8 * cap : 4 * cap;
+    // fresh: `running` only receives the result (its content is unspecified on entry)
     S *share = reinterpret_cast<S *>(pools + region);                   // 4
     int *counts = reinterpret_cast<int *>(share + 4);                   // 4
 
@@ -398,7 +399,7 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
     const S *row = scores + (int64_t)blockIdx.x * ld;
     key_t *run = running ? running + (int64_t)blockIdx.x * ksel : nullptr;
     S start = ScoreOps<S>::worst();
-    if (run) {
+    if (run && !fresh) {
         const key_t last = run[ksel - 1];
         if (last != kEmptyKey) {
             start = key_score_as<S>(last);
@@ -474,7 +475,7 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
     if (lane == 0) {
         counts[wave] = pool.count;
     }
-    const int total = block_merge_pools<4>(pools, cap, counts, run, run ? ksel : 0, tid);
+    const int total = block_merge_pools<4>(pools, cap, counts, run, (run && !fresh) ? ksel : 0, tid);
     for (int i = tid; i < ksel; i += 256) {
         key_t kk = i < total ? pools[i] : kEmptyKey;
         if (out_idx) {
@@ -489,10 +490,10 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
 template <typename S>
 __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
                                                           int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                          int64_t col_base, key_t *__restrict__ running)
+                                                          int64_t col_base, key_t *__restrict__ running, bool fresh)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running);
+    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -560,7 +561,7 @@ __device__ __forceinline__ void rank_select_256(key_t *src, int n, key_t *dst, i
 template <typename S, int G>
 __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
     const S *__restrict__ scores, int64_t ld, int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
-    int64_t col_base, key_t *__restrict__ running)
+    int64_t col_base, key_t *__restrict__ running, bool fresh)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     key_t *cand = reinterpret_cast<key_t *>(smem_raw);            // kSelRegCap + 2
@@ -576,7 +577,7 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
 
     // the running result so far (sorted, kEmptyKey-padded) opens the candidate list
     int have = 0;   // workgroup-uniform: keys in cand[] before this segment, sorted
-    if (run) {
+    if (run && !fresh) {
         for (int i = tid; i < ksel; i += 256) {
             cand[i] = run[i];
         }
@@ -715,7 +716,7 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
         if (ctl[4]) {
             // too many equal scores for the list: the streaming selection redoes the row
             __syncthreads();
-            select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running);
+            select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh);
             return;
         }
         int before = have, total = 0;
@@ -755,7 +756,7 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
 
 template <typename S>
 static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                                 int64_t col_base, unsigned long long *running, hipStream_t s)
+                                 int64_t col_base, unsigned long long *running, bool fresh, hipStream_t s)
 {
     if (nrows == 0) {
         return;
@@ -773,7 +774,7 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
         auto kern = ksel <= 96 ? select_rows_reg_kernel<S, 1>
                                : (ksel <= 192 ? select_rows_reg_kernel<S, 2> : select_rows_reg_kernel<S, 4>);
         hipLaunchKernelGGL(kern, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap, out_idx,
-                           col_base, running);
+                           col_base, running, fresh);
         return;
     }
     if (smem > 48 * 1024) {
@@ -781,19 +782,19 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     }
     hipLaunchKernelGGL(select_rows_kernel<S>, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
-                       out_idx, col_base, running);
+                       out_idx, col_base, running, fresh);
 }
 
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                        int64_t col_base, unsigned long long *running, hipStream_t s)
+                        int64_t col_base, unsigned long long *running, hipStream_t s, bool fresh)
 {
-    launch_select_rows_t<float>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, s);
+    launch_select_rows_t<float>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, fresh, s);
 }
 
 void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
-                            int64_t col_base, unsigned long long *running, hipStream_t s)
+                            int64_t col_base, unsigned long long *running, hipStream_t s, bool fresh)
 {
-    launch_select_rows_t<int32_t>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, s);
+    launch_select_rows_t<int32_t>(scores, nrows, ld, nc, ksel, out_idx, col_base, running, fresh, s);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -541,7 +541,6 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
     ws_idx_.resize((size_t)n * k);
     IXA_HIP(hipEventRecord(ev_[0], stream_));
     launch_sqnorm_rows(xd, n, d_, ws_qn_.data(), stream_);
-    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
     const int launches = stream_select_f32(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), metric_,
                                            ncand, ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
@@ -641,7 +640,6 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     IXA_HIP(hipEventRecord(ev_[0], stream_));
     hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_, xd, n, d_,
                        ws_qn_.data());
-    IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
     const int launches = stream_select_i8(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), (int)k,
                                           ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
     hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,

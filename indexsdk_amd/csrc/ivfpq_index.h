@@ -82,7 +82,8 @@ private:
     void upload_trained(const float *centroids, const float *codebook);
     // best `nout` lists of every row of device matrix x (canonical arithmetic), device outputs
     void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
-                       float *out_dist, bool set_only = false);
+                       float *out_dist, bool set_only = false, bool defer_check = false);
+    int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist);
     void coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
                            int32_t *out_ids, float *out_dist);
     void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev);

@@ -314,7 +314,7 @@ void IvfpqIndex::coarse_exact_rows(const float *x_dev, const std::vector<int64_t
 // proof.  Queries whose proof fails (near-tied centroids) are redone exactly from canonical scores of
 // all centroids.
 void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
-                               float *out_dist, bool set_only)
+                               float *out_dist, bool set_only, bool defer_check)
 {
     if (n == 0) {
         return;
@@ -325,7 +325,6 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     bool approx = false;
     if (cfg_.coarse_bf16) {
         ws_running_.resize((size_t)n * ncand);
-        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
         ws_xsplit_.resize((size_t)n * 3 * dp_);
         launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
         approx = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
@@ -335,7 +334,6 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     if (!approx) {
         ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
         ws_running_.resize((size_t)n * ncand);
-        IXA_HIP(hipMemsetAsync(ws_running_.data(), 0xff, ws_running_.bytes(), stream_));
         stream_select_f32(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric, ncand,
                           ws_running_.data(), ws_sel_, cfg_.scratch_bytes, stream_);
     }
@@ -354,8 +352,12 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     const float err_scale = approx ? dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * u)
                                    : dots * (float)(2 * d_ + 8) * u;
     const float round_scale = select_metric == kMetricL2 ? 4.0f * u : 0.0f;
-    ws_flag_.resize((size_t)n + 1);
-    IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+    // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
+    // when it was not, so the common case needs no fill in front of the kernels that append to it
+    if (ws_flag_.size() < (size_t)n + 1) {   // grows only, so its first word stays what the last call left
+        ws_flag_.resize((size_t)n + 1);
+        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+    }
     if (approx && set_only && !out_dist && ncand > nout) {
         // search: only the SET of probed lists matters, so only the candidates the approximate scores
         // cannot decide are re-evaluated
@@ -377,17 +379,30 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
                                    select_metric, n, ws_flag_.data(), stream_);
         }
     }
+    if (!defer_check) {
+        coarse_finish(x_dev, nout, select_metric, out_ids, out_dist);
+    }
+}
+
+// Second half of coarse_select(): waits for the stream, and redoes the queries whose candidate list
+// could not be proven complete from canonical scores of all centroids.  Returns how many there were.
+// search() calls it after it has queued the scan behind the coarse stage, so that the common case (no
+// such query) has no host round trip between the two.
+int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist)
+{
     int32_t nfail = 0;
     ws_flag_.download(&nfail, 1, stream_);
     if (nfail == 0) {
-        return;
+        return 0;
     }
     last_coarse_reruns_ += nfail;
     std::vector<int32_t> rows32((size_t)nfail);
     IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
+    IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
     IXA_HIP(hipStreamSynchronize(stream_));
     std::sort(rows32.begin(), rows32.end());   // the order of the appends is not deterministic
     coarse_exact_rows(x_dev, std::vector<int64_t>(rows32.begin(), rows32.end()), nout, select_metric, out_ids, out_dist);
+    return nfail;
 }
 
 void IvfpqIndex::assign(int64_t n, const float *x, int64_t *out, bool on_device)
@@ -736,8 +751,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
 
     IXA_HIP(hipEventRecord(ev_[0], stream_));
     last_coarse_reruns_ = 0;
-    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true);
-    stats_.coarse_reruns = last_coarse_reruns_;
+    coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true, true);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
 
     ScanParams p{};
@@ -773,6 +787,12 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     p.order = nullptr;
     p.xcd_chunks = (getenv("IXA_XCD_CHUNKS") && nsplit == 1) ? 1 : 0;
     launch_scan(p, n, stream_);
+    // the scan is queued; only now does the host look at the coarse stage's verdict.  Queries that had to
+    // be redone exactly (near-tied centroids: rare) have new probe lists, and the scan runs again.
+    if (coarse_finish(xd, nprobe_, metric_, ws_probes_.data(), nullptr) > 0) {
+        launch_scan(p, n, stream_);
+    }
+    stats_.coarse_reruns = last_coarse_reruns_;
     {
         ScanParams planned = p;
         plan_scan(planned);

@@ -12,8 +12,9 @@ struct StreamSelectWorkspace {
     DeviceBuffer<unsigned long long> filter;
 };
 
-// running[nq][ncand] must be filled with 0xff bytes by the caller; on return (the stream has been
-// synchronised) it holds each query's best ncand keys (ordered score << 32 | base row), ascending.
+// running[nq][ncand] is written only: once the work queued on the stream has run it holds each query's
+// best ncand keys (ordered score << 32 | base row), ascending, kEmptyKey-padded.  The call waits for
+// the stream only when it used filtered launches (whose overflow flag decides about a second attempt).
 // A first stretch of the base goes through a score scratch of at most scratch_bytes and seeds
 // the running keys; afterwards the score kernel admits only what beats each query's current
 // ncand-th score and the admitted keys are merged.  If a query ever admits more keys than its

@@ -59,9 +59,10 @@ struct F32Ops {
     {
         launch_score_tiles_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, metric, flt, s);
     }
-    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
+                hipStream_t s) const
     {
-        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s);
+        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
     void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
     {
@@ -88,9 +89,10 @@ struct Bf16Ops {
         const bool ok = launch_score_ring_bf16(Q, nq, B, nb, d, qn + q0, bn + b0, metric, nullptr, 0, true, flt, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
     }
-    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
+                hipStream_t s) const
     {
-        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s);
+        launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
     void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
     {
@@ -118,9 +120,10 @@ struct I8Ops {
     {
         launch_score_tiles_i8_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, flt, s);
     }
-    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, hipStream_t s) const
+    void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
+                hipStream_t s) const
     {
-        launch_select_rows_i32(sc, nq, ld, nc, k, nullptr, base, run, s);
+        launch_select_rows_i32(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
     void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
     {
@@ -135,6 +138,10 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
 {
     using S = typename Ops::S;
     if (nq_total == 0) {
+        return 0;
+    }
+    if (nb_total == 0) {   // no chunk will start the running keys
+        IXA_HIP(hipMemsetAsync(running, 0xff, (size_t)nq_total * ncand * sizeof(key_t), s));
         return 0;
     }
     const int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
@@ -160,7 +167,9 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     if (can_fuse) {
         ws.filter.resize((size_t)qb * cap);
     }
-    IXA_HIP(hipMemsetAsync(ws.cnt.data(), 0, ws.cnt.bytes(), s));
+    if (can_fuse) {   // per-query candidate counters and the overflow flag of the filtered launches
+        IXA_HIP(hipMemsetAsync(ws.cnt.data(), 0, ws.cnt.bytes(), s));
+    }
     int *overflow = ws.cnt.data() + nq_total;
     int launches = 0;
     bool fused = can_fuse;
@@ -176,7 +185,8 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             for (int64_t b0 = 0; b0 < head; b0 += ldo) {
                 const int64_t nbc = std::min(ldo, head - b0);
                 ops.scores(Q + q0 * d, nq, q0, B + b0 * d, nbc, b0, d, ws.scores.data(), ldo, s);
-                ops.select(ws.scores.data(), nq, ldo, nbc, ncand, b0, running + q0 * ncand, s);
+                // the first chunk of a query block starts its running keys (whatever `running` held)
+                ops.select(ws.scores.data(), nq, ldo, nbc, ncand, b0, running + q0 * ncand, b0 == 0, s);
                 launches++;
             }
             if (!fused) {
@@ -195,16 +205,16 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
                 seen += nbc;
             }
         }
-        int ovf = 0;
-        if (fused) {
-            IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, s));
+        if (!fused) {
+            break;   // nothing can overflow: no host synchronisation, the caller's stream carries on
         }
+        int ovf = 0;
+        IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, s));
         IXA_HIP(hipStreamSynchronize(s));
         if (!ovf) {
             break;
         }
         fused = false;
-        IXA_HIP(hipMemsetAsync(running, 0xff, (size_t)nq_total * ncand * sizeof(key_t), s));
     }
     return launches;
 }
