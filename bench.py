@@ -269,6 +269,18 @@ def main():
                      "kernel": "ivfpq_scan_kernel", "bytes_per_launch": scan_bytes, "ms_per_launch": scan_ms_avg},
     }
 
+    # The same batch through the host-pointer entry point (queries and results in pageable host memory, as a
+    # caller of the reference's API holds them): reported beside `value`, never as `value`.
+    qh_io = queries.cpu().numpy()
+    index.search(qh_io, k)
+    t0 = time.perf_counter()
+    for _ in range(3):
+        index.search(qh_io, k)
+    host_io_ms = (time.perf_counter() - t0) / 3 * 1e3
+    result["host_io"] = {"ms_per_step": host_io_ms, "queries_per_s": nq / (host_io_ms * 1e-3),
+                         "note": "ivfpq_search with host pointers: H2D of the queries and D2H of the results included"}
+    log(f"host-pointer search: {host_io_ms:.3f} ms per batch, {nq / (host_io_ms * 1e-3):.0f} QPS")
+
     if not args.no_cpu:
         from oracle import oracle as orc
         t0 = time.time()
