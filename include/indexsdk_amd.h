@@ -62,6 +62,40 @@ int ixa_merge_search_results(int ndev, int64_t n, int64_t k, int metric, const f
                              const int64_t *const *labels, float *distances, int64_t *out_labels);
 
 /* ---------------------------------------------------------------------------------------------
+ * Stage operators.  The reference runs the search path as named device operators through
+ * AscendOperator::exec(inputs, outputs, stream) (FR/ascenddaemon/utils/AscendOperator.cpp:33-45,
+ * 110-121; descriptors FR/ascenddaemon/impl/IndexIVFPQ.cpp:1633-1755).  The entry points below take the
+ * same tensors as plain DEVICE pointers, allocate nothing, and only queue work on `stream` (a
+ * hipStream_t, NULL = the null stream): a host layer that keeps the reference's staging can call them
+ * where it called exec.  Arithmetic: the reference's scalar order (left to right, no FMA).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Operator "DistanceFlatL2MinsAtFP32" (FR/ops/ascendc/op_kernel/distance_flat_l2_mins_at_fp32.cpp:95-251).
+ * inputs: queries [batch][d], codes [n][d], codesSqrSum [n];  outputs: dist [batch][n] =
+ * (|q|^2 + codesSqrSum[j]) - g - g, and min [batch][ceil(n/64)*2] (may be NULL): per burst of 64 codes
+ * the smallest distance followed by its position in the burst (uint32 bit pattern), as WholeReduceMin
+ * leaves them.  The operator's third output (a completion flag for the AICPU top-k that polls it) has
+ * no counterpart: stream order does that job here. */
+int ixa_op_distance_flat_l2_mins_fp32(const float *queries_dev, int64_t batch, const float *codes_dev, int64_t n,
+                                      int d, const float *codes_sqr_sum_dev, float *dist_dev, float *min_dev,
+                                      void *stream);
+
+/* Operator "TopkFlatFp32" (FR/ops/cpukernel/impl/topk_flat_fp32_cpu_kernel.cpp:223-384) as the IVFPQ
+ * path uses it (attrs asc = 1, k = nprobe, one block, one page; IndexIVFPQ.cpp:2127-2136).
+ * input: dists [batch][ld], the first n columns of a row are valid;  outputs: outdists [batch][k]
+ * ascending and outlabel [batch][k] (column numbers, int64), padded with (FLT_MAX, -1) when n < k.
+ * Equal distances go to the lower column (the reference's heap leaves that order unspecified).
+ * k <= 2048; asc must be 1. */
+int ixa_op_topk_flat_fp32(const float *dists_dev, int64_t batch, int64_t n, int64_t ld, int k, int asc,
+                          float *out_dists_dev, int64_t *out_labels_dev, void *stream);
+
+/* Operator "AscendcIvfpqSubspaceDistance" (FR/ops/ascendc/op_kernel/ascendc_ivfpq_subspace_distance.cpp:
+ * 197-477).  inputs: queries [batch][d], codeBook [msubs][256][d/msubs];  output: lut [batch][msubs][256]
+ * = (|cb|^2 + |q_m|^2) + (-2 q_m.cb) for IXA_METRIC_L2, q_m.cb for IXA_METRIC_INNER_PRODUCT. */
+int ixa_op_ivfpq_subspace_distance(const float *queries_dev, int64_t batch, int d, const float *codebook_dev,
+                                   int msubs, int metric, float *lut_dev, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
  * IVFPQ
  * ------------------------------------------------------------------------------------------- */
 
@@ -139,6 +173,12 @@ int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out);
 int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
 int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
                         int64_t *labels_dev);
+/* Stages 2-4 only, on probe lists the caller selected: operators "AscendcIvfpqSearchDistanceL2" +
+ * "TopkIvfpqL3" (IndexIVFPQ::searchImplL3, FR/ascenddaemon/impl/IndexIVFPQ.cpp:2162-2347), the LUT being
+ * built inside the launch.  probes_dev: [n][nprobe] list ids (int32, DEVICE), -1 = no list; a list
+ * named twice is scanned twice.  Results as ivfpq_search_device.  Waits for the results. */
+int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe,
+                               int64_t k, float *distances_dev, int64_t *labels_dev);
 
 /* Coarse assignment used by add (nearest centroid under L2), FR/ascend/impl/AscendIndexIVFPQImpl.cpp:603-672;
  * out[n]. */

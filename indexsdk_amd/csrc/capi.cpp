@@ -10,6 +10,7 @@
 
 #include "flat_index.h"
 #include "ivfpq_index.h"
+#include "ops.h"
 
 namespace ixa {
 void write_faiss_ivfpq(const IvfpqIndex &idx, const char *path);
@@ -383,6 +384,36 @@ IXA_EXPORT int ixa_merge_search_results(int ndev, int64_t n, int64_t k, int metr
             }
         }
     });
+}
+IXA_EXPORT int ixa_op_distance_flat_l2_mins_fp32(const float *queries_dev, int64_t batch, const float *codes_dev,
+                                                 int64_t n, int d, const float *codes_sqr_sum_dev, float *dist_dev,
+                                                 float *min_dev, void *stream)
+{
+    return guarded([&] {
+        ixa::op_distance_flat_l2_mins_fp32(queries_dev, batch, codes_dev, n, d, codes_sqr_sum_dev, dist_dev, min_dev,
+                                           static_cast<hipStream_t>(stream));
+    });
+}
+IXA_EXPORT int ixa_op_topk_flat_fp32(const float *dists_dev, int64_t batch, int64_t n, int64_t ld, int k, int asc,
+                                     float *out_dists_dev, int64_t *out_labels_dev, void *stream)
+{
+    return guarded([&] {
+        IXA_REQUIRE(asc == 1, ixa::kErrInvalidParam, "TopkFlatFp32: only ascending selection (asc = 1) is supported");
+        ixa::op_topk_flat_fp32(dists_dev, batch, n, ld, k, out_dists_dev, out_labels_dev, static_cast<hipStream_t>(stream));
+    });
+}
+IXA_EXPORT int ixa_op_ivfpq_subspace_distance(const float *queries_dev, int64_t batch, int d, const float *codebook_dev,
+                                              int msubs, int metric, float *lut_dev, void *stream)
+{
+    return guarded([&] {
+        ixa::op_ivfpq_subspace_distance(queries_dev, batch, d, codebook_dev, msubs, metric, lut_dev,
+                                        static_cast<hipStream_t>(stream));
+    });
+}
+IXA_EXPORT int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev,
+                                          int nprobe, int64_t k, float *distances_dev, int64_t *labels_dev)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search_probes(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev); });
 }
 IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
 {

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "scan.h"
 #include "stream_select.h"
 
 namespace ixa {
@@ -65,6 +66,9 @@ public:
     // n codes for arbitrary lists in one arena rebuild; list order inside a list = input order (host pointers)
     void add_codes_bulk(int64_t n, const int32_t *list_no, const uint8_t *codes, const int64_t *ids);
     void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
+    // stages 2-4 only, on probe lists the caller selected (device pointers)
+    void search_probes(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k, float *dist_dev,
+                       int64_t *labels_dev);
     void assign(int64_t n, const float *x, int64_t *out, bool on_device);               // out: host
     void coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device);  // out: host
     void encode(int64_t n, const float *x, uint8_t *codes, bool on_device);             // codes: host
@@ -84,6 +88,8 @@ private:
     void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
                        float *out_dist, bool set_only = false, bool defer_check = false);
     int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist);
+    ScanParams scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
+                           int64_t *ld);
     void coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
                            int32_t *out_ids, float *out_dist);
     void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev);

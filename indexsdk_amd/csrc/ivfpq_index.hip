@@ -723,6 +723,63 @@ void IvfpqIndex::reset()
     sync_list_tables();
 }
 
+// Parameters of the fused LUT + scan + top-k launch for `n` queries and their probe lists.
+ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
+                                   int64_t *ld)
+{
+    ScanParams p{};
+    p.queries = xd;
+    p.probes = probes;
+    p.nprobe = nprobe;
+    p.codebook = codebook_.data();
+    p.cb_norms = cbnorm_.data();
+    p.d = d_;
+    p.M = M_;
+    p.dsub = dsub_;
+    p.metric = metric_;
+    p.lut_fp16 = cfg_.lut_fp16;
+    p.codes = codes_.data();
+    p.ids = ids_.data();
+    p.list_off = list_off_dev_.data();
+    p.list_len = list_len_dev_.data();
+    p.code_layout = layout_;
+    p.k = (int)k;
+    // enough workgroups to fill 256 CUs several times over, bounded by what one merge pass can hold
+    int nsplit = 1;
+    if (n < 2048) {
+        nsplit = (int)std::min<int64_t>((2048 + n - 1) / n, nprobe);
+        nsplit = (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));
+    }
+    p.nsplit = nsplit;
+    if (nsplit > 1) {
+        ws_partial_.resize((size_t)n * nsplit * k);
+        p.partial = ws_partial_.data();
+    }
+    p.out_dist = dd;
+    p.out_labels = ld;
+    p.order = nullptr;
+    p.xcd_chunks = 0;   // contiguous query chunks per XCD: measured +6 % only with queries sorted by locality
+    return p;
+}
+
+// Stages 2-4 on caller-supplied probe lists (AscendcIvfpqSearchDistanceL2 + TopkIvfpqL3 of the
+// reference, FR/ascenddaemon/impl/IndexIVFPQ.cpp:2162-2347, with the LUT built inside the launch):
+// probes[n][nprobe] list ids on the device, -1 = no list.
+void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k,
+                               float *dist_dev, int64_t *labels_dev)
+{
+    check_trained();
+    IXA_REQUIRE(x_dev && probes_dev && dist_dev && labels_dev, kErrInvalidParam,
+                "x, probes, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+    IXA_REQUIRE(nprobe > 0 && nprobe <= nlist_, kErrInvalidParam, "nprobe must be > 0 and <= nlist");
+    flush_stats();
+    ScanParams p = scan_params(x_dev, n, probes_dev, nprobe, k, dist_dev, labels_dev);
+    launch_scan(p, n, stream_);
+    IXA_HIP(hipStreamSynchronize(stream_));
+}
+
 // -------------------------------------------------------------------------------------------------
 // search (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2351-2411): the whole batch goes through three
 // launches on one stream -- no per-8-query batching, no host round trip for the probe lists.
@@ -754,38 +811,8 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true, true);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
 
-    ScanParams p{};
-    p.queries = xd;
-    p.probes = ws_probes_.data();
-    p.nprobe = nprobe_;
-    p.codebook = codebook_.data();
-    p.cb_norms = cbnorm_.data();
-    p.d = d_;
-    p.M = M_;
-    p.dsub = dsub_;
-    p.metric = metric_;
-    p.lut_fp16 = cfg_.lut_fp16;
-    p.codes = codes_.data();
-    p.ids = ids_.data();
-    p.list_off = list_off_dev_.data();
-    p.list_len = list_len_dev_.data();
-    p.code_layout = layout_;
-    p.k = (int)k;
-    // enough workgroups to fill 256 CUs several times over, bounded by what one merge pass can hold
-    int nsplit = 1;
-    if (n < 2048) {
-        nsplit = (int)std::min<int64_t>((2048 + n - 1) / n, nprobe_);
-        nsplit = (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));
-    }
-    p.nsplit = nsplit;
-    if (nsplit > 1) {
-        ws_partial_.resize((size_t)n * nsplit * k);
-        p.partial = ws_partial_.data();
-    }
-    p.out_dist = dd;
-    p.out_labels = ld;
-    p.order = nullptr;
-    p.xcd_chunks = 0;   // contiguous query chunks per XCD: measured +6 % only with queries sorted by locality
+    ScanParams p = scan_params(xd, n, ws_probes_.data(), nprobe_, k, dd, ld);
+    const int nsplit = p.nsplit;
     launch_scan(p, n, stream_);
     // the scan is queued; only now does the host look at the coarse stage's verdict.  Queries that had to
     // be redone exactly (near-tied centroids: rare) have new probe lists, and the scan runs again.
