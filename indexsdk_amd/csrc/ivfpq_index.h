@@ -112,6 +112,7 @@ private:
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
     DeviceBuffer<int32_t> ws_flag_;
     int last_coarse_reruns_ = 0;
+    bool flag_pending_ = true;   // ws_flag_[0] may be non-zero: clear it before the next coarse stage
     bool stats_pending_ = false;
     int64_t stats_rows_ = 0;
     int stats_nprobe_ = 0;

@@ -430,8 +430,12 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     // when it was not, so the common case needs no fill in front of the kernels that append to it
     if (ws_flag_.size() < (size_t)n + 1) {   // grows only, so its first word stays what the last call left
         ws_flag_.resize((size_t)n + 1);
+        flag_pending_ = true;
+    }
+    if (flag_pending_) {   // new memory, or a deferred verdict that was never read (a failed call in between)
         IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
     }
+    flag_pending_ = true;
     if (approx && set_only && !out_dist && ncand > nout) {
         // search: only the SET of probed lists matters, so only the candidates the approximate scores
         // cannot decide are re-evaluated
@@ -467,6 +471,7 @@ int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, i
     int32_t nfail = 0;
     ws_flag_.download(&nfail, 1, stream_);
     if (nfail == 0) {
+        flag_pending_ = false;
         return 0;
     }
     last_coarse_reruns_ += nfail;
@@ -474,6 +479,7 @@ int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, i
     IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
     IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
     IXA_HIP(hipStreamSynchronize(stream_));
+    flag_pending_ = false;
     std::sort(rows32.begin(), rows32.end());   // the order of the appends is not deterministic
     coarse_exact_rows(x_dev, std::vector<int64_t>(rows32.begin(), rows32.end()), nout, select_metric, out_ids, out_dist);
     return nfail;
