@@ -218,6 +218,7 @@ typedef struct ivfpq_search_stats {
     double shared_pool;   /* 1: one workgroup-wide candidate pool (large k), 0: one pool per wavefront */
     double coarse_reruns; /* queries whose matrix-core coarse result could not be proven complete and that were
                              redone from canonical scores of all centroids */
+    double ordered;       /* 1: the scan started its queries in order of decreasing work (few, heavy workgroups) */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 /* Device times of the last search only (HIP events on the index's stream, in ms); either output may be NULL.

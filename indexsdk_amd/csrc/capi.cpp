@@ -283,6 +283,7 @@ IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stat
         out->scan_waves = s.scan_waves;
         out->shared_pool = s.shared_pool;
         out->coarse_reruns = s.coarse_reruns;
+        out->ordered = s.ordered;
     });
 }
 

@@ -37,6 +37,7 @@ struct SearchStats {
     double scan_waves = 0;
     double shared_pool = 0;
     double coarse_reruns = 0;
+    double ordered = 0;
 };
 
 class IvfpqIndex {
@@ -111,6 +112,8 @@ private:
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
     DeviceBuffer<int32_t> ws_flag_;
+    DeviceBuffer<int32_t> ws_order_, ws_order_hist_;   // execution order of the scan (heaviest queries first)
+    int32_t max_list_len_ = 0;
     int last_coarse_reruns_ = 0;
     bool flag_pending_ = true;   // ws_flag_[0] may be non-zero: clear it before the next coarse stage
     bool stats_pending_ = false;

@@ -298,6 +298,7 @@ void IvfpqIndex::check_trained() const
 
 void IvfpqIndex::sync_list_tables()
 {
+    max_list_len_ = list_len_.empty() ? 0 : *std::max_element(list_len_.begin(), list_len_.end());
     list_off_dev_.upload(list_off_.data(), (size_t)nlist_, stream_);
     list_len_dev_.upload(list_len_.data(), (size_t)nlist_, stream_);
     IXA_HIP(hipStreamSynchronize(stream_));
@@ -837,7 +838,22 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     }
     p.out_dist = dd;
     p.out_labels = ld;
+    // Few workgroups (at most eight rounds of a full GPU), each with enough work that a late heavy one
+    // shows: start the heaviest queries first.  Measured on 100M Zipf-skewed vectors, 1024 queries, nprobe 256: scan 5.4 -> 4.95 ms;
+    // no effect on 10000 queries over even lists.
     p.order = nullptr;
+    const int64_t codes_per_group = nlist_ > 0 ? ntotal_ / nlist_ * nprobe / nsplit : 0;   // average work of a workgroup
+    if (n * nsplit <= 8192 && n >= 64 && codes_per_group >= 16384) {
+        ws_order_.resize((size_t)n * 2);   // order | class
+        if (ws_order_hist_.size() == 0) {
+            ws_order_hist_.resize(2 * 1024);   // histogram (kept zero between calls) | cursors
+            IXA_HIP(hipMemsetAsync(ws_order_hist_.data(), 0, ws_order_hist_.bytes(), stream_));
+        }
+        launch_order_by_work(probes, n, nprobe, list_len_dev_.data(), (long long)nprobe * max_list_len_,
+                             ws_order_.data() + n, ws_order_hist_.data(), ws_order_hist_.data() + 1024,
+                             ws_order_.data(), stream_);
+        p.order = ws_order_.data();
+    }
     p.xcd_chunks = 0;   // contiguous query chunks per XCD: measured +6 % only with queries sorted by locality
     return p;
 }
@@ -900,6 +916,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
         launch_scan(p, n, stream_);
     }
     stats_.coarse_reruns = last_coarse_reruns_;
+    stats_.ordered = p.order ? 1 : 0;
     {
         ScanParams planned = p;
         plan_scan(planned);

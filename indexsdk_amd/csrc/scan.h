@@ -48,6 +48,12 @@ size_t plan_scan(ScanParams &p);
 
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s);
 
+// order[0 .. nq) = the queries by descending work class (work = sum of the probed lists' lengths, at most
+// max_work).  cls: nq ints; hist: 1024 ints that are ZERO on entry and zero again afterwards;
+// cursor: 1024 ints (scratch).
+void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, long long max_work,
+                          int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s);
+
 // *out += sum over probes of list_len[probe]  (probe < 0 contributes nothing).
 void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, unsigned long long *out,
                           hipStream_t s);

@@ -493,6 +493,79 @@ void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_
     hipLaunchKernelGGL(count_scanned_kernel, dim3(grid), dim3(256), 0, s, probes, n, list_len, out);
 }
 
+// ---- execution order: heaviest queries first ------------------------------------------------------
+// A launch of few workgroups with very different amounts of work (skewed lists, large nprobe) ends
+// with a long tail when a heavy query happens to start late.  Three small kernels order the queries
+// by descending work class (work = codes to scan, 1024 classes up to max_work) with a counting sort;
+// the order inside a class is whatever the atomics give -- it only decides when a workgroup runs.
+constexpr int kWorkClasses = 1024;
+
+// one wavefront per query: cls[q] and the class histogram
+__global__ __launch_bounds__(256) void work_class_kernel(const int32_t *__restrict__ probes, int64_t nq, int nprobe,
+                                                         const int32_t *__restrict__ list_len, long long max_work,
+                                                         int32_t *__restrict__ cls, int32_t *__restrict__ hist)
+{
+    const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (q >= nq) {
+        return;
+    }
+    long long w = 0;
+    for (int j = lane; j < nprobe; j += 64) {
+        const int l = probes[q * nprobe + j];
+        w += l >= 0 ? list_len[l] : 0;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        w += __shfl_xor(w, o);
+    }
+    if (lane == 0) {
+        long long c = w * kWorkClasses / (max_work + 1);
+        c = c < 0 ? 0 : (c > kWorkClasses - 1 ? kWorkClasses - 1 : c);
+        cls[q] = (int32_t)c;
+        atomicAdd(&hist[c], 1);
+    }
+}
+
+// one workgroup: cursor[c] = queries in classes above c; the histogram is left zeroed for the next call
+__global__ __launch_bounds__(kWorkClasses) void class_offsets_kernel(int32_t *__restrict__ hist,
+                                                                    int32_t *__restrict__ cursor)
+{
+    __shared__ int32_t scan[kWorkClasses];
+    const int t = threadIdx.x, c = kWorkClasses - 1 - t;   // thread 0 owns the heaviest class
+    const int32_t mine = hist[c];
+    hist[c] = 0;
+    scan[t] = mine;
+    __syncthreads();
+    for (int o = 1; o < kWorkClasses; o <<= 1) {
+        const int32_t add = t >= o ? scan[t - o] : 0;
+        __syncthreads();
+        scan[t] += add;
+        __syncthreads();
+    }
+    cursor[c] = scan[t] - mine;
+}
+
+__global__ __launch_bounds__(256) void scatter_order_kernel(const int32_t *__restrict__ cls, int64_t nq,
+                                                            int32_t *__restrict__ cursor, int32_t *__restrict__ order)
+{
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q < nq) {
+        order[atomicAdd(&cursor[cls[q]], 1)] = (int32_t)q;
+    }
+}
+
+void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, long long max_work,
+                          int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    hipLaunchKernelGGL(work_class_kernel, dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, s, probes, nq, nprobe, list_len,
+                       max_work, cls, hist);
+    hipLaunchKernelGGL(class_offsets_kernel, dim3(1), dim3(kWorkClasses), 0, s, hist, cursor);
+    hipLaunchKernelGGL(scatter_order_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, cls, nq, cursor, order);
+}
+
 template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
