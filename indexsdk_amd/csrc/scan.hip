@@ -654,7 +654,10 @@ static size_t plan_with_waves(ScanParams &p, int waves, bool shared)
     p.off_hist = (int)off;
     off += shared ? 4096 : 0;
     p.off_misc = (int)off;
-    off += 128;   // share[W], counts[W], BlockPoolCtl
+    // share[W] + counts[W] + BlockPoolCtl.  (Sized for eight waves this region ended 32 bytes short with
+    // sixteen: harmless while the plan's total is rounded up by the LDS allocation granule, a workgroup
+    // that never finishes when the total is an exact multiple of it.)
+    off += (size_t)round_up(8 * waves + (int64_t)sizeof(BlockPoolCtl), 64);
     return off;
 }
 

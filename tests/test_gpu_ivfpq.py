@@ -528,3 +528,16 @@ def test_few_heavy_workgroups_run_heaviest_first(ix, oracle):
     gpu.setNumProbes(1)
     gpu.search(q[:70], 20)
     assert gpu.last_search_stats()["ordered"] == 0
+
+
+def test_sixteen_wave_pool_with_an_lds_plan_that_fills_whole_allocation_granules(ix, oracle):
+    """M = 48 (64 KB LUT), d = 96, k = 1024 and 64 lists per workgroup make the scan's LDS plan end within
+    a few bytes of a multiple of 1280: the control words of the sixteen-wave pool must lie inside it."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 91, 30000, 2100, 96, 64, 48, ix.METRIC_L2)
+    gpu.setNumProbes(64)
+    D, I = gpu.search(q, 1024)
+    st = gpu.last_search_stats()
+    assert st["shared_pool"] == 1 and st["nsplit"] == 1 and st["scan_waves"] == 16
+    sub = slice(0, 2100, 21)
+    Dr, Ir = ref.search(q[sub], 1024, 64)
+    assert_topk_parity(oracle, ref, q[sub], D[sub], I[sub], Dr, Ir, TOL_FP32)
