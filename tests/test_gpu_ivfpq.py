@@ -519,12 +519,13 @@ def test_few_heavy_workgroups_run_heaviest_first(ix, oracle):
     results are those of the oracle, whatever the order)."""
     gpu, ref, x, q, ids = build_pair(ix, oracle, 81, 200000, 600, 32, 16, 8, ix.METRIC_L2, niter=3)
     gpu.setNumProbes(8)
-    D, I = gpu.search(q, 20)
-    st = gpu.last_search_stats()
-    assert st["ordered"] == 1 and st["nsplit"] > 1
-    Dr, Ir = ref.search(q, 20, 8)
-    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
-    assert st["scanned_codes"] == ref.last_scanned
+    for nq, split in ((600, False), (150, True)):      # one workgroup per query, and several
+        D, I = gpu.search(q[:nq], 20)
+        st = gpu.last_search_stats()
+        assert st["ordered"] == 1 and (st["nsplit"] > 1) == split
+        Dr, Ir = ref.search(q[:nq], 20, 8)
+        assert_topk_parity(oracle, ref, q[:nq], D, I, Dr, Ir, TOL_FP32)
+        assert st["scanned_codes"] == ref.last_scanned
     gpu.setNumProbes(1)
     gpu.search(q[:70], 20)
     assert gpu.last_search_stats()["ordered"] == 0
