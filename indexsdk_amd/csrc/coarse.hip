@@ -518,30 +518,54 @@ constexpr int kSelRegStage = 160;     // new candidates per wave and segment
 constexpr int kSelRegMaxK = 384;
 constexpr int kSelRegCap = kSelRegMaxK + 4 * kSelRegStage;   // 1024
 
-// dst[0 .. min(n, keep)) = the smallest keys of src[0 .. n) in ascending order.  n <= 1024, src is
-// 16-byte aligned with src[n] writable; all 256 threads call it; barriers inside.
-__device__ __forceinline__ void rank_select_256(key_t *src, int n, key_t *dst, int keep, int tid)
+// dst[0 .. min(n, keep)) = the smallest keys of src[0 .. n) in ascending order, by counting ranks (the
+// keys are distinct).  src[0 .. have) is already ascending: those keys know their rank among
+// themselves, the others find theirs among them by bisection, and only the n - have new keys are
+// counted against one by one.  n <= 1024, src is 16-byte aligned with src[n] writable; all 256
+// threads call it; barriers inside.
+__device__ __forceinline__ void rank_select_256(key_t *src, int have, int n, key_t *dst, int keep, int tid)
 {
+    const int first = have & ~1;              // new keys are read in aligned pairs from here on
     if (tid == 0 && (n & 1)) {
-        src[n] = kEmptyKey;   // never below a key
+        src[n] = kEmptyKey;                   // never below a key
     }
     __syncthreads();
     key_t mine[4];
     int rank[4];
+    const int owned = (n + 255 - tid) >> 8;   // entries tid, tid + 256, ... below n
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        mine[e] = tid + 256 * e < n ? src[tid + 256 * e] : 0;   // 0: rank stays 0 and is not used
-        rank[e] = 0;
+        const int i = tid + 256 * e;
+        mine[e] = i < n ? src[i] : 0;         // 0: its rank is not used
+        if (i < have) {
+            rank[e] = i - (first < have ? (src[first] < mine[e]) : 0);   // src[first] is counted again below
+        } else {
+            int lo = 0, hi = have;            // keys of the sorted part below mine
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (src[mid] < mine[e]) {
+                    lo = mid + 1;
+                } else {
+                    hi = mid;
+                }
+            }
+            rank[e] = lo - (first < have && first < lo ? 1 : 0);
+        }
     }
-    const int owned = (n + 255 - tid) >> 8;   // entries tid, tid + 256, ... below n
     const ulonglong2 *pairs = reinterpret_cast<const ulonglong2 *>(src);
     if (n <= 256) {
-        for (int f = 0; f < (n + 1) >> 1; f++) {
+        for (int f = first >> 1; f < (n + 1) >> 1; f++) {
             const ulonglong2 pr = pairs[f];   // same address in every lane: one broadcast read
             rank[0] += (pr.x < mine[0]) + (pr.y < mine[0]);
         }
+    } else if (n <= 512) {
+        for (int f = first >> 1; f < (n + 1) >> 1; f++) {
+            const ulonglong2 pr = pairs[f];
+            rank[0] += (pr.x < mine[0]) + (pr.y < mine[0]);
+            rank[1] += (pr.x < mine[1]) + (pr.y < mine[1]);
+        }
     } else {
-        for (int f = 0; f < (n + 1) >> 1; f++) {
+        for (int f = first >> 1; f < (n + 1) >> 1; f++) {
             const ulonglong2 pr = pairs[f];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -731,7 +755,7 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
                 cand[before + i] = stage[wave * kSelRegStage + i];
             }
             const int n = have + total;
-            rank_select_256(cand, n, best, ksel, tid);
+            rank_select_256(cand, have, n, best, ksel, tid);
             have = n < ksel ? n : ksel;
             for (int i = tid; i < have; i += 256) {
                 cand[i] = best[i];
