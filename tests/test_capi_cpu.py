@@ -28,7 +28,7 @@ def capi():
     return _capi
 
 
-def test_header_declares_the_survey_boundary():
+def test_header_declares_the_index_level_boundary():
     names = declared_functions()
     for need in ["ivfpq_create", "ivfpq_destroy", "ivfpq_train", "ivfpq_set_trained", "ivfpq_add_with_ids",
                  "ivfpq_add_codes", "ivfpq_set_nprobe", "ivfpq_get_nprobe", "ivfpq_search", "ivfpq_assign",
