@@ -125,6 +125,16 @@ def load():
         if not os.path.exists(LIB_PATH):
             raise OSError(f"{LIB_PATH} is missing: build it with indexsdk_amd/csrc/build.sh "
                           "(there is no CPU fallback)")
+        # PyTorch-ROCm brings its own copy of the HIP runtime: when it initialises after this library has
+        # started the system's runtime, torch.cuda reports no GPU.  If the caller has imported torch
+        # already, let it start first (it costs nothing when it has).
+        import sys
+        torch = sys.modules.get("torch")
+        if torch is not None and hasattr(torch, "cuda") and torch.cuda.device_count() > 0:
+            try:
+                torch.cuda.init()
+            except Exception:
+                pass
         lib = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(lib, name)

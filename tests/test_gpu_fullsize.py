@@ -1,0 +1,103 @@
+"""The headline configuration at its full size (10M x 128, nlist 16384, M 32, 10000 queries, nprobe 64,
+k 100) through properties that do not need a full-size reference run, plus oracle parity on a sample of
+the queries against the index copied back to the host."""
+import numpy as np
+import pytest
+
+from tests.parity import assert_topk_parity
+
+pytestmark = pytest.mark.gpu
+
+N, D, NLIST, M, NQ, NPROBE, K = 10_000_000, 128, 16384, 32, 10_000, 64, 100
+
+
+@pytest.fixture(scope="module")
+def big():
+    import indexsdk_amd as ix
+    rng = np.random.default_rng(1236)
+    centres = rng.standard_normal((1024, D), dtype=np.float32)
+
+    def draw(n):
+        x = rng.standard_normal((n, D), dtype=np.float32)
+        x *= np.float32(0.25)
+        x += centres[rng.integers(0, 1024, n)]
+        return x
+
+    cfg = ix.AscendIndexIVFPQConfig(niter=4, train_samples_per_list=1 << 20)
+    index = ix.AscendIndexIVFPQ(D, ix.METRIC_L2, NLIST, M, 8, cfg)
+    index.train(draw(500_000))
+    keep = {}
+    for c in range(10):
+        x = draw(N // 10)
+        if c == 3:
+            keep["rows"] = x[:2000].copy()                  # database vectors used as queries later
+            keep["first_id"] = c * (N // 10)
+        index.add(x)
+    del x
+    q = draw(NQ)
+    index.setNumProbes(NPROBE)
+    return ix, index, q, keep
+
+
+def test_full_size_result_properties(big):
+    ix, index, q, keep = big
+    assert index.ntotal == N
+    lens = np.array([index.getListLength(l) for l in range(NLIST)], dtype=np.int64)
+    assert lens.sum() == N
+    Dm, Im = index.search(q, K)
+    st = index.last_search_stats()
+    assert (Im >= 0).all() and (Im < N).all()
+    assert (np.diff(Dm, axis=1) >= 0).all()                                   # best first
+    assert (np.diff(np.sort(Im, axis=1), axis=1) > 0).all()                   # no id twice
+    # idempotence, and k = 10 is a prefix of k = 100
+    D2, I2 = index.search(q, K)
+    assert np.array_equal(I2, Im) and np.array_equal(D2.view(np.uint32), Dm.view(np.uint32))
+    D10, I10 = index.search(q, 10)
+    assert np.array_equal(I10, Im[:, :10]) and np.array_equal(D10.view(np.uint32), Dm[:, :10].view(np.uint32))
+    # the scanned-code count is the sum of the probed lists' lengths
+    probes, _ = index.coarse_probe(q)
+    assert st["scanned_codes"] == lens[probes].sum()
+    # fewer probes can only make the k-th distance worse
+    index.setNumProbes(16)
+    D16, _ = index.search(q, K)
+    index.setNumProbes(NPROBE)
+    assert (D16[:, K - 1] >= Dm[:, K - 1]).all()
+
+
+def test_full_size_self_queries_come_back_first(big):
+    """A database vector's own code minimises every term of its ADC sum, and its own list is its first
+    probe: it is the top result unless another vector of a probed list has the same code
+    (FR/test/ascend/TestAscendIndexIVFPQ.cpp:150-166)."""
+    ix, index, q, keep = big
+    rows, first = keep["rows"], keep["first_id"]
+    Ds, Is = index.search(rows, 5)
+    own = np.arange(first, first + len(rows))
+    hit = Is[:, 0] == own
+    assert hit.mean() > 0.995
+    # where another id came first it ties with the vector's own entry
+    for i in np.flatnonzero(~hit):
+        pos = np.flatnonzero(Is[i] == own[i])
+        assert len(pos) == 1 and Ds[i, pos[0]] == Ds[i, 0]
+
+
+def test_full_size_sample_against_the_oracle(big, oracle):
+    ix, index, q, keep = big
+    cent, cb = index.get_trained()
+    lens = np.array([index.getListLength(l) for l in range(NLIST)], dtype=np.int64)
+    off = np.zeros(NLIST + 1, dtype=np.int64)
+    np.cumsum(lens, out=off[1:])
+    codes = np.empty((N, M), dtype=np.uint8)
+    ids = np.empty(N, dtype=np.int64)
+    for l in range(NLIST):
+        if lens[l]:
+            codes[off[l]:off[l + 1]], ids[off[l]:off[l + 1]] = index.getListCodesAndIds(l)
+    assert np.array_equal(np.sort(ids), np.arange(N))
+    ref = oracle.CsrIndex(D, M, ix.METRIC_L2, cent, cb, off, codes, ids)
+    sample = q[::50]
+    Dg, Ig = index.search(sample, K)
+    Dr, Ir = ref.search(sample, K, NPROBE)
+    exempt = assert_topk_parity(oracle, ref, sample, Dg, Ig, Dr, Ir, 1e-4)
+    assert exempt <= 0.002 * Ig.size + 5
+    pi, pd = index.coarse_probe(sample)
+    oi, od = oracle.coarse_probe(sample, cent, NPROBE, ix.METRIC_L2)
+    assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
