@@ -101,3 +101,37 @@ def test_full_size_sample_against_the_oracle(big, oracle):
     pi, pd = index.coarse_probe(sample)
     oi, od = oracle.coarse_probe(sample, cent, NPROBE, ix.METRIC_L2)
     assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
+
+
+def test_full_size_flat_int8_exact(oracle):
+    """Flat int8 at its full size (10M x 512, 2048 queries, k 100): every returned distance is the exact
+    integer distance of the returned id, rows are ordered by (distance, id), planted copies of base
+    vectors come back at distance 0, and a sample of the queries equals brute force over the whole base."""
+    import indexsdk_amd as ix
+    n, d, nq, k = 10_000_000, 512, 2048, 100
+    rng = np.random.default_rng(1238)
+    index = ix.AscendIndexInt8Flat(d)
+    chunks = []
+    for c in range(10):
+        b = rng.integers(-127, 128, size=(n // 10, d), dtype=np.int8)
+        index.add(b)
+        chunks.append(b)
+    base = np.concatenate(chunks)
+    del chunks
+    q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    planted = rng.integers(0, n, 64)
+    q[:64] = base[planted]
+    Dg, Ig = index.search_int32(q, k)
+    assert index.ntotal == n and (Ig >= 0).all() and (Ig < n).all()
+    assert (Dg[:64, 0] == 0).all() and (Ig[:64, 0] == planted).all()
+    # ordered by (distance, id); no id twice
+    dd, di = np.diff(Dg, axis=1), np.diff(Ig, axis=1)
+    assert ((dd > 0) | ((dd == 0) & (di > 0))).all()
+    # returned distances are the exact integer distances of the returned ids (a sample of rows)
+    for i in range(0, nq, 97):
+        diff = base[Ig[i]].astype(np.int32) - q[i].astype(np.int32)
+        assert np.array_equal((diff * diff).sum(axis=1), Dg[i])
+    # brute force over the whole base for a few queries
+    sample = np.arange(0, nq, 128)
+    Dr, Ir = oracle.flat_i8(base, q[sample], k)
+    assert np.array_equal(Ig[sample], Ir) and np.array_equal(Dg[sample], Dr)
