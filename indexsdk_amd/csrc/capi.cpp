@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <cstring>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -18,7 +19,12 @@ std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig
 }  // namespace ixa
 
 // The handle owns the index through a pointer so that a loader can hand over a finished one.
+// Every call on a handle holds the handle's mutex: the reference guards an index with one shared_mutex
+// when MX_INDEX_MULTITHREAD is set (FR/ascend/impl/AscendIndexImpl.h:62, 230); here calls on one index
+// are always serialised (a search uses the index's workspace and stream), calls on different indexes
+// run concurrently.
 struct ivfpq_index {
+    mutable std::mutex mu;
     std::unique_ptr<ixa::IvfpqIndex> owned;
     ixa::IvfpqIndex &impl;
     ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
@@ -29,10 +35,12 @@ struct ivfpq_index {
 };
 
 struct flat_index {
+    mutable std::mutex mu;
     ixa::FlatIndex impl;
     flat_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
 };
 struct flat_i8_index {
+    mutable std::mutex mu;
     ixa::FlatI8Index impl;
     flat_i8_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
 };
@@ -59,7 +67,9 @@ int guarded(F &&f)
     }
 }
 
-#define IXA_HANDLE(h) IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.")
+#define IXA_HANDLE(h)                                                                             \
+    IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.");      \
+    std::lock_guard<std::mutex> ixa_handle_lock((h)->mu)
 
 ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
 {

@@ -542,3 +542,26 @@ def test_sixteen_wave_pool_with_an_lds_plan_that_fills_whole_allocation_granules
     sub = slice(0, 2100, 21)
     Dr, Ir = ref.search(q[sub], 1024, 64)
     assert_topk_parity(oracle, ref, q[sub], D[sub], I[sub], Dr, Ir, TOL_FP32)
+
+
+def test_concurrent_callers_of_one_index_are_serialised(ix, oracle):
+    """Searches from several threads on the same index (ctypes releases the GIL): every call holds the
+    handle's lock, so each thread gets the result a lone caller gets
+    (FR/ascend/impl/AscendIndexImpl.h:62, 230: the reference's optional per-index lock)."""
+    import threading
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 93, 20000, 400, 64, 32, 16, ix.METRIC_L2)
+    gpu.setNumProbes(8)
+    want = [gpu.search(q[i::4], 10 + i) for i in range(4)]
+    got = [None] * 4
+
+    def work(i):
+        for _ in range(5):
+            got[i] = gpu.search(q[i::4], 10 + i)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for i in range(4):
+        assert np.array_equal(got[i][1], want[i][1]) and np.array_equal(got[i][0].view(np.uint32), want[i][0].view(np.uint32))
