@@ -10,9 +10,9 @@ def rel_close(a, b, tol):
     return np.abs(a - b) <= tol * np.maximum(np.maximum(np.abs(a), np.abs(b)), 1e-30)
 
 
-def candidate_distances(orc, idx, q_row, ids):
+def candidate_distances(orc, idx, q_row, ids, lut_fp16=False):
     """Oracle ADC distance of arbitrary database ids for one query (for the tie exemption)."""
-    lut = orc.lut(q_row[None, :], idx.codebook, idx.metric)[0]
+    lut = orc.lut(q_row[None, :], idx.codebook, idx.metric, lut_fp16=lut_fp16)[0]
     pos = {int(v): i for i, v in enumerate(idx.ids)}
     out = []
     for i in ids:
@@ -20,11 +20,13 @@ def candidate_distances(orc, idx, q_row, ids):
     return np.array(out, dtype=np.float32)
 
 
-def assert_topk_parity(orc, idx, q, D_gpu, I_gpu, D_ref, I_ref, tol):
+def assert_topk_parity(orc, idx, q, D_gpu, I_gpu, D_ref, I_ref, tol, lut_fp16=None):
     """Position-wise id equality; a mismatch is accepted only between candidates whose oracle
     distances tie within ``tol`` (relative), including across the k-th boundary.  Distances at
     equal rank must agree within ``tol``.  Returns the number of exempted positions."""
     assert D_gpu.shape == D_ref.shape and I_gpu.shape == I_ref.shape
+    if lut_fp16 is None:
+        lut_fp16 = tol > 1e-3          # the fp16-LUT tests are the ones that use the wide tolerance
     # padding must be identical
     assert np.array_equal(I_gpu == -1, I_ref == -1), "padding differs"
     pad = I_ref == -1
@@ -36,7 +38,7 @@ def assert_topk_parity(orc, idx, q, D_gpu, I_gpu, D_ref, I_ref, tol):
         bad = np.flatnonzero(I_gpu[qi] != I_ref[qi])
         # each id the GPU reports there must be a real candidate whose oracle distance ties with
         # the oracle's entry at that rank
-        d_or = candidate_distances(orc, idx, q[qi], I_gpu[qi, bad])
+        d_or = candidate_distances(orc, idx, q[qi], I_gpu[qi, bad], lut_fp16)
         assert rel_close(d_or, D_ref[qi, bad], tol).all(), f"query {qi}: non-tied id mismatch at ranks {bad}"
         assert len(set(I_gpu[qi][I_gpu[qi] >= 0].tolist())) == (I_gpu[qi] >= 0).sum(), "duplicate ids"
         exempt += len(bad)
