@@ -126,3 +126,103 @@ def test_coarse_probe_sweep(oracle, seed, d, nlist, nprobe, nq, metric_l2, near_
     assert np.array_equal(gi, oi)
     assert np.array_equal(gd.view(np.uint32), od.view(np.uint32))
     assert np.array_equal(gpu.assign(q), oracle.assign(q, cent))
+
+
+@pytest.mark.parametrize("d,M,fp16", [(64, 16, 0), (64, 32, 0), (96, 48, 0), (192, 96, 1), (128, 64, 0)])
+def test_write_side_random_sequences_against_a_host_model(oracle, d, M, fp16):
+    """Random sequences of add, remove, update, add_codes and a file round trip, mirrored in a plain host
+    model of the inverted lists (reference encoder, input order inside a list, survivors keep their
+    order): after every step lists read back equal the model, under every code layout (row, rot32,
+    xor48) whose byte order depends on the position inside the list."""
+    import os
+    import tempfile
+    import indexsdk_amd as ix
+    rng = np.random.default_rng(d * 7 + M)
+    nlist = 12
+    centres = rng.standard_normal((20, d)).astype(np.float32)
+
+    def draw(n):
+        return (centres[rng.integers(0, 20, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+
+    x0 = draw(4000)
+    cent, _ = oracle.kmeans(x0, nlist, niter=3, seed=3)
+    cb = oracle.train_pq(x0, M, niter=2, seed=3)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(lut_fp16=fp16))
+    gpu.set_trained(cent, cb)
+    lists = [([], []) for _ in range(nlist)]          # per list: ids, codes (rows)
+    next_id = [1000]
+
+    def fresh_ids(n):
+        out = np.arange(next_id[0], next_id[0] + n, dtype=np.int64) * 3 + 1
+        next_id[0] += n
+        return out
+
+    def model_add(x, ids):
+        asg = oracle.assign(x, cent)
+        codes = oracle.pq_encode(x, cb)
+        for i in range(len(ids)):
+            lists[asg[i]][0].append(int(ids[i]))
+            lists[asg[i]][1].append(codes[i])
+
+    def model_remove(victims):
+        vs = set(int(v) for v in victims)
+        n = 0
+        for l in range(nlist):
+            keep = [j for j, v in enumerate(lists[l][0]) if v not in vs]
+            n += len(lists[l][0]) - len(keep)
+            lists[l] = ([lists[l][0][j] for j in keep], [lists[l][1][j] for j in keep])
+        return n
+
+    def check(which):
+        assert gpu.ntotal == sum(len(l[0]) for l in lists)
+        for l in which:
+            codes, lid = gpu.getListCodesAndIds(l)
+            assert lid.tolist() == lists[l][0], f"list {l}: ids differ"
+            want = np.array(lists[l][1], dtype=np.uint8).reshape(-1, M)
+            assert np.array_equal(codes, want), f"list {l}: codes differ"
+
+    for step in range(14):
+        op = ["add", "add", "remove", "update", "add_codes", "file"][int(rng.integers(0, 6))] if step else "add"
+        present = np.array([v for l in lists for v in l[0]], dtype=np.int64)
+        if op == "add":
+            n = int(rng.integers(1, 1500))
+            x, ids = draw(n), fresh_ids(n)
+            gpu.add_with_ids(x, ids)
+            model_add(x, ids)
+        elif op == "remove" and len(present):
+            victims = np.concatenate([rng.choice(present, min(len(present), int(rng.integers(1, 400))), replace=False),
+                                      np.array([7, 8], dtype=np.int64)])          # two ids that do not exist
+            assert gpu.remove_ids(victims) == model_remove(victims)
+        elif op == "update" and len(present):
+            ids = np.concatenate([rng.choice(present, min(len(present), int(rng.integers(1, 150))), replace=False),
+                                  np.array([5], dtype=np.int64)])
+            x = draw(len(ids))
+            missing = gpu.update(x, ids)
+            assert missing.tolist() == [5]
+            model_remove(ids[:-1])
+            model_add(x[:-1], ids[:-1])
+        elif op == "add_codes":
+            l, n = int(rng.integers(0, nlist)), int(rng.integers(1, 90))
+            codes = rng.integers(0, 256, size=(n, M), dtype=np.uint8)
+            ids = fresh_ids(n)
+            gpu.add_codes(l, codes, ids)
+            lists[l][0].extend(int(v) for v in ids)
+            lists[l][1].extend(list(codes))
+        elif op == "file":
+            with tempfile.TemporaryDirectory() as tmp:
+                path = os.path.join(tmp, "index.faiss")
+                gpu.write_faiss(path)
+                gpu = ix.AscendIndexIVFPQ.read_faiss(path, ix.AscendIndexIVFPQConfig(lut_fp16=fp16))
+        check(rng.choice(nlist, 4, replace=False))
+    check(range(nlist))
+    # the lists as they stand, searched: parity with the oracle on the model's content
+    off = np.zeros(nlist + 1, dtype=np.int64)
+    np.cumsum([len(l[0]) for l in lists], out=off[1:])
+    codes = np.concatenate([np.array(l[1], dtype=np.uint8).reshape(-1, M) for l in lists])
+    ids = np.concatenate([np.array(l[0], dtype=np.int64) for l in lists])
+    ref = oracle.CsrIndex(d, M, ix.METRIC_L2, cent, cb, off, codes, ids)
+    q = draw(60)
+    gpu.setNumProbes(5)
+    D, I = gpu.search(q, 30)
+    Dr, Ir = ref.search(q, 30, 5, lut_fp16=bool(fp16))
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, 1e-2 if fp16 else 1e-4)
