@@ -226,3 +226,28 @@ def test_write_side_random_sequences_against_a_host_model(oracle, d, M, fp16):
     D, I = gpu.search(q, 30)
     Dr, Ir = ref.search(q, 30, 5, lut_fp16=bool(fp16))
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, 1e-2 if fp16 else 1e-4)
+
+
+def test_search_with_more_queries_than_one_coarse_block(oracle):
+    """40000 queries: the coarse stage walks them in blocks of 16384 rows (the score scratch never holds
+    more), the scan takes them in one launch."""
+    import indexsdk_amd as ix
+    d, M, nlist, nq, nprobe, k = 32, 8, 4100, 40000, 6, 10
+    rng = np.random.default_rng(31)
+    centres = rng.standard_normal((50, d)).astype(np.float32)
+    cent = (centres[rng.integers(0, 50, nlist)] + 0.5 * rng.standard_normal((nlist, d))).astype(np.float32)
+    x = (centres[rng.integers(0, 50, 60000)] + 0.5 * rng.standard_normal((60000, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 50, nq)] + 0.5 * rng.standard_normal((nq, d))).astype(np.float32)
+    cb = oracle.train_pq(x[:5000], M, niter=2, seed=1)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add(x)
+    gpu.setNumProbes(nprobe)
+    D, I = gpu.search(q, k)
+    gi, gd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
+    assert np.array_equal(gi, oi) and np.array_equal(gd.view(np.uint32), od.view(np.uint32))
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, np.arange(60000, dtype=np.int64))
+    Dr, Ir = ref.search(q, k, nprobe)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, 1e-4)
+    assert gpu.last_search_stats()["scanned_codes"] == ref.last_scanned
