@@ -132,8 +132,8 @@ def run_flat_i8(args, torch, ix, _capi, lib):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"],
                     help="benchmark configuration; C2 (default) is the one the metric is quoted on")
     ap.add_argument("--n", type=int, default=0, help="override the number of base vectors")
