@@ -50,8 +50,11 @@ namespace {
 thread_local std::string g_last_error;
 
 template <typename F>
-int guarded(F &&f)
+int guarded(F &&f, bool uses_gpu = true)
 {
+    if (uses_gpu) {
+        (void)hipGetLastError();   // an error some earlier caller on this thread left behind is not this call's
+    }
     try {
         f();
         return IXA_OK;
@@ -63,6 +66,9 @@ int guarded(F &&f)
         return IXA_ERR_BAD_ALLOC;
     } catch (const std::exception &e) {
         g_last_error = e.what();
+        return IXA_ERR_INNER_ERROR;
+    } catch (...) {   // nothing may unwind through a C caller
+        g_last_error = "unknown exception";
         return IXA_ERR_INNER_ERROR;
     }
 }
@@ -394,7 +400,7 @@ IXA_EXPORT int ixa_merge_search_results(int ndev, int64_t n, int64_t k, int metr
                 settle(from);
             }
         }
-    });
+    }, false);
 }
 IXA_EXPORT int ixa_op_distance_flat_l2_mins_fp32(const float *queries_dev, int64_t batch, const float *codes_dev,
                                                  int64_t n, int d, const float *codes_sqr_sum_dev, float *dist_dev,

@@ -59,6 +59,15 @@ struct Error : std::runtime_error {
         }                                                                                               \
     } while (0)
 
+// Waits for the stream.  A launch the device rejects (a grid or LDS size it cannot run) is reported by
+// no later call except hipGetLastError, so that is asked first: a kernel that never ran must not pass
+// for one that did.
+inline void sync_stream(hipStream_t s)
+{
+    IXA_HIP(hipGetLastError());
+    IXA_HIP(hipStreamSynchronize(s));
+}
+
 // Owning device allocation.  Grows by reallocation (contents are NOT preserved by reserve()).
 template <typename T>
 class DeviceBuffer {
@@ -117,7 +126,7 @@ public:
     {
         if (n) {
             IXA_HIP(hipMemcpyAsync(host, p_, n * sizeof(T), hipMemcpyDeviceToHost, s));
-            IXA_HIP(hipStreamSynchronize(s));
+            sync_stream(s);
         }
     }
 

@@ -328,6 +328,7 @@ void launch_copy_probe(const void *src, void *dst, int64_t bytes)
     IXA_REQUIRE(src && dst && bytes > 0 && bytes % 16 == 0, kErrInvalidParam, "copy probe needs a multiple of 16 bytes");
     hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 16), dim3(256), 0, nullptr, static_cast<const uint4 *>(src),
                        static_cast<uint4 *>(dst), bytes / 16);
+    IXA_HIP(hipGetLastError());
     IXA_HIP(hipDeviceSynchronize());
 }
 
@@ -379,7 +380,7 @@ void FlatBase<T>::reserve(int64_t n)
         IXA_HIP(hipMemcpyAsync(nb.data(), base_.data(), (size_t)ntotal_ * d_ * sizeof(T), hipMemcpyDeviceToDevice,
                                stream_));
         IXA_HIP(hipMemcpyAsync(ni.data(), ids_.data(), (size_t)ntotal_ * 8, hipMemcpyDeviceToDevice, stream_));
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
     }
     base_ = std::move(nb);
     ids_ = std::move(ni);
@@ -402,7 +403,7 @@ void FlatBase<T>::add(int64_t n, const T *x, const int64_t *ids, bool on_device)
         hipLaunchKernelGGL(iota_ids_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, ids_.data() + ntotal_, n,
                            ntotal_);
     }
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     ntotal_ += n;
 }
 
@@ -414,7 +415,7 @@ void FlatBase<T>::get_base(int64_t offset, int64_t n, T *out) const
     if (n) {
         IXA_HIP(hipMemcpyAsync(out, base_.data() + offset * d_, (size_t)n * d_ * sizeof(T), hipMemcpyDeviceToHost,
                                stream_));
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
     }
 }
 
@@ -425,14 +426,14 @@ void FlatBase<T>::get_ids(int64_t offset, int64_t n, int64_t *out) const
                 "range [%ld, %ld) is outside the index (ntotal %ld)", (long)offset, (long)(offset + n), (long)ntotal_);
     if (n) {
         IXA_HIP(hipMemcpyAsync(out, ids_.data() + offset, (size_t)n * 8, hipMemcpyDeviceToHost, stream_));
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
     }
 }
 
 template <typename T>
 void FlatBase<T>::reset()
 {
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     base_.release();
     ids_.release();
     ntotal_ = capacity_ = 0;
@@ -504,7 +505,7 @@ void FlatIndex::exact_rows(const float *xd, const std::vector<int64_t> &rows, in
         hipLaunchKernelGGL(scatter_result_rows_kernel, dim3(blocks_for(m * k)), dim3(256), 0, stream_, dsub.data(),
                            lsub.data(), rows_dev.data() + r0, m, (int)k, dist_dev, labels_dev);
     }
-    IXA_HIP(hipStreamSynchronize(stream_));   // the temporaries above are freed on return
+    sync_stream(stream_);   // the temporaries above are freed on return
 }
 
 void FlatIndex::reset()
@@ -568,14 +569,14 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
         if (nfail > 0) {
             std::vector<int32_t> rows32((size_t)nfail);
             IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
-            IXA_HIP(hipStreamSynchronize(stream_));
+            sync_stream(stream_);
             std::sort(rows32.begin(), rows32.end());
             exact_rows(xd, std::vector<int64_t>(rows32.begin(), rows32.end()), k, dd, ld);
             stats_.exact_reruns = nfail;
         }
     }
     IXA_HIP(hipEventRecord(ev_[2], stream_));
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     if (!on_device) {
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);
@@ -607,7 +608,7 @@ void FlatI8Index::add(int64_t n, const int8_t *x, const int64_t *ids, bool on_de
     }
     hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_,
                        base_.data() + before * d_, n, d_, nn.data() + before);
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     norms_ = std::move(nn);
 }
 
@@ -645,7 +646,7 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,
                        ws_running_.data(), n * k, kMetricL2, ids_.data(), (int32_t)0x7fffffff, dd, ld);
     IXA_HIP(hipEventRecord(ev_[1], stream_));
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     if (!on_device) {
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);

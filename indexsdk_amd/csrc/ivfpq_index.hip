@@ -225,6 +225,18 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
     out[e] = x[idx[e / d] * d + e % d];
 }
 
+// probe lists handed in by a caller: anything that is not a list id becomes -1 ("no list"), so that no
+// later kernel indexes the list tables with it
+__global__ __launch_bounds__(256) void sanitize_probes_kernel(const int32_t *__restrict__ in, int64_t n, int32_t nlist,
+                                                              int32_t *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e < n) {
+        const int32_t l = in[e];
+        out[e] = (l >= 0 && l < nlist) ? l : -1;
+    }
+}
+
 inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
 
 }  // namespace
@@ -301,7 +313,7 @@ void IvfpqIndex::sync_list_tables()
     max_list_len_ = list_len_.empty() ? 0 : *std::max_element(list_len_.begin(), list_len_.end());
     list_off_dev_.upload(list_off_.data(), (size_t)nlist_, stream_);
     list_len_dev_.upload(list_len_.data(), (size_t)nlist_, stream_);
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
 }
 
 // Centroid and codeword norms are produced on the device in the same left-to-right fp32 order the
@@ -324,7 +336,7 @@ void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
         cbnorm_.resize((size_t)M_ * 256);
         launch_sqnorm_rows(codebook_.data(), (int64_t)M_ * 256, dsub_, cbnorm_.data(), stream_);
     }
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
 }
 
 void IvfpqIndex::set_trained(const float *centroids, const float *codebook)
@@ -379,7 +391,7 @@ void IvfpqIndex::coarse_exact_rows(const float *x_dev, const std::vector<int64_t
         hipLaunchKernelGGL(scatter_rows_kernel, dim3(blocks_for(mr * nout)), dim3(256), 0, stream_, idx.data(),
                            out_dist ? dist.data() : nullptr, rows_dev.data() + r0, mr, nout, out_ids, out_dist);
     }
-    IXA_HIP(hipStreamSynchronize(stream_));   // the temporaries above are freed on return
+    sync_stream(stream_);   // the temporaries above are freed on return
 }
 
 // Candidate generation with matrix-core products -- bf16 x 3 (error bound below, 16 spare candidates)
@@ -479,7 +491,7 @@ int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, i
     std::vector<int32_t> rows32((size_t)nfail);
     IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
     IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     flag_pending_ = false;
     std::sort(rows32.begin(), rows32.end());   // the order of the appends is not deterministic
     coarse_exact_rows(x_dev, std::vector<int64_t>(rows32.begin(), rows32.end()), nout, select_metric, out_ids, out_dist);
@@ -631,7 +643,7 @@ void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *co
 {
     std::vector<int32_t> list_no((size_t)n), pos((size_t)n);
     IXA_HIP(hipMemcpyAsync(list_no.data(), list_no_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream_));
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     std::vector<int32_t> new_len(list_len_);
     for (int64_t i = 0; i < n; i++) {
         const int32_t l = list_no[(size_t)i];
@@ -660,7 +672,7 @@ void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *co
     }
     hipLaunchKernelGGL(scatter_new_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, n, list_no_dev, pos_dev.data(),
                        codes_dev, ids_dev, ntotal_, new_off_dev.data(), M_, layout_, new_codes.data(), new_ids.data());
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     codes_ = std::move(new_codes);
     ids_ = std::move(new_ids);
     list_off_ = std::move(new_off);
@@ -692,7 +704,7 @@ void IvfpqIndex::get_list(int64_t list, uint8_t *codes, int64_t *ids) const
     }
     if (ids) {
         IXA_HIP(hipMemcpyAsync(ids, ids_.data() + off, (size_t)len * 8, hipMemcpyDeviceToHost, stream_));
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
     }
 }
 
@@ -709,7 +721,7 @@ int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
     std::unordered_set<int64_t> del(ids, ids + n);
     std::vector<int64_t> all_ids((size_t)total_slots_);
     IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     std::vector<int32_t> keep_list;
     std::vector<int64_t> keep_ids;
     std::vector<uint8_t> keep_codes, buf;
@@ -765,7 +777,7 @@ std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t
     if (ntotal_ > 0) {
         std::vector<int64_t> all_ids((size_t)total_slots_);
         IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
         for (int64_t l = 0; l < nlist_; l++) {
             const int64_t off = list_off_[(size_t)l];
             for (int64_t i = 0; i < list_len_[(size_t)l]; i++) {
@@ -794,7 +806,7 @@ std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t
 void IvfpqIndex::reset()
 {
     flush_stats();
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
     codes_.release();
     ids_.release();
     list_off_.assign((size_t)nlist_ + 1, 0);
@@ -872,9 +884,12 @@ void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *pro
     IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
     IXA_REQUIRE(nprobe > 0 && nprobe <= nlist_, kErrInvalidParam, "nprobe must be > 0 and <= nlist");
     flush_stats();
-    ScanParams p = scan_params(x_dev, n, probes_dev, nprobe, k, dist_dev, labels_dev);
+    ws_probes_.resize((size_t)n * nprobe);
+    hipLaunchKernelGGL(sanitize_probes_kernel, dim3(blocks_for(n * nprobe)), dim3(256), 0, stream_, probes_dev,
+                       n * nprobe, (int32_t)nlist_, ws_probes_.data());
+    ScanParams p = scan_params(x_dev, n, ws_probes_.data(), nprobe, k, dist_dev, labels_dev);
     launch_scan(p, n, stream_);
-    IXA_HIP(hipStreamSynchronize(stream_));
+    sync_stream(stream_);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -930,7 +945,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);
     } else {
-        IXA_HIP(hipStreamSynchronize(stream_));
+        sync_stream(stream_);
     }
     stats_.scan_launches = nsplit > 1 ? 2 : 1;
     stats_.nsplit = nsplit;

@@ -116,6 +116,7 @@ void op_distance_flat_l2_mins_fp32(const float *queries, int64_t batch, const fl
     const int64_t bursts = (n + 63) / 64;
     hipLaunchKernelGGL(op_distance_l2_mins_kernel, dim3((unsigned)((bursts + 3) / 4), (unsigned)batch), dim3(256), 0, s,
                        queries, batch, codes, n, d, codes_sqr_sum, dist, mins);
+    IXA_HIP(hipGetLastError());
 }
 
 void op_ivfpq_subspace_distance(const float *queries, int64_t batch, int d, const float *codebook, int M, int metric,
@@ -130,6 +131,7 @@ void op_ivfpq_subspace_distance(const float *queries, int64_t batch, int d, cons
     }
     hipLaunchKernelGGL(op_subspace_distance_kernel, dim3((unsigned)M, (unsigned)batch), dim3(256), 0, s, queries, batch,
                        d, codebook, M, d / M, metric, lut);
+    IXA_HIP(hipGetLastError());
 }
 
 void op_topk_flat_fp32(const float *dists, int64_t batch, int64_t n, int64_t ld, int k, float *out_dist,
@@ -145,6 +147,7 @@ void op_topk_flat_fp32(const float *dists, int64_t batch, int64_t n, int64_t ld,
     launch_select_rows(dists, batch, ld, n, k, nullptr, 0, reinterpret_cast<unsigned long long *>(out_label), s, true);
     hipLaunchKernelGGL(op_topk_finish_kernel, dim3((unsigned)((batch * k + 255) / 256)), dim3(256), 0, s, out_label,
                        out_dist, batch * k);
+    IXA_HIP(hipGetLastError());
 }
 
 }  // namespace ixa

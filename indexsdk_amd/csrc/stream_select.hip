@@ -210,7 +210,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
         }
         int ovf = 0;
         IXA_HIP(hipMemcpyAsync(&ovf, overflow, sizeof(int), hipMemcpyDeviceToHost, s));
-        IXA_HIP(hipStreamSynchronize(s));
+        sync_stream(s);
         if (!ovf) {
             break;
         }

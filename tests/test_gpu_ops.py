@@ -160,9 +160,12 @@ def test_operators_chained_equal_the_fused_search(env, oracle):
     assert np.array_equal(I2.get(), I) and np.array_equal(D2.get().view(np.uint32), D.view(np.uint32))
     Dr, Ir = ref.search(q, k, nprobe)
     assert_topk_parity(oracle, ref, q, D2.get(), I2.get(), Dr, Ir, 1e-4)
-    # a probe list with holes: -1 entries are skipped
+    # a probe list with holes: -1 entries, and values that name no list, are skipped
     holes = probes_h.copy()
     holes[:, ::2] = -1
+    holes[:, ::4] = nlist
+    holes[0, 0] = 2 ** 31 - 1
+    holes[1, 0] = -(2 ** 31)
     _capi.check(lib.ivfpq_search_probes_device(gpu._h, nq, _p(dq), _p(hip.put(holes)), nprobe, k, _p(D2), _p(I2)))
     keep = np.ascontiguousarray(probes_h[:, 1::2])
     D3 = hip.empty((nq, k), np.float32)
