@@ -132,6 +132,23 @@ def test_search_ip_fp16_lut(ix, oracle):
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP16)
 
 
+def test_search_ip_sums_that_cancel_to_almost_nothing(ix, oracle):
+    """Inner product with one dimension per sub-quantizer: 96 terms of both signs, many results within
+    1e-4 of zero.  There the association order of the fp32 sum shows at the scale of the terms, which is
+    what the parity rule measures against; ids and ranks still have to match."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 31241, 300, 65, 96, 16, 96, ix.METRIC_INNER_PRODUCT, niter=2)
+    gpu.setNumProbes(16)
+    D, I = gpu.search(q, 1000)
+    Dr, Ir = ref.search(q, 1000, 16)
+    assert (np.abs(Dr[:, :300]) < 1e-4).sum() > 20           # the case is what it claims to be
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    # the rule is no blank cheque: an error of 1e-3 of the terms' scale is still caught
+    Dbad = D.copy()
+    Dbad[0, 5] += 1e-3
+    with pytest.raises(AssertionError):
+        assert_topk_parity(oracle, ref, q, Dbad, I, Dr, Ir, TOL_FP32)
+
+
 def test_search_sentinels_k_larger_than_candidates(ix, oracle):
     gpu, ref, x, q, ids = build_pair(ix, oracle, 25, 600, 20, 64, 32, 8, ix.METRIC_L2)
     gpu.setNumProbes(2)

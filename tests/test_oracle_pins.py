@@ -329,3 +329,32 @@ def test_merge_results_skips_invalid_labels_anywhere_and_pads(oracle):
     got_d, got_l = oracle.merge_results(d[:, :, ::-1].copy(), lab[:, :, ::-1].copy(), oracle.METRIC_INNER_PRODUCT)
     assert got_l.tolist() == [[12, 21, 10, -1]]
     assert got_d.tolist() == [[3.0, 2.0, 1.0, float(FLT_MAX)]]
+
+
+def test_parity_rule_measures_cancelling_sums_against_their_terms(oracle):
+    """tests/parity.py: term_scale is the sum of |LUT entries| of an id's code (brute force here), and
+    assert_topk_parity accepts association noise on a sum that cancels but not a real error."""
+    from tests.parity import assert_topk_parity, term_scale
+    rng = np.random.default_rng(5)
+    d = M = 8
+    x = rng.standard_normal((200, d)).astype(np.float32)
+    cent, _ = oracle.kmeans(x, 4, niter=2, seed=1)
+    cb = oracle.train_pq(x, M, niter=2, seed=1)
+    idx = oracle.CsrIndex.build(d, M, oracle.METRIC_INNER_PRODUCT, cent, cb, x)
+    q = rng.standard_normal((3, d)).astype(np.float32)
+    D, I = idx.search(q, 20, 4)
+    lut = oracle.lut(q[:1], cb, oracle.METRIC_INNER_PRODUCT)[0]
+    pos = {int(v): i for i, v in enumerate(idx.ids)}
+    want = [sum(abs(float(lut[m, idx.codes[pos[int(i)]][m]])) for m in range(M)) for i in I[0, :5]]
+    assert np.allclose(term_scale(oracle, idx, q[0], I[0, :5]), want, rtol=1e-12)
+    # the entry closest to zero, moved by a few ulps of its terms: beyond 1e-4 of itself, within 1e-4 of the terms
+    r = int(np.argmin(np.abs(D[0])))
+    scale = term_scale(oracle, idx, q[0], [I[0, r]])[0]
+    noisy = D.copy()
+    noisy[0, r] += np.float32(3e-5 * scale)
+    if abs(noisy[0, r] - D[0, r]) > 1e-4 * max(abs(noisy[0, r]), abs(D[0, r])):
+        assert_topk_parity(oracle, idx, q, noisy, I, D, I, 1e-4)
+    wrong = D.copy()
+    wrong[0, r] += np.float32(1e-3 * scale)
+    with pytest.raises(AssertionError):
+        assert_topk_parity(oracle, idx, q, wrong, I, D, I, 1e-4)
