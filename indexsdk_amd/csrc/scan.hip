@@ -680,6 +680,8 @@ size_t plan_scan(ScanParams &p)
         return best_smem;
     }
     int best_waves = best_smem <= 160 * 1024 ? resident_waves(best_smem, 8) : 0;
+    ScanParams smallest = best;   // reported when nothing fits
+    size_t smallest_smem = best_smem;
     const struct {
         int waves;
         bool shared;
@@ -698,6 +700,14 @@ size_t plan_scan(ScanParams &p)
             best_smem = smem;
             best_waves = rw;
         }
+        if (smem < smallest_smem) {
+            smallest = q;
+            smallest_smem = smem;
+        }
+    }
+    if (best_waves == 0) {
+        p = smallest;
+        return smallest_smem;
     }
     p = best;
     return best_smem;
@@ -711,7 +721,7 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
     p.nq = nq;
     const size_t smem = plan_scan(p);
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam,
-                "IVFPQ scan needs %zu bytes of LDS (M=%d, k=%d, %s LUT); the limit is 163840", smem, p.M, p.k,
+                "IVFPQ scan needs at least %zu bytes of LDS (M=%d, k=%d, %s LUT); the limit is 163840", smem, p.M, p.k,
                 p.lut_fp16 ? "fp16" : "fp32");
     IXA_REQUIRE(nq * p.nsplit < ((int64_t)1 << 31), kErrInvalidParam, "scan grid too large");
     if (p.lut_fp16) {

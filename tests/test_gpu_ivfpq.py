@@ -358,6 +358,24 @@ def test_large_k_shared_pool_layouts_and_workgroup_sizes(ix, oracle, d, M, layou
     assert_topk_parity(oracle, ref, q[sub], D[sub], I[sub], Dr, Ir, TOL_FP32)
 
 
+def test_k_beyond_what_the_lds_holds_next_to_the_largest_lut_is_refused(ix, oracle):
+    """128 sub-quantizers with an fp32 LUT take 128 of the 160 KB of LDS: pools for k <= 1024 fit beside it
+    (previous test), larger k is refused with a message that names the need; an fp16 LUT makes room."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 77, 3000, 5, 128, 8, 128, ix.METRIC_L2)
+    gpu.setNumProbes(4)
+    with pytest.raises(ix.IndexSdkError, match="bytes of LDS") as err:
+        gpu.search(q, 1025)
+    assert err.value.code == 2001
+    D, I = gpu.search(q, 1024)                  # the index is still usable
+    Dr, Ir = ref.search(q, 1024, 4)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    half, ref16, _, _, _ = build_pair(ix, oracle, 77, 3000, 5, 128, 8, 128, ix.METRIC_L2, lut_fp16=1)
+    half.setNumProbes(4)
+    D, I = half.search(q, 2048)
+    Dr, Ir = ref16.search(q, 2048, 4, lut_fp16=True)
+    assert_topk_parity(oracle, ref16, q, D, I, Dr, Ir, TOL_FP16)
+
+
 def test_xor48_layout_is_the_default_for_m48_and_lists_read_back_in_row_order(ix, oracle):
     gpu, ref, x, q, ids = build_pair(ix, oracle, 47, 20000, 64, 96, 32, 48, ix.METRIC_L2)
     row, _, _, _, _ = build_pair(ix, oracle, 47, 20000, 64, 96, 32, 48, ix.METRIC_L2, layout=0)
