@@ -4,7 +4,12 @@ The reference ships no data; its python harness reads SIFT1M from disk
 (FR/test/python/datasets.py:71-84).  Here every configuration is a seeded mixture so that tests,
 golden fixtures and the benchmark draw base, train and query vectors from the same distribution.
 ``scale`` shrinks the base/query counts for CI-sized twins; the distribution is unchanged.
+
+``evaluate`` is the reference harness's recall measurement with the same contract, and ``ground_truth``
+produces the exact-neighbour array it is measured against.
 """
+import time
+
 import numpy as np
 
 
@@ -69,3 +74,31 @@ def make(name, scale=1.0, nq=None):
     if c["kind"] == "vmf":
         return vmf_like_mixture(c["seed"], n, nq, c["d"], c["comp"], c["sigma"])
     return int8_uniform(c["seed"], n, nq, c["d"])
+
+
+def ground_truth(xb, xq, k=1, metric="L2", ids=None):
+    """Exact k nearest neighbours of every query by brute force on the GPU (AscendIndexFlat, fp32):
+    the ``gt`` array of ``evaluate``; ``gt[:, 0]`` is the true nearest neighbour.  The reference reads
+    this array from SIFT1M's ground-truth file (FR/test/python/datasets.py:43-45)."""
+    from . import ascendfaiss
+    flat = ascendfaiss.AscendIndexFlat(xb.shape[1], ascendfaiss.METRIC_L2 if metric == "L2"
+                                       else ascendfaiss.METRIC_INNER_PRODUCT)
+    flat.add_with_ids(xb, ids)
+    return flat.search(xq, k)[1]
+
+
+def evaluate(index, xq, gt, k):
+    """(milliseconds per query, {r: recall@r}) for r = 1, 10, 100, ... <= k, where recall@r is the
+    fraction of queries whose true nearest neighbour ``gt[:, 0]`` is among the first r results of
+    ``index.search(xq, k)`` -- the measure of the reference's harness (FR/test/python/datasets.py:71-84)."""
+    nq = xq.shape[0]
+    t0 = time.time()
+    _, labels = index.search(xq, k)
+    t1 = time.time()
+    truth = np.asarray(gt)[:, :1]
+    recalls = {}
+    r = 1
+    while r <= k:
+        recalls[r] = float((labels[:, :r] == truth).any(axis=1).sum()) / nq
+        r *= 10
+    return (t1 - t0) * 1000.0 / nq, recalls

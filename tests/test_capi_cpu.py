@@ -126,3 +126,24 @@ def test_merge_search_results_rejects_bad_arguments(capi):
     lib = capi.load()
     rc = lib.ixa_merge_search_results(0, 1, 1, 1, None, None, None, None)
     assert rc != 0 and "ndev" in lib.ixa_last_error().decode()
+
+
+def test_evaluate_counts_queries_whose_true_neighbour_is_in_the_first_r_results():
+    """indexsdk_amd.datasets.evaluate (the reference harness's recall@r, FR/test/python/datasets.py:71-84)
+    on a hand-made result list: true neighbours 7, 8, 9, 10; found at ranks 1, 3, 11 and never."""
+    import numpy as np
+    from indexsdk_amd.datasets import evaluate
+
+    class Canned:
+        def search(self, xq, k):
+            lab = np.full((4, k), -1, dtype=np.int64)
+            lab[0, 0] = 7
+            lab[1, 2] = 8
+            lab[2, 10] = 9
+            lab[3, :] = np.arange(100, 100 + k)
+            return np.zeros((4, k), dtype=np.float32), lab
+
+    gt = np.array([[7, 1], [8, 2], [9, 3], [10, 4]], dtype=np.int64)
+    ms, rec = evaluate(Canned(), np.zeros((4, 2), dtype=np.float32), gt, 100)
+    assert ms >= 0 and rec == {1: 0.25, 10: 0.5, 100: 0.75}
+    assert set(evaluate(Canned(), np.zeros((4, 2), dtype=np.float32), gt, 50)[1]) == {1, 10}

@@ -600,3 +600,26 @@ def test_concurrent_callers_of_one_index_are_serialised(ix, oracle):
         t.join()
     for i in range(4):
         assert np.array_equal(got[i][1], want[i][1]) and np.array_equal(got[i][0].view(np.uint32), want[i][0].view(np.uint32))
+
+
+def test_recall_harness_against_exact_neighbours(ix, oracle):
+    """evaluate() / ground_truth() of indexsdk_amd.datasets, the counterpart of the reference's SIFT1M
+    recall harness (FR/test/python/datasets.py:71-84, TestAscendIndexIVFPQ.py:33-72): the GPU brute force
+    agrees with the oracle's, recall grows with r and with nprobe, and probing every list with fine
+    codes finds almost every true neighbour."""
+    from indexsdk_amd.datasets import evaluate, ground_truth
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 90, 20000, 300, 64, 64, 32, ix.METRIC_L2)
+    gt = ground_truth(x, q, 1, "L2", ids)
+    Do, Io = oracle.flat_f32(x, q, 1, ix.METRIC_L2)
+    assert np.array_equal(gt[:, 0], ids[Io[:, 0]])
+    gpu.setNumProbes(1)
+    _, r1 = evaluate(gpu, q, gt, 100)
+    gpu.setNumProbes(64)
+    ms, r64 = evaluate(gpu, q, gt, 100)
+    assert list(r64) == [1, 10, 100] and ms > 0
+    assert r64[1] <= r64[10] <= r64[100] and r1[1] <= r1[10] <= r1[100]
+    assert r64[100] >= r1[100] and r64[100] >= 0.99 and r64[1] >= 0.3
+    # the same figures from the oracle's result lists: parity of ids makes the recall identical
+    Dr, Ir = ref.search(q, 100, 64)
+    want = {r: float((Ir[:, :r] == gt[:, :1]).any(axis=1).mean()) for r in (1, 10, 100)}
+    assert all(abs(r64[r] - want[r]) <= 1.0 / len(q) for r in want)
