@@ -24,6 +24,18 @@ def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
+def cpu_model():
+    """Model name of the host CPU the baseline leg runs on (/proc/cpuinfo), or "unknown"."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def gen_mixture_gpu(torch, seed, n, d, comp, sigma, centres=None, chunk=1 << 20, weights=None, unit=False,
                     out=None):
     """Mixture rows generated on the device in chunks: centres ~ N(0, I) (normalised when ``unit``),
@@ -121,7 +133,8 @@ def run_flat_i8(args, torch, ix, _capi, lib):
         exact = bool(np.array_equal(Dg, Dr) and np.array_equal(Ig, Ir))
         cpu_ops = 2.0 * sample_q * sample_n * d
         result["cpu_baseline"] = {"value": sample_q / t_cpu * (sample_n / n), "unit": "queries/s", "cores": orc.num_threads(),
-                                  "kind": "port", "sample": f"{sample_q} queries x first {sample_n} base rows in {t_cpu:.1f}s, "
+                                  "kind": "port", "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
+                                  "sample": f"{sample_q} queries x first {sample_n} base rows in {t_cpu:.1f}s, "
                                   f"scaled by {sample_n}/{n} to the full base; {cpu_ops / t_cpu / 1e9:.1f} GOP/s"}
         result["parity_sample"] = {"queries": sample_q, "rows": sample_n, "bit_exact": exact}
         log(f"CPU oracle flat int8: {t_cpu:.2f}s for {sample_q}x{sample_n}; GPU bit-exact on the sample: {exact}")
@@ -320,6 +333,7 @@ def main():
         log(f"CPU oracle: {sample} queries x {passes} passes, median {t_cpu:.2f}s on {orc.num_threads()} threads = "
             f"{cpu_qps:.0f} QPS; GPU ids equal at {same:.6f} of positions, distances within {tol}: {dist_ok}")
         result["cpu_baseline"] = {"value": cpu_qps, "unit": "queries/s", "cores": orc.num_threads(), "kind": "port",
+                                  "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
                                   "sample": f"first {sample} of the {nq} queries, same index, OpenMP over queries, "
                                             f"median of {passes} passes of {t_cpu:.1f}s",
                                   "adc_scan_GBps": ref.last_scanned * M / t_cpu / 1e9}

@@ -47,6 +47,8 @@ extern "C" {
 
 /* Message of the last failed call on this thread ("" if none). */
 const char *ixa_last_error(void);
+/* The same string under the index family's prefix. */
+const char *ivfpq_last_error(void);
 
 /* Copies bytes (a multiple of 16) between two DEVICE buffers with a plain copy kernel and waits for
  * it.  No counterpart in the reference: it is the kernel of known size that hardware traffic

@@ -106,6 +106,7 @@ extern "C" {
 #define IXA_EXPORT __attribute__((visibility("default")))
 
 IXA_EXPORT const char *ixa_last_error(void) { return g_last_error.c_str(); }
+IXA_EXPORT const char *ivfpq_last_error(void) { return g_last_error.c_str(); }
 
 IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
 {

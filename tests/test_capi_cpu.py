@@ -33,7 +33,7 @@ def test_header_declares_the_index_level_boundary():
     for need in ["ivfpq_create", "ivfpq_destroy", "ivfpq_train", "ivfpq_set_trained", "ivfpq_add_with_ids",
                  "ivfpq_add_codes", "ivfpq_set_nprobe", "ivfpq_get_nprobe", "ivfpq_search", "ivfpq_assign",
                  "ivfpq_coarse_probe", "ivfpq_list_length", "ivfpq_get_list", "ivfpq_remove_ids", "ivfpq_reset",
-                 "ixa_last_error"]:
+                 "ixa_last_error", "ivfpq_last_error"]:
         assert need in names
 
 
