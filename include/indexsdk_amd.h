@@ -166,12 +166,14 @@ int ivfpq_add_with_ids_device(ivfpq_index_t *h, int64_t n, const float *x_dev, c
  * codes row-major [n][msubs]. */
 int ivfpq_add_codes(ivfpq_index_t *h, int64_t list, int64_t n, const uint8_t *codes, const int64_t *ids);
 
-/* AscendIndexIVF::setNumProbes / getNumProbes  FR/ascend/AscendIndexIVF.h:96-99 */
+/* AscendIndexIVF::setNumProbes / getNumProbes  FR/ascend/AscendIndexIVF.h:96-99.  nprobe >= 1; a value above
+ * the number of lists is clamped to it; more than 2048 probed lists are refused. */
 int ivfpq_set_nprobe(ivfpq_index_t *h, int nprobe);
 int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out);
 
 /* AscendIndex::search(n, x, k, distances, labels)  FR/ascend/AscendIndex.h:79-80 ->
- * ascend::IndexIVFPQ::searchImpl  FR/ascenddaemon/impl/IndexIVFPQ.cpp:2373-2411 */
+ * ascend::IndexIVFPQ::searchImpl  FR/ascenddaemon/impl/IndexIVFPQ.cpp:2373-2411.  0 < n < 1e9, 0 < k <= 2048
+ * (the reference's device limit is 320); with 128 sub-quantizers and an fp32 LUT, k <= 1024. */
 int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
 int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
                         int64_t *labels_dev);

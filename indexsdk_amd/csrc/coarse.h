@@ -60,6 +60,9 @@ void launch_verify_superset(const unsigned long long *running, int ncand, const 
                             int *flag,
                             hipStream_t s);
 
+// Largest selection size of launch_select_rows*: the private pools of its wavefronts hold 4096 keys.
+constexpr int kSelectMaxK = 3072;
+
 // Best `ksel` columns of every row of a score matrix.  out_idx (may be null) receives the column
 // indices (+ col_base), best first.  running (may be null) is a [nrows][ksel] array of keys
 // (ordered score << 32) | (col_base + column): its content takes part in the selection and is

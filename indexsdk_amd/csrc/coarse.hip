@@ -383,13 +383,27 @@ void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter
 // column chunks) take part in the merge and provide the initial bound, which turns a sequence of
 // calls over column chunks into a streaming top-k.  Output: ksel column indices per row (best
 // first, -1 where the row has fewer than ksel columns) and/or the keys themselves.
+// Keys the pool region of a streaming selection holds: the pools of the scanning wavefronts plus the
+// running keys merged in at the end, rounded up to the power of two the merge sorts.
+__host__ __device__ inline int select_region_keys(int active, int cap, int extra)
+{
+    int n = 2;
+    while (n < active * cap + extra) {
+        n <<= 1;
+    }
+    return n;
+}
+
 template <typename S>
 __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, const S *__restrict__ scores, int64_t ld,
                                                      int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                     int64_t col_base, key_t *__restrict__ running, bool fresh)
+                                                     int64_t col_base, key_t *__restrict__ running, bool fresh,
+                                                     int active = 4)
 {
-    key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // pow2_ceil(4 * cap + ksel)
-    const int region = running ? 8 * cap : 4 * cap;
+    // `active` of the four wavefronts scan (each with a private pool of `cap` keys), all four merge: a
+    // selection too large for four pools in LDS runs on two or one
+    key_t *pools = reinterpret_cast<key_t *>(smem_raw);                 // select_region_keys() keys
+    const int region = select_region_keys(active, cap, running ? ksel : 0);
     // fresh: `running` only receives the result (its content is unspecified on entry)
     S *share = reinterpret_cast<S *>(pools + region);                   // 4
     int *counts = reinterpret_cast<int *>(share + 4);                   // 4
@@ -409,13 +423,14 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
         share[tid] = ScoreOps<S>::worst();
     }
     __syncthreads();
+    const bool scans = wave < active;
     WavePool<S> pool;
-    pool.init(pools + wave * cap, cap, ksel);
+    pool.init(pools + (scans ? wave : 0) * cap, cap, ksel);
     pool.bound = wave_uniform(start);
-    const int share_rank = (ksel + 3) / 4;
+    const int share_rank = (ksel + active - 1) / active;
     auto adopt_shared = [&]() {
         S b = share[0];
-        for (int i = 1; i < 4; i++) {
+        for (int i = 1; i < active; i++) {
             b = share[i] > b ? share[i] : b;
         }
         b = wave_uniform(b);
@@ -423,9 +438,11 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
     };
     const bool vec4 = (ld % 4 == 0) && (reinterpret_cast<uintptr_t>(scores) % 16 == 0);
     int iter = 0;
-    if (vec4) {
+    if (!scans) {
+        // no work for this wavefront until the merge
+    } else if (vec4) {
         // 128-bit loads: a wavefront covers 256 consecutive columns per step
-        for (int64_t base = (int64_t)wave * 256; base < nc; base += 1024, iter++) {
+        for (int64_t base = (int64_t)wave * 256; base < nc; base += active * 256, iter++) {
             const int64_t c = base + lane * 4;
             S v[4];
             if (c + 3 < nc) {
@@ -459,7 +476,7 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
             }
         }
     } else {
-        for (int64_t base = (int64_t)wave * 64; base < nc; base += 256, iter++) {
+        for (int64_t base = (int64_t)wave * 64; base < nc; base += active * 64, iter++) {
             int64_t c = base + lane;
             S v = c < nc ? row[c] : ScoreOps<S>::worst();
             const bool compacted =
@@ -470,10 +487,12 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
         }
     }
     __syncthreads();
-    adopt_shared();
-    pool.finish(lane);
+    if (scans) {
+        adopt_shared();
+        pool.finish(lane);
+    }
     if (lane == 0) {
-        counts[wave] = pool.count;
+        counts[wave] = scans ? pool.count : 0;
     }
     const int total = block_merge_pools<4>(pools, cap, counts, run, (run && !fresh) ? ksel : 0, tid);
     for (int i = tid; i < ksel; i += 256) {
@@ -490,10 +509,11 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
 template <typename S>
 __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
                                                           int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                          int64_t col_base, key_t *__restrict__ running, bool fresh)
+                                                          int64_t col_base, key_t *__restrict__ running, bool fresh,
+                                                          int active)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh);
+    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh, active);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -785,9 +805,15 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
     if (nrows == 0) {
         return;
     }
-    IXA_REQUIRE(ksel >= 1 && ksel <= 2048, kErrInvalidParam, "selection size %d out of range [1, 2048]", ksel);
+    IXA_REQUIRE(ksel >= 1 && ksel <= kSelectMaxK, kErrInvalidParam, "selection size %d out of range [1, %d]", ksel,
+                kSelectMaxK);
     const int cap = wave_pool_capacity(ksel);
-    size_t smem = (size_t)(running ? 8 : 4) * cap * sizeof(key_t) + 64;
+    // four scanning wavefronts when their pools and the merge fit LDS, else two, else one
+    int active = 4;
+    while (active > 1 && (size_t)select_region_keys(active, cap, running ? ksel : 0) * sizeof(key_t) + 64 > 160 * 1024) {
+        active >>= 1;
+    }
+    size_t smem = (size_t)select_region_keys(active, cap, running ? ksel : 0) * sizeof(key_t) + 64;
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "selection size %d needs %zu bytes of LDS", ksel, smem);
     const bool vec4 = ld % 4 == 0 && reinterpret_cast<uintptr_t>(scores) % 16 == 0;
     // measured: the register kernel wins on rows of up to a few segments (16384 columns: 0.17 ms against
@@ -806,7 +832,7 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     }
     hipLaunchKernelGGL(select_rows_kernel<S>, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
-                       out_idx, col_base, running, fresh);
+                       out_idx, col_base, running, fresh, active);
 }
 
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,

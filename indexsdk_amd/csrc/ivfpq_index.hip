@@ -36,6 +36,7 @@ bool contains(const int (&a)[N], int64_t v)
 
 constexpr int64_t kMaxN = 1000000000;   // MAX_N, FR/ascend/AscendIndex.h
 constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this build (reference device limit: 320)
+constexpr int kMaxNprobe = 2048;        // probed lists per query (the reference's L3 operator takes 128 per tile)
 constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
 
 // ---- arena kernels ------------------------------------------------------------------------------
@@ -300,7 +301,10 @@ void IvfpqIndex::set_nprobe(int nprobe)
 {
     flush_stats();
     IXA_REQUIRE(nprobe >= 1, kErrInvalidParam, "nprobe must be >= 1, got %d", nprobe);
-    nprobe_ = (int)std::min<int64_t>(nprobe, nlist_);
+    const int clamped = (int)std::min<int64_t>(nprobe, nlist_);
+    // the probe selection keeps nprobe + 16 + nprobe / 8 candidates per query in LDS
+    IXA_REQUIRE(clamped <= kMaxNprobe, kErrInvalidParam, "nprobe must be <= %d, got %d", kMaxNprobe, clamped);
+    nprobe_ = clamped;
 }
 
 void IvfpqIndex::check_trained() const

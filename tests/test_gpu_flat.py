@@ -214,3 +214,31 @@ def test_flat_i8_rows_selected_from_registers(ix, oracle):
     D, I = index.search_int32(q, k)
     Dr, Ir = oracle.flat_i8(base, q, k)
     assert np.array_equal(I, Ir) and np.array_equal(D, Dr)
+
+
+@pytest.mark.parametrize("n,nq,scratch", [(9000, 37, 0), (2049, 129, 1 << 20), (50000, 5, 4 << 20), (1500, 3, 0)])
+def test_flat_largest_k(ix, oracle, n, nq, scratch):
+    """k = 2048, the API's maximum, on all three Flat variants: the streaming selection then runs on two
+    scanning wavefronts (four pools of 4096 keys do not fit LDS), over one block of the base or several,
+    and with fewer rows than k the tail is padding."""
+    d, k = 64, 2048
+    rng = np.random.default_rng(n + nq)
+    bi = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    qi = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    bi[n // 3] = bi[1]
+    index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=scratch)
+    index.add(bi)
+    D, I = index.search_int32(qi, k)
+    Dr, Ir = oracle.flat_i8(bi, qi, k)
+    assert np.array_equal(I, Ir) and np.array_equal(D, Dr)
+    centres = rng.standard_normal((16, d)).astype(np.float32)
+    base = (centres[rng.integers(0, 16, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 16, nq)] + 0.3 * rng.standard_normal((nq, d))).astype(np.float32)
+    base[n // 3] = base[1]
+    for metric in (ix.METRIC_L2, ix.METRIC_INNER_PRODUCT):
+        flat = ix.AscendIndexFlat(d, metric, scratch_bytes=scratch)
+        flat.add(base)
+        D, I = flat.search(q, k)
+        Dr, Ir = oracle.flat_f32(base, q, k, metric)
+        assert np.array_equal(I, Ir)
+        assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))

@@ -623,3 +623,32 @@ def test_recall_harness_against_exact_neighbours(ix, oracle):
     Dr, Ir = ref.search(q, 100, 64)
     want = {r: float((Ir[:, :r] == gt[:, :1]).any(axis=1).mean()) for r in (1, 10, 100)}
     assert all(abs(r64[r] - want[r]) <= 1.0 / len(q) for r in want)
+
+
+def test_largest_nprobe(ix, oracle):
+    """nprobe = 2048 of 2500 lists (the limit: 2048 + 16 + 256 candidates per query go through the probe
+    selection): probe ids and distances bit-exact, search parity; one more is refused, and a request
+    beyond the number of lists is clamped to it first."""
+    nlist, d, M = 2500, 32, 8
+    rng = np.random.default_rng(12)
+    centres = rng.standard_normal((40, d)).astype(np.float32)
+    cent = (centres[rng.integers(0, 40, nlist)] + 0.5 * rng.standard_normal((nlist, d))).astype(np.float32)
+    x = (centres[rng.integers(0, 40, 30000)] + 0.5 * rng.standard_normal((30000, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 40, 20)] + 0.5 * rng.standard_normal((20, d))).astype(np.float32)
+    cb = oracle.train_pq(x[:4000], M, niter=2, seed=2)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add(x)
+    with pytest.raises(ix.IndexSdkError, match="nprobe must be <= 2048"):
+        gpu.setNumProbes(2049)
+    gpu.setNumProbes(2048)
+    gi, gd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, 2048, ix.METRIC_L2)
+    assert np.array_equal(gi, oi) and np.array_equal(gd.view(np.uint32), od.view(np.uint32))
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x)
+    D, I = gpu.search(q, 100)
+    Dr, Ir = ref.search(q, 100, 2048)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    small = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, 64, M, 8, ix.AscendIndexIVFPQConfig())
+    small.setNumProbes(100000)
+    assert small.getNumProbes() == 64

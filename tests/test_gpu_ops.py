@@ -95,7 +95,7 @@ def test_distance_flat_l2_mins(env, oracle, batch, n, d):
 
 
 @pytest.mark.parametrize("batch,n,ld,k", [(33, 1013, 1013, 70), (4, 50, 64, 128), (9, 20000, 20000, 100),
-                                          (6, 5000, 5120, 300), (2, 1, 4, 3)])
+                                          (6, 5000, 5120, 300), (2, 1, 4, 3), (5, 30000, 30000, 2048), (3, 3000, 3000, 1100)])
 def test_topk_flat_fp32(env, batch, n, ld, k):
     hip, ix, _capi, lib = env
     rng = np.random.default_rng(n + k)
