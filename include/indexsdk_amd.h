@@ -180,7 +180,8 @@ int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t
 /* Stages 2-4 only, on probe lists the caller selected: operators "AscendcIvfpqSearchDistanceL2" +
  * "TopkIvfpqL3" (IndexIVFPQ::searchImplL3, FR/ascenddaemon/impl/IndexIVFPQ.cpp:2162-2347), the LUT being
  * built inside the launch.  probes_dev: [n][nprobe] list ids (int32, DEVICE); -1, like any other value
- * outside [0, nlist), means no list; a list named twice is scanned twice.  Results as ivfpq_search_device.  Waits for the results. */
+ * outside [0, nlist), means no list; a list named twice is scanned twice.  Results as ivfpq_search_device.  Waits for the results.
+ * ivfpq_last_search_stats afterwards reports the plan of the scan only (no stage timings are taken here). */
 int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe,
                                int64_t k, float *distances_dev, int64_t *labels_dev);
 

@@ -894,6 +894,14 @@ void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *pro
     ScanParams p = scan_params(x_dev, n, ws_probes_.data(), nprobe, k, dist_dev, labels_dev);
     launch_scan(p, n, stream_);
     sync_stream(stream_);
+    // the plan of this launch; no stage timings are taken here
+    stats_ = SearchStats{};
+    stats_.nsplit = p.nsplit;
+    stats_.scan_launches = p.nsplit > 1 ? 2 : 1;
+    stats_.ordered = p.order ? 1 : 0;
+    plan_scan(p);
+    stats_.scan_waves = p.waves;
+    stats_.shared_pool = p.shared_pool;
 }
 
 // -------------------------------------------------------------------------------------------------

@@ -441,14 +441,48 @@ __global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restric
                                                           int64_t *__restrict__ out_labels)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    key_t *merge = reinterpret_cast<key_t *>(smem_raw);
+    key_t *lists = reinterpret_cast<key_t *>(smem_raw);   // [nsplit][k], each ascending, empty keys last
+    key_t *merge = lists + merge_n;                        // [k] the result
     const int tid = threadIdx.x;
     const int64_t q = blockIdx.x;
     const int total = nsplit * k;
-    for (int i = tid; i < merge_n; i += 256) {
-        merge[i] = i < total ? partial[q * total + i] : kEmptyKey;
+    for (int i = tid; i < total; i += 256) {
+        lists[i] = partial[q * total + i];
     }
-    block_bitonic_sort(merge, merge_n, tid, 256);
+    for (int i = tid; i < k; i += 256) {
+        merge[i] = kEmptyKey;
+    }
+    __syncthreads();
+    // Every key finds its own rank in the union: its position in its list plus, for every other list,
+    // the number of keys below it (binary search; no barriers, where a sort of the union takes dozens).
+    // Equal keys (one list probed twice) are ordered by split so that ranks stay distinct.
+    for (int e = tid; e < total; e += 256) {
+        const int sp = e / k, pos = e - sp * k;
+        const key_t mine = lists[e];
+        if (mine == kEmptyKey) {
+            continue;
+        }
+        int rank = pos;
+        for (int o = 0; o < nsplit && rank < k; o++) {
+            if (o == sp) {
+                continue;
+            }
+            const key_t *other = lists + o * k;
+            int lo = 0, hi = k;   // first index whose key is not below `mine` (o > sp) / above it (o < sp)
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                const key_t v = other[mid];
+                const bool below = o < sp ? v <= mine : v < mine;
+                lo = below ? mid + 1 : lo;
+                hi = below ? hi : mid;
+            }
+            rank += lo;
+        }
+        if (rank < k) {
+            merge[rank] = mine;
+        }
+    }
+    __syncthreads();
     for (int i = tid; i < k; i += 256) {
         const key_t kk = merge[i];
         const bool ok = kk != kEmptyKey;
@@ -730,8 +764,8 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
         dispatch_m<float>(p, nq, smem, s);
     }
     if (p.nsplit > 1) {
-        const int merge_n = pow2_ceil(p.nsplit * p.k);
-        const size_t msmem = (size_t)merge_n * sizeof(key_t);
+        const int merge_n = p.nsplit * p.k;
+        const size_t msmem = (size_t)(merge_n + p.k) * sizeof(key_t);
         IXA_REQUIRE(msmem <= 160 * 1024, kErrInner, "merge of %d x %d candidates exceeds LDS", p.nsplit, p.k);
         if (msmem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(ivfpq_merge_kernel),

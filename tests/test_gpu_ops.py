@@ -173,3 +173,15 @@ def test_operators_chained_equal_the_fused_search(env, oracle):
     _capi.check(lib.ivfpq_search_probes_device(gpu._h, nq, _p(dq), _p(hip.put(keep)), keep.shape[1], k, _p(D3), _p(I3)))
     assert np.array_equal(I2.get(), I3.get())
     assert np.array_equal(D2.get().view(np.uint32), D3.get().view(np.uint32))
+    # one list named twice is scanned twice: every result of the single scan comes back doubled, the two
+    # copies next to each other (the two scans run in different workgroups here and meet in the split merge)
+    one = np.ascontiguousarray(probes_h[:, :1])
+    two = np.ascontiguousarray(np.repeat(one, 2, axis=1))
+    kk = 16
+    D1, I1 = hip.empty((nq, kk), np.float32), hip.empty((nq, kk), np.int64)
+    Dd, Id = hip.empty((nq, 2 * kk), np.float32), hip.empty((nq, 2 * kk), np.int64)
+    _capi.check(lib.ivfpq_search_probes_device(gpu._h, nq, _p(dq), _p(hip.put(one)), 1, kk, _p(D1), _p(I1)))
+    _capi.check(lib.ivfpq_search_probes_device(gpu._h, nq, _p(dq), _p(hip.put(two)), 2, 2 * kk, _p(Dd), _p(Id)))
+    assert gpu.last_search_stats()["nsplit"] == 2
+    assert np.array_equal(Id.get(), np.repeat(I1.get(), 2, axis=1))
+    assert np.array_equal(Dd.get().view(np.uint32), np.repeat(D1.get(), 2, axis=1).view(np.uint32))
