@@ -394,11 +394,10 @@ __host__ __device__ inline int select_region_keys(int active, int cap, int extra
     return n;
 }
 
-template <typename S>
+template <typename S, int active = 4>
 __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, const S *__restrict__ scores, int64_t ld,
                                                      int64_t nc, int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                     int64_t col_base, key_t *__restrict__ running, bool fresh,
-                                                     int active = 4)
+                                                     int64_t col_base, key_t *__restrict__ running, bool fresh)
 {
     // `active` of the four wavefronts scan (each with a private pool of `cap` keys), all four merge: a
     // selection too large for four pools in LDS runs on two or one
@@ -506,14 +505,13 @@ __device__ __forceinline__ void select_row_streaming(unsigned char *smem_raw, co
     }
 }
 
-template <typename S>
+template <typename S, int ACTIVE>
 __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ scores, int64_t ld, int64_t nc,
                                                           int ksel, int cap, int32_t *__restrict__ out_idx,
-                                                          int64_t col_base, key_t *__restrict__ running, bool fresh,
-                                                          int active)
+                                                          int64_t col_base, key_t *__restrict__ running, bool fresh)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    select_row_streaming<S>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh, active);
+    select_row_streaming<S, ACTIVE>(smem_raw, scores, ld, nc, ksel, cap, out_idx, col_base, running, fresh);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -827,12 +825,13 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
                            col_base, running, fresh);
         return;
     }
+    auto kern = active == 4 ? select_rows_kernel<S, 4> : (active == 2 ? select_rows_kernel<S, 2> : select_rows_kernel<S, 1>);
     if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(select_rows_kernel<S>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
     }
-    hipLaunchKernelGGL(select_rows_kernel<S>, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap,
-                       out_idx, col_base, running, fresh, active);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap, out_idx, col_base,
+                       running, fresh);
 }
 
 void launch_select_rows(const float *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
