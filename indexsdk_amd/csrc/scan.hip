@@ -43,29 +43,32 @@ __device__ __forceinline__ float from_lut(float v) { return v; }
 __device__ __forceinline__ float from_lut(__half v) { return __half2float(v); }
 
 // Half-precision LUT under the rot32 code layout.  Two halves share one 32-bit LDS word, so "32
-// lanes read 32 different sub-quantizers" only means 32 different banks if the two halves of a word
-// never belong to different sub-quantizer offsets of a 32-block.
-//   * Even number of 32-blocks (M = 64): blocks are paired.  Block pair p owns 32 KB, codeword kk a row
-//     of 32 words in it, word r holds sub-quantizer r of the even block (low half) and of the odd
-//     block (high half).  A lane's word index is row * 32 + r with r distinct across the 32 lanes: no
-//     bank conflicts for any code values; the address is one shift-add of the code.
-//   * Odd number (M = 32, 96): a block has no partner, and pairing codewords instead (row kk / 2, half
-//     kk % 2) costs two more address instructions per lookup.  Rows of 64 bytes do not: row
-//     g = block * 256 + kk starts at byte 64 g and sub-quantizer r sits in half (r >> 4) of word r of
-//     the row, so r >= 16 reaches into the next row's words, whose own sub-quantizers 0..15 use the
-//     other half.  The address is (code << 6) + a per-lane constant again, for every block; lanes r and
-//     r ^ 16 now share a bank whenever their codes differ in parity (a two-way conflict on most reads).
-//     The scan is bound by vector instructions, not by LDS: measured on 20M x 768, M = 96: 5.31 -> 5.19 ms.
-//     (Giving the unpaired block 32 KB of its own with fp32 words has neither cost, but the larger LUT
-//     costs a resident workgroup at M = 96: measured slower.)
+// lanes read 32 different sub-quantizers" only means 32 different banks if the words they read are
+// 32 different words modulo the 32 banks, whatever the code values.  Sub-quantizer r of a 32-block
+// sits at byte R(r) = 4 r + 2 (r >> 4) of its codeword's row: word r, low half for r < 16, high half
+// above.
+//   * Blocks are paired.  Block pair p owns 32 KB, codeword kk a row of 128 bytes in it; the even
+//     block starts at byte 0 of the row, the odd block at byte 64, so that its sub-quantizers 16..31
+//     land in words 0..15 of the NEXT row -- in the half that row's even block (r < 16) leaves free.
+//     A lane's bank is r (even block) or r + 16 mod 32 (odd block): no conflicts.
+//   * A last block without partner has rows of 64 bytes, so that its sub-quantizers 16..31 reach into
+//     the next row in the same way.  Lanes r and r ^ 16 then share a bank whenever their codes differ
+//     in parity (a two-way conflict on most reads of that block), which costs less than the two extra
+//     address instructions per lookup of the conflict-free alternative, pairing codewords (row kk / 2,
+//     half kk % 2): the scan is bound by vector instructions.
+// Every address is (code << 7 or 6) + a per-lane constant + an immediate: one shift-add.  The last
+// row's upper half needs 64 bytes beyond M * 512.
+// (Giving the unpaired block 32 KB of its own with fp32 words has neither cost, but the larger LUT
+// costs a resident workgroup at M = 96: measured slower.)
 __host__ __device__ __forceinline__ int rot32_half_slot(int nblocks, int m, int kk)
 {
     const int b = m >> 5, r = m & 31;
+    const int in_row = r * 4 + 2 * (r >> 4);
     int byte;
-    if ((nblocks & 1) == 0) {
-        byte = (b >> 1) * 32768 + kk * 128 + r * 4 + 2 * (b & 1);
+    if (b < (nblocks & ~1)) {
+        byte = (b >> 1) * 32768 + kk * 128 + 64 * (b & 1) + in_row;
     } else {
-        byte = (b * 256 + kk) * 64 + r * 4 + 2 * (r >> 4);
+        byte = (nblocks >> 1) * 32768 + kk * 64 + in_row;
     }
     return byte >> 1;
 }
@@ -267,8 +270,7 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
 #pragma unroll
         for (int j = 0; j < 32; j++) {
             const uint32_t r = (uint32_t)((j + l32) & 31);
-            // odd number of blocks: rows of 64 bytes, sub-quantizer r in half (r >> 4) of word r
-            rot4[j] = lut_base + (r << 2) + ((MT / 32) % 2 == 1 ? (r >> 4) << 1 : 0u);
+            rot4[j] = lut_base + (r << 2) + ((r >> 4) << 1);   // byte R(r) of a row (rot32_half_slot)
             asm volatile("" : "+v"(rot4[j]));
         }
     }
@@ -294,10 +296,10 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
                 uint32_t off;
                 uint32_t code = (ww >> (8 * (m & 3))) & 0xffu;
                 asm("" : "+v"(code));   // keep extract-then-shift-add (two instructions for every byte)
-                if (NB % 2 == 0) {
-                    off = ((code << 7) + r4) + (uint32_t)((b >> 1) * 32768 + 2 * (b & 1));
+                if (b < (NB & ~1)) {
+                    off = ((code << 7) + r4) + (uint32_t)((b >> 1) * 32768 + 64 * (b & 1));
                 } else {
-                    off = ((code << 6) + r4) + (uint32_t)(b * 16384);
+                    off = ((code << 6) + r4) + (uint32_t)((NB >> 1) * 32768);
                 }
                 const uint32_t raw = *(lds_half_t *)off;
                 asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(acc[m & 3]) : "v"(raw));
@@ -677,8 +679,8 @@ static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
 static size_t plan_with_waves(ScanParams &p, int waves, bool shared)
 {
     size_t lut_bytes = (size_t)p.M * 256 * (p.lut_fp16 ? 2 : 4);
-    if (p.code_layout == 1 && p.lut_fp16 && (p.M / 32) % 2 == 1) {
-        lut_bytes += 64;   // rows of 64 bytes whose second half reaches into the next row: one half row more
+    if (p.code_layout == 1 && p.lut_fp16) {
+        lut_bytes += 64;   // the upper half of the last row lies in the row after it (rot32_half_slot)
     }
     if (p.code_layout == 2) {
         lut_bytes = (size_t)64 * 256 * 4;
