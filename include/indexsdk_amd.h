@@ -54,6 +54,13 @@ const char *ivfpq_last_error(void);
  * it.  No counterpart in the reference: it is the kernel of known size that hardware traffic
  * counters (FETCH_SIZE / WRITE_SIZE) of the search kernels are scaled by. */
 int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes);
+/* Reads bytes (a multiple of 16) of a DEVICE buffer `passes` times with a plain streaming kernel (16 bytes
+ * per lane and step, grid-stride) and returns the average duration of a pass in *ms_per_pass: the rate
+ * at which this GPU's memory system delivers a sequential read, the practical ceiling that the scan
+ * kernel's achieved bytes per second are to be read against (the published peak is not reachable by
+ * any kernel).  The buffer should be several times larger than the last-level cache.  No counterpart in
+ * the reference. */
+int ixa_read_probe(const void *src_dev, int64_t bytes, int passes, double *ms_per_pass);
 
 /* AscendIndexImpl::mergeSearchResult  FR/ascend/impl/AscendIndexImpl.cpp:587-640: merges the result
  * lists that `ndev` devices (or index shards) returned for the same n queries into one list of k per

@@ -50,6 +50,7 @@ _SIGNATURES = {
     "ixa_last_error": (ctypes.c_char_p, []),
     "ivfpq_last_error": (ctypes.c_char_p, []),
     "ixa_copy_probe": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]),
+    "ixa_read_probe": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]),
     "ixa_merge_search_results": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                 ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p),
                                                 ctypes.c_void_p, ctypes.c_void_p]),

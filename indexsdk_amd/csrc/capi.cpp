@@ -437,6 +437,13 @@ IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
 {
     return guarded([&] { ixa::launch_copy_probe(src_dev, dst_dev, bytes); });
 }
+IXA_EXPORT int ixa_read_probe(const void *src_dev, int64_t bytes, int passes, double *ms_per_pass)
+{
+    return guarded([&] {
+        IXA_REQUIRE(ms_per_pass != nullptr, ixa::kErrInvalidParam, "ms_per_pass can not be nullptr.");
+        *ms_per_pass = ixa::launch_read_probe(src_dev, bytes, passes);
+    });
+}
 IXA_EXPORT int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });

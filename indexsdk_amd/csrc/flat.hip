@@ -323,6 +323,53 @@ __global__ __launch_bounds__(256) void copy_probe_kernel(const uint4 *__restrict
     }
 }
 
+// Plain streaming read: the lanes only fold what they load, and the impossible comparison keeps the loads
+// alive without a store.
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict__ src, int64_t n16,
+                                                         uint32_t *__restrict__ sink)
+{
+    uint32_t acc = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) {
+        const uint4 v = src[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9e3779b9u && sink) {
+        *sink = acc;
+    }
+}
+
+double launch_read_probe(const void *src, int64_t bytes, int passes)
+{
+    IXA_REQUIRE(src && bytes > 0 && bytes % 16 == 0 && passes >= 1 && passes <= 1000, kErrInvalidParam,
+                "read probe needs a multiple of 16 bytes and 1..1000 passes");
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    IXA_HIP(hipEventCreate(&e0));
+    IXA_HIP(hipEventCreate(&e1));
+    float ms = 0.f;
+    // eight workgroups per CU: measured best of 4 / 8 / 16 / 32 on an 8 GiB buffer
+    hipLaunchKernelGGL(read_probe_kernel, dim3(256 * 8), dim3(256), 0, nullptr, static_cast<const uint4 *>(src),
+                       bytes / 16, static_cast<uint32_t *>(nullptr));   // warm-up
+    hipError_t err = hipEventRecord(e0, nullptr);
+    for (int p = 0; p < passes && err == hipSuccess; p++) {
+        hipLaunchKernelGGL(read_probe_kernel, dim3(256 * 8), dim3(256), 0, nullptr, static_cast<const uint4 *>(src),
+                           bytes / 16, static_cast<uint32_t *>(nullptr));
+    }
+    if (err == hipSuccess) {
+        err = hipEventRecord(e1, nullptr);
+    }
+    if (err == hipSuccess) {
+        err = hipEventSynchronize(e1);
+    }
+    if (err == hipSuccess) {
+        err = hipEventElapsedTime(&ms, e0, e1);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    IXA_HIP(err);
+    IXA_HIP(hipGetLastError());
+    return (double)ms / passes;
+}
+
 void launch_copy_probe(const void *src, void *dst, int64_t bytes)
 {
     IXA_REQUIRE(src && dst && bytes > 0 && bytes % 16 == 0, kErrInvalidParam, "copy probe needs a multiple of 16 bytes");

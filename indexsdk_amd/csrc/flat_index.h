@@ -85,5 +85,7 @@ private:
 
 // dst[0:bytes] = src[0:bytes] on the device with a plain copy kernel (traffic-counter yardstick).
 void launch_copy_probe(const void *src, void *dst, int64_t bytes);
+// Average duration (ms) of one plain streaming read of src[0:bytes] over `passes` passes.
+double launch_read_probe(const void *src, int64_t bytes, int passes);
 
 }  // namespace ixa

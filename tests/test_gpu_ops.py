@@ -185,3 +185,15 @@ def test_operators_chained_equal_the_fused_search(env, oracle):
     assert gpu.last_search_stats()["nsplit"] == 2
     assert np.array_equal(Id.get(), np.repeat(I1.get(), 2, axis=1))
     assert np.array_equal(Dd.get().view(np.uint32), np.repeat(D1.get(), 2, axis=1).view(np.uint32))
+
+
+def test_read_probe_reports_a_duration_and_rejects_bad_sizes(env):
+    hip, ix, _capi, lib = env
+    import ctypes
+    buf = hip.empty((1 << 22,), np.float32)          # 16 MiB
+    ms = ctypes.c_double(-1.0)
+    _capi.check(lib.ixa_read_probe(_p(buf), (1 << 22) * 4, 3, ctypes.byref(ms)))
+    assert 0.0 < ms.value < 50.0
+    assert lib.ixa_read_probe(_p(buf), 24, 3, ctypes.byref(ms)) != 0            # not a multiple of 16
+    assert lib.ixa_read_probe(_p(buf), 1 << 20, 0, ctypes.byref(ms)) != 0       # no passes
+    assert lib.ixa_read_probe(None, 1 << 20, 1, ctypes.byref(ms)) != 0
