@@ -22,6 +22,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "topk.h"
 
@@ -155,21 +156,15 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     }
 
     // ---- stage 2: LUT into LDS.  Thread t owns codeword k = t % 256 of every (NT/256)-th sub-quantizer.
+    // For the usual sub-vector lengths the codewords of four entries are loaded before the first is
+    // used: one memory round trip per four entries instead of one per entry, which is most of a
+    // workgroup's start-up time (and of a small batch's latency).  The arithmetic is the same either way.
     {
-        const int dsub = p.dsub;
         const int kk = tid & 255;
-        for (int m = tid >> 8; m < M; m += NT / 256) {
-            const float *qm = qs + m * dsub;
-            const float *cw = p.codebook + ((int64_t)m * 256 + kk) * dsub;
-            float ip = 0.f, qn = 0.f;
-            for (int t = 0; t < dsub; t++) {
-                float qv = qm[t];
-                ip = __fadd_rn(ip, __fmul_rn(qv, cw[t]));
-                qn = __fadd_rn(qn, __fmul_rn(qv, qv));
-            }
+        auto store_entry = [&](int m, float ip, float qn, float cbn) {
             float v;
             if (p.metric == kMetricL2) {
-                v = __fadd_rn(__fadd_rn(p.cb_norms[m * 256 + kk], qn), __fmul_rn(ip, -2.0f));
+                v = __fadd_rn(__fadd_rn(cbn, qn), __fmul_rn(ip, -2.0f));
             } else {
                 v = -ip;  // minimise the negated inner product
             }
@@ -185,6 +180,81 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
                     slot = rot32_half_slot(M / 32, m, kk);
                 }
                 lut[slot] = to_lut<LutT>(v);
+            }
+        };
+        const bool l2 = p.metric == kMetricL2;
+        auto build = [&](auto dsc) {
+            constexpr int DS = decltype(dsc)::value;
+            constexpr int kAhead = 4, kStep = NT / 256;
+            for (int m0 = tid >> 8; m0 < M; m0 += kAhead * kStep) {
+                float cwv[kAhead][DS], cbn[kAhead];
+#pragma unroll
+                for (int u = 0; u < kAhead; u++) {
+                    const int m = m0 + u * kStep;
+                    cbn[u] = 0.f;
+                    if (m < M) {
+                        const float *cw = p.codebook + ((int64_t)m * 256 + kk) * DS;
+                        if constexpr (DS % 4 == 0) {
+#pragma unroll
+                            for (int t = 0; t < DS; t += 4) {
+                                const float4 x = *reinterpret_cast<const float4 *>(cw + t);
+                                cwv[u][t] = x.x;
+                                cwv[u][t + 1] = x.y;
+                                cwv[u][t + 2] = x.z;
+                                cwv[u][t + 3] = x.w;
+                            }
+                        } else if constexpr (DS == 2) {
+                            const float2 x = *reinterpret_cast<const float2 *>(cw);
+                            cwv[u][0] = x.x;
+                            cwv[u][1] = x.y;
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < DS; t++) {
+                                cwv[u][t] = cw[t];
+                            }
+                        }
+                        if (l2) {
+                            cbn[u] = p.cb_norms[m * 256 + kk];
+                        }
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kAhead; u++) {
+                    const int m = m0 + u * kStep;
+                    if (m < M) {
+                        const float *qm = qs + m * DS;
+                        float ip = 0.f, qn = 0.f;
+#pragma unroll
+                        for (int t = 0; t < DS; t++) {
+                            const float qv = qm[t];
+                            ip = __fadd_rn(ip, __fmul_rn(qv, cwv[u][t]));
+                            qn = __fadd_rn(qn, __fmul_rn(qv, qv));
+                        }
+                        store_entry(m, ip, qn, cbn[u]);
+                    }
+                }
+            }
+        };
+        const int dsub = p.dsub;
+        if (dsub == 4) {
+            build(std::integral_constant<int, 4>{});
+        } else if (dsub == 8) {
+            build(std::integral_constant<int, 8>{});
+        } else if (dsub == 2) {
+            build(std::integral_constant<int, 2>{});
+        } else if (dsub == 1) {
+            build(std::integral_constant<int, 1>{});
+        } else {
+            for (int m = tid >> 8; m < M; m += NT / 256) {
+                const float *qm = qs + m * dsub;
+                const float *cw = p.codebook + ((int64_t)m * 256 + kk) * dsub;
+                float ip = 0.f, qn = 0.f;
+                for (int t = 0; t < dsub; t++) {
+                    float qv = qm[t];
+                    ip = __fadd_rn(ip, __fmul_rn(qv, cw[t]));
+                    qn = __fadd_rn(qn, __fmul_rn(qv, qv));
+                }
+                store_entry(m, ip, qn, l2 ? p.cb_norms[m * 256 + kk] : 0.f);
             }
         }
     }
