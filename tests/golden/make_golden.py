@@ -59,5 +59,40 @@ def main():
     print(path, os.path.getsize(path), "bytes")
 
 
+def layouts():
+    """tests/golden/ivfpq_layouts.npz: the three shapes whose scan kernels re-order the code bytes and the
+    LUT (32 sub-quantizers: rot32; 48: xor48; 96 with a half-precision LUT: rot32 with paired blocks and
+    64-byte rows), as small as they can be.  Results do not depend on a layout; the fixture holds what the
+    oracle returns, and the GPU test compares through the tolerance of a re-associated sum."""
+    out = {}
+    for tag, d, M, metric, lut16, seed in (("m32", 32, 32, orc.METRIC_L2, False, 1),
+                                           ("m48", 48, 48, orc.METRIC_L2, False, 2),
+                                           ("m96", 96, 96, orc.METRIC_INNER_PRODUCT, True, 3)):
+        rng = np.random.default_rng(777 + seed)
+        nlist, n, nq, k, nprobe = 8, 400, 12, 20, 3
+        centres = rng.standard_normal((6, d)).astype(np.float32)
+        x = (centres[rng.integers(0, 6, n)] + 0.3 * rng.standard_normal((n, d))).astype(np.float16)
+        q = (centres[rng.integers(0, 6, nq)] + 0.3 * rng.standard_normal((nq, d))).astype(np.float16)
+        xf, qf = x.astype(np.float32), q.astype(np.float32)
+        if metric == orc.METRIC_INNER_PRODUCT:
+            # unit vectors, as far as halves allow: the stored halves are the input
+            x = (xf / np.linalg.norm(xf, axis=1, keepdims=True)).astype(np.float16)
+            q = (qf / np.linalg.norm(qf, axis=1, keepdims=True)).astype(np.float16)
+            xf, qf = x.astype(np.float32), q.astype(np.float32)
+        cent = (np.round(orc.kmeans(xf, nlist, niter=4, seed=seed)[0] * 1024) / 1024).astype(np.float32)
+        cb = (np.round(orc.train_pq(xf, M, niter=3, seed=seed) * 1024) / 1024).astype(np.float16)
+        ids = rng.permutation(50000)[:n].astype(np.int64)
+        idx = orc.CsrIndex.build(d, M, metric, cent, cb.astype(np.float32), xf, ids)
+        D, I = idx.search(qf, k, nprobe, lut_fp16=lut16)
+        out.update({f"{tag}_base": x, f"{tag}_queries": q, f"{tag}_centroids": cent, f"{tag}_codebook": cb,
+                    f"{tag}_ids": ids, f"{tag}_codes": orc.pq_encode(xf, cb.astype(np.float32)),
+                    f"{tag}_assign": orc.assign(xf, cent).astype(np.int32), f"{tag}_D": D, f"{tag}_I": I,
+                    f"{tag}_meta": np.array([d, M, nlist, k, nprobe, metric, int(lut16)], dtype=np.int64)})
+    path = os.path.join(ROOT, "tests", "golden", "ivfpq_layouts.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes")
+
+
 if __name__ == "__main__":
     main()
+    layouts()

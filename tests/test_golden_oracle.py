@@ -39,3 +39,21 @@ def test_oracle_reproduces_flat_fixture(oracle, g):
     x, q = g["base"].astype(np.float32), g["queries"].astype(np.float32)
     D, I = oracle.flat_f32(x[:400], q[:6], 12, oracle.METRIC_L2)
     assert np.array_equal(D, g["flat_f32_D"]) and np.array_equal(I, g["flat_f32_I"])
+
+
+LAYOUTS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ivfpq_layouts.npz")
+
+
+@pytest.mark.parametrize("tag", ["m32", "m48", "m96"])
+def test_oracle_reproduces_layouts_fixture(oracle, tag):
+    """32, 48 and 96 sub-quantizers (the shapes whose GPU kernels re-order code bytes and LUT)."""
+    g = np.load(LAYOUTS, allow_pickle=False)
+    d, M, nlist, k, nprobe, metric, lut16 = (int(v) for v in g[f"{tag}_meta"])
+    x, q = g[f"{tag}_base"].astype(np.float32), g[f"{tag}_queries"].astype(np.float32)
+    cent, cb = g[f"{tag}_centroids"], g[f"{tag}_codebook"].astype(np.float32)
+    assert cent.shape == (nlist, d) and cb.shape == (M, 256, d // M)
+    assert np.array_equal(oracle.assign(x, cent), g[f"{tag}_assign"])
+    assert np.array_equal(oracle.pq_encode(x, cb), g[f"{tag}_codes"])
+    idx = oracle.CsrIndex.build(d, M, metric, cent, cb, x, g[f"{tag}_ids"])
+    D, I = idx.search(q, k, nprobe, lut_fp16=bool(lut16))
+    assert np.array_equal(D, g[f"{tag}_D"]) and np.array_equal(I, g[f"{tag}_I"])
