@@ -46,6 +46,7 @@ __global__ __launch_bounds__(256) void threshold_i32_kernel(const int32_t *__res
 struct F32Ops {
     using T = float;
     using S = float;
+    static constexpr int64_t kMinChunk = 1;   // its score launchers serve any chunk of base rows
     const float *qn, *bn;
     int metric;
     const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
@@ -73,6 +74,7 @@ struct F32Ops {
 struct Bf16Ops {
     using T = uint16_t;
     using S = float;
+    static constexpr int64_t kMinChunk = 2048;   // the ring kernel is the only one for split operands
     const float *qn, *bn;
     int metric;
     const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
@@ -103,6 +105,7 @@ struct Bf16Ops {
 struct I8Ops {
     using T = int8_t;
     using S = int32_t;
+    static constexpr int64_t kMinChunk = 1;
     const int32_t *qn, *bn;
     const S *threshold(StreamSelectWorkspace<S> &ws, int64_t q0, int64_t nq, hipStream_t s) const
     {
@@ -144,7 +147,11 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
         IXA_HIP(hipMemsetAsync(running, 0xff, (size_t)nq_total * ncand * sizeof(key_t), s));
         return 0;
     }
-    const int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
+    int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
+    if (scratch_bytes / (qb * (int64_t)sizeof(S)) < Ops::kMinChunk) {
+        // a small scratch: fewer query rows per block rather than chunks narrower than the kernel serves
+        qb = std::max<int64_t>(128, scratch_bytes / (Ops::kMinChunk * (int64_t)sizeof(S)) / 128 * 128);
+    }
     int64_t nb = scratch_bytes / (qb * (int64_t)sizeof(S));
     nb = std::max<int64_t>(128, nb / 128 * 128);
     nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(nb_total, 1), 128));
@@ -158,6 +165,29 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query; keep
     // that expectation below a quarter of the candidate buffer
     const int64_t growth = std::max<int64_t>(2, cap / (4 * (int64_t)ncand));
+    if (Ops::kMinChunk > 1) {
+        // Dry run of the chunking below (the filtered plan and the materialised one it falls back to): every
+        // chunk must be one the score kernel serves, or the caller takes another route.
+        const int64_t ld_plan = can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb;
+        bool ok = true;
+        auto walk = [&](int64_t head, int64_t width) {
+            for (int64_t b0 = 0; b0 < head; b0 += width) {
+                ok = ok && std::min(width, head - b0) >= Ops::kMinChunk;
+            }
+        };
+        walk(nb_total, nb);
+        if (can_fuse) {
+            walk(seed_rows, ld_plan);
+            for (int64_t seen = seed_rows; seen < nb_total;) {
+                const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * growth, (int64_t)1 << 23});
+                ok = ok && nbc >= Ops::kMinChunk;
+                seen += nbc;
+            }
+        }
+        if (!ok) {
+            return -1;
+        }
+    }
     // the scratch only has to hold the seeding stretch unless the fallback is taken
     ws.scores.resize((size_t)qb * (can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb));
     const int64_t ld = can_fuse ? std::min(nb, round_up(seed_rows, 128)) : nb;
@@ -232,8 +262,8 @@ int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int
                          const float *bn, int metric, int ncand, unsigned long long *running,
                          StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, hipStream_t s)
 {
-    // the ring kernel needs whole K-steps and at least 1024 base rows in every launch; the plan below
-    // only produces launches of the whole base or of >= 2048 rows
+    // the ring kernel needs whole K-steps and at least 2048 base rows in every launch; a plan with a
+    // narrower chunk (a small scratch, a short remainder) answers -1 as well
     if (d3 % 32 != 0 || nb < 2048 || reinterpret_cast<uintptr_t>(Qs) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(Bs) % 16 != 0) {
         return -1;

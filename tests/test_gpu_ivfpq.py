@@ -652,3 +652,25 @@ def test_largest_nprobe(ix, oracle):
     small = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, 64, M, 8, ix.AscendIndexIVFPQConfig())
     small.setNumProbes(100000)
     assert small.getNumProbes() == 64
+
+
+@pytest.mark.parametrize("nlist,nq,scratch", [(2600, 3000, 4 << 20), (5000, 3000, 32 << 20), (12900, 3000, 32 << 20),
+                                              (12900, 700, 64 << 20), (4096, 10000, 64 << 20)])
+def test_coarse_probe_with_a_small_score_scratch(ix, oracle, nlist, nq, scratch):
+    """A score scratch (the reference's resourceSize) far below the default makes the coarse stage walk the
+    centroids in chunks.  The matrix-core kernel for split operands only serves chunks of 2048 rows or more:
+    the plan narrows the query block instead of the chunk, and where a remainder would still be too short it
+    leaves the whole call to the fp32 kernels.  Either way probes and distances are the oracle's."""
+    d, M, nprobe = 32, 8, 24
+    rng = np.random.default_rng(nlist + nq)
+    centres = rng.standard_normal((30, d)).astype(np.float32)
+    cent = (centres[rng.integers(0, 30, nlist)] + 0.4 * rng.standard_normal((nlist, d))).astype(np.float32)
+    q = (centres[rng.integers(0, 30, nq)] + 0.4 * rng.standard_normal((nq, d))).astype(np.float32)
+    cb = rng.standard_normal((M, 256, d // M)).astype(np.float32)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(scratch_bytes=scratch))
+    gpu.set_trained(cent, cb)
+    gpu.setNumProbes(nprobe)
+    gi, gd = gpu.coarse_probe(q)
+    oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
+    assert np.array_equal(gi, oi) and np.array_equal(gd.view(np.uint32), od.view(np.uint32))
+    assert np.array_equal(gpu.assign(q), oracle.assign(q, cent))
