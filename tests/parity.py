@@ -10,13 +10,22 @@ def rel_close(a, b, tol):
     return np.abs(a - b) <= tol * np.maximum(np.maximum(np.abs(a), np.abs(b)), 1e-30)
 
 
+def positions_of(idx, ids):
+    """Rows of ``idx.codes`` that hold the given database ids.  The lookup (ids sorted once, then a binary
+    search) is kept on the index object, so that an index of 10^8 vectors costs one sort, not one per query."""
+    if getattr(idx, "_ids_sorter", None) is None or len(idx._ids_sorter) != len(idx.ids):
+        idx._ids_sorter = np.argsort(idx.ids, kind="stable")
+        idx._ids_sorted = idx.ids[idx._ids_sorter]
+    ids = np.asarray(ids, dtype=np.int64)
+    at = np.searchsorted(idx._ids_sorted, ids)
+    assert (at < len(idx._ids_sorted)).all() and (idx._ids_sorted[at] == ids).all(), "an id that is not in the index"
+    return idx._ids_sorter[at]
+
+
 def candidate_distances(orc, idx, q_row, ids, lut_fp16=False):
     """Oracle ADC distance of arbitrary database ids for one query (for the tie exemption)."""
     lut = orc.lut(q_row[None, :], idx.codebook, idx.metric, lut_fp16=lut_fp16)[0]
-    pos = {int(v): i for i, v in enumerate(idx.ids)}
-    out = []
-    for i in ids:
-        out.append(orc.adc_list(lut, idx.codes[pos[int(i)]][None, :])[0])
+    out = [orc.adc_list(lut, idx.codes[p][None, :])[0] for p in positions_of(idx, ids)]
     return np.array(out, dtype=np.float32)
 
 
@@ -26,9 +35,8 @@ def term_scale(orc, idx, q_row, ids, lut_fp16=False):
     is the distance itself; for inner product the entries have both signs and the sum can cancel to
     almost nothing, where a different association order moves it by ulps of the entries, not of the sum."""
     lut = orc.lut(q_row[None, :], idx.codebook, idx.metric, lut_fp16=lut_fp16)[0].astype(np.float64)
-    pos = {int(v): i for i, v in enumerate(idx.ids)}
     m = np.arange(lut.shape[0])
-    return np.array([np.abs(lut[m, idx.codes[pos[int(i)]]]).sum() for i in ids])
+    return np.array([np.abs(lut[m, idx.codes[p]]).sum() for p in positions_of(idx, ids)])
 
 
 def close_at_scale(orc, idx, q, I, a, b, tol, lut_fp16):
