@@ -159,6 +159,8 @@ def main():
     ap.add_argument("--layout", type=int, default=-1)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--scratch-mb", type=int, default=0,
+                    help="score scratch of the coarse stage in MiB (the reference's resourceSize); 0 = library default")
     ap.add_argument("--same-queries", action="store_true",
                     help="diagnostic: every query is a copy of the first, so the scanned lists stay in L2 "
                          "(the scan kernel's own ceiling, without HBM); not the benchmark")
@@ -204,7 +206,8 @@ def main():
         queries = queries[:1].repeat(nq, 1).contiguous()
     torch.cuda.synchronize()
     cfg = ix.AscendIndexIVFPQConfig(niter=args.niter, train_samples_per_list=1 << 20, code_layout=args.layout,
-                                    lut_fp16=w["lut_fp16"], spherical=1 if metric == ix.METRIC_INNER_PRODUCT else 0)
+                                    lut_fp16=w["lut_fp16"], spherical=1 if metric == ix.METRIC_INNER_PRODUCT else 0,
+                                    **({"scratch_bytes": args.scratch_mb << 20} if args.scratch_mb else {}))
     index = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, cfg)
     _capi.check(lib.ivfpq_train_device(index._h, ntrain, ctypes.c_void_p(train.data_ptr())))
     log(f"trained (nlist={nlist}, M={M}, {ntrain} samples, {args.niter} iters) in {time.time() - t0:.1f}s")
