@@ -159,6 +159,8 @@ def main():
     ap.add_argument("--layout", type=int, default=-1)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target CPU time of the baseline sample")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--locality", type=int, default=-1,
+                    help="scan workgroups ordered by locality: 1, 0, -1 = library default")
     ap.add_argument("--scratch-mb", type=int, default=0,
                     help="score scratch of the coarse stage in MiB (the reference's resourceSize); 0 = library default")
     ap.add_argument("--same-queries", action="store_true",
@@ -206,7 +208,7 @@ def main():
         queries = queries[:1].repeat(nq, 1).contiguous()
     torch.cuda.synchronize()
     cfg = ix.AscendIndexIVFPQConfig(niter=args.niter, train_samples_per_list=1 << 20, code_layout=args.layout,
-                                    lut_fp16=w["lut_fp16"], spherical=1 if metric == ix.METRIC_INNER_PRODUCT else 0,
+                                    lut_fp16=w["lut_fp16"], scan_locality=args.locality, spherical=1 if metric == ix.METRIC_INNER_PRODUCT else 0,
                                     **({"scratch_bytes": args.scratch_mb << 20} if args.scratch_mb else {}))
     index = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, cfg)
     _capi.check(lib.ivfpq_train_device(index._h, ntrain, ctypes.c_void_p(train.data_ptr())))
@@ -273,10 +275,11 @@ def main():
         del src, dst
 
     # HBM traffic of the scan kernel per launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by the
-    # copy probe (profiles/ivfpq_scan_kernel_c2_10M_traffic.md): 1.030 x the algorithmic bytes are fetched,
-    # 12.2 MB are written.  Only quoted for the default workload it was measured on.
+    # copy probe (profiles/ivfpq_scan_kernel_c2_10M_traffic.md): with the workgroups in locality order 0.731 x
+    # the algorithmic bytes are fetched (1.030 x in input order), 12.2 MB are written.  Only quoted for the
+    # default workload it was measured on.
     default_c2 = args.workload == "C2" and not any(getattr(args, key) for key in ("n", "nq", "nlist", "nprobe", "k"))
-    traffic = 1.030 * scan_bytes + 12.2e6 if default_c2 else None
+    traffic = (0.731 if args.locality != 0 else 1.030) * scan_bytes + 12.2e6 if default_c2 else None
     if args.layout in (-1, 1) and M in (32, 64, 96):
         layout_name = "rot32"
     elif args.layout in (-1, 2) and M == 48 and not w["lut_fp16"]:
@@ -299,7 +302,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
                      "streaming_read_GBps": stream_read, "frac_of_streaming_read": achieved / stream_read,
-                     "kernel": "ivfpq_scan_kernel", "bytes_per_launch": scan_bytes, "ms_per_launch": scan_ms_avg},
+                     "kernel": "ivfpq_scan_kernel", "bytes_per_launch": scan_bytes, "ms_per_launch": scan_ms_avg,
+                     "fetched_GBps": None if traffic is None else traffic / (scan_ms_avg * 1e-3) / 1e9},
     }
 
     # The same batch through the host-pointer entry point (queries and results in pageable host memory, as a

@@ -129,6 +129,9 @@ typedef struct ivfpq_config {
                                        {1024..16384, 262144, 524288}, M in {2,4,8,16,32} */
     int32_t coarse_fp32_only;       /* 0 = coarse candidates from bf16 x 3 matrix products, re-evaluated in fp32 and
                                        verified (results identical to the fp32 plan); 1 = fp32 matrix products only */
+    int32_t scan_locality;          /* execution order of the scan's workgroups in large batches (results do not
+                                       depend on it): 1 = queries that probe the same lists run side by side on one
+                                       XCD, 0 = input order, -1 = choose */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */

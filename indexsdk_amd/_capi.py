@@ -30,6 +30,7 @@ class IvfpqConfig(ctypes.Structure):
         ("seed", ctypes.c_uint64),
         ("strict_reference_params", ctypes.c_int32),
         ("coarse_fp32_only", ctypes.c_int32),
+        ("scan_locality", ctypes.c_int32),
     ]
 
 

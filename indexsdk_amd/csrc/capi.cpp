@@ -95,6 +95,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.seed = cfg->seed;
         c.strict_reference_params = cfg->strict_reference_params;
         c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
+        c.scan_locality = cfg->scan_locality;
     }
     return c;
 }
@@ -126,6 +127,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->seed = d.seed;
     cfg->strict_reference_params = d.strict_reference_params;
     cfg->coarse_fp32_only = d.coarse_bf16 ? 0 : 1;
+    cfg->scan_locality = d.scan_locality;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,

@@ -22,6 +22,7 @@ struct IvfpqConfig {
     int64_t scratch_bytes = (int64_t)1 << 30;  // budget of the coarse score scratch
     uint64_t seed = 1234;
     int strict_reference_params = 0;  // 1 = enforce the reference's d / nlist / M whitelists
+    int scan_locality = -1;           // scan workgroups of large batches ordered by locality: 1, 0, -1 = choose
     int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
                                       // stay exact: candidates are re-evaluated in fp32 and the superset
                                       // property is verified, with an fp32 rerun if it cannot be proven)

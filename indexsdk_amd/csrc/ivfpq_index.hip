@@ -871,7 +871,22 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
                              ws_order_.data(), stream_);
         p.order = ws_order_.data();
     }
-    p.xcd_chunks = 0;   // contiguous query chunks per XCD: measured +6 % only with queries sorted by locality
+    // Large batches, one workgroup per query: queries that probe the same lists are made neighbours in the
+    // execution order and every XCD takes a contiguous chunk of it, so that lists shared by neighbours are
+    // fetched into that XCD's L2 once.
+    p.xcd_chunks = 0;
+    const bool by_locality = cfg_.scan_locality < 0 ? n >= 2048 : cfg_.scan_locality > 0;
+    if (!p.order && nsplit == 1 && n >= 16 && by_locality) {
+        ws_order_.resize((size_t)n * 2);
+        if (ws_order_hist_.size() == 0) {
+            ws_order_hist_.resize(2 * 1024);
+            IXA_HIP(hipMemsetAsync(ws_order_hist_.data(), 0, ws_order_hist_.bytes(), stream_));
+        }
+        launch_order_by_locality(probes, n, nprobe, ws_order_.data() + n, ws_order_hist_.data(),
+                                 ws_order_hist_.data() + 1024, ws_order_.data(), stream_);
+        p.order = ws_order_.data();
+        p.xcd_chunks = 1;
+    }
     return p;
 }
 
@@ -898,7 +913,7 @@ void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *pro
     stats_ = SearchStats{};
     stats_.nsplit = p.nsplit;
     stats_.scan_launches = p.nsplit > 1 ? 2 : 1;
-    stats_.ordered = p.order ? 1 : 0;
+    stats_.ordered = p.order ? (p.xcd_chunks ? 2 : 1) : 0;   // 1 = heaviest first, 2 = by locality
     plan_scan(p);
     stats_.scan_waves = p.waves;
     stats_.shared_pool = p.shared_pool;
@@ -944,7 +959,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
         launch_scan(p, n, stream_);
     }
     stats_.coarse_reruns = last_coarse_reruns_;
-    stats_.ordered = p.order ? 1 : 0;
+    stats_.ordered = p.order ? (p.xcd_chunks ? 2 : 1) : 0;   // 1 = heaviest first, 2 = by locality
     {
         ScanParams planned = p;
         plan_scan(planned);

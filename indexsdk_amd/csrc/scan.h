@@ -48,6 +48,11 @@ size_t plan_scan(ScanParams &p);
 
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s);
 
+// order[0 .. nq) = the queries grouped by the lists they probe (class = hash of the smallest probed list id).
+// cls, hist, cursor as below.
+void launch_order_by_locality(const int32_t *probes, int64_t nq, int nprobe, int32_t *cls, int32_t *hist,
+                              int32_t *cursor, int32_t *order, hipStream_t s);
+
 // order[0 .. nq) = the queries by descending work class (work = sum of the probed lists' lengths, at most
 // max_work).  cls: nq ints; hist: 1024 ints that are ZERO on entry and zero again afterwards;
 // cursor: 1024 ints (scratch).

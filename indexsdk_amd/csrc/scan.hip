@@ -668,6 +668,51 @@ __global__ __launch_bounds__(256) void scatter_order_kernel(const int32_t *__res
     }
 }
 
+// ---- execution order: queries that probe the same lists side by side ---------------------------------
+// Queries drawn from one cluster of the data probe nearly the same lists, and the smallest list id
+// among a query's probes is then the same for most of them.  A hash of that id is the query's class,
+// so the counting sort above puts such queries next to each other (with a few strangers whose hash
+// collides, which does no harm: only neighbourhood in time matters, and a class is much shorter than
+// the set of workgroups an XCD runs at once).  Results do not depend on the order.  (Sorting every
+// query's probe list by list id as well, so that neighbours walk their common lists in the same
+// sequence, was measured and is slower: 1.79 against 1.71 ms on 10000 queries x 64 lists of a 10M index.)
+__global__ __launch_bounds__(256) void locality_class_kernel(const int32_t *__restrict__ probes, int64_t nq, int nprobe,
+                                                             int32_t *__restrict__ cls, int32_t *__restrict__ hist)
+{
+    const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (q >= nq) {
+        return;
+    }
+    uint32_t lowest = 0xffffffffu;   // -1 (no list) is the largest value as unsigned
+    for (int j = lane; j < nprobe; j += 64) {
+        const uint32_t l = (uint32_t)probes[q * nprobe + j];
+        lowest = l < lowest ? l : lowest;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)lowest, o);
+        lowest = other < lowest ? other : lowest;
+    }
+    if (lane == 0) {
+        const int c = (int)((lowest * 2654435761u) >> 22);   // 1024 classes
+        cls[q] = c;
+        atomicAdd(&hist[c], 1);
+    }
+}
+
+void launch_order_by_locality(const int32_t *probes, int64_t nq, int nprobe, int32_t *cls, int32_t *hist,
+                              int32_t *cursor, int32_t *order, hipStream_t s)
+{
+    static_assert(kWorkClasses == 1024, "the class hash keeps ten bits");
+    if (nq == 0) {
+        return;
+    }
+    hipLaunchKernelGGL(locality_class_kernel, dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, s, probes, nq, nprobe, cls,
+                       hist);
+    hipLaunchKernelGGL(class_offsets_kernel, dim3(1), dim3(kWorkClasses), 0, s, hist, cursor);
+    hipLaunchKernelGGL(scatter_order_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, cls, nq, cursor, order);
+}
+
 void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, long long max_work,
                           int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s)
 {

@@ -3,6 +3,14 @@ import sys
 
 import pytest
 
+# The full-size tests generate their data with torch on the device.  A process can hold one HIP runtime:
+# torch ships its own, and it has to be the one that is loaded first (the library then binds to it, as it
+# does under bench.py); loaded after the library's, torch finds no device.
+try:
+    import torch  # noqa: F401
+except ImportError:
+    pass
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -566,6 +566,31 @@ def test_few_heavy_workgroups_run_heaviest_first(ix, oracle):
     assert gpu.last_search_stats()["ordered"] == 0
 
 
+def test_large_batches_run_in_locality_order_with_the_same_results(ix, oracle):
+    """Large batches: the scan's workgroups run in an order that puts queries probing the same lists side by
+    side, one contiguous chunk of that order per XCD (a scheduling matter only).  Results are bit-identical
+    to those in input order, for a query count that is no multiple of eight, and equal the oracle's."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 83, 60000, 2051, 64, 128, 16, ix.METRIC_L2, niter=3)
+    cent, cb = gpu.get_trained()
+    results = {}
+    for mode, nq, want in ((0, 2051, 0), (-1, 2051, 2), (1, 2051, 2), (1, 501, 2), (0, 501, 0), (-1, 501, 0)):
+        g = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 128, 16, 8, ix.AscendIndexIVFPQConfig(scan_locality=mode))
+        g.set_trained(cent, cb)
+        g.add_with_ids(x, ids)
+        g.setNumProbes(12)
+        D, I = g.search(q[:nq], 50)
+        st = g.last_search_stats()
+        assert st["ordered"] == want and st["nsplit"] == 1
+        assert st["scanned_codes"] == np.diff(ref.list_off)[oracle.coarse_probe(q[:nq], cent, 12, ix.METRIC_L2)[0]].sum()
+        if nq in results:
+            assert np.array_equal(I, results[nq][1])
+            assert np.array_equal(D.view(np.uint32), results[nq][0].view(np.uint32))
+        else:
+            results[nq] = (D, I)
+            Dr, Ir = ref.search(q[:nq], 50, 12)
+            assert_topk_parity(oracle, ref, q[:nq], D, I, Dr, Ir, TOL_FP32)
+
+
 def test_sixteen_wave_pool_with_an_lds_plan_that_fills_whole_allocation_granules(ix, oracle):
     """M = 48 (64 KB LUT), d = 96, k = 1024 and 64 lists per workgroup make the scan's LDS plan end within
     a few bytes of a multiple of 1280: the control words of the sixteen-wave pool must lie inside it."""
