@@ -195,6 +195,20 @@ int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t
 int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe,
                                int64_t k, float *distances_dev, int64_t *labels_dev);
 
+/* ivfpq_search_probes_device for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments, same results bit for bit; it calls no hipMalloc / hipFree: the intermediates of the launch
+ * (sanitised probe lists, execution order, split partials) lie in a static device array of
+ * IVFPQ_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.  A call that
+ * needs more (8192 + 8 n + 4 n nprobe + 8 n nsplit k bytes, each term rounded up to 256; nsplit <= 8 is
+ * the number of workgroups a query of a small batch is split over) fails with IXA_ERR_INVALID_PARAM and a
+ * message that names the need and the limit.  All calls on one GPU share the array; inside one process
+ * they take turns (a lock), and the array's contents mean nothing between calls.  It leaves
+ * ivfpq_last_search_stats alone.  Waits for the results. */
+#define IVFPQ_NOALLOC_SCRATCH_BYTES (8u << 20)
+int ivfpq_search_probes_device_noalloc(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev,
+                                       int nprobe, int64_t k, float *distances_dev, int64_t *labels_dev);
+
 /* Coarse assignment used by add (nearest centroid under L2), FR/ascend/impl/AscendIndexIVFPQImpl.cpp:603-672;
  * out[n]. */
 int ivfpq_assign(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out_list_ids);

@@ -65,6 +65,9 @@ _SIGNATURES = {
                                                       ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_search_probes_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
                                                   ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
+    "ivfpq_search_probes_device_noalloc": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+                                                          ctypes.c_int, ctypes.c_int64, ctypes.c_void_p,
+                                                          ctypes.c_void_p]),
     "ivfpq_config_default": (None, [ctypes.POINTER(IvfpqConfig)]),
     "ivfpq_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(IvfpqConfig), ctypes.POINTER(_H)]),

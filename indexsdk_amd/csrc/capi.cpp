@@ -435,6 +435,15 @@ IXA_EXPORT int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const flo
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.search_probes(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev); });
 }
+IXA_EXPORT int ivfpq_search_probes_device_noalloc(ivfpq_index_t *h, int64_t n, const float *x_dev,
+                                                  const int32_t *probes_dev, int nprobe, int64_t k,
+                                                  float *distances_dev, int64_t *labels_dev)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        h->impl.search_probes_noalloc(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev);
+    });
+}
 IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
 {
     return guarded([&] { ixa::launch_copy_probe(src_dev, dst_dev, bytes); });

@@ -41,6 +41,13 @@ struct SearchStats {
     double ordered = 0;
 };
 
+// Scratch of one scan launch when the caller of scan_params() provides it.
+struct ScanScratch {
+    int32_t *order;               // 2 n ints: execution order | class of every query
+    int32_t *hist;                // 2048 ints, the first 1024 zero on entry: class histogram | cursors
+    unsigned long long *partial;  // n * nsplit * k keys (only read when a query is split over workgroups)
+};
+
 class IvfpqIndex {
 public:
     IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const IvfpqConfig &cfg);
@@ -71,6 +78,11 @@ public:
     // stages 2-4 only, on probe lists the caller selected (device pointers)
     void search_probes(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k, float *dist_dev,
                        int64_t *labels_dev);
+    // search_probes() with every intermediate in the library's static device scratch: no allocation; sizes
+    // beyond kNoAllocScratchBytes are refused; leaves the statistics of the last search alone
+    void search_probes_noalloc(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k,
+                               float *dist_dev, int64_t *labels_dev);
+    static constexpr size_t kNoAllocScratchBytes = (size_t)8 << 20;
     void assign(int64_t n, const float *x, int64_t *out, bool on_device);               // out: host
     void coarse_probe(int64_t n, const float *x, int64_t *out_ids, float *out_dist, bool on_device);  // out: host
     void encode(int64_t n, const float *x, uint8_t *codes, bool on_device);             // codes: host
@@ -91,7 +103,8 @@ private:
                        float *out_dist, bool set_only = false, bool defer_check = false);
     int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist);
     ScanParams scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
-                           int64_t *ld);
+                           int64_t *ld, const ScanScratch *ext = nullptr);
+    static int scan_nsplit(int64_t n, int nprobe, int64_t k);
     void coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
                            int32_t *out_ids, float *out_dist);
     void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev);
@@ -108,6 +121,7 @@ private:
     bool trained_ = false;
     int64_t ntotal_ = 0;
     hipStream_t stream_ = nullptr;
+    unsigned char *noalloc_scratch_ = nullptr;   // this device's copy of the static scratch (resolved at construction)
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;

@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <numeric>
 #include <random>
 #include <unordered_set>
@@ -14,9 +15,47 @@
 #include "scan.h"
 #include "stream_select.h"
 
+// Scratch of ivfpq_search_probes_device_noalloc (IvfpqIndex::search_probes_noalloc): sanitised probe lists,
+// execution order and split partials of one scan launch.  Every GPU the library runs on holds its own copy
+// at its own address until the process ends; in host code the name below is only a handle for
+// hipGetSymbolAddress, never a device address.  (No `used` attribute: the compiler gives a static device
+// variable that host code refers to a global symbol in the code object, which is what the runtime looks up;
+// with the attribute the symbol stays local and the runtime aborts when the code object is loaded.)
+static __device__ __align__(256) unsigned char scratch[ixa::IvfpqIndex::kNoAllocScratchBytes];
+
 namespace ixa {
 
 namespace {
+
+// Address of the current device's copy of `scratch`, resolved once per device.
+unsigned char *noalloc_scratch_of_current_device()
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static unsigned char *ptr[kMaxDevices] = {};
+    int dev = 0;
+    IXA_HIP(hipGetDevice(&dev));
+    IXA_REQUIRE(dev >= 0 && dev < kMaxDevices, kErrInner, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        IXA_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        IXA_REQUIRE(p != nullptr, kErrInner, "hipGetSymbolAddress returned no address for the static scratch");
+        ptr[dev] = static_cast<unsigned char *>(p);
+    }
+    return ptr[dev];
+}
+
+// Calls that use the static scratch of a device share it; inside one process they take turns.
+std::mutex g_noalloc_mu;
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t *__restrict__ p, int n, int32_t v)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
 
 // Parameter whitelists of the reference (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:130-140).
 const int kRefDims[] = {128};
@@ -277,6 +316,7 @@ IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const
     for (auto &ev : ev_) {
         IXA_HIP(hipEventCreate(&ev));
     }
+    noalloc_scratch_ = noalloc_scratch_of_current_device();
     list_off_.assign(nlist_ + 1, 0);
     list_len_.assign(nlist_, 0);
     sync_list_tables();
@@ -820,9 +860,23 @@ void IvfpqIndex::reset()
     sync_list_tables();
 }
 
-// Parameters of the fused LUT + scan + top-k launch for `n` queries and their probe lists.
+// Workgroups per query of the scan.  Small batches are split over several workgroups per query, about 384
+// workgroups in all and at most eight per query: every workgroup builds the query's whole LUT, so more of
+// them cost more than they balance.  Measured at nlist 16384, nprobe 64: 8 queries 0.31 -> 0.16 ms and 64
+// queries 0.33 -> 0.17 ms against a rule that aimed at 2048 workgroups; from about 400 queries on one
+// workgroup per query is best.
+int IvfpqIndex::scan_nsplit(int64_t n, int nprobe, int64_t k)
+{
+    int nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(8, (384 + n / 2) / n));
+    nsplit = std::min(nsplit, nprobe);
+    return (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));   // one merge pass holds them
+}
+
+// Parameters of the fused LUT + scan + top-k launch for `n` queries and their probe lists.  With `ext` the
+// launch's scratch (split partials, execution order) lies in memory the caller provides and nothing is
+// allocated here.
 ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
-                                   int64_t *ld)
+                                   int64_t *ld, const ScanScratch *ext)
 {
     ScanParams p{};
     p.queries = xd;
@@ -841,17 +895,15 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     p.list_len = list_len_dev_.data();
     p.code_layout = layout_;
     p.k = (int)k;
-    // Small batches are split over several workgroups per query, about 384 workgroups in all and at most
-    // eight per query: every workgroup builds the query's whole LUT, so more of them cost more than they
-    // balance.  Measured at nlist 16384, nprobe 64: 8 queries 0.31 -> 0.16 ms and 64 queries 0.33 -> 0.17 ms
-    // against a rule that aimed at 2048 workgroups; from about 400 queries on one workgroup per query is best.
-    int nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(8, (384 + n / 2) / n));
-    nsplit = std::min(nsplit, nprobe);
-    nsplit = (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));   // one merge pass holds them
+    const int nsplit = scan_nsplit(n, nprobe, k);
     p.nsplit = nsplit;
     if (nsplit > 1) {
-        ws_partial_.resize((size_t)n * nsplit * k);
-        p.partial = ws_partial_.data();
+        if (ext) {
+            p.partial = ext->partial;
+        } else {
+            ws_partial_.resize((size_t)n * nsplit * k);
+            p.partial = ws_partial_.data();
+        }
     }
     p.out_dist = dd;
     p.out_labels = ld;
@@ -860,16 +912,25 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     // no effect on 10000 queries over even lists.
     p.order = nullptr;
     const int64_t codes_per_group = nlist_ > 0 ? ntotal_ / nlist_ * nprobe / nsplit : 0;   // average work of a workgroup
-    if (n * nsplit <= 8192 && n >= 64 && codes_per_group >= 16384) {
-        ws_order_.resize((size_t)n * 2);   // order | class
+    // order | class of every query, and histogram (zero between calls) | cursors of the counting sort
+    int32_t *order = ext ? ext->order : nullptr, *hist = ext ? ext->hist : nullptr;
+    auto own_order_buffers = [&]() {
+        if (ext) {
+            return;
+        }
+        ws_order_.resize((size_t)n * 2);
         if (ws_order_hist_.size() == 0) {
-            ws_order_hist_.resize(2 * 1024);   // histogram (kept zero between calls) | cursors
+            ws_order_hist_.resize(2 * 1024);
             IXA_HIP(hipMemsetAsync(ws_order_hist_.data(), 0, ws_order_hist_.bytes(), stream_));
         }
-        launch_order_by_work(probes, n, nprobe, list_len_dev_.data(), (long long)nprobe * max_list_len_,
-                             ws_order_.data() + n, ws_order_hist_.data(), ws_order_hist_.data() + 1024,
-                             ws_order_.data(), stream_);
-        p.order = ws_order_.data();
+        order = ws_order_.data();
+        hist = ws_order_hist_.data();
+    };
+    if (n * nsplit <= 8192 && n >= 64 && codes_per_group >= 16384) {
+        own_order_buffers();
+        launch_order_by_work(probes, n, nprobe, list_len_dev_.data(), (long long)nprobe * max_list_len_, order + n, hist,
+                             hist + 1024, order, stream_);
+        p.order = order;
     }
     // Large batches, one workgroup per query: queries that probe the same lists are made neighbours in the
     // execution order and every XCD takes a contiguous chunk of it, so that lists shared by neighbours are
@@ -877,14 +938,9 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     p.xcd_chunks = 0;
     const bool by_locality = cfg_.scan_locality < 0 ? n >= 2048 : cfg_.scan_locality > 0;
     if (!p.order && nsplit == 1 && n >= 16 && by_locality) {
-        ws_order_.resize((size_t)n * 2);
-        if (ws_order_hist_.size() == 0) {
-            ws_order_hist_.resize(2 * 1024);
-            IXA_HIP(hipMemsetAsync(ws_order_hist_.data(), 0, ws_order_hist_.bytes(), stream_));
-        }
-        launch_order_by_locality(probes, n, nprobe, ws_order_.data() + n, ws_order_hist_.data(),
-                                 ws_order_hist_.data() + 1024, ws_order_.data(), stream_);
-        p.order = ws_order_.data();
+        own_order_buffers();
+        launch_order_by_locality(probes, n, nprobe, order + n, hist, hist + 1024, order, stream_);
+        p.order = order;
         p.xcd_chunks = 1;
     }
     return p;
@@ -917,6 +973,44 @@ void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *pro
     plan_scan(p);
     stats_.scan_waves = p.waves;
     stats_.shared_pool = p.shared_pool;
+}
+
+// The same call with nothing allocated, for callers that cannot call hipMalloc (HIP graph capture, tight
+// serving loops): the sanitised probe lists, the execution order and the split partials lie in the static
+// device scratch, laid out as [histogram | cursors: 8 KB][order | class: 8 n][probes: 4 n nprobe]
+// [partials: 8 n nsplit k], each part rounded up to 256 bytes.
+void IvfpqIndex::search_probes_noalloc(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k,
+                                       float *dist_dev, int64_t *labels_dev)
+{
+    check_trained();
+    IXA_REQUIRE(x_dev && probes_dev && dist_dev && labels_dev, kErrInvalidParam,
+                "x, probes, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+    IXA_REQUIRE(nprobe > 0 && nprobe <= nlist_, kErrInvalidParam, "nprobe must be > 0 and <= nlist");
+    const int nsplit = scan_nsplit(n, nprobe, k);
+    const int64_t hist_bytes = 2 * 1024 * 4, order_bytes = round_up(n * 8, 256),
+                  probes_bytes = round_up(n * nprobe * 4, 256), partial_bytes = nsplit > 1 ? n * nsplit * k * 8 : 0;
+    const int64_t need = hist_bytes + order_bytes + probes_bytes + partial_bytes;
+    IXA_REQUIRE(need <= (int64_t)kNoAllocScratchBytes, kErrInvalidParam,
+                "n = %ld queries with nprobe = %d and k = %ld need %ld bytes of scratch; the static scratch of the "
+                "no-allocation entry point holds %zu (use ivfpq_search_probes_device, or fewer queries per call)",
+                (long)n, nprobe, (long)k, (long)need, kNoAllocScratchBytes);
+    std::lock_guard<std::mutex> lock(g_noalloc_mu);
+    unsigned char *base = noalloc_scratch_;
+    ScanScratch ext{};
+    ext.hist = reinterpret_cast<int32_t *>(base);
+    ext.order = reinterpret_cast<int32_t *>(base + hist_bytes);
+    int32_t *probes = reinterpret_cast<int32_t *>(base + hist_bytes + order_bytes);
+    ext.partial = reinterpret_cast<unsigned long long *>(base + hist_bytes + order_bytes + probes_bytes);
+    // the array keeps what the last call left: the histogram has to start at zero (a fill kernel, not a
+    // memset node, so that the sequence can be captured into a graph)
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(8), dim3(256), 0, stream_, ext.hist, 2 * 1024, 0);
+    hipLaunchKernelGGL(sanitize_probes_kernel, dim3(blocks_for(n * nprobe)), dim3(256), 0, stream_, probes_dev,
+                       n * nprobe, (int32_t)nlist_, probes);
+    ScanParams p = scan_params(x_dev, n, probes, nprobe, k, dist_dev, labels_dev, &ext);
+    launch_scan(p, n, stream_);
+    sync_stream(stream_);
 }
 
 // -------------------------------------------------------------------------------------------------
