@@ -132,6 +132,11 @@ typedef struct ivfpq_config {
     int32_t scan_locality;          /* execution order of the scan's workgroups in large batches (results do not
                                        depend on it): 1 = queries that probe the same lists run side by side on one
                                        XCD, 0 = input order, -1 = choose */
+    int32_t coarse_sampled_bound;   /* coarse stage of large batches (results do not depend on it): 1 or -1 = the
+                                       admission bound of the score kernel comes from a seed stretch of the centroids
+                                       and every query's candidate list is proven complete by count, so that no
+                                       query x centroid score matrix is written; 0 = the score matrix of a query
+                                       block is written and selected from */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */
@@ -247,7 +252,10 @@ typedef struct ivfpq_search_stats {
     double shared_pool;   /* 1: one workgroup-wide candidate pool (large k), 0: one pool per wavefront */
     double coarse_reruns; /* queries whose matrix-core coarse result could not be proven complete and that were
                              redone from canonical scores of all centroids */
-    double ordered;       /* 1: the scan started its queries in order of decreasing work (few, heavy workgroups) */
+    double ordered;       /* 1: the scan started its queries in order of decreasing work (few, heavy workgroups),
+                             2: in locality order */
+    double coarse_plan;   /* 0: the coarse stage wrote the score matrix and selected from it, 1: sampled bound +
+                             proof by count (queries without proof are part of coarse_reruns) */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 /* Device times of the last search only (HIP events on the index's stream, in ms); either output may be NULL.

@@ -31,13 +31,14 @@ class IvfpqConfig(ctypes.Structure):
         ("strict_reference_params", ctypes.c_int32),
         ("coarse_fp32_only", ctypes.c_int32),
         ("scan_locality", ctypes.c_int32),
+        ("coarse_sampled_bound", ctypes.c_int32),
     ]
 
 
 class IvfpqSearchStats(ctypes.Structure):
     _fields_ = [(n, ctypes.c_double) for n in
                 ("scanned_codes", "ms_coarse", "ms_scan", "ms_total", "scan_launches", "nsplit", "scan_waves",
-                 "shared_pool", "coarse_reruns", "ordered")]
+                 "shared_pool", "coarse_reruns", "ordered", "coarse_plan")]
 
 
 class FlatSearchStats(ctypes.Structure):

@@ -96,6 +96,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.strict_reference_params = cfg->strict_reference_params;
         c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
         c.scan_locality = cfg->scan_locality;
+        c.coarse_sampled_bound = cfg->coarse_sampled_bound;
     }
     return c;
 }
@@ -128,6 +129,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->strict_reference_params = d.strict_reference_params;
     cfg->coarse_fp32_only = d.coarse_bf16 ? 0 : 1;
     cfg->scan_locality = d.scan_locality;
+    cfg->coarse_sampled_bound = d.coarse_sampled_bound;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,
@@ -303,6 +305,7 @@ IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stat
         out->shared_pool = s.shared_pool;
         out->coarse_reruns = s.coarse_reruns;
         out->ordered = s.ordered;
+        out->coarse_plan = s.coarse_plan;
     });
 }
 

@@ -49,6 +49,36 @@ bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, in
                             const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                             hipStream_t s);
 
+// Record mode of the bf16 ring kernel: nothing is stored; every run of four consecutive base rows (first
+// row a multiple of four) whose smallest score is at or below flt.tau[row] is appended to the row's
+// record list: 32 bytes {four fp32 scores, uint32 col_base + first base row, unused} at
+// (unsigned char *)flt.cand + (row * flt.cap + i) * 32, i counted in flt.cnt[row] (which may run past
+// flt.cap: the excess is dropped and the folds below treat such a row as unproven).  nb % 4 == 0.
+bool launch_score_ring_bf16_records(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                                    const float *bn, int metric, ScoreFilter<float> flt, hipStream_t s);
+// Group-minima mode: out[row * ldo + g] = the smallest score of the row among the 32 base rows of group g, for
+// the 8 * ceil(nb / 256) groups of the base (+inf for a group past its end); each base row is in exactly one
+// group.  Nothing else is written.  nb % 4 == 0.
+bool launch_score_ring_bf16_minima(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                                   const float *bn, int metric, float *out, int64_t ldo, hipStream_t s);
+// tau[row] = the rank-th smallest (1-based) of gm[row * G .. + G); G <= 512.
+void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s);
+
+// Largest k of launch_fold_records.
+constexpr int kFoldMaxK = 384;
+// Turns the records of a launch over the WHOLE base into every row's best-k keys (running[nq][k], sorted,
+// kEmptyKey padded; written only), resets cnt[row], and appends every row whose result is not PROVEN to be
+// the k smallest keys of the base (fewer than k scores <= tau[row] on record, or records dropped) to
+// flag[1 + flag[0]++] as row_base + row, marking it by kEmptyKey in its last key.
+void launch_fold_records(unsigned long long *running, int k, ScoreFilter<float> flt, int64_t nq, int *flag,
+                         int64_t row_base, hipStream_t s);
+// launch_fold_records and launch_refine_boundary in one launch, without the sort in between: the exact best
+// nout SET of every row; capk = scores <= tau a row may have on record (at most 2048); rows without proof
+// are appended to flag.  Resets cnt[row].
+void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
+                                 int metric, ScoreFilter<float> flt, int capk, int nout, float cmax, float err_scale,
+                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s);
+
 // out[row] = [hi | hi | lo] (query side) or [hi | lo | hi] (base side) of x[row], each segment
 // zero-padded from d to dp elements of bf16 (stored as uint16_t); out has n * 3 * dp elements.
 void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s);

@@ -534,13 +534,15 @@ __global__ __launch_bounds__(256) void select_rows_kernel(const S *__restrict__ 
 constexpr int kSelRegSeg = 16384;     // columns per segment: 64 per lane
 constexpr int kSelRegStage = 160;     // new candidates per wave and segment
 constexpr int kSelRegMaxK = 384;
+static_assert(kFoldMaxK == kSelRegMaxK, "the record fold ranks with the register selection's key arrays");
 constexpr int kSelRegCap = kSelRegMaxK + 4 * kSelRegStage;   // 1024
 
 // dst[0 .. min(n, keep)) = the smallest keys of src[0 .. n) in ascending order, by counting ranks (the
 // keys are distinct).  src[0 .. have) is already ascending: those keys know their rank among
 // themselves, the others find theirs among them by bisection, and only the n - have new keys are
-// counted against one by one.  n <= 1024, src is 16-byte aligned with src[n] writable; all 256
+// counted against one by one.  n <= 256 E, src is 16-byte aligned with src[n] writable; all 256
 // threads call it; barriers inside.
+template <int E = 4>
 __device__ __forceinline__ void rank_select_256(key_t *src, int have, int n, key_t *dst, int keep, int tid)
 {
     const int first = have & ~1;              // new keys are read in aligned pairs from here on
@@ -548,11 +550,11 @@ __device__ __forceinline__ void rank_select_256(key_t *src, int have, int n, key
         src[n] = kEmptyKey;                   // never below a key
     }
     __syncthreads();
-    key_t mine[4];
-    int rank[4];
+    key_t mine[E];
+    int rank[E];
     const int owned = (n + 255 - tid) >> 8;   // entries tid, tid + 256, ... below n
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
+    for (int e = 0; e < E; e++) {
         const int i = tid + 256 * e;
         mine[e] = i < n ? src[i] : 0;         // 0: its rank is not used
         if (i < have) {
@@ -582,17 +584,25 @@ __device__ __forceinline__ void rank_select_256(key_t *src, int have, int n, key
             rank[0] += (pr.x < mine[0]) + (pr.y < mine[0]);
             rank[1] += (pr.x < mine[1]) + (pr.y < mine[1]);
         }
+    } else if (n <= 1024 || E <= 4) {
+        for (int f = first >> 1; f < (n + 1) >> 1; f++) {
+            const ulonglong2 pr = pairs[f];
+#pragma unroll
+            for (int e = 0; e < (E < 4 ? E : 4); e++) {
+                rank[e] += (pr.x < mine[e]) + (pr.y < mine[e]);
+            }
+        }
     } else {
         for (int f = first >> 1; f < (n + 1) >> 1; f++) {
             const ulonglong2 pr = pairs[f];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
+            for (int e = 0; e < E; e++) {
                 rank[e] += (pr.x < mine[e]) + (pr.y < mine[e]);
             }
         }
     }
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
+    for (int e = 0; e < E; e++) {
         if (e < owned && rank[e] < keep) {
             dst[rank[e]] = mine[e];
         }
@@ -796,6 +806,140 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Fold of the records a record-mode score launch over the WHOLE base appended (runs of four
+// consecutive columns whose smallest score was at or below the row's bound tau) into the row's best-k
+// keys, sorted, with the proof that makes a bound of ANY origin safe: every score <= tau of the base is
+// in the records, so if they hold at least k scores <= tau, their k smallest keys are the k smallest of
+// the whole base.  A row without that proof (or with dropped records) is appended to
+// flag[1 + flag[0]++] and its last key is set to kEmptyKey, which is how the later stages recognise a
+// list they must not judge.  One workgroup per row; k <= kSelRegMaxK.
+constexpr int kFoldCap = 2048;   // scores <= tau the fold ranks at once
+
+__global__ __launch_bounds__(256) void fold_records_kernel(key_t *__restrict__ running, int k, ScoreFilter<float> flt,
+                                                           int *__restrict__ flag, int64_t row_base)
+{
+    __shared__ __align__(16) key_t cand[kFoldCap + 2];
+    __shared__ __align__(16) key_t best[kSelRegMaxK];
+    __shared__ int n_keys;
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    int nrec = flt.cnt[row];
+    bool lost = false;        // workgroup-uniform: something admitted is not among the keys
+    if (nrec > flt.cap) {
+        nrec = flt.cap;
+        lost = true;
+    }
+    if (tid == 0) {
+        n_keys = 0;
+    }
+    __syncthreads();
+    const float tau = flt.tau[row];
+    const unsigned char *records = reinterpret_cast<const unsigned char *>(flt.cand) + (int64_t)row * flt.cap * 32;
+    for (int r = tid; r < nrec; r += 256) {
+        const float4 sc = *reinterpret_cast<const float4 *>(records + (int64_t)r * 32);
+        const uint32_t col = *reinterpret_cast<const uint32_t *>(records + (int64_t)r * 32 + 16);
+        const float v[4] = {sc.x, sc.y, sc.z, sc.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            if (v[t] <= tau) {
+                const int pos = atomicAdd(&n_keys, 1);
+                if (pos < kFoldCap) {
+                    cand[pos] = make_key(v[t], col + (uint32_t)t);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    int n = n_keys;
+    if (n > kFoldCap) {
+        n = kFoldCap;
+        lost = true;
+    }
+    if (n <= 1024) {
+        rank_select_256<4>(cand, 0, n, best, k, tid);
+    } else {
+        rank_select_256<8>(cand, 0, n, best, k, tid);
+    }
+    // proof: at least k scores at or below the bound the launch admitted by
+    const bool proven = !lost && n >= k;
+    key_t *run = running + row * k;
+    for (int i = tid; i < k; i += 256) {
+        key_t kk = i < n ? best[i] : kEmptyKey;
+        if (!proven && i == k - 1) {
+            kk = kEmptyKey;
+        }
+        run[i] = kk;
+    }
+    if (tid == 0) {
+        flt.cnt[row] = 0;
+        if (!proven) {
+            flag[1 + atomicAdd(flag, 1)] = (int)(row_base + row);
+        }
+    }
+}
+
+void launch_fold_records(unsigned long long *running, int k, ScoreFilter<float> flt, int64_t nq, int *flag,
+                         int64_t row_base, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    IXA_REQUIRE(k >= 1 && k <= kSelRegMaxK && k < kFoldCap, kErrInner, "record fold of %d keys", k);
+    hipLaunchKernelGGL(fold_records_kernel, dim3((unsigned)nq), dim3(256), 0, s, running, k, flt, flag, row_base);
+}
+
+// tau[row] = the `rank`-th smallest (1-based) of the row's G group minima gm[row * G .. + G): an upper bound
+// of the rank-th smallest score of the columns the groups cover.  One wavefront per row, the minima in
+// registers, bisection over the ordered score bits.  G <= 64 E.
+template <int E>
+__global__ __launch_bounds__(256) void tau_from_minima_kernel(const float *__restrict__ gm, int G, int rank, int64_t n,
+                                                              float *__restrict__ tau)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n) {
+        return;
+    }
+    uint32_t u[E];
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+        const int i = e * 64 + lane;
+        u[e] = i < G ? ordered_bits(gm[row * G + i]) : 0xffffffffu;
+    }
+    uint32_t p = 0;   // the largest value with fewer than `rank` minima below it = the rank-th smallest
+    for (int bit = 31; bit >= 0; bit--) {
+        const uint32_t c = p | (1u << bit);
+        int below = 0;
+#pragma unroll
+        for (int e = 0; e < E; e++) {
+            below += __popcll(__ballot(u[e] < c));
+        }
+        p = below < rank ? c : p;
+    }
+    if (lane == 0) {
+        tau[row] = unordered_bits(p);
+    }
+}
+
+void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    IXA_REQUIRE(G >= 1 && G <= 512 && rank >= 1 && rank <= G, kErrInner, "rank %d of %d group minima", rank, G);
+    const dim3 grid((unsigned)((nq + 3) / 4)), block(256);
+    if (G <= 64) {
+        hipLaunchKernelGGL(tau_from_minima_kernel<1>, grid, block, 0, s, gm, G, rank, nq, tau);
+    } else if (G <= 128) {
+        hipLaunchKernelGGL(tau_from_minima_kernel<2>, grid, block, 0, s, gm, G, rank, nq, tau);
+    } else if (G <= 256) {
+        hipLaunchKernelGGL(tau_from_minima_kernel<4>, grid, block, 0, s, gm, G, rank, nq, tau);
+    } else {
+        hipLaunchKernelGGL(tau_from_minima_kernel<8>, grid, block, 0, s, gm, G, rank, nq, tau);
+    }
+}
+
 template <typename S>
 static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int64_t nc, int ksel, int32_t *out_idx,
                                  int64_t col_base, unsigned long long *running, bool fresh, hipStream_t s)
@@ -816,7 +960,7 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
     const bool vec4 = ld % 4 == 0 && reinterpret_cast<uintptr_t>(scores) % 16 == 0;
     // measured: the register kernel wins on rows of up to a few segments (16384 columns: 0.17 ms against
     // 0.27 ms for 10000 rows, ksel 88), the streaming kernel on rows of hundreds of thousands of columns
-    if (vec4 && ksel <= kSelRegMaxK && nc >= 4096 && nc <= 6 * kSelRegSeg) {
+    if (vec4 && ksel <= kSelRegMaxK && nc >= 2048 && nc <= 6 * kSelRegSeg) {
         smem = std::max(smem, (size_t)(kSelRegCap + 2 + kSelRegMaxK + 4 * kSelRegStage) * sizeof(key_t) + 4 * 64 * 4 * 4 + 64);
         // groups per lane: ksel / (256 G) stays near 1/3
         auto kern = ksel <= 96 ? select_rows_reg_kernel<S, 1>
@@ -1069,6 +1213,219 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
                        ncand, nout, cmax, err_scale, round_scale, out_ids, flag);
+}
+
+// The boundary refinement above straight from the records of a record-mode score launch over the whole
+// base (see launch_fold_records), without a sorted list in between: one wavefront per query compacts the
+// recorded scores at or below tau into LDS, finds T = the approximate score at rank nout by bisection
+// over the ordered score bits (the scores in registers), classifies against T -+ 2 err and re-evaluates
+// the undecided as above.  The records hold EVERY centroid whose approximate score is at or below tau,
+// so the set is proven complete when tau > T + 2 err -- whatever tau was derived from.  A query without
+// proof (that, dropped records, more scores than the wave's 64 E places, more undecided candidates than
+// amb_cap) is appended to flag[1 + flag[0]++] for the caller's exact plan.
+template <bool VEC4, int E>
+__global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
+    const float *__restrict__ Q, int64_t nq, const float *__restrict__ C, int d, const float *__restrict__ qn,
+    const float *__restrict__ cn, int metric, ScoreFilter<float> flt, int amb_cap, int nout, float cmax,
+    float err_scale, float round_scale, int32_t *__restrict__ out_ids, int *__restrict__ flag, int64_t row_base)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    constexpr int capk = 64 * E;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= nq) {
+        return;
+    }
+    const size_t per_wave = (size_t)capk * sizeof(key_t) + (size_t)amb_cap * (sizeof(key_t) + sizeof(int32_t));
+    key_t *keys = reinterpret_cast<key_t *>(smem_raw + wave * per_wave);
+    key_t *ekeys = keys + capk;
+    int32_t *amb = reinterpret_cast<int32_t *>(ekeys + amb_cap);
+    int32_t *out = out_ids + row * nout;
+    const float tau = flt.tau[row];
+    int nrec = flt.cnt[row];
+    bool fail = nrec > flt.cap;   // wave-uniform: records were dropped
+    nrec = nrec > flt.cap ? flt.cap : nrec;
+    nrec = __builtin_amdgcn_readfirstlane(nrec);
+    // ---- every recorded score at or below tau, compacted; four loads of 64 records in flight at a time
+    int n = 0;
+    const unsigned char *records = reinterpret_cast<const unsigned char *>(flt.cand) + (int64_t)row * flt.cap * 32;
+    for (int base = 0; base < nrec; base += 4 * kWave) {
+        float4 sc[4];
+        uint32_t col[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int r = base + b * kWave + lane;
+            sc[b] = make_float4(0.f, 0.f, 0.f, 0.f);
+            col[b] = 0;
+            if (r < nrec) {
+                sc[b] = *reinterpret_cast<const float4 *>(records + (int64_t)r * 32);
+                col[b] = *reinterpret_cast<const uint32_t *>(records + (int64_t)r * 32 + 16);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const int r = base + b * kWave + lane;
+            const float v[4] = {sc[b].x, sc[b].y, sc[b].z, sc[b].w};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const bool pass = r < nrec && v[t] <= tau;
+                const unsigned long long m = __ballot(pass);
+                if (m) {
+                    const int pos = n + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                                       __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+                    if (pass && pos < capk) {
+                        keys[pos] = make_key(v[t], col[b] + (uint32_t)t);
+                    }
+                    n += __popcll(m);
+                }
+            }
+        }
+    }
+    if (lane == 0) {
+        flt.cnt[row] = 0;   // the next launch's records start at zero
+    }
+    fail = fail || n > capk || n < nout;
+    wave_lds_fence();
+    float lo = 0.f, hi = 0.f;
+    if (!fail) {
+        // ordered bits of the score at rank nout: the largest value with fewer than nout scores below it,
+        // built from the top bit down
+        uint32_t u[E];
+#pragma unroll
+        for (int e = 0; e < E; e++) {
+            const int i = e * kWave + lane;
+            u[e] = i < n ? (uint32_t)(keys[i] >> 32) : 0xffffffffu;
+        }
+        uint32_t p = 0;
+        for (int bit = 31; bit >= 0; bit--) {
+            const uint32_t c = p | (1u << bit);
+            int below = 0;
+#pragma unroll
+            for (int e = 0; e < E; e++) {
+                below += __popcll(__ballot(u[e] < c));
+            }
+            p = below < nout ? c : p;
+        }
+        const float T = unordered_bits(p);
+        const float qlen = sqrtf(qn[row]);
+        const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
+        lo = T - 2.0f * err;
+        hi = T + 2.0f * err;
+        fail = !(tau > hi);
+    }
+    int n_in = 0, n_amb = 0;
+    if (!fail) {
+        for (int base = 0; base < n; base += kWave) {
+            const int i = base + lane;
+            const key_t kk = i < n ? keys[i] : kEmptyKey;
+            const float sc = key_score(kk);
+            const bool in = i < n && sc < lo;
+            const bool und = i < n && !in && sc <= hi;
+            const unsigned long long m_in = __ballot(in), m_und = __ballot(und);
+            const int p_in =
+                __builtin_amdgcn_mbcnt_hi((uint32_t)(m_in >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m_in, 0));
+            const int p_und =
+                __builtin_amdgcn_mbcnt_hi((uint32_t)(m_und >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m_und, 0));
+            if (in) {
+                out[n_in + p_in] = (int32_t)key_index(kk);   // fewer than nout scores lie below T
+            }
+            if (und && n_amb + p_und < amb_cap) {
+                amb[n_amb + p_und] = (int32_t)key_index(kk);
+            }
+            n_in += __popcll(m_in);
+            n_amb += __popcll(m_und);
+        }
+        fail = n_amb > amb_cap;
+    }
+    if (fail) {
+        if (lane == 0) {
+            flag[1 + atomicAdd(flag, 1)] = (int)(row_base + row);   // the list of queries that need another plan
+        }
+        return;
+    }
+    wave_lds_fence();
+    const float *q = Q + row * d;
+    for (int j = lane; j < n_amb; j += kWave) {
+        const int32_t c = amb[j];
+        const float *cv = C + (int64_t)c * d;
+        float g = 0.f;
+        if (VEC4) {
+#pragma unroll 8
+            for (int t = 0; t < d; t += 4) {
+                const float4 a = *reinterpret_cast<const float4 *>(q + t);
+                const float4 b = *reinterpret_cast<const float4 *>(cv + t);
+                g = __fadd_rn(g, __fmul_rn(a.x, b.x));
+                g = __fadd_rn(g, __fmul_rn(a.y, b.y));
+                g = __fadd_rn(g, __fmul_rn(a.z, b.z));
+                g = __fadd_rn(g, __fmul_rn(a.w, b.w));
+            }
+        } else {
+            for (int t = 0; t < d; t++) {
+                g = __fadd_rn(g, __fmul_rn(q[t], cv[t]));
+            }
+        }
+        float v;
+        if (metric == kMetricL2) {
+            v = __fadd_rn(qn[row], cn[c]);
+            v = __fsub_rn(v, g);
+            v = __fsub_rn(v, g);
+        } else {
+            v = -g;
+        }
+        ekeys[j] = make_key(v, (uint32_t)c);
+    }
+    wave_lds_fence();
+    const int need = nout - n_in;   // >= 1: the candidate at rank nout is itself undecided
+    for (int j = lane; j < n_amb; j += kWave) {
+        const key_t mine = ekeys[j];
+        int rank = 0;
+        for (int t = 0; t < n_amb; t++) {
+            rank += ekeys[t] < mine ? 1 : 0;
+        }
+        if (rank < need) {
+            out[n_in + rank] = (int32_t)key_index(mine);
+        }
+    }
+}
+
+template <bool VEC4>
+static void launch_fold_refine_boundary_t(const float *Q, int64_t nq, const float *C, int d, const float *qn,
+                                          const float *cn, int metric, ScoreFilter<float> flt, int capk, int nout,
+                                          float cmax, float err_scale, float round_scale, int32_t *out_ids, int *flag,
+                                          int64_t row_base, hipStream_t s)
+{
+    const int amb_cap = 128;
+    const int E = capk <= 256 ? 4 : (capk <= 512 ? 8 : (capk <= 1024 ? 16 : 32));
+    const size_t smem = (size_t)4 * ((size_t)64 * E * sizeof(key_t) + (size_t)amb_cap * (sizeof(key_t) + sizeof(int32_t)));
+    auto kern = E == 4 ? fold_refine_boundary_kernel<VEC4, 4>
+                       : (E == 8 ? fold_refine_boundary_kernel<VEC4, 8>
+                                 : (E == 16 ? fold_refine_boundary_kernel<VEC4, 16> : fold_refine_boundary_kernel<VEC4, 32>));
+    if (smem > 48 * 1024) {
+        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, flt,
+                       amb_cap, nout, cmax, err_scale, round_scale, out_ids, flag, row_base);
+}
+
+void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
+                                 int metric, ScoreFilter<float> flt, int capk, int nout, float cmax, float err_scale,
+                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s)
+{
+    if (nq == 0) {
+        return;
+    }
+    IXA_REQUIRE(nout >= 1 && capk >= nout && capk <= 2048, kErrInner, "fold refine of %d from %d keys", nout, capk);
+    const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
+                      (reinterpret_cast<uintptr_t>(C) % 16 == 0);
+    if (vec4) {
+        launch_fold_refine_boundary_t<true>(Q, nq, C, d, qn, cn, metric, flt, capk, nout, cmax, err_scale, round_scale,
+                                            out_ids, flag, row_base, s);
+    } else {
+        launch_fold_refine_boundary_t<false>(Q, nq, C, d, qn, cn, metric, flt, capk, nout, cmax, err_scale,
+                                             round_scale, out_ids, flag, row_base, s);
+    }
 }
 
 // Canonical scores of whole rows: out[row * ldo + col] for every centroid, one lane per score, in the

@@ -23,6 +23,9 @@ struct IvfpqConfig {
     uint64_t seed = 1234;
     int strict_reference_params = 0;  // 1 = enforce the reference's d / nlist / M whitelists
     int scan_locality = -1;           // scan workgroups of large batches ordered by locality: 1, 0, -1 = choose
+    int coarse_sampled_bound = -1;    // coarse stage of large batches: 1 / -1 = admission bound from a seed stretch of
+                                      // the centroids and a proof by count (no score matrix is written), 0 = the
+                                      // whole score matrix of a query block is written and selected from
     int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
                                       // stay exact: candidates are re-evaluated in fp32 and the superset
                                       // property is verified, with an fp32 rerun if it cannot be proven)
@@ -39,6 +42,7 @@ struct SearchStats {
     double shared_pool = 0;
     double coarse_reruns = 0;
     double ordered = 0;
+    double coarse_plan = 0;     // 0: score matrix materialised and selected from, 1: sampled bound + proof by count
 };
 
 // Scratch of one scan launch when the caller of scan_params() provides it.
@@ -101,6 +105,7 @@ private:
     // best `nout` lists of every row of device matrix x (canonical arithmetic), device outputs
     void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
                        float *out_dist, bool set_only = false, bool defer_check = false);
+    float bf16x3_err_scale(int select_metric) const;
     int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist);
     ScanParams scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
                            int64_t *ld, const ScanScratch *ext = nullptr);
@@ -130,6 +135,9 @@ private:
     DeviceBuffer<int32_t> ws_order_, ws_order_hist_;   // execution order of the scan (heaviest queries first)
     int32_t max_list_len_ = 0;
     int last_coarse_reruns_ = 0;
+    int last_coarse_plan_ = 0;        // plan of the last coarse_select(): 0 materialised, 1 sampled bound
+    int64_t last_coarse_n_ = 0;       // its number of queries
+    bool sampled_bound_ok_ = true;    // cleared when the sampled bound failed too many proofs on this index
     bool flag_pending_ = true;   // ws_flag_[0] may be non-zero: clear it before the next coarse stage
     bool stats_pending_ = false;
     int64_t stats_rows_ = 0;

@@ -453,14 +453,46 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
     int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 16 + nout / 8);
+    // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
+    // when it was not, so the common case needs no fill in front of the kernels that append to it
+    if (ws_flag_.size() < (size_t)n + 1) {   // grows only, so its first word stays what the last call left
+        ws_flag_.resize((size_t)n + 1);
+        flag_pending_ = true;
+    }
+    if (flag_pending_) {   // new memory, or a deferred verdict that was never read (a failed call in between)
+        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
+    }
+    flag_pending_ = true;
     bool approx = false;
+    last_coarse_plan_ = 0;
+    last_coarse_n_ = n;
     if (cfg_.coarse_bf16) {
         ws_running_.resize((size_t)n * ncand);
         ws_xsplit_.resize((size_t)n * 3 * dp_);
         launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
-        approx = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
-                                      cnorm_.data(), select_metric, ncand, ws_running_.data(), ws_sel_,
-                                      cfg_.scratch_bytes, stream_) >= 0;   // < 0: shape not served
+        // large products: admission bound from a seed stretch, result proven by count, nothing but the seed's
+        // scores written (rows without proof join the list of queries that coarse_finish() redoes exactly)
+        const bool set_wanted = set_only && !out_dist && ncand > nout;   // search: only the SET of lists matters
+        BoundaryRefine br{x_dev, centroids_.data(), d_, nout, cmax_, bf16x3_err_scale(select_metric),
+                          select_metric == kMetricL2 ? 4.0f * 5.9604645e-8f : 0.0f, out_ids};
+        if (sampled_bound_ok_ && cfg_.coarse_sampled_bound != 0 &&
+            stream_select_bf16x3_sampled(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
+                                         cnorm_.data(), select_metric, ncand, ws_running_.data(), ws_sel_,
+                                         cfg_.scratch_bytes, ws_flag_.data(), set_wanted ? &br : nullptr,
+                                         stream_) >= 0) {
+            approx = true;
+            last_coarse_plan_ = 1;
+            if (set_wanted) {   // the plan has written out_ids itself
+                if (!defer_check) {
+                    coarse_finish(x_dev, nout, select_metric, out_ids, out_dist);
+                }
+                return;
+            }
+        } else {
+            approx = stream_select_bf16x3(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
+                                          cnorm_.data(), select_metric, ncand, ws_running_.data(), ws_sel_,
+                                          cfg_.scratch_bytes, stream_) >= 0;   // < 0: shape not served
+        }
     }
     if (!approx) {
         ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 8 + nout / 8);
@@ -480,19 +512,8 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     // (|q| + |c|)^2, the same on both sides up to one unit each.
     const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
     const float u = 5.9604645e-8f;
-    const float err_scale = approx ? dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * u)
-                                   : dots * (float)(2 * d_ + 8) * u;
+    const float err_scale = approx ? bf16x3_err_scale(select_metric) : dots * (float)(2 * d_ + 8) * u;
     const float round_scale = select_metric == kMetricL2 ? 4.0f * u : 0.0f;
-    // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
-    // when it was not, so the common case needs no fill in front of the kernels that append to it
-    if (ws_flag_.size() < (size_t)n + 1) {   // grows only, so its first word stays what the last call left
-        ws_flag_.resize((size_t)n + 1);
-        flag_pending_ = true;
-    }
-    if (flag_pending_) {   // new memory, or a deferred verdict that was never read (a failed call in between)
-        IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
-    }
-    flag_pending_ = true;
     if (approx && set_only && !out_dist && ncand > nout) {
         // search: only the SET of probed lists matters, so only the candidates the approximate scores
         // cannot decide are re-evaluated
@@ -523,6 +544,13 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
 // could not be proven complete from canonical scores of all centroids.  Returns how many there were.
 // search() calls it after it has queued the scan behind the coarse stage, so that the common case (no
 // such query) has no host round trip between the two.
+// Bound on |bf16 x 3 score - canonical score| per unit of |q||c| (derivation in coarse_select()).
+float IvfpqIndex::bf16x3_err_scale(int select_metric) const
+{
+    const float dots = select_metric == kMetricL2 ? 2.0f : 1.0f;
+    return dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * 5.9604645e-8f);
+}
+
 int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist)
 {
     int32_t nfail = 0;
@@ -532,6 +560,11 @@ int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, i
         return 0;
     }
     last_coarse_reruns_ += nfail;
+    if (last_coarse_plan_ == 1 && (int64_t)nfail * 16 > last_coarse_n_) {
+        // the seed stretch does not represent this index's centroids (they come in some order): every
+        // such query costs an exact rerun, so the plan that writes the score matrix is the cheaper one
+        sampled_bound_ok_ = false;
+    }
     std::vector<int32_t> rows32((size_t)nfail);
     IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
     IXA_HIP(hipMemsetAsync(ws_flag_.data(), 0, sizeof(int32_t), stream_));
@@ -1053,6 +1086,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
         launch_scan(p, n, stream_);
     }
     stats_.coarse_reruns = last_coarse_reruns_;
+    stats_.coarse_plan = last_coarse_plan_;
     stats_.ordered = p.order ? (p.xcd_chunks ? 2 : 1) : 0;   // 1 = heaviest first, 2 = by locality
     {
         ScanParams planned = p;

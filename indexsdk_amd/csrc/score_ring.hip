@@ -160,7 +160,14 @@ __host__ __device__ constexpr int ring_vmcnt(int n)
     return 0x0f70 | ((n > 63 ? 63 : n) & 15) | (((n > 63 ? 63 : n) >> 4) << 14);
 }
 
-template <typename Tr, bool FILTER>
+// MODE 0: the scores are stored.  MODE 1: scores at or below the row's bound are appended as keys, one
+// atomic per key.  MODE 2 (fp32 scores): runs of four consecutive columns whose smallest score is at or below
+// the row's bound are appended as 32-byte records {four scores, first column, unused x 3}; a lane counts its
+// passing runs of a query row first and reserves their places with ONE atomic, so a tile costs a wave four
+// atomic round trips whatever the admission rate.  MODE 3 (fp32 scores): nothing but group minima leave the
+// kernel: out[row * ldo + 8 * base tile + 2 * (wave column) + lane half] = the smallest score of the row among
+// that lane's 32 columns of the tile (+inf where it has none).
+template <typename Tr, int MODE>
 __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void score_ring_kernel(
     const typename Tr::T *__restrict__ Q, int64_t nq, const typename Tr::T *__restrict__ B, int64_t nb, int d,
     const typename Tr::S *__restrict__ qn, const typename Tr::S *__restrict__ bn, int metric,
@@ -169,6 +176,8 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
     using T = typename Tr::T;
     using S = typename Tr::S;
     constexpr bool kInt = sizeof(T) == 1;
+    constexpr bool FILTER = MODE != 0, DUMP = MODE == 2, MINIMA = MODE == 3;
+    static_assert(!(DUMP || MINIMA) || !kInt, "record and group-minima epilogues: floating-point scores only");
     extern __shared__ __align__(16) unsigned char ring[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -425,6 +434,110 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
                 }
             }
             wave_lds_fence();
+            if constexpr (MINIMA) {
+#pragma unroll
+                for (int ra = 0; ra < 4; ra++) {
+                    asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
+                    const int64_t row = i0 + (wr * 128 + ra * 32 + l32);
+                    const float rowv = *reinterpret_cast<const float *>(aux + 768 + (ra * 32 + l32) * 4);
+                    int cb = wc * 64 + 4 * half;
+                    asm volatile("" : "+v"(cb));
+                    float best = __builtin_inff();
+#pragma unroll
+                    for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                        for (int rq = 0; rq < 4; rq++) {
+                            const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
+                            const float bnq[4] = {__builtin_bit_cast(float, u.x), __builtin_bit_cast(float, u.y),
+                                                  __builtin_bit_cast(float, u.z), __builtin_bit_cast(float, u.w)};
+                            float m = __builtin_inff();
+#pragma unroll
+                            for (int t = 0; t < 4; t++) {
+                                const float g = acc[ra][rb][rq * 4 + t];
+                                float w;
+                                if (metric == kMetricL2) {
+                                    w = __fadd_rn(rowv, bnq[t]);
+                                    w = __fsub_rn(w, g);
+                                    w = __fsub_rn(w, g);
+                                } else {
+                                    w = -g;
+                                }
+                                m = fminf(m, w);
+                            }
+                            // columns past the end of the base re-read its last row: they count for nothing
+                            // (the base has a multiple of four rows, so a run of four is inside or outside)
+                            best = j0 + cb + rb * 32 + 8 * rq < nb ? fminf(best, m) : best;
+                        }
+                    }
+                    if (row < nq) {
+                        out[row * ldo + (tn * 8 + wc * 2 + half)] = best;
+                    }
+                }
+            } else if constexpr (DUMP) {
+                unsigned char *records = reinterpret_cast<unsigned char *>(flt.cand);
+#pragma unroll
+                for (int ra = 0; ra < 4; ra++) {
+                    asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
+                    const int64_t row = i0 + (wr * 128 + ra * 32 + l32);
+                    const bool row_ok = row < nq;
+                    const float tauv = *reinterpret_cast<const float *>(aux + 256 + (ra * 32 + l32) * 4);
+                    const float rowv = *reinterpret_cast<const float *>(aux + 768 + (ra * 32 + l32) * 4);
+                    float v[2][16];
+                    int npass = 0;
+                    int cb = wc * 64 + 4 * half;   // opaque: no column offsets live across the main loop
+                    asm volatile("" : "+v"(cb));
+#pragma unroll
+                    for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                        for (int rq = 0; rq < 4; rq++) {
+                            const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
+                            const float bnq[4] = {__builtin_bit_cast(float, u.x), __builtin_bit_cast(float, u.y),
+                                                  __builtin_bit_cast(float, u.z), __builtin_bit_cast(float, u.w)};
+#pragma unroll
+                            for (int t = 0; t < 4; t++) {
+                                const float g = acc[ra][rb][rq * 4 + t];
+                                float w;
+                                if (metric == kMetricL2) {
+                                    w = __fadd_rn(rowv, bnq[t]);
+                                    w = __fsub_rn(w, g);
+                                    w = __fsub_rn(w, g);
+                                } else {
+                                    w = -g;
+                                }
+                                v[rb][rq * 4 + t] = w;
+                            }
+                            const float m = fminf(fminf(v[rb][rq * 4], v[rb][rq * 4 + 1]),
+                                                  fminf(v[rb][rq * 4 + 2], v[rb][rq * 4 + 3]));
+                            // columns past the end of the base re-read its last row: never admitted
+                            const bool pass = row_ok && m <= tauv && j0 + cb + rb * 32 + 8 * rq < nb;
+                            npass += pass ? 1 : 0;
+                        }
+                    }
+                    int pos = 0;
+                    if (npass > 0) {
+                        pos = atomicAdd(&flt.cnt[row], npass);
+                    }
+                    unsigned char *rec = records + ((int64_t)row * flt.cap + pos) * 32;
+#pragma unroll
+                    for (int rb = 0; rb < 2; rb++) {
+#pragma unroll
+                        for (int rq = 0; rq < 4; rq++) {
+                            const float m = fminf(fminf(v[rb][rq * 4], v[rb][rq * 4 + 1]),
+                                                  fminf(v[rb][rq * 4 + 2], v[rb][rq * 4 + 3]));
+                            const int64_t col = j0 + cb + rb * 32 + 8 * rq;
+                            if (row_ok && m <= tauv && col < nb) {
+                                if (pos < flt.cap) {
+                                    *reinterpret_cast<float4 *>(rec) = make_float4(v[rb][rq * 4], v[rb][rq * 4 + 1],
+                                                                                   v[rb][rq * 4 + 2], v[rb][rq * 4 + 3]);
+                                    *reinterpret_cast<uint32_t *>(rec + 16) = (uint32_t)(col + flt.col_base);
+                                }
+                                pos++;
+                                rec += 32;
+                            }
+                        }
+                    }
+                }
+            } else {
 #pragma unroll
             for (int ra = 0; ra < 4; ra++) {
                 asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
@@ -497,6 +610,7 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
                     }
                 }
             }
+            }   // !DUMP
         }
         if (!FILTER && last_step) {
             // The stores below queue up behind the loads in flight, and how many of them a wave issues
@@ -585,10 +699,25 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
     }
 }
 
+template <typename Tr, int MODE>
+void launch_ring_mode(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, int64_t nb, int d,
+                      const typename Tr::S *qn, const typename Tr::S *bn, int metric, typename Tr::S *out, int64_t ldo,
+                      ScoreFilter<typename Tr::S> flt, int64_t rt_m, int64_t rt_n, unsigned grid, hipStream_t s)
+{
+    const size_t smem = (size_t)kRingStages * kRingStageBytes + (MODE != 0 ? kRingWaves * kRingAuxBytes : 0);
+    auto kern = score_ring_kernel<Tr, MODE>;
+    IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)smem));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
+                       (int)rt_m, (int)rt_n, flt);
+}
+
+// mode: 0 = store the scores, 1 = append admitted keys, 2 = append admitted runs of four as records
+// (floating-point scores only)
 template <typename Tr>
 bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, int64_t nb, int d,
                  const typename Tr::S *qn, const typename Tr::S *bn, int metric, typename Tr::S *out, int64_t ldo,
-                 bool filter, ScoreFilter<typename Tr::S> flt, hipStream_t s)
+                 int mode, ScoreFilter<typename Tr::S> flt, hipStream_t s)
 {
     if (d % Tr::kElemsPerStep != 0 || nb < 8 * kRingTN || reinterpret_cast<uintptr_t>(Q) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(B) % 16 != 0) {
@@ -605,19 +734,21 @@ bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, i
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
     }
     const unsigned grid = (unsigned)((cus + 7) / 8 * 8);   // one persistent workgroup per CU
-    const size_t smem = (size_t)kRingStages * kRingStageBytes + (filter ? kRingWaves * kRingAuxBytes : 0);
-    if (filter) {
-        auto kern = score_ring_kernel<Tr, true>;
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
-                           (int)rt_m, (int)rt_n, flt);
+    if (mode == 2 || mode == 3) {
+        if constexpr (sizeof(typename Tr::T) == 2) {
+            if (mode == 2) {
+                launch_ring_mode<Tr, 2>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, flt, rt_m, rt_n, grid, s);
+            } else {
+                launch_ring_mode<Tr, 3>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, flt, rt_m, rt_n, grid, s);
+            }
+            return true;
+        }
+        return false;
+    }
+    if (mode == 1) {
+        launch_ring_mode<Tr, 1>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, flt, rt_m, rt_n, grid, s);
     } else {
-        auto kern = score_ring_kernel<Tr, false>;
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
-                           (int)rt_m, (int)rt_n, flt);
+        launch_ring_mode<Tr, 0>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, flt, rt_m, rt_n, grid, s);
     }
     return true;
 }
@@ -628,14 +759,28 @@ bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t 
                           const int32_t *bn, int32_t *out, int64_t ldo, bool filter, ScoreFilter<int32_t> flt,
                           hipStream_t s)
 {
-    return launch_ring<I8Traits>(Q, nq, B, nb, d, qn, bn, kMetricL2, out, ldo, filter, flt, s);
+    return launch_ring<I8Traits>(Q, nq, B, nb, d, qn, bn, kMetricL2, out, ldo, filter ? 1 : 0, flt, s);
 }
 
 bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
                             const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                             hipStream_t s)
 {
-    return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter, flt, s);
+    return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter ? 1 : 0, flt, s);
+}
+
+bool launch_score_ring_bf16_minima(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                                   const float *bn, int metric, float *out, int64_t ldo, hipStream_t s)
+{
+    ScoreFilter<float> flt{};
+    flt.tau = qn;   // the epilogue's operand staging wants a bound array; this mode reads none of it
+    return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, 3, flt, s);
+}
+
+bool launch_score_ring_bf16_records(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
+                                    const float *bn, int metric, ScoreFilter<float> flt, hipStream_t s)
+{
+    return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, nullptr, 0, 2, flt, s);
 }
 
 // ---- bf16 x 3 split --------------------------------------------------------------------------------
@@ -719,7 +864,7 @@ bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t n
                            const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                            hipStream_t s)
 {
-    return launch_ring<F32Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter, flt, s);
+    return launch_ring<F32Traits>(Q, nq, B, nb, d, qn, bn, metric, out, ldo, filter ? 1 : 0, flt, s);
 }
 
 }  // namespace ixa

@@ -10,6 +10,7 @@ struct StreamSelectWorkspace {
     DeviceBuffer<S> scores, tau, thr;
     DeviceBuffer<int32_t> cnt;                    // per-query admitted-candidate counters + overflow flag
     DeviceBuffer<unsigned long long> filter;
+    bool cnt_zero = false;                        // every counter is zero (the sampled-bound plan keeps them so)
 };
 
 // running[nq][ncand] is written only: once the work queued on the stream has run it holds each query's
@@ -29,6 +30,25 @@ int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, in
 int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3, const float *qn,
                          const float *bn, int metric, int ncand, unsigned long long *running,
                          StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, hipStream_t s);
+// The same selection without a score matrix: the score kernel's admission bound comes from group minima
+// over a seed stretch of the base (a bound that holds with overwhelming probability when base rows come in
+// no particular order), the admitted scores are appended as records, and every row's result is PROVEN
+// afterwards; rows without proof are appended to flag[1 + flag[0]++] (flag: 1 + nq ints, flag[0] zero or the
+// count so far) with kEmptyKey in their last key, for the caller's exact plan.  Never waits for the stream.
+// Returns -1 without doing anything when the plan does not apply (short bases, small products, more than
+// 384 keys, unaligned operands, a scratch too small for 128 rows of records).
+// With `refine` the call ends in the exact best-nout SET of every row instead (refine->out_ids[nq][nout],
+// unordered; see launch_fold_refine_boundary) and `running` is not touched.
+struct BoundaryRefine {
+    const float *Q, *C;   // fp32 operands: queries [nq][d], base rows [nb][d]
+    int d, nout;
+    float cmax, err_scale, round_scale;
+    int32_t *out_ids;
+};
+int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3,
+                                 const float *qn, const float *bn, int metric, int ncand, unsigned long long *running,
+                                 StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, int *flag,
+                                 const BoundaryRefine *refine, hipStream_t s);
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
                      int64_t scratch_bytes, hipStream_t s);

@@ -2,6 +2,7 @@
 #include "stream_select.h"
 
 #include <algorithm>
+#include <cmath>
 
 #include "topk.h"
 
@@ -194,6 +195,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     ws.tau.resize((size_t)nq_total);
     ws.thr.resize((size_t)nq_total);
     ws.cnt.resize((size_t)nq_total + 1);
+    ws.cnt_zero = false;
     if (can_fuse) {
         ws.filter.resize((size_t)qb * cap);
     }
@@ -269,6 +271,91 @@ int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int
         return -1;
     }
     return stream_select(Bf16Ops{qn, bn, metric}, Qs, nq, Bs, nb, d3, ncand, running, ws, scratch_bytes, s);
+}
+
+// ---- bound by sample, proof afterwards --------------------------------------------------------------
+// The plan for large query x base products that need only a few keys per row (the IVFPQ coarse stage):
+// no score is ever written to memory except the few a row admits.
+//   1. a group-minima launch over a seed stretch (the first `seed` base rows) leaves, per row, the
+//      smallest score of each group of 32 seed rows: G = seed / 32 values;
+//   2. tau = the j-th smallest of them, an upper bound of the j-th smallest seed score.  j is chosen so
+//      that tau lies at or above the row's r-th smallest score over the WHOLE base with overwhelming
+//      probability (r = the rank the caller's proof needs): the seed holds m = r seed / nb of the true
+//      best r on average (hypergeometric, variance < m), and j = m + 4.5 sqrt(m) + 3;
+//   3. one record-mode launch over the whole base appends every run of four scores with a score <= tau;
+//   4. a fold turns the records into the result and PROVES it per row (launch_fold_records: at least
+//      ncand scores <= tau; launch_fold_refine_boundary: tau above the decision band of rank nout).
+//      Rows without proof (tau too low after all, or records dropped) are appended to `flag` for the
+//      caller's exact plan.
+// About nb (1 - (1 - j / G)^(1/32)) scores per row are admitted instead of nb written and read again.
+// Base rows are assumed to come in no particular order (k-means centroids do); an order that makes the
+// seed unrepresentative only costs proofs, never correctness.  No host synchronisation.
+// Returns the number of score launches, or -1 when the plan does not apply (nothing has been queued).
+int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uint16_t *Bs, int64_t nb_total, int d3,
+                                 const float *qn, const float *bn, int metric, int ncand, unsigned long long *running,
+                                 StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, int *flag,
+                                 const BoundaryRefine *refine, hipStream_t s)
+{
+    if (!flag || d3 % 32 != 0 || nb_total % 4 != 0 || ncand > kFoldMaxK || reinterpret_cast<uintptr_t>(Qs) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(Bs) % 16 != 0) {
+        return -1;
+    }
+    const int64_t seed = round_up(std::max<int64_t>(2048, 16 * (int64_t)ncand), 256);
+    if (nb_total < 4 * seed || nq_total * nb_total < ((int64_t)16 << 20)) {
+        return -1;   // short bases and small products: one materialised pass is cheaper
+    }
+    const int G = (int)(seed / 32);
+    // the rank tau has to reach: the whole candidate list, or rank nout plus room for its decision band
+    const int r = refine ? std::min(ncand, refine->nout + 8 + refine->nout / 16) : ncand;
+    const double m = (double)r * (double)seed / (double)nb_total;
+    const int j = (int)std::ceil(m + 4.5 * std::sqrt(m) + 3.0);
+    if (4 * j > 3 * G) {
+        return -1;   // the seed is too small a sample for this rank
+    }
+    // expected scores <= tau per row: a group's minimum is <= tau with probability j / G
+    const double admitted = (1.0 - std::pow(1.0 - (double)j / G, 1.0 / 32.0)) * (double)nb_total;
+    if (r + 2.0 * admitted > 2048.0) {
+        return -1;   // more than a fold holds
+    }
+    const int capk = (int)std::ceil(r + 2.0 * admitted);                     // scores <= tau a row may have
+    const int cap = std::max(256, pow2_ceil((int)std::ceil(2.0 * admitted)));   // records per row
+    int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
+    if (scratch_bytes / ((int64_t)cap * 32) < qb) {   // the records of a query block stay inside the scratch budget
+        qb = scratch_bytes / ((int64_t)cap * 32) / 128 * 128;
+        if (qb < 128) {
+            return -1;
+        }
+    }
+    ws.scores.resize((size_t)qb * G);
+    ws.tau.resize((size_t)nq_total);
+    const bool fresh_cnt = ws.cnt.size() < (size_t)nq_total + 1;
+    ws.cnt.resize((size_t)nq_total + 1);
+    ws.filter.resize((size_t)qb * cap * 4);   // 32-byte records
+    if (fresh_cnt || !ws.cnt_zero) {
+        IXA_HIP(hipMemsetAsync(ws.cnt.data(), 0, ws.cnt.bytes(), s));   // the folds leave the counters at zero
+    }
+    ws.cnt_zero = false;   // until every fold below has been queued
+    int launches = 0;
+    for (int64_t q0 = 0; q0 < nq_total; q0 += qb) {
+        const int64_t nq = std::min(qb, nq_total - q0);
+        bool ok = launch_score_ring_bf16_minima(Qs + q0 * d3, nq, Bs, seed, d3, qn + q0, bn, metric, ws.scores.data(), G, s);
+        IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
+        launch_tau_from_minima(ws.scores.data(), G, j, nq, ws.tau.data() + q0, s);
+        ScoreFilter<float> flt{ws.tau.data() + q0, nullptr, ws.cnt.data() + q0, ws.filter.data(), cap, 0};
+        ok = launch_score_ring_bf16_records(Qs + q0 * d3, nq, Bs, nb_total, d3, qn + q0, bn, metric, flt, s);
+        IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
+        if (refine) {
+            // only the exact best-nout SET is wanted: no sorted list in between
+            launch_fold_refine_boundary(refine->Q + q0 * refine->d, nq, refine->C, refine->d, qn + q0, bn, metric, flt,
+                                        capk, refine->nout, refine->cmax, refine->err_scale, refine->round_scale,
+                                        refine->out_ids + q0 * refine->nout, flag, q0, s);
+        } else {
+            launch_fold_records(running + q0 * ncand, ncand, flt, nq, flag, q0, s);
+        }
+        launches += 2;
+    }
+    ws.cnt_zero = true;
+    return launches;
 }
 
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
