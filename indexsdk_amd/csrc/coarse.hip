@@ -1247,14 +1247,16 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
     bool fail = nrec > flt.cap;   // wave-uniform: records were dropped
     nrec = nrec > flt.cap ? flt.cap : nrec;
     nrec = __builtin_amdgcn_readfirstlane(nrec);
-    // ---- every recorded score at or below tau, compacted; four loads of 64 records in flight at a time
+    const float qnorm = qn[row];
+    // ---- every recorded score at or below tau, compacted; eight loads of 64 records in flight at a time
     int n = 0;
     const unsigned char *records = reinterpret_cast<const unsigned char *>(flt.cand) + (int64_t)row * flt.cap * 32;
-    for (int base = 0; base < nrec; base += 4 * kWave) {
-        float4 sc[4];
-        uint32_t col[4];
+    constexpr int kBatch = 8;
+    for (int base = 0; base < nrec; base += kBatch * kWave) {
+        float4 sc[kBatch];
+        uint32_t col[kBatch];
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
+        for (int b = 0; b < kBatch; b++) {
             const int r = base + b * kWave + lane;
             sc[b] = make_float4(0.f, 0.f, 0.f, 0.f);
             col[b] = 0;
@@ -1264,7 +1266,10 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
             }
         }
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
+        for (int b = 0; b < kBatch; b++) {
+            if (base + b * kWave >= nrec) {
+                break;   // wave-uniform
+            }
             const int r = base + b * kWave + lane;
             const float v[4] = {sc[b].x, sc[b].y, sc[b].z, sc[b].w};
 #pragma unroll
@@ -1308,7 +1313,7 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
             p = below < nout ? c : p;
         }
         const float T = unordered_bits(p);
-        const float qlen = sqrtf(qn[row]);
+        const float qlen = sqrtf(qnorm);
         const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
         lo = T - 2.0f * err;
         hi = T + 2.0f * err;
@@ -1367,7 +1372,7 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
         }
         float v;
         if (metric == kMetricL2) {
-            v = __fadd_rn(qn[row], cn[c]);
+            v = __fadd_rn(qnorm, cn[c]);
             v = __fsub_rn(v, g);
             v = __fsub_rn(v, g);
         } else {
