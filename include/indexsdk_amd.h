@@ -235,6 +235,16 @@ int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *r
  * missing_ids (room for n entries, may be NULL) and counted in *n_missing (may be NULL). */
 int ivfpq_update(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids, int64_t *missing_ids,
                  int64_t *n_missing);
+/* AscendIndexIVF::reserveMemory(numVecs)  FR/ascend/AscendIndexIVF.h:101-102: makes room for num_vecs more vectors, so
+ * that adding them does not replace the code arena (lists still move inside it as they outgrow their slack). */
+int ivfpq_reserve_memory(ivfpq_index_t *h, int64_t num_vecs);
+/* AscendIndexIVF::reclaimMemory()  FR/ascend/AscendIndexIVF.h:104-106: shrinks the code arena to what the lists hold
+ * (their slack and the holes moved lists left are given back); *bytes_reclaimed may be NULL. */
+int ivfpq_reclaim_memory(ivfpq_index_t *h, int64_t *bytes_reclaimed);
+/* Fill state of the code arena, in slots of msubs + 8 bytes: allocated, handed out to lists (their slack included)
+ * or abandoned, and abandoned by lists that moved.  Any output may be NULL.  No counterpart in the reference
+ * (whose lists are separate device vectors): a diagnostic of the amortised add path. */
+int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocated, int64_t *slots_used, int64_t *slots_holes);
 /* AscendIndexIVF::reset()  FR/ascend/AscendIndexIVF.h:93: drops the lists, keeps the quantizers. */
 int ivfpq_reset(ivfpq_index_t *h);
 int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out);

@@ -69,6 +69,9 @@ _SIGNATURES = {
     "ivfpq_search_probes_device_noalloc": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
                                                           ctypes.c_int, ctypes.c_int64, ctypes.c_void_p,
                                                           ctypes.c_void_p]),
+    "ivfpq_reserve_memory": (ctypes.c_int, [_H, ctypes.c_int64]),
+    "ivfpq_reclaim_memory": (ctypes.c_int, [_H, c_i64p]),
+    "ivfpq_arena_state": (ctypes.c_int, [_H, c_i64p, c_i64p, c_i64p]),
     "ivfpq_config_default": (None, [ctypes.POINTER(IvfpqConfig)]),
     "ivfpq_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(IvfpqConfig), ctypes.POINTER(_H)]),

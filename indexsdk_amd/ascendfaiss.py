@@ -198,6 +198,22 @@ class AscendIndexIVFPQ:
     def reset(self):
         _capi.check(self._lib.ivfpq_reset(self._h))
 
+    def reserveMemory(self, num_vecs):
+        """AscendIndexIVF::reserveMemory: room for num_vecs more vectors without replacing the code arena."""
+        _capi.check(self._lib.ivfpq_reserve_memory(self._h, int(num_vecs)))
+
+    def reclaimMemory(self):
+        """AscendIndexIVF::reclaimMemory: shrinks the code arena to what the lists hold; returns the bytes released."""
+        out = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_reclaim_memory(self._h, ctypes.byref(out)))
+        return out.value
+
+    def arena_state(self):
+        """(slots allocated, slots handed out, slots abandoned by lists that moved) of the code arena."""
+        a, u, h = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_arena_state(self._h, ctypes.byref(a), ctypes.byref(u), ctypes.byref(h)))
+        return a.value, u.value, h.value
+
     def last_search_timings(self):
         """(ms_coarse, ms_scan) of the last search; no device work, usable inside a timed loop."""
         a, b = ctypes.c_double(), ctypes.c_double()

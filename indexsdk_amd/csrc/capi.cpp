@@ -281,6 +281,38 @@ IXA_EXPORT int ivfpq_update(ivfpq_index_t *h, int64_t n, const float *x, const i
         }
     });
 }
+IXA_EXPORT int ivfpq_reserve_memory(ivfpq_index_t *h, int64_t num_vecs)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.reserve_memory(num_vecs); });
+}
+IXA_EXPORT int ivfpq_reclaim_memory(ivfpq_index_t *h, int64_t *bytes_reclaimed)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        const int64_t b = h->impl.reclaim_memory();
+        if (bytes_reclaimed) {
+            *bytes_reclaimed = b;
+        }
+    });
+}
+IXA_EXPORT int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocated, int64_t *slots_used,
+                                 int64_t *slots_holes)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        int64_t a = 0, u = 0, ho = 0;
+        h->impl.arena_state(&a, &u, &ho);
+        if (slots_allocated) {
+            *slots_allocated = a;
+        }
+        if (slots_used) {
+            *slots_used = u;
+        }
+        if (slots_holes) {
+            *slots_holes = ho;
+        }
+    });
+}
 IXA_EXPORT int ivfpq_reset(ivfpq_index_t *h)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.reset(); });

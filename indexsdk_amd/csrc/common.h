@@ -135,6 +135,39 @@ private:
     size_t n_ = 0, cap_ = 0;
 };
 
+// Page-locked host memory for the small copies of latency-bound paths (a copy to or from pageable memory
+// goes through a staging buffer of the runtime).  Grows by reallocation; contents are not preserved.
+class PinnedBuffer {
+public:
+    PinnedBuffer() = default;
+    PinnedBuffer(const PinnedBuffer &) = delete;
+    PinnedBuffer &operator=(const PinnedBuffer &) = delete;
+    ~PinnedBuffer()
+    {
+        if (p_) {
+            (void)hipHostFree(p_);
+        }
+    }
+    void *reserve(size_t bytes)
+    {
+        if (bytes > cap_) {
+            if (p_) {
+                (void)hipHostFree(p_);
+                p_ = nullptr;
+                cap_ = 0;
+            }
+            const size_t want = bytes + bytes / 2 + 4096;
+            IXA_HIP(hipHostMalloc(&p_, want, hipHostMallocDefault));
+            cap_ = want;
+        }
+        return p_;
+    }
+
+private:
+    void *p_ = nullptr;
+    size_t cap_ = 0;
+};
+
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 inline int pow2_ceil(int v)
 {

@@ -93,6 +93,15 @@ public:
     int64_t list_length(int64_t list) const;
     void get_list(int64_t list, uint8_t *codes, int64_t *ids) const;                    // host pointers
     int64_t remove_ids(int64_t n, const int64_t *ids);
+    void reserve_memory(int64_t num_vecs);   // AscendIndexIVF::reserveMemory
+    int64_t reclaim_memory();                // AscendIndexIVF::reclaimMemory: bytes released
+    // slots allocated / handed out / abandoned by lists that moved (the arena's fill state)
+    void arena_state(int64_t *slots, int64_t *used, int64_t *holes) const
+    {
+        *slots = arena_slots_;
+        *used = arena_used_;
+        *holes = hole_slots_;
+    }
     // replaces the vectors of ids that exist; returns the ids that do not (host pointers)
     std::vector<int64_t> update(int64_t n, const float *x, const int64_t *ids);
     void reset();
@@ -112,7 +121,10 @@ private:
     static int scan_nsplit(int64_t n, int nprobe, int64_t k);
     void coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
                            int32_t *out_ids, float *out_dist);
-    void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev);
+    void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev,
+                const float *assigned_from = nullptr);
+    int64_t remove_sorted_ids(const std::vector<int64_t> &gone, std::vector<uint8_t> *found);
+    void relayout(const std::vector<int32_t> &cap, int64_t min_slots);
     void sync_list_tables();
     void kmeans_coarse(const std::vector<float> &sample, int64_t ns);
     void kmeans_pq(const std::vector<float> &sample, int64_t ns);
@@ -156,9 +168,18 @@ private:
     DeviceBuffer<int64_t> ids_;
     DeviceBuffer<int64_t> list_off_dev_;
     DeviceBuffer<int32_t> list_len_dev_;
-    std::vector<int64_t> list_off_;   // first slot of each list (host mirror), size nlist + 1
-    std::vector<int32_t> list_len_;
-    int64_t total_slots_ = 0;
+    std::vector<int64_t> list_off_;   // first slot of each list (host mirror)
+    std::vector<int32_t> list_len_;   // its valid entries
+    std::vector<int32_t> list_cap_;   // the slots it owns (a multiple of 64, >= its length)
+    std::vector<int32_t> touch_mark_; // scratch of append(): -1, or the list's place among the touched lists
+    std::vector<int32_t> add_pos_;    // scratch of append(): position of every new vector inside its list
+    PinnedBuffer add_stage_, add_pack_;   // append(): assignments coming down, kernel inputs going up
+    DeviceBuffer<int64_t> ws_add_pack_, ws_add_ids_;
+    DeviceBuffer<int32_t> ws_add_lists_;
+    DeviceBuffer<uint8_t> ws_add_codes_;
+    int64_t arena_slots_ = 0;         // slots allocated
+    int64_t arena_used_ = 0;          // slots handed out so far (lists and holes)
+    int64_t hole_slots_ = 0;          // slots inside the used part that no list owns any more
     // search workspaces (grown on demand, reused between calls)
     DeviceBuffer<float> ws_x_, ws_qn_, ws_dist_, ws_exact_;
     StreamSelectWorkspace<float> ws_sel_;

@@ -80,31 +80,143 @@ constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
 
 // ---- arena kernels ------------------------------------------------------------------------------
 
-// Copies every list from the old arena to its place in the new one (16-byte units; a list's slot
-// range is a multiple of 64 slots, so both ends are 16-byte aligned for every M).
-__global__ __launch_bounds__(256) void copy_lists_kernel(const uint8_t *__restrict__ old_codes,
-                                                         const int64_t *__restrict__ old_ids,
-                                                         const int64_t *__restrict__ old_off,
-                                                         const int32_t *__restrict__ old_len,
-                                                         uint8_t *__restrict__ new_codes,
-                                                         int64_t *__restrict__ new_ids,
-                                                         const int64_t *__restrict__ new_off, int M)
+// Moves lists inside one arena or from an old arena to a new one: job j copies list lists[j] (its
+// src_len[j] valid entries, whole 64-slot groups) from slot src_off[j] to slot dst_off[j].  Source
+// and destination ranges never overlap (a list moves to free space).  16-byte units; a list starts
+// on a 64-slot boundary, so both ends are 16-byte aligned for every M.
+__global__ __launch_bounds__(256) void move_lists_kernel(const uint8_t *__restrict__ src_codes,
+                                                         const int64_t *__restrict__ src_ids,
+                                                         const int64_t *__restrict__ src_off,
+                                                         const int32_t *__restrict__ src_len,
+                                                         uint8_t *__restrict__ dst_codes, int64_t *__restrict__ dst_ids,
+                                                         const int64_t *__restrict__ dst_off, int M)
 {
-    const int l = blockIdx.x;
-    const int len = old_len[l];
+    const int j = blockIdx.x;
+    const int len = src_len[j];
     if (len == 0) {
         return;
     }
-    const int64_t so = old_off[l], dn = new_off[l];
+    const int64_t so = src_off[j], dn = dst_off[j];
     const int64_t slots = ((int64_t)len + 63) / 64 * 64;
-    const uint4 *src = reinterpret_cast<const uint4 *>(old_codes + so * M);
-    uint4 *dst = reinterpret_cast<uint4 *>(new_codes + dn * M);
+    const uint4 *src = reinterpret_cast<const uint4 *>(src_codes + so * M);
+    uint4 *dst = reinterpret_cast<uint4 *>(dst_codes + dn * M);
     const int64_t n16 = slots * M / 16;
     for (int64_t i = threadIdx.x; i < n16; i += 256) {
         dst[i] = src[i];
     }
     for (int64_t i = threadIdx.x; i < len; i += 256) {
-        new_ids[dn + i] = old_ids[so + i];
+        dst_ids[dn + i] = src_ids[so + i];
+    }
+}
+
+// list_off[lists[j]] = off[j], list_len[lists[j]] = len[j]: the device tables follow the host's for the
+// lists an add touched.
+__global__ __launch_bounds__(256) void update_list_tables_kernel(const int32_t *__restrict__ lists,
+                                                                 const int64_t *__restrict__ off,
+                                                                 const int32_t *__restrict__ len, int n,
+                                                                 int64_t *__restrict__ list_off,
+                                                                 int32_t *__restrict__ list_len)
+{
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j < n) {
+        list_off[lists[j]] = off[j];
+        list_len[lists[j]] = len[j];
+    }
+}
+
+// remove_ids on the device (FR/ascenddaemon/impl/IndexIVFPQ.cpp:346-506 compacts on the device too): one
+// workgroup per list walks it in chunks of 256 entries; an entry whose id is in `gone` (sorted, unique) is
+// dropped, the others close ranks in place keeping their order.  An entry that moves from position p to
+// p2 has its code bytes re-ordered for the position-dependent layouts.  A chunk is read completely (ids
+// and codes into LDS) before any of its survivors is written, and survivors only move towards the list's
+// start, so in-place is safe.  Writes list_len[l], adds to *removed, and marks found[i] = 1 for every
+// gone[i] it met (found may be null).
+__global__ __launch_bounds__(256) void remove_ids_kernel(uint8_t *__restrict__ codes, int64_t *__restrict__ ids,
+                                                         const int64_t *__restrict__ list_off,
+                                                         int32_t *__restrict__ list_len, int M, int layout,
+                                                         const int64_t *__restrict__ gone, int64_t n_gone,
+                                                         uint8_t *__restrict__ found,
+                                                         unsigned long long *__restrict__ removed)
+{
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    uint8_t *stage = smem_raw;                                              // 256 x M code bytes of the chunk
+    int *wsum = reinterpret_cast<int *>(smem_raw + (size_t)256 * M);        // 4 wave totals
+    const int l = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int len = list_len[l];
+    if (len == 0) {
+        return;
+    }
+    const int64_t off = list_off[l];
+    int kept = 0;   // survivors so far (workgroup-uniform)
+    for (int c0 = 0; c0 < len; c0 += 256) {
+        const int p = c0 + tid;
+        const bool valid = p < len;
+        int64_t id = 0;
+        bool drop = false;
+        if (valid) {
+            id = ids[off + p];
+            int64_t lo = 0, hi = n_gone;   // first element not below id
+            while (lo < hi) {
+                const int64_t mid = (lo + hi) >> 1;
+                if (gone[mid] < id) {
+                    lo = mid + 1;
+                } else {
+                    hi = mid;
+                }
+            }
+            drop = lo < n_gone && gone[lo] == id;
+            if (drop && found) {
+                found[lo] = 1;
+            }
+        }
+        const bool keep = valid && !drop;
+        const unsigned long long m = __ballot(keep);
+        const int in_wave = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+        if (lane == 0) {
+            wsum[wave] = __popcll(m);
+        }
+        const int chunk = len - c0 < 256 ? len - c0 : 256;
+        const bool moving = kept < c0 || __syncthreads_or(valid && drop);   // an earlier drop, or one in this chunk
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            before += w < wave ? wsum[w] : 0;
+            total += wsum[w];
+        }
+        if (moving) {
+            // the chunk's code bytes are contiguous: stage them, then every survivor writes its own
+            // (whole 64-slot groups in 16-byte units: a list owns its slots up to the next multiple of 64)
+            const uint4 *src = reinterpret_cast<const uint4 *>(codes + (off + c0) * M);
+            const int n16 = (chunk + 63) / 64 * 64 * M / 16;
+            for (int i = tid; i < n16; i += 256) {
+                reinterpret_cast<uint4 *>(stage)[i] = src[i];
+            }
+            __syncthreads();
+            if (keep) {
+                const int p2 = kept + before + in_wave;
+                uint8_t *dst = codes + (off + p2) * M;
+                const uint8_t *mine = stage + tid * M;
+                for (int j = 0; j < M; j++) {
+                    // byte j of the new slot holds sub-quantizer m2, which the old slot keeps at byte j1
+                    int j1 = j;
+                    if (layout == 1) {
+                        const int m2 = (j & ~31) | ((j + p2) & 31);
+                        j1 = (m2 & ~31) | ((m2 - p) & 31);
+                    } else if (layout == 2) {
+                        j1 = xor48_byte_of_sq(xor48_sq_of_byte(j, p2), p);
+                    }
+                    dst[j] = mine[j1];
+                }
+                ids[off + p2] = id;
+            }
+        }
+        kept += total;
+        __syncthreads();   // the staging area and the wave totals are reused by the next chunk
+    }
+    if (tid == 0 && kept != len) {
+        list_len[l] = kept;
+        atomicAdd(removed, (unsigned long long)(len - kept));
     }
 }
 
@@ -317,8 +429,9 @@ IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const
         IXA_HIP(hipEventCreate(&ev));
     }
     noalloc_scratch_ = noalloc_scratch_of_current_device();
-    list_off_.assign(nlist_ + 1, 0);
-    list_len_.assign(nlist_, 0);
+    list_off_.assign((size_t)nlist_, 0);
+    list_len_.assign((size_t)nlist_, 0);
+    list_cap_.assign((size_t)nlist_, 0);
     sync_list_tables();
 }
 
@@ -652,9 +765,10 @@ void IvfpqIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_devi
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     IXA_REQUIRE(ntotal_ + n < ((int64_t)1 << 32) - 64 * nlist_, kErrInvalidParam,
                 "index would exceed the 32-bit slot space");
-    DeviceBuffer<int32_t> list_no;
-    DeviceBuffer<uint8_t> codes;
-    DeviceBuffer<int64_t> ids_dev;
+    // (workspaces of the add path live in the index: a small add must not pay for allocations)
+    DeviceBuffer<int32_t> &list_no = ws_add_lists_;
+    DeviceBuffer<uint8_t> &codes = ws_add_codes_;
+    DeviceBuffer<int64_t> &ids_dev = ws_add_ids_;
     for (int64_t p0 = 0; p0 < n; p0 += kAddPage) {
         const int64_t np = std::min(kAddPage, n - p0);
         const float *xd = x + p0 * d_;
@@ -672,10 +786,11 @@ void IvfpqIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_devi
             }
         }
         list_no.resize((size_t)np);
-        coarse_select(xd, np, 1, kMetricL2, list_no.data(), nullptr);
+        // the verdict of the assignment's proof is read together with the assignments (one wait, not two)
+        coarse_select(xd, np, 1, kMetricL2, list_no.data(), nullptr, false, true);
         codes.resize((size_t)np * M_);
         launch_pq_encode(xd, np, d_, M_, codebook_.data(), codes.data(), stream_);
-        append(np, list_no.data(), codes.data(), idd);
+        append(np, list_no.data(), codes.data(), idd, xd);
     }
 }
 
@@ -716,47 +831,224 @@ void IvfpqIndex::add_codes_bulk(int64_t n, const int32_t *list_no, const uint8_t
     append(n, ln.data(), cd.data(), idd.data());
 }
 
-void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev)
+// Appends n encoded vectors to their lists, positions inside a list following input order.  Lists have
+// slack: a list whose new length fits its capacity is extended in place; one that does not moves to free
+// space at the end of the arena with half as much room again (a list that is new gets what it needs); when
+// the arena itself is full, a new one (at least half as large again) takes every list in id order, which
+// also reclaims the holes that moved lists left.  An add therefore touches the lists it extends and, now
+// and then, pays for a compaction that its predecessors' growth amortises
+// (FR/ascenddaemon/impl/IndexIVFPQ.cpp:210-235 appends to per-list device vectors in the same way).  Host
+// tables change only after the device work has succeeded.
+void IvfpqIndex::append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev,
+                        const float *assigned_from)
 {
-    std::vector<int32_t> list_no((size_t)n), pos((size_t)n);
-    IXA_HIP(hipMemcpyAsync(list_no.data(), list_no_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream_));
+    // assigned_from: the vectors whose coarse assignment (queued with a deferred verdict) produced list_no_dev
+    int32_t *stage = static_cast<int32_t *>(add_stage_.reserve(((size_t)n + 1) * 4));
+    int32_t *list_no = stage + 1;
+    stage[0] = 0;
+    if (assigned_from) {
+        IXA_HIP(hipMemcpyAsync(stage, ws_flag_.data(), 4, hipMemcpyDeviceToHost, stream_));
+    }
+    IXA_HIP(hipMemcpyAsync(list_no, list_no_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream_));
     sync_stream(stream_);
-    std::vector<int32_t> new_len(list_len_);
+    if (assigned_from) {
+        if (stage[0] != 0) {
+            // some assignments could not be proven: they are redone exactly, and read again
+            coarse_finish(assigned_from, 1, kMetricL2, const_cast<int32_t *>(list_no_dev), nullptr);
+            IXA_HIP(hipMemcpyAsync(list_no, list_no_dev, (size_t)n * 4, hipMemcpyDeviceToHost, stream_));
+            sync_stream(stream_);
+        } else {
+            flag_pending_ = false;
+        }
+    }
+    std::vector<int32_t> &pos = add_pos_;
+    pos.resize((size_t)n);
+    // positions of the new vectors, and the lists they touch (in order of first appearance)
+    std::vector<int32_t> touched, new_len_t;
+    if (touch_mark_.size() != (size_t)nlist_) {
+        touch_mark_.assign((size_t)nlist_, -1);
+    }
     for (int64_t i = 0; i < n; i++) {
-        const int32_t l = list_no[(size_t)i];
-        IXA_REQUIRE(l >= 0 && l < nlist_, kErrInner, "coarse assignment produced list %d", l);
-        pos[(size_t)i] = new_len[(size_t)l]++;
+        const int32_t l = list_no[i];
+        if (!(l >= 0 && l < nlist_)) {
+            for (int32_t t : touched) {
+                touch_mark_[(size_t)t] = -1;
+            }
+            fail(kErrInner, "coarse assignment produced list %d", l);
+        }
+        int32_t &slot = touch_mark_[(size_t)l];
+        if (slot < 0) {
+            slot = (int32_t)touched.size();
+            touched.push_back(l);
+            new_len_t.push_back(list_len_[(size_t)l]);
+        }
+        pos[(size_t)i] = new_len_t[(size_t)slot]++;
     }
-    std::vector<int64_t> new_off((size_t)nlist_ + 1, 0);
-    for (int64_t l = 0; l < nlist_; l++) {
-        new_off[(size_t)l + 1] = new_off[(size_t)l] + round_up(new_len[(size_t)l], 64);
+    for (int32_t t : touched) {
+        touch_mark_[(size_t)t] = -1;
     }
-    const int64_t slots = new_off[(size_t)nlist_];
-    IXA_REQUIRE(slots < ((int64_t)1 << 32) - 1, kErrInvalidParam, "index exceeds the 32-bit slot space");
+    // lists that outgrow their capacity
+    std::vector<int32_t> grow;          // indices into `touched`
+    std::vector<int64_t> new_cap_t(touched.size());
+    int64_t grow_slots = 0, freed_slots = 0;
+    for (size_t t = 0; t < touched.size(); t++) {
+        const int32_t l = touched[t];
+        new_cap_t[t] = list_cap_[(size_t)l];
+        if (new_len_t[t] > list_cap_[(size_t)l]) {
+            const int64_t want = list_cap_[(size_t)l] == 0 ? new_len_t[t] : (int64_t)new_len_t[t] + new_len_t[t] / 2;
+            new_cap_t[t] = round_up(want, 64);
+            grow.push_back((int32_t)t);
+            grow_slots += new_cap_t[t];
+            freed_slots += list_cap_[(size_t)l];
+        }
+    }
+    IXA_REQUIRE(arena_used_ - hole_slots_ - freed_slots + grow_slots < ((int64_t)1 << 32) - 1, kErrInvalidParam,
+                "index exceeds the 32-bit slot space");
+    if (arena_used_ + grow_slots > arena_slots_ || (hole_slots_ + freed_slots) * 2 > arena_used_ + grow_slots) {
+        // the arena is full, or half of it would be holes: a new one takes every list in id order, the growing
+        // lists with their new capacities, and leaves half as much room again for lists that move later
+        std::vector<int32_t> cap_all(list_cap_);
+        for (size_t t = 0; t < touched.size(); t++) {
+            cap_all[(size_t)touched[t]] = (int32_t)new_cap_t[t];
+        }
+        const int64_t live = arena_used_ - hole_slots_ - freed_slots + grow_slots;
+        relayout(cap_all, live + live / 2);
+        grow.clear();
+        freed_slots = 0;
+    }
+    std::vector<int64_t> new_off_t(touched.size());
+    for (size_t t = 0; t < touched.size(); t++) {
+        new_off_t[t] = list_off_[(size_t)touched[t]];
+    }
+    int64_t new_used = arena_used_;
+    // everything the kernels below read goes up in ONE copy of 64-bit words:
+    //   [move jobs: src, dst, len of each growing list][touched lists: list, new first slot, new length][positions]
+    const size_t ng = grow.size(), nt = touched.size();
+    const size_t pack_words = 3 * ng + 3 * nt + ((size_t)n + 1) / 2;
+    int64_t *pack = static_cast<int64_t *>(add_pack_.reserve(pack_words * 8));
+    for (size_t g = 0; g < ng; g++) {
+        const size_t t = (size_t)grow[g];
+        const int32_t l = touched[t];
+        pack[g] = list_off_[(size_t)l];
+        pack[ng + g] = new_used;
+        reinterpret_cast<int32_t *>(pack + 2 * ng)[g] = list_len_[(size_t)l];
+        new_off_t[t] = new_used;
+        new_used += new_cap_t[t];
+    }
+    int64_t *pt = pack + 3 * ng;
+    for (size_t t = 0; t < nt; t++) {
+        pt[t] = new_off_t[t];
+        reinterpret_cast<int32_t *>(pt + nt)[t] = touched[t];
+        reinterpret_cast<int32_t *>(pt + 2 * nt)[t] = new_len_t[t];
+    }
+    std::memcpy(pt + 3 * nt, pos.data(), (size_t)n * 4);
+    try {
+        ws_add_pack_.upload(pack, pack_words, stream_);
+        const int64_t *dp = ws_add_pack_.data();
+        if (ng > 0) {
+            // the lists that outgrew their place move to the end of the used part
+            hipLaunchKernelGGL(move_lists_kernel, dim3((unsigned)ng), dim3(256), 0, stream_, codes_.data(), ids_.data(),
+                               dp, reinterpret_cast<const int32_t *>(dp + 2 * ng), codes_.data(), ids_.data(), dp + ng,
+                               M_);
+        }
+        // the device tables follow for the touched lists, then the new vectors are placed by them
+        const int64_t *dt = dp + 3 * ng;
+        hipLaunchKernelGGL(update_list_tables_kernel, dim3(blocks_for((int64_t)nt)), dim3(256), 0, stream_,
+                           reinterpret_cast<const int32_t *>(dt + nt), dt, reinterpret_cast<const int32_t *>(dt + 2 * nt),
+                           (int)nt, list_off_dev_.data(), list_len_dev_.data());
+        hipLaunchKernelGGL(scatter_new_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, n, list_no_dev,
+                           reinterpret_cast<const int32_t *>(dt + 3 * nt), codes_dev, ids_dev, ntotal_,
+                           list_off_dev_.data(), M_, layout_, codes_.data(), ids_.data());
+        sync_stream(stream_);
+    } catch (...) {
+        sync_list_tables();   // the device tables go back to what the host says (the lists themselves are untouched)
+        throw;
+    }
+    // success: the host's view follows
+    for (size_t t = 0; t < touched.size(); t++) {
+        const int32_t l = touched[t];
+        list_off_[(size_t)l] = new_off_t[t];
+        list_len_[(size_t)l] = new_len_t[t];
+        list_cap_[(size_t)l] = (int32_t)new_cap_t[t];
+        max_list_len_ = std::max(max_list_len_, new_len_t[t]);
+    }
+    arena_used_ = new_used;
+    hole_slots_ += freed_slots;
+    ntotal_ += n;
+}
 
-    DeviceBuffer<uint8_t> new_codes((size_t)std::max<int64_t>(slots, 64) * M_);
-    DeviceBuffer<int64_t> new_ids((size_t)std::max<int64_t>(slots, 64));
-    DeviceBuffer<int64_t> new_off_dev;
-    DeviceBuffer<int32_t> pos_dev;
-    new_off_dev.upload(new_off.data(), (size_t)nlist_, stream_);
-    pos_dev.upload(pos.data(), (size_t)n, stream_);
+// A new arena of at least min_slots slots takes every list in id order, list l with cap[l] slots (>= its
+// length rounded up to 64).  The old arena is released only after the new one is complete, so a failure
+// (no memory for the second copy) leaves the index as it was.
+void IvfpqIndex::relayout(const std::vector<int32_t> &cap, int64_t min_slots)
+{
+    std::vector<int64_t> off((size_t)nlist_);
+    int64_t at = 0;
+    for (int64_t l = 0; l < nlist_; l++) {
+        off[(size_t)l] = at;
+        at += cap[(size_t)l];
+    }
+    int64_t slots = round_up(std::max<int64_t>({at, min_slots, 1024}), 64);
+    slots = std::min<int64_t>(slots, ((int64_t)1 << 32) - 64);
+    IXA_REQUIRE(slots >= at, kErrInvalidParam, "index exceeds the 32-bit slot space");
+    DeviceBuffer<uint8_t> new_codes((size_t)slots * M_);
+    DeviceBuffer<int64_t> new_ids((size_t)slots);
+    DeviceBuffer<int64_t> off_dev;
     IXA_HIP(hipMemsetAsync(new_codes.data(), 0, new_codes.bytes(), stream_));
     IXA_HIP(hipMemsetAsync(new_ids.data(), 0xff, new_ids.bytes(), stream_));
+    off_dev.upload(off.data(), (size_t)nlist_, stream_);
     if (ntotal_ > 0) {
-        hipLaunchKernelGGL(copy_lists_kernel, dim3((unsigned)nlist_), dim3(256), 0, stream_, codes_.data(),
-                           ids_.data(), list_off_dev_.data(), list_len_dev_.data(), new_codes.data(), new_ids.data(),
-                           new_off_dev.data(), M_);
+        hipLaunchKernelGGL(move_lists_kernel, dim3((unsigned)nlist_), dim3(256), 0, stream_, codes_.data(), ids_.data(),
+                           list_off_dev_.data(), list_len_dev_.data(), new_codes.data(), new_ids.data(), off_dev.data(),
+                           M_);
     }
-    hipLaunchKernelGGL(scatter_new_kernel, dim3(blocks_for(n)), dim3(256), 0, stream_, n, list_no_dev, pos_dev.data(),
-                       codes_dev, ids_dev, ntotal_, new_off_dev.data(), M_, layout_, new_codes.data(), new_ids.data());
     sync_stream(stream_);
     codes_ = std::move(new_codes);
     ids_ = std::move(new_ids);
-    list_off_ = std::move(new_off);
-    list_len_ = std::move(new_len);
-    total_slots_ = slots;
-    ntotal_ += n;
-    sync_list_tables();
+    list_off_ = std::move(off);
+    list_cap_ = cap;
+    arena_slots_ = slots;
+    arena_used_ = at;
+    hole_slots_ = 0;
+    list_off_dev_.upload(list_off_.data(), (size_t)nlist_, stream_);
+    sync_stream(stream_);
+}
+
+// AscendIndexIVF::reserveMemory(numVecs) (FR/ascend/AscendIndexIVF.h): room for num_vecs more vectors before
+// the arena has to be replaced (spread over the lists in proportion to nothing: lists still move inside the
+// arena as they grow; what is reserved is the arena itself).
+void IvfpqIndex::reserve_memory(int64_t num_vecs)
+{
+    flush_stats();
+    IXA_REQUIRE(num_vecs >= 0 && num_vecs < kMaxN, kErrInvalidParam, "numVecs must be >= 0 and < %ld", (long)kMaxN);
+    // every list may round its share up to a multiple of 64 and move once with half as much room again
+    const int64_t want = arena_used_ + num_vecs + num_vecs / 2 + 64 * nlist_;
+    if (want > arena_slots_) {
+        relayout(list_cap_, std::min<int64_t>(want, ((int64_t)1 << 32) - 64));
+    }
+}
+
+// AscendIndexIVF::reclaimMemory() (FR/ascend/AscendIndexIVF.h): gives back what the lists do not use; returns
+// the bytes released.
+int64_t IvfpqIndex::reclaim_memory()
+{
+    flush_stats();
+    const int64_t before = arena_slots_;
+    std::vector<int32_t> cap((size_t)nlist_);
+    int64_t need = 0;
+    for (int64_t l = 0; l < nlist_; l++) {
+        cap[(size_t)l] = (int32_t)round_up(list_len_[(size_t)l], 64);
+        need += cap[(size_t)l];
+    }
+    if (ntotal_ == 0) {
+        reset();
+        return before * (M_ + 8);
+    }
+    if (round_up(std::max<int64_t>(need, 1024), 64) >= before) {
+        return 0;
+    }
+    relayout(cap, 0);
+    return (before - arena_slots_) * (M_ + 8);
 }
 
 int64_t IvfpqIndex::list_length(int64_t list) const
@@ -785,9 +1077,45 @@ void IvfpqIndex::get_list(int64_t list, uint8_t *codes, int64_t *ids) const
     }
 }
 
-// remove_ids: every list is filtered in place keeping the order of the survivors
-// (FR/ascenddaemon/impl/IndexIVFPQ.cpp:346-506).  Host-mediated: the arena is read back, filtered
-// and re-appended list by list.
+// remove_ids: every list is filtered in place on the device, keeping the order of the survivors
+// (FR/ascenddaemon/impl/IndexIVFPQ.cpp:346-506).  The ids go up sorted; one workgroup per list looks its
+// entries up by bisection and compacts.  `found`, when given, receives for every entry of the SORTED
+// UNIQUE id list whether the index held it.
+int64_t IvfpqIndex::remove_sorted_ids(const std::vector<int64_t> &gone, std::vector<uint8_t> *found)
+{
+    if (gone.empty() || ntotal_ == 0) {
+        if (found) {
+            found->assign(gone.size(), 0);
+        }
+        return 0;
+    }
+    DeviceBuffer<int64_t> gone_dev;
+    DeviceBuffer<uint8_t> found_dev;
+    DeviceBuffer<unsigned long long> removed_dev(1);
+    gone_dev.upload(gone.data(), gone.size(), stream_);
+    if (found) {
+        found_dev.resize(gone.size());
+        IXA_HIP(hipMemsetAsync(found_dev.data(), 0, found_dev.bytes(), stream_));
+    }
+    IXA_HIP(hipMemsetAsync(removed_dev.data(), 0, 8, stream_));
+    const size_t smem = (size_t)256 * M_ + 64;
+    hipLaunchKernelGGL(remove_ids_kernel, dim3((unsigned)nlist_), dim3(256), smem, stream_, codes_.data(), ids_.data(),
+                       list_off_dev_.data(), list_len_dev_.data(), M_, layout_, gone_dev.data(), (int64_t)gone.size(),
+                       found ? found_dev.data() : nullptr, removed_dev.data());
+    unsigned long long removed = 0;
+    removed_dev.download(&removed, 1, stream_);
+    if (found) {
+        found->resize(gone.size());
+        found_dev.download(found->data(), gone.size(), stream_);
+    }
+    if (removed > 0) {
+        list_len_dev_.download(list_len_.data(), (size_t)nlist_, stream_);
+        max_list_len_ = *std::max_element(list_len_.begin(), list_len_.end());
+        ntotal_ -= (int64_t)removed;
+    }
+    return (int64_t)removed;
+}
+
 int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
 {
     flush_stats();
@@ -795,50 +1123,10 @@ int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
     if (n == 0 || ntotal_ == 0) {
         return 0;
     }
-    std::unordered_set<int64_t> del(ids, ids + n);
-    std::vector<int64_t> all_ids((size_t)total_slots_);
-    IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
-    sync_stream(stream_);
-    std::vector<int32_t> keep_list;
-    std::vector<int64_t> keep_ids;
-    std::vector<uint8_t> keep_codes, buf;
-    int64_t removed = 0;
-    for (int64_t l = 0; l < nlist_; l++) {
-        const int64_t len = list_len_[(size_t)l], off = list_off_[(size_t)l];
-        if (len == 0) {
-            continue;
-        }
-        bool any = false;
-        for (int64_t i = 0; i < len && !any; i++) {
-            any = del.count(all_ids[(size_t)(off + i)]) != 0;
-        }
-        buf.resize((size_t)len * M_);
-        get_list(l, buf.data(), nullptr);
-        for (int64_t i = 0; i < len; i++) {
-            const int64_t id = all_ids[(size_t)(off + i)];
-            if (any && del.count(id)) {
-                removed++;
-                continue;
-            }
-            keep_list.push_back((int32_t)l);
-            keep_ids.push_back(id);
-            keep_codes.insert(keep_codes.end(), buf.begin() + i * M_, buf.begin() + (i + 1) * M_);
-        }
-    }
-    if (removed == 0) {
-        return 0;
-    }
-    reset();
-    if (!keep_ids.empty()) {
-        DeviceBuffer<int32_t> ln;
-        DeviceBuffer<uint8_t> cd;
-        DeviceBuffer<int64_t> idd;
-        ln.upload(keep_list.data(), keep_list.size(), stream_);
-        cd.upload(keep_codes.data(), keep_codes.size(), stream_);
-        idd.upload(keep_ids.data(), keep_ids.size(), stream_);
-        append((int64_t)keep_ids.size(), ln.data(), cd.data(), idd.data());
-    }
-    return removed;
+    std::vector<int64_t> gone(ids, ids + n);
+    std::sort(gone.begin(), gone.end());
+    gone.erase(std::unique(gone.begin(), gone.end()), gone.end());
+    return remove_sorted_ids(gone, nullptr);
 }
 
 // update (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:540-601): ids that exist are deleted and re-added with
@@ -850,22 +1138,16 @@ std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t
     IXA_REQUIRE(x, kErrInvalidParam, "vector list is nullptr!");
     IXA_REQUIRE(ids, kErrInvalidParam, "vector ID list is nullptr!");
     IXA_REQUIRE(n > 0, kErrInvalidParam, "update vector number must be greater than 0!");
-    std::unordered_set<int64_t> present;
-    if (ntotal_ > 0) {
-        std::vector<int64_t> all_ids((size_t)total_slots_);
-        IXA_HIP(hipMemcpyAsync(all_ids.data(), ids_.data(), all_ids.size() * 8, hipMemcpyDeviceToHost, stream_));
-        sync_stream(stream_);
-        for (int64_t l = 0; l < nlist_; l++) {
-            const int64_t off = list_off_[(size_t)l];
-            for (int64_t i = 0; i < list_len_[(size_t)l]; i++) {
-                present.insert(all_ids[(size_t)(off + i)]);
-            }
-        }
-    }
+    std::vector<int64_t> gone(ids, ids + n);
+    std::sort(gone.begin(), gone.end());
+    gone.erase(std::unique(gone.begin(), gone.end()), gone.end());
+    std::vector<uint8_t> found;
+    remove_sorted_ids(gone, &found);   // the removal itself tells which ids the index held
     std::vector<int64_t> missing, exist_ids;
     std::vector<float> exist_x;
     for (int64_t i = 0; i < n; i++) {
-        if (present.count(ids[i])) {
+        const size_t at = (size_t)(std::lower_bound(gone.begin(), gone.end(), ids[i]) - gone.begin());
+        if (found[at]) {
             exist_ids.push_back(ids[i]);
             exist_x.insert(exist_x.end(), x + i * d_, x + (i + 1) * d_);
         } else {
@@ -873,7 +1155,6 @@ std::vector<int64_t> IvfpqIndex::update(int64_t n, const float *x, const int64_t
         }
     }
     if (!exist_ids.empty()) {
-        remove_ids((int64_t)exist_ids.size(), exist_ids.data());
         add((int64_t)exist_ids.size(), exist_x.data(), exist_ids.data(), false);
     }
     return missing;
@@ -886,9 +1167,10 @@ void IvfpqIndex::reset()
     sync_stream(stream_);
     codes_.release();
     ids_.release();
-    list_off_.assign((size_t)nlist_ + 1, 0);
+    list_off_.assign((size_t)nlist_, 0);
     list_len_.assign((size_t)nlist_, 0);
-    total_slots_ = 0;
+    list_cap_.assign((size_t)nlist_, 0);
+    arena_slots_ = arena_used_ = hole_slots_ = 0;
     ntotal_ = 0;
     sync_list_tables();
 }

@@ -103,6 +103,46 @@ def test_full_size_sample_against_the_oracle(big, oracle):
     assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
 
 
+def test_full_size_incremental_writes(big):
+    """On the 10M index: small adds extend lists in place (the arena is not replaced every time), a removal
+    of 1000 ids is a device-side compaction that takes milliseconds, removed ids never come back, and vectors
+    added afterwards are found by their own queries.  (Runs last of the tests that share the index: it
+    changes it.)"""
+    import time
+    ix, index, q, keep = big
+    rng = np.random.default_rng(99)
+    sizes = {index.arena_state()[0]}
+    t0 = time.perf_counter()
+    new_rows = []
+    for c in range(20):
+        x = (keep["rows"][rng.integers(0, 2000, 10_000)] + 0.25 * rng.standard_normal((10_000, D))).astype(np.float32)
+        ids = np.arange(N + c * 10_000, N + (c + 1) * 10_000, dtype=np.int64)
+        index.add_with_ids(x, ids)
+        sizes.add(index.arena_state()[0])
+        new_rows.append(x[:50])
+    t_add = time.perf_counter() - t0
+    assert index.ntotal == N + 200_000
+    assert len(sizes) <= 2, f"20 small adds replaced the arena {len(sizes) - 1} times"
+    assert t_add < 5.0, f"20 adds of 10000 vectors took {t_add:.2f} s"
+    victims = rng.choice(N, 1000, replace=False).astype(np.int64)
+    t0 = time.perf_counter()
+    assert index.remove_ids(victims) == 1000
+    t_rm = time.perf_counter() - t0
+    assert t_rm < 0.5, f"remove_ids(1000) on 10M vectors took {t_rm * 1e3:.0f} ms"
+    assert index.ntotal == N + 199_000 and index.remove_ids(victims) == 0
+    Dm, Im = index.search(q, K)
+    assert not np.isin(Im, victims).any()
+    assert (np.diff(Dm, axis=1) >= 0).all() and (Im >= 0).all()
+    rows = np.concatenate(new_rows)
+    own = np.concatenate([np.arange(N + c * 10_000, N + c * 10_000 + 50) for c in range(20)])
+    Ds, Is = index.search(rows, 5)
+    hit = Is[:, 0] == own
+    assert hit.mean() > 0.98
+    for i in np.flatnonzero(~hit):
+        pos = np.flatnonzero(Is[i] == own[i])
+        assert len(pos) == 1 and Ds[i, pos[0]] == Ds[i, 0]
+
+
 def test_full_size_flat_int8_exact(oracle):
     """Flat int8 at its full size (10M x 512, 2048 queries, k 100): every returned distance is the exact
     integer distance of the returned id, rows are ordered by (distance, id), planted copies of base
