@@ -188,7 +188,9 @@ int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out);
 
 /* AscendIndex::search(n, x, k, distances, labels)  FR/ascend/AscendIndex.h:79-80 ->
  * ascend::IndexIVFPQ::searchImpl  FR/ascenddaemon/impl/IndexIVFPQ.cpp:2373-2411.  0 < n < 1e9, 0 < k <= 2048
- * (the reference's device limit is 320); with 128 sub-quantizers and an fp32 LUT, k <= 1024. */
+ * (the reference's device limit is 320); with 128 sub-quantizers and an fp32 LUT, k <= 1024.  A batch whose
+ * per-query workspaces would exceed config.scratch_bytes is served page by page (AscendIndexImpl::searchPaged,
+ * FR/ascend/impl/AscendIndexImpl.cpp:296-346); the results do not depend on the paging. */
 int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
 int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
                         int64_t *labels_dev);
@@ -266,6 +268,8 @@ typedef struct ivfpq_search_stats {
                              2: in locality order */
     double coarse_plan;   /* 0: the coarse stage wrote the score matrix and selected from it, 1: sampled bound +
                              proof by count (queries without proof are part of coarse_reruns) */
+    double pages;         /* query pages the search was served in (more than one: the sums of the pages' times,
+                             scanned codes and reruns are reported; the plan fields are the last page's) */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
 /* Device times of the last search only (HIP events on the index's stream, in ms); either output may be NULL.

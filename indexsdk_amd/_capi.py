@@ -38,7 +38,7 @@ class IvfpqConfig(ctypes.Structure):
 class IvfpqSearchStats(ctypes.Structure):
     _fields_ = [(n, ctypes.c_double) for n in
                 ("scanned_codes", "ms_coarse", "ms_scan", "ms_total", "scan_launches", "nsplit", "scan_waves",
-                 "shared_pool", "coarse_reruns", "ordered", "coarse_plan")]
+                 "shared_pool", "coarse_reruns", "ordered", "coarse_plan", "pages")]
 
 
 class FlatSearchStats(ctypes.Structure):

@@ -338,6 +338,7 @@ IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stat
         out->coarse_reruns = s.coarse_reruns;
         out->ordered = s.ordered;
         out->coarse_plan = s.coarse_plan;
+        out->pages = s.pages;
     });
 }
 

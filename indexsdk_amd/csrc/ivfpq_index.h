@@ -43,6 +43,7 @@ struct SearchStats {
     double coarse_reruns = 0;
     double ordered = 0;
     double coarse_plan = 0;     // 0: score matrix materialised and selected from, 1: sampled bound + proof by count
+    double pages = 0;           // query pages the search was served in
 };
 
 // Scratch of one scan launch when the caller of scan_params() provides it.
@@ -110,12 +111,15 @@ public:
 
 private:
     void check_trained() const;
+    void search_page(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
     void upload_trained(const float *centroids, const float *codebook);
     // best `nout` lists of every row of device matrix x (canonical arithmetic), device outputs
     void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
                        float *out_dist, bool set_only = false, bool defer_check = false);
     float bf16x3_err_scale(int select_metric) const;
-    int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist);
+    // redone (may be null): receives the rows that were redone, ascending
+    int coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist,
+                      std::vector<int32_t> *redone = nullptr);
     ScanParams scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
                            int64_t *ld, const ScanScratch *ext = nullptr);
     static int scan_nsplit(int64_t n, int nprobe, int64_t k);
@@ -144,6 +148,7 @@ private:
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
     DeviceBuffer<int32_t> ws_flag_;
+    DeviceBuffer<int32_t> ws_redo_;                    // rows of the queries a search scans a second time
     DeviceBuffer<int32_t> ws_order_, ws_order_hist_;   // execution order of the scan (heaviest queries first)
     int32_t max_list_len_ = 0;
     int last_coarse_reruns_ = 0;

@@ -664,7 +664,8 @@ float IvfpqIndex::bf16x3_err_scale(int select_metric) const
     return dots * (3.0f / 262144.0f + (float)(3 * dp_ + d_ + 8) * 5.9604645e-8f);
 }
 
-int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist)
+int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist,
+                              std::vector<int32_t> *redone)
 {
     int32_t nfail = 0;
     ws_flag_.download(&nfail, 1, stream_);
@@ -685,6 +686,9 @@ int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, i
     flag_pending_ = false;
     std::sort(rows32.begin(), rows32.end());   // the order of the appends is not deterministic
     coarse_exact_rows(x_dev, std::vector<int64_t>(rows32.begin(), rows32.end()), nout, select_metric, out_ids, out_dist);
+    if (redone) {
+        *redone = std::move(rows32);
+    }
     return nfail;
 }
 
@@ -1337,7 +1341,41 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
+    // Query paging (AscendIndexImpl::searchPaged, FR/ascend/impl/AscendIndexImpl.cpp:296-346): the workspaces
+    // of a search grow with the number of queries -- staged queries and results (host callers), split
+    // operands, probe lists, candidate keys -- and stay within the scratch budget (the reference's
+    // resourceSize) by serving a very large batch page by page.  Results do not depend on the paging.
+    const int64_t ncand = std::min<int64_t>(nlist_, (int64_t)nprobe_ + 16 + nprobe_ / 8);
+    const int64_t per_query = (on_device ? 0 : (int64_t)d_ * 4 + k * 12) + (int64_t)3 * dp_ * 2 + ncand * 8 +
+                              (int64_t)nprobe_ * 4 + 64;
+    const int64_t page = std::max<int64_t>(256, cfg_.scratch_bytes / per_query / 256 * 256);
+    if (n <= page) {
+        search_page(n, x, k, dist, labels, on_device);
+        return;
+    }
+    SearchStats total{};
+    for (int64_t p0 = 0; p0 < n; p0 += page) {
+        const int64_t np = std::min(page, n - p0);
+        search_page(np, x + p0 * d_, k, dist + p0 * k, labels + p0 * k, on_device);
+        const SearchStats &s = stats();   // of this page (a small launch and a wait: nothing beside a page's work)
+        total.scanned_codes += s.scanned_codes;
+        total.ms_coarse += s.ms_coarse;
+        total.ms_scan += s.ms_scan;
+        total.ms_total += s.ms_total;
+        total.scan_launches += s.scan_launches;
+        total.coarse_reruns += s.coarse_reruns;
+        total.nsplit = s.nsplit;
+        total.scan_waves = s.scan_waves;
+        total.shared_pool = s.shared_pool;
+        total.ordered = s.ordered;
+        total.coarse_plan = s.coarse_plan;
+        total.pages += 1;
+    }
+    stats_ = total;
+}
 
+void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
+{
     const float *xd = x;
     if (!on_device) {
         ws_x_.upload(x, (size_t)n * d_, stream_);
@@ -1364,8 +1402,14 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     launch_scan(p, n, stream_);
     // the scan is queued; only now does the host look at the coarse stage's verdict.  Queries that had to
     // be redone exactly (near-tied centroids: rare) have new probe lists, and the scan runs again.
-    if (coarse_finish(xd, nprobe_, metric_, ws_probes_.data(), nullptr) > 0) {
-        launch_scan(p, n, stream_);
+    std::vector<int32_t> redone;
+    if (coarse_finish(xd, nprobe_, metric_, ws_probes_.data(), nullptr, &redone) > 0) {
+        // only the redone queries are scanned again: their rows are the execution order of a second launch
+        ws_redo_.upload(redone.data(), redone.size(), stream_);
+        ScanParams again = p;
+        again.order = ws_redo_.data();
+        again.xcd_chunks = 0;
+        launch_scan(again, (int64_t)redone.size(), stream_);
     }
     stats_.coarse_reruns = last_coarse_reruns_;
     stats_.coarse_plan = last_coarse_plan_;
@@ -1386,6 +1430,7 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
     }
     stats_.scan_launches = nsplit > 1 ? 2 : 1;
     stats_.nsplit = nsplit;
+    stats_.pages = 1;
     stats_pending_ = true;   // timings and the scanned-code count are worked out when somebody asks
     stats_rows_ = n;
     stats_nprobe_ = nprobe_;

@@ -517,6 +517,7 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
 // Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3).
 __global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restrict__ partial, int nsplit, int k,
                                                           int merge_n, int metric, const int64_t *__restrict__ ids,
+                                                          const int32_t *__restrict__ order,
                                                           float *__restrict__ out_dist,
                                                           int64_t *__restrict__ out_labels)
 {
@@ -524,7 +525,7 @@ __global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restric
     key_t *lists = reinterpret_cast<key_t *>(smem_raw);   // [nsplit][k], each ascending, empty keys last
     key_t *merge = lists + merge_n;                        // [k] the result
     const int tid = threadIdx.x;
-    const int64_t q = blockIdx.x;
+    const int64_t q = order ? order[blockIdx.x] : blockIdx.x;   // the scan's own numbering of the queries it served
     const int total = nsplit * k;
     for (int i = tid; i < total; i += 256) {
         lists[i] = partial[q * total + i];
@@ -900,7 +901,7 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem));
         }
         hipLaunchKernelGGL(ivfpq_merge_kernel, dim3((unsigned)nq), dim3(256), msmem, s, p.partial, p.nsplit, p.k,
-                           merge_n, p.metric, p.ids, p.out_dist, p.out_labels);
+                           merge_n, p.metric, p.ids, p.order, p.out_dist, p.out_labels);
     }
 }
 

@@ -485,6 +485,15 @@ def test_search_redoes_only_the_queries_whose_coarse_proof_fails(ix, oracle):
     pi, pd = gpu.coarse_probe(q)
     oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
     assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
+    # a small batch: every query is split over eight workgroups, and the second scan (of the redone queries
+    # only) goes through the split merge under its own numbering
+    q2 = np.ascontiguousarray(np.concatenate([near[:20], far[:10]]))
+    D2, I2 = gpu.search(q2, 20)
+    st = gpu.last_search_stats()
+    assert st["nsplit"] == 8 and 1 <= st["coarse_reruns"] <= 20, st
+    Dr2, Ir2 = ref.search(q2, 20, nprobe)
+    assert st["scanned_codes"] == ref.last_scanned
+    assert_topk_parity(oracle, ref, q2, D2, I2, Dr2, Ir2, TOL_FP32)
 
 
 def test_reset_keeps_quantizers_and_readd_reproduces_codes(ix, oracle):
@@ -699,3 +708,26 @@ def test_coarse_probe_with_a_small_score_scratch(ix, oracle, nlist, nq, scratch)
     oi, od = oracle.coarse_probe(q, cent, nprobe, ix.METRIC_L2)
     assert np.array_equal(gi, oi) and np.array_equal(gd.view(np.uint32), od.view(np.uint32))
     assert np.array_equal(gpu.assign(q), oracle.assign(q, cent))
+
+
+def test_search_in_query_pages_equals_one_batch(ix, oracle):
+    """A scratch budget (the reference's resourceSize) of 1 MiB holds the workspaces of 768 of these queries:
+    2500 queries are served in four pages, with the answers of the unpaged search bit for bit and the
+    statistics summed over the pages (AscendIndexImpl::searchPaged, FR/ascend/impl/AscendIndexImpl.cpp:296-346)."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 83, 30000, 2500, 64, 96, 16, ix.METRIC_L2)
+    cent, cb = gpu.get_trained()
+    small = ix.AscendIndexIVFPQ(64, ix.METRIC_L2, 96, 16, 8, ix.AscendIndexIVFPQConfig(scratch_bytes=1 << 20))
+    small.set_trained(cent, cb)
+    small.add_with_ids(x, ids)
+    for g in (gpu, small):
+        g.setNumProbes(8)
+    D, I = gpu.search(q, 20)
+    one = gpu.last_search_stats()
+    Dp, Ip = small.search(q, 20)
+    paged = small.last_search_stats()
+    assert one["pages"] == 1 and paged["pages"] == 4, (one["pages"], paged["pages"])
+    assert np.array_equal(Ip, I) and np.array_equal(Dp.view(np.uint32), D.view(np.uint32))
+    assert paged["scanned_codes"] == one["scanned_codes"]
+    Dr, Ir = ref.search(q, 20, 8)
+    assert paged["scanned_codes"] == ref.last_scanned
+    assert_topk_parity(oracle, ref, q, Dp, Ip, Dr, Ir, TOL_FP32)
