@@ -251,6 +251,23 @@ int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocated, int64_t 
 int ivfpq_reset(ivfpq_index_t *h);
 int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out);
 
+/* LDS plan of the fused LUT + scan + top-k kernel for a shape, as the launcher lays it out: byte offsets of the
+ * regions the kernel addresses inside its dynamic LDS, and the total.  Host code only (no GPU is touched; it
+ * works without one): what a test holds against the regions' sizes to prove that no region ends outside the
+ * allocation.  waves = 0 asks for the plan the launcher would choose; 4, 8 or 16 with shared_pool 0 / 1 for
+ * the layout of that workgroup size and pool kind.  No counterpart in the reference. */
+typedef struct ivfpq_scan_lds_plan {
+    int32_t waves, shared_pool; /* wavefronts per workgroup; 1 = one workgroup-wide candidate pool */
+    int32_t cap;                /* keys per pool */
+    int32_t merge_n;            /* keys of the pool region (waves x cap private pools, or cap) */
+    int32_t table_n;            /* probed lists per workgroup */
+    int32_t off_query, off_pools, off_table, off_hist, off_misc; /* the LUT starts at 0 */
+    int32_t ctl_bytes;          /* control block of the shared pool, at off_misc + 8 x waves */
+    int32_t total_bytes;
+} ivfpq_scan_lds_plan_t;
+int ivfpq_plan_scan_lds(int d, int msubs, int lut_fp16, int code_layout, int nprobe, int nsplit, int k, int waves,
+                        int shared_pool, ivfpq_scan_lds_plan_t *out);
+
 /* Device timings of the last ivfpq_search* call, measured with HIP events on the index's stream.
  * No counterpart in the reference (it prints std::chrono timers when verbose). */
 typedef struct ivfpq_search_stats {

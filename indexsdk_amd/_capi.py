@@ -41,6 +41,12 @@ class IvfpqSearchStats(ctypes.Structure):
                  "shared_pool", "coarse_reruns", "ordered", "coarse_plan", "pages")]
 
 
+class ScanLdsPlan(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in
+                ("waves", "shared_pool", "cap", "merge_n", "table_n", "off_query", "off_pools", "off_table", "off_hist",
+                 "off_misc", "ctl_bytes", "total_bytes")]
+
+
 class FlatSearchStats(ctypes.Structure):
     _fields_ = [(n, ctypes.c_double) for n in ("ms_score", "ms_select", "ms_total", "score_launches",
                                                      "exact_reruns")]
@@ -72,6 +78,7 @@ _SIGNATURES = {
     "ivfpq_reserve_memory": (ctypes.c_int, [_H, ctypes.c_int64]),
     "ivfpq_reclaim_memory": (ctypes.c_int, [_H, c_i64p]),
     "ivfpq_arena_state": (ctypes.c_int, [_H, c_i64p, c_i64p, c_i64p]),
+    "ivfpq_plan_scan_lds": (ctypes.c_int, [ctypes.c_int] * 9 + [ctypes.POINTER(ScanLdsPlan)]),
     "ivfpq_config_default": (None, [ctypes.POINTER(IvfpqConfig)]),
     "ivfpq_create": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     ctypes.POINTER(IvfpqConfig), ctypes.POINTER(_H)]),

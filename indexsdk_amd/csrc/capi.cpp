@@ -12,6 +12,7 @@
 #include "flat_index.h"
 #include "ivfpq_index.h"
 #include "ops.h"
+#include "scan.h"
 
 namespace ixa {
 void write_faiss_ivfpq(const IvfpqIndex &idx, const char *path);
@@ -479,6 +480,32 @@ IXA_EXPORT int ivfpq_search_probes_device_noalloc(ivfpq_index_t *h, int64_t n, c
         IXA_HANDLE(h);
         h->impl.search_probes_noalloc(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev);
     });
+}
+IXA_EXPORT int ivfpq_plan_scan_lds(int d, int msubs, int lut_fp16, int code_layout, int nprobe, int nsplit, int k,
+                                   int waves, int shared_pool, ivfpq_scan_lds_plan_t *out)
+{
+    return guarded([&] {
+        IXA_REQUIRE(out != nullptr, ixa::kErrInvalidParam, "out can not be nullptr.");
+        IXA_REQUIRE(d >= 1 && msubs >= 1 && msubs <= 128 && nprobe >= 1 && nsplit >= 1 && k >= 1 &&
+                        (waves == 0 || waves == 4 || waves == 8 || waves == 16) && code_layout >= 0 && code_layout <= 2,
+                    ixa::kErrInvalidParam, "invalid scan shape");
+        ixa::ScanParams p{};
+        int ctl = 0;
+        const size_t total = ixa::scan_lds_plan(d, msubs, lut_fp16, code_layout, nprobe, nsplit, k, waves, shared_pool,
+                                                &p, &ctl);
+        out->waves = p.waves;
+        out->shared_pool = p.shared_pool;
+        out->cap = p.cap;
+        out->merge_n = p.merge_n;
+        out->table_n = p.table_n;
+        out->off_query = p.off_query;
+        out->off_pools = p.off_pools;
+        out->off_table = p.off_table;
+        out->off_hist = p.off_hist;
+        out->off_misc = p.off_misc;
+        out->ctl_bytes = ctl;
+        out->total_bytes = (int32_t)total;
+    }, false);
 }
 IXA_EXPORT int ixa_copy_probe(const void *src_dev, void *dst_dev, int64_t bytes)
 {

@@ -48,6 +48,12 @@ size_t plan_scan(ScanParams &p);
 
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s);
 
+// The LDS plan of a launch (host only).  waves = 0: the plan plan_scan() chooses; else the layout for that
+// workgroup size (4, 8, 16 wavefronts) and pool kind.  Returns the dynamic LDS bytes; *ctl_bytes = size of the
+// shared pool's control block, which follows the 2 x waves words at off_misc.
+size_t scan_lds_plan(int d, int M, int lut_fp16, int code_layout, int nprobe, int nsplit, int k, int waves,
+                     int shared_pool, ScanParams *out, int *ctl_bytes);
+
 // order[0 .. nq) = the queries grouped by the lists they probe (class = hash of the smallest probed list id).
 // cls, hist, cursor as below.
 void launch_order_by_locality(const int32_t *probes, int64_t nq, int nprobe, int32_t *cls, int32_t *hist,

@@ -876,6 +876,25 @@ size_t plan_scan(ScanParams &p)
     return best_smem;
 }
 
+// The LDS plan of a launch as plain numbers (host only: no device is touched).  waves = 0 lets plan_scan()
+// choose; otherwise the plan for that workgroup size and pool kind is returned as it would be laid out.
+size_t scan_lds_plan(int d, int M, int lut_fp16, int code_layout, int nprobe, int nsplit, int k, int waves,
+                     int shared_pool, ScanParams *out, int *ctl_bytes)
+{
+    ScanParams p{};
+    p.d = d;
+    p.M = M;
+    p.lut_fp16 = lut_fp16;
+    p.code_layout = code_layout;
+    p.nprobe = nprobe;
+    p.nsplit = nsplit;
+    p.k = k;
+    const size_t smem = waves == 0 ? plan_scan(p) : plan_with_waves(p, waves, shared_pool != 0);
+    *out = p;
+    *ctl_bytes = (int)sizeof(BlockPoolCtl);
+    return smem;
+}
+
 void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
 {
     if (nq == 0) {

@@ -147,3 +147,64 @@ def test_evaluate_counts_queries_whose_true_neighbour_is_in_the_first_r_results(
     ms, rec = evaluate(Canned(), np.zeros((4, 2), dtype=np.float32), gt, 100)
     assert ms >= 0 and rec == {1: 0.25, 10: 0.5, 100: 0.75}
     assert set(evaluate(Canned(), np.zeros((4, 2), dtype=np.float32), gt, 50)[1]) == {1, 10}
+
+
+def _pool_capacity(k, waves, shared):
+    """Keys a candidate pool must hold (the rule the selection code states: k plus two rounds of what the
+    wavefronts that share the pool can append between prunes), as a power of two."""
+    cap, need = (1024, k + 2 * waves * 64) if shared else (256, k + 2 * 64)
+    while cap < need:
+        cap *= 2
+    return cap
+
+
+def test_scan_lds_plan_keeps_every_region_inside_the_allocation(capi):
+    """The fused scan kernel addresses its dynamic LDS through offsets the launcher computes by hand.  Over
+    sub-quantizer counts, k, probe counts, splits, workgroup sizes, both pool kinds, both LUT types and every
+    code layout: each region (LUT, query, candidate pools, list table, histogram, per-wave words + control
+    block), sized here from what the kernel stores in it, ends inside the allocation, starts 16-byte aligned,
+    and overlaps no other region."""
+    lib = capi.load()
+    plan = capi.ScanLdsPlan()
+    checked = 0
+    for M in (4, 8, 16, 32, 48, 64, 96, 128):
+        for lut_fp16 in (0, 1):
+            layouts = [0]
+            if M in (32, 64, 96):
+                layouts.append(1)
+            if M == 48 and not lut_fp16:
+                layouts.append(2)
+            for layout in layouts:
+                for k in (1, 10, 100, 129, 320, 1000, 1024, 2048):
+                    for nprobe, nsplit in ((1, 1), (16, 1), (64, 8), (256, 1), (2048, 1), (2048, 8), (100, 3)):
+                        for waves, shared in ((0, 0), (4, 0), (8, 0), (8, 1), (16, 1)):
+                            d = M * 4
+                            rc = lib.ivfpq_plan_scan_lds(d, M, lut_fp16, layout, nprobe, nsplit, k, waves, shared,
+                                                         ctypes.byref(plan))
+                            assert rc == 0, lib.ixa_last_error()
+                            W, sh = plan.waves, plan.shared_pool
+                            if waves:
+                                assert (W, sh) == (waves, shared)
+                            assert plan.cap == _pool_capacity(k, W, sh)
+                            assert plan.table_n == -(-nprobe // nsplit)
+                            lut = 64 * 256 * 4 if layout == 2 else M * 256 * (2 if lut_fp16 else 4)
+                            if layout == 1 and lut_fp16:
+                                lut += 64          # the upper half of the last row's sub-quantizers 16..31
+                            regions = [
+                                ("lut", 0, lut),
+                                ("query", plan.off_query, d * 4),
+                                ("pools", plan.off_pools, (plan.cap if sh else W * plan.cap) * 8),
+                                ("table", plan.off_table, plan.table_n * 12),
+                                ("misc", plan.off_misc, 8 * W + plan.ctl_bytes),
+                            ]
+                            if sh:
+                                regions.append(("hist", plan.off_hist, 1024 * 4))
+                            assert plan.ctl_bytes >= 32
+                            spans = sorted((off, off + size, name) for name, off, size in regions)
+                            for off, end, name in spans:
+                                assert off % 16 == 0 or name == "misc" and off % 8 == 0, (name, off)
+                                assert end <= plan.total_bytes, (name, end, plan.total_bytes, M, k, nprobe, W, sh)
+                            for (a0, a1, an), (b0, b1, bn) in zip(spans, spans[1:]):
+                                assert a1 <= b0, (an, bn, M, k, nprobe, W, sh)
+                            checked += 1
+    assert checked > 5000
