@@ -1,0 +1,74 @@
+// Header-only C++ face of the MI355X search path with the reference's class shape, root of the hierarchy:
+//   faiss::ascend::AscendIndex : faiss::Index      (FR/ascend/AscendIndex.h:41-110)
+// Every method of the classes built on it forwards to the C ABI (include/indexsdk_amd.h) and throws
+// faiss::FaissException on a non-zero status, as the reference's public layer does (FAISS_THROW_IF_NOT_FMT).
+#pragma once
+#include <cstdint>
+#include <initializer_list>
+#include <string>
+#include <vector>
+
+#include "../faiss_shim.h"
+#include "../indexsdk_amd.h"
+
+namespace faiss {
+namespace ascend {
+
+using ascend_idx_t = uint64_t;  // FR/ascend/AscendIndex.h:45
+
+const idx_t MAX_N = 1000000000;
+const idx_t MAX_K = 4096;
+const int64_t INDEX_DEFAULT_MEM = 0x2000000;   // 32M
+const uint32_t DEFAULT_BLOCK_SIZE = 16384 * 16;
+
+inline void ixaThrowIfError(int status)
+{
+    if (status != IXA_OK) {
+        throw faiss::FaissException(ixa_last_error());
+    }
+}
+
+// AscendIndexConfig (FR/ascend/AscendIndex.h:51-71).  deviceList is accepted for source compatibility: this
+// build serves exactly one GPU, the current HIP device.  resourceSize bounds the scratch of a search
+// (raised to this build's minimum where smaller).
+struct AscendIndexConfig {
+    inline AscendIndexConfig() : deviceList({0}), resourceSize(INDEX_DEFAULT_MEM), dBlockSize(DEFAULT_BLOCK_SIZE) {}
+    inline AscendIndexConfig(std::initializer_list<int> devices, int64_t resources = INDEX_DEFAULT_MEM,
+                             uint32_t blockSize = DEFAULT_BLOCK_SIZE)
+        : deviceList(devices), resourceSize(resources), dBlockSize(blockSize)
+    {
+    }
+    inline AscendIndexConfig(std::vector<int> devices, int64_t resources = INDEX_DEFAULT_MEM,
+                             uint32_t blockSize = DEFAULT_BLOCK_SIZE)
+        : deviceList(std::move(devices)), resourceSize(resources), dBlockSize(blockSize)
+    {
+    }
+    std::vector<int> deviceList;
+    int64_t resourceSize;
+    bool slim = false;
+    bool filterable = false;
+    uint32_t dBlockSize = DEFAULT_BLOCK_SIZE;
+};
+
+class AscendIndex : public faiss::Index {
+public:
+    AscendIndex(int dims, faiss::MetricType metric, AscendIndexConfig config)
+        : faiss::Index(dims, metric), indexConfig(std::move(config))
+    {
+    }
+    virtual ~AscendIndex() {}
+    AscendIndex(const AscendIndex &) = delete;
+    AscendIndex &operator=(const AscendIndex &) = delete;
+
+    // reserve memory for the database (FR/ascend/AscendIndex.h:91-92); a family without growable storage ignores it
+    virtual void reserveMemory(size_t /*numVecs*/) {}
+    // reclaim device memory to exactly the amount needed; returns the bytes released (:94-96)
+    virtual size_t reclaimMemory() { return 0; }
+    std::vector<int> getDeviceList() { return indexConfig.deviceList; }
+
+protected:
+    AscendIndexConfig indexConfig;
+};
+
+}  // namespace ascend
+}  // namespace faiss

@@ -1,25 +1,84 @@
 // Header-only C++ faces of the Flat paths with the reference's class shapes:
-//   faiss::ascend::AscendIndexFlat / AscendIndexFlatL2   (FR/ascend/AscendIndexFlat.h:48-90)
-//   faiss::ascend::AscendIndexInt8Flat                   (FR/ascend/AscendIndexInt8.h:53-96, AscendIndexInt8Flat.h)
+//   faiss::ascend::AscendIndexFlat : AscendIndex, AscendIndexFlatL2   (FR/ascend/AscendIndexFlat.h:34-110)
+//   faiss::ascend::AscendIndexInt8Flat : AscendIndexInt8              (FR/ascend/AscendIndexInt8Flat.h:30-100)
 // forwarding to the C ABI (include/indexsdk_amd.h).
 #pragma once
 #include <cfloat>
 #include <vector>
 
-#include "AscendIndexIVFPQ.h"
+#include "AscendIndex.h"
+#include "AscendIndexInt8.h"
 
 namespace faiss {
 namespace ascend {
 
-class AscendIndexFlat : public faiss::Index {
-public:
-    AscendIndexFlat(int dims, faiss::MetricType metric, int64_t resourceSize = 0) : faiss::Index(dims, metric)
+const int64_t FLAT_DEFAULT_MEM = 0x8000000;   // 128M
+
+// The score scratch of a Flat search: the library's default (0) unless the caller's resourceSize asks for more
+// (the reference's defaults of 32M / 128M size a different kind of pool).
+inline int64_t scratchOf(int64_t resourceSize) { return resourceSize > ((int64_t)1 << 30) ? resourceSize : 0; }
+
+// AscendIndexFlatConfig (FR/ascend/AscendIndexFlat.h:34-45)
+struct AscendIndexFlatConfig : public AscendIndexConfig {
+    inline AscendIndexFlatConfig() {}
+    inline AscendIndexFlatConfig(std::initializer_list<int> devices, int64_t resourceSize = FLAT_DEFAULT_MEM)
+        : AscendIndexConfig(devices, resourceSize)
     {
-        ixaThrowIfError(flat_create(dims, (int)metric, resourceSize, &h_));
+    }
+    inline AscendIndexFlatConfig(std::vector<int> devices, int64_t resourceSize = FLAT_DEFAULT_MEM)
+        : AscendIndexConfig(std::move(devices), resourceSize)
+    {
+    }
+};
+
+class AscendIndexFlat : public AscendIndex {
+public:
+    // Construct an empty instance that can be added to
+    AscendIndexFlat(int dims, faiss::MetricType metric, AscendIndexFlatConfig config = AscendIndexFlatConfig())
+        : AscendIndex(dims, metric, config)
+    {
+        ixaThrowIfError(flat_create(dims, (int)metric, scratchOf(config.resourceSize), &h_));
+    }
+    // Construct from a pre-existing faiss::IndexFlat instance
+    explicit AscendIndexFlat(const faiss::IndexFlat *index, AscendIndexFlatConfig config = AscendIndexFlatConfig())
+        : AscendIndex(index ? index->d : 0, index ? index->metric_type : faiss::METRIC_L2, config)
+    {
+        if (index == nullptr) {
+            throw FaissException("index is nullptr.");
+        }
+        ixaThrowIfError(flat_create(index->d, (int)index->metric_type, scratchOf(config.resourceSize), &h_));
+        copyFrom(index);
     }
     virtual ~AscendIndexFlat() { flat_destroy(h_); }
     AscendIndexFlat(const AscendIndexFlat &) = delete;
     AscendIndexFlat &operator=(const AscendIndexFlat &) = delete;
+
+    // Initialize ourselves from the given CPU index; will overwrite all data in ourselves
+    void copyFrom(const faiss::IndexFlat *index)
+    {
+        if (index == nullptr || index->d != d || index->metric_type != metric_type) {
+            throw FaissException("copyFrom: the source index must have this index's dims and metric");
+        }
+        reset();
+        if (index->ntotal > 0) {
+            add(index->ntotal, index->get_xb());
+        }
+    }
+    // Copy ourselves to the given CPU index; will overwrite all data in the index instance
+    void copyTo(faiss::IndexFlat *index) const
+    {
+        if (index == nullptr) {
+            throw FaissException("index is nullptr.");
+        }
+        index->reset();
+        index->d = d;
+        index->metric_type = metric_type;
+        std::vector<float> xb((size_t)ntotal * d);
+        if (ntotal > 0) {
+            ixaThrowIfError(flat_get_base(h_, 0, ntotal, xb.data()));
+            index->add(ntotal, xb.data());
+        }
+    }
     void add(idx_t n, const float *x) override { add_with_ids(n, x, nullptr); }
     void add_with_ids(idx_t n, const float *x, const idx_t *ids) override
     {
@@ -36,11 +95,23 @@ public:
         ixaThrowIfError(flat_reset(h_));
         ntotal = 0;
     }
+    // Returns the number of vectors we contain
     size_t getBaseSize(int /*deviceId*/ = 0) const { return (size_t)ntotal; }
+    // Returns the vectors we contain (the reference hands them out as fp16 bytes; here they are fp32)
     void getBase(int /*deviceId*/, std::vector<float> &xb) const
     {
         xb.resize((size_t)ntotal * d);
-        ixaThrowIfError(flat_get_base(h_, 0, ntotal, xb.data()));
+        if (ntotal > 0) {
+            ixaThrowIfError(flat_get_base(h_, 0, ntotal, xb.data()));
+        }
+    }
+    // Returns the ids of the vectors we contain, in base order
+    void getIdxMap(int /*deviceId*/, std::vector<idx_t> &idxMap) const
+    {
+        idxMap.resize((size_t)ntotal);
+        if (ntotal > 0) {
+            ixaThrowIfError(flat_get_ids(h_, 0, ntotal, reinterpret_cast<int64_t *>(idxMap.data())));
+        }
     }
 
 protected:
@@ -55,41 +126,50 @@ protected:
 
 class AscendIndexFlatL2 : public AscendIndexFlat {
 public:
-    explicit AscendIndexFlatL2(int dims, int64_t resourceSize = 0) : AscendIndexFlat(dims, faiss::METRIC_L2, resourceSize)
+    explicit AscendIndexFlatL2(int dims, AscendIndexFlatConfig config = AscendIndexFlatConfig())
+        : AscendIndexFlat(dims, faiss::METRIC_L2, config)
     {
     }
 };
 
-// int8 vectors; L2 only.  search() keeps the reference's float signature (exact below 2^24,
-// rounded to nearest above); searchInt32() returns the exact int32 distances.
-class AscendIndexInt8Flat {
-public:
-    using idx_t = faiss::idx_t;
-    AscendIndexInt8Flat(int dims, faiss::MetricType metric = faiss::METRIC_L2, int64_t resourceSize = 0) : d(dims)
+const int64_t INT8_FLAT_DEFAULT_MEM = 0x8000000;
+
+// AscendIndexInt8FlatConfig (FR/ascend/AscendIndexInt8Flat.h:30-57); the block size and index mode steer the
+// reference's device layout and have no counterpart here.
+struct AscendIndexInt8FlatConfig : public AscendIndexInt8Config {
+    inline AscendIndexInt8FlatConfig() : AscendIndexInt8Config({0}, INT8_FLAT_DEFAULT_MEM) {}
+    inline AscendIndexInt8FlatConfig(std::initializer_list<int> devices, int64_t resourceSize = INT8_FLAT_DEFAULT_MEM)
+        : AscendIndexInt8Config(devices, resourceSize)
     {
-        ixaThrowIfError(flat_i8_create(dims, (int)metric, resourceSize, &h_));
+    }
+    inline AscendIndexInt8FlatConfig(std::vector<int> devices, int64_t resourceSize = INT8_FLAT_DEFAULT_MEM)
+        : AscendIndexInt8Config(std::move(devices), resourceSize)
+    {
+    }
+    uint32_t dBlockSize = 16384 * 16;
+};
+
+// int8 vectors; L2 only.  search() keeps the reference's float signature (exact below 2^24, rounded to
+// nearest above; the reference returns a scaled fp16 value); searchInt32() returns the exact int32 distances.
+class AscendIndexInt8Flat : public AscendIndexInt8 {
+public:
+    explicit AscendIndexInt8Flat(int dims, faiss::MetricType metric = faiss::METRIC_L2,
+                                 AscendIndexInt8FlatConfig config = AscendIndexInt8FlatConfig())
+        : AscendIndexInt8(dims, metric, config)
+    {
+        ixaThrowIfError(flat_i8_create(dims, (int)metric, scratchOf(config.resourceSize), &h_));
     }
     virtual ~AscendIndexInt8Flat() { flat_i8_destroy(h_); }
-    AscendIndexInt8Flat(const AscendIndexInt8Flat &) = delete;
-    AscendIndexInt8Flat &operator=(const AscendIndexInt8Flat &) = delete;
-    void add(idx_t n, const int8_t *x) { add_with_ids(n, x, nullptr); }
-    void add_with_ids(idx_t n, const int8_t *x, const idx_t *ids)
-    {
-        ixaThrowIfError(flat_i8_add_with_ids(h_, n, x, reinterpret_cast<const int64_t *>(ids)));
-        int64_t v = 0;
-        ixaThrowIfError(flat_i8_ntotal(h_, &v));
-        ntotal = v;
-    }
     void searchInt32(idx_t n, const int8_t *x, idx_t k, int32_t *distances, idx_t *labels) const
     {
         ixaThrowIfError(flat_i8_search(h_, n, x, k, distances, reinterpret_cast<int64_t *>(labels)));
     }
-    void search(idx_t n, const int8_t *x, idx_t k, float *distances, idx_t *labels) const
+    size_t getBaseSize(int /*deviceId*/ = 0) const { return (size_t)ntotal; }
+    void getBase(int /*deviceId*/, std::vector<int8_t> &xb) const
     {
-        std::vector<int32_t> tmp((size_t)n * k);
-        searchInt32(n, x, k, tmp.data(), labels);
-        for (size_t i = 0; i < tmp.size(); i++) {
-            distances[i] = labels[i] < 0 ? FLT_MAX : (float)tmp[i];
+        xb.resize((size_t)ntotal * d);
+        if (ntotal > 0) {
+            ixaThrowIfError(flat_i8_get_base(h_, 0, ntotal, xb.data()));
         }
     }
     void reset()
@@ -97,10 +177,23 @@ public:
         ixaThrowIfError(flat_i8_reset(h_));
         ntotal = 0;
     }
-    int d;
-    idx_t ntotal = 0;
 
 protected:
+    void addImpl(idx_t n, const int8_t *x, const idx_t *ids) override
+    {
+        ixaThrowIfError(flat_i8_add_with_ids(h_, n, x, reinterpret_cast<const int64_t *>(ids)));
+        int64_t v = 0;
+        ixaThrowIfError(flat_i8_ntotal(h_, &v));
+        ntotal = v;
+    }
+    void searchImpl(idx_t n, const int8_t *x, idx_t k, float *distances, idx_t *labels) const override
+    {
+        std::vector<int32_t> tmp((size_t)n * k);
+        searchInt32(n, x, k, tmp.data(), labels);
+        for (size_t i = 0; i < tmp.size(); i++) {
+            distances[i] = labels[i] < 0 ? FLT_MAX : (float)tmp[i];
+        }
+    }
     flat_i8_index_t *h_ = nullptr;
 };
 

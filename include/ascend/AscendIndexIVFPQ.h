@@ -1,80 +1,47 @@
-// Header-only C++ face of the MI355X IVFPQ path with the reference's class shape:
-//   faiss::ascend::AscendIndexIVFPQ : AscendIndexIVF : AscendIndex : faiss::Index
-//   (FR/ascend/AscendIndexIVFPQ.h:71-96, FR/ascend/AscendIndexIVF.h:75-118, FR/ascend/AscendIndex.h:62-110).
-// Every method forwards to the C ABI (include/indexsdk_amd.h) and throws faiss::FaissException on
-// a non-zero status, as the reference's public layer does (FAISS_THROW_IF_NOT_FMT).
+// faiss::ascend::AscendIndexIVFPQ : AscendIndexIVF : AscendIndex : faiss::Index
+//   (FR/ascend/AscendIndexIVFPQ.h:32-96, FR/ascend/AscendIndexIVF.h:75-118, FR/ascend/AscendIndex.h:62-110).
+// Header-only; every method forwards to the C ABI (include/indexsdk_amd.h).
 #pragma once
-#include <cstdint>
-#include <initializer_list>
-#include <string>
-#include <vector>
+#include <algorithm>
+#include <cstring>
 
-#include "../faiss_shim.h"
-#include "../indexsdk_amd.h"
+#include "AscendIndexIVF.h"
 
 namespace faiss {
 namespace ascend {
 
-using ascend_idx_t = uint64_t;  // FR/ascend/utils/AscendUtils.h
-
-inline void ixaThrowIfError(int status)
-{
-    if (status != IXA_OK) {
-        throw faiss::FaissException(ixa_last_error());
-    }
-}
-
-const int64_t IVF_DEFAULT_MEM = 0x8000000;
-
-// AscendIndexIVFPQConfig (FR/ascend/AscendIndexIVFPQ.h:32-68).  deviceList is accepted for source
-// compatibility; this build serves exactly one GPU and uses the current HIP device.
-struct AscendIndexIVFPQConfig {
-    AscendIndexIVFPQConfig() : deviceList({0}), resourceSize(IVF_DEFAULT_MEM) {}
-    explicit AscendIndexIVFPQConfig(std::initializer_list<int> devices, int64_t resources = IVF_DEFAULT_MEM)
-        : deviceList(devices), resourceSize(resources)
+// AscendIndexIVFPQConfig (FR/ascend/AscendIndexIVFPQ.h:32-68)
+struct AscendIndexIVFPQConfig : public AscendIndexIVFConfig {
+    inline AscendIndexIVFPQConfig() : AscendIndexIVFConfig({0}, IVF_DEFAULT_MEM) {}
+    explicit inline AscendIndexIVFPQConfig(std::initializer_list<int> devices, int64_t resourceSize = IVF_DEFAULT_MEM)
+        : AscendIndexIVFConfig(devices, resourceSize)
     {
     }
-    explicit AscendIndexIVFPQConfig(std::vector<int> devices, int64_t resources = IVF_DEFAULT_MEM)
-        : deviceList(std::move(devices)), resourceSize(resources)
+    explicit inline AscendIndexIVFPQConfig(std::vector<int> devices, int64_t resourceSize = IVF_DEFAULT_MEM)
+        : AscendIndexIVFConfig(std::move(devices), resourceSize)
     {
     }
-    std::vector<int> deviceList;
-    int64_t resourceSize;
-    bool useKmeansPP = false;
     int trainSamplesPerList = 40;
     int maxTrainSamples = 10000000;
-    int pqNiter = -1;
+    int pqNiter = -1;                        // -1: cp.niter
     bool useDistributedCoarse = false;       // no counterpart on one GPU
     bool enableQueryParallelSearch = false;  // no counterpart on one GPU
     // additions of this build
-    int niter = 25;               // coarse k-means iterations (the reference's CPU mode uses 25)
-    bool spherical = false;       // the reference trains spherical k-means; plain Lloyd is the default here
-    bool lutFp16 = false;         // per-query LUT stored as IEEE half
-    bool strictReferenceParams = true;  // enforce the reference's d / nlist / msubs whitelists
+    bool lutFp16 = false;                // per-query LUT stored as IEEE half (distances within 1e-2)
+    bool strictReferenceParams = false;  // true: enforce the reference's whitelists (dims 128, nlist 1024..16384 /
+                                         // 262144 / 524288, msubs 2..32) with its "Unsupported ..." messages
 };
 
-class AscendIndexIVFPQ : public faiss::Index {
+class AscendIndexIVFPQ : public AscendIndexIVF {
 public:
     AscendIndexIVFPQ(int dims, faiss::MetricType metric, int nlist, int msubs, int nbits,
                      AscendIndexIVFPQConfig config = AscendIndexIVFPQConfig())
-        : faiss::Index(dims, metric), nlist_(nlist), msubs_(msubs)
+        : AscendIndexIVF(dims, metric, nlist, config), ivfPQConfig(config), msubs_(msubs), nbits_(nbits)
     {
-        ivfpq_config_t c;
-        ivfpq_config_default(&c);
-        c.niter = config.niter;
-        c.pq_niter = config.pqNiter;
-        c.spherical = config.spherical ? 1 : 0;
-        c.train_samples_per_list = config.trainSamplesPerList;
-        c.max_train_samples = config.maxTrainSamples;
-        c.lut_fp16 = config.lutFp16 ? 1 : 0;
-        c.strict_reference_params = config.strictReferenceParams ? 1 : 0;
-        if (config.resourceSize > c.scratch_bytes) {
-            c.scratch_bytes = config.resourceSize;
-        }
-        ixaThrowIfError(ivfpq_create(dims, (int)metric, nlist, msubs, nbits, &c, &h_));
+        create(dims, metric, nlist, msubs, nbits);
         is_trained = false;
     }
-    virtual ~AscendIndexIVFPQ() { ivfpq_destroy(h_); }
+    virtual ~AscendIndexIVFPQ() {}
     AscendIndexIVFPQ(const AscendIndexIVFPQ &) = delete;
     AscendIndexIVFPQ &operator=(const AscendIndexIVFPQ &) = delete;
 
@@ -83,28 +50,10 @@ public:
         ixaThrowIfError(ivfpq_train(h_, n, x));
         is_trained = true;
     }
-    void add(idx_t n, const float *x) override { add_with_ids(n, x, nullptr); }
-    void add_with_ids(idx_t n, const float *x, const idx_t *ids) override
+    void remove_ids(size_t n, const idx_t *ids)
     {
-        ixaThrowIfError(ivfpq_add_with_ids(h_, n, x, reinterpret_cast<const int64_t *>(ids)));
+        ixaThrowIfError(ivfpq_remove_ids(h_, (int64_t)n, reinterpret_cast<const int64_t *>(ids), nullptr));
         syncTotal();
-    }
-    void search(idx_t n, const float *x, idx_t k, float *distances, idx_t *labels,
-                const SearchParameters * = nullptr) const override
-    {
-        ixaThrowIfError(ivfpq_search(h_, n, x, k, distances, reinterpret_cast<int64_t *>(labels)));
-    }
-    void reset() override
-    {
-        ixaThrowIfError(ivfpq_reset(h_));
-        syncTotal();
-    }
-    size_t remove_ids(size_t n, const idx_t *ids)
-    {
-        int64_t removed = 0;
-        ixaThrowIfError(ivfpq_remove_ids(h_, (int64_t)n, reinterpret_cast<const int64_t *>(ids), &removed));
-        syncTotal();
-        return (size_t)removed;
     }
     std::vector<idx_t> update(idx_t n, const float *x, const idx_t *ids)
     {
@@ -116,30 +65,115 @@ public:
         syncTotal();
         return missing;
     }
-    // AscendIndexIVF
-    int getNumLists() const { return nlist_; }
-    virtual void setNumProbes(int nprobes) { ixaThrowIfError(ivfpq_set_nprobe(h_, nprobes)); }
-    int getNumProbes() const
+
+    // Initialize ourselves from the given CPU index; will overwrite (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:392-425).
+    // The reference copies the codes as they are and searches them against the RAW query, which is only right
+    // for an index built with by_residual = false: here an index with by_residual = true is refused.
+    void copyFrom(const faiss::IndexIVFPQ *index)
     {
-        int v = 0;
-        ixaThrowIfError(ivfpq_get_nprobe(h_, &v));
-        return v;
+        if (index == nullptr) {
+            throw FaissException("index is nullptr.");
+        }
+        if (!index->is_trained) {
+            throw FaissException("Source index is not trained");
+        }
+        if (index->by_residual) {
+            throw FaissException("copyFrom: the source index encodes residuals (by_residual = true); this index "
+                                 "searches codes of the raw vectors (by_residual = false)");
+        }
+        if (index->pq.nbits != 8 || index->quantizer == nullptr || index->invlists == nullptr ||
+            index->quantizer->ntotal != (idx_t)index->nlist || index->invlists->code_size != index->pq.M) {
+            throw FaissException("copyFrom: the source index must have 8-bit codes, a filled coarse quantizer and "
+                                 "inverted lists of pq.M bytes per entry");
+        }
+        const auto *flat = dynamic_cast<const faiss::IndexFlat *>(index->quantizer);
+        if (flat == nullptr) {
+            throw FaissException("copyFrom: the coarse quantizer must be an IndexFlat");
+        }
+        // a new device index of the source's shape replaces ours (the reference overwrites d, nlist, metric too)
+        ivfpq_index_t *old = h_;
+        h_ = nullptr;
+        try {
+            metric_type = index->metric_type;
+            create(index->d, index->metric_type, (int)index->nlist, (int)index->pq.M, 8);
+        } catch (...) {
+            h_ = old;
+            throw;
+        }
+        ivfpq_destroy(old);
+        d = index->d;
+        nlist = (int)index->nlist;
+        msubs_ = (int)index->pq.M;
+        ivfConfig.cp = index->cp;
+        ixaThrowIfError(ivfpq_set_trained(h_, flat->get_xb(), index->pq.centroids.data()));
+        is_trained = true;
+        setNumProbes((int)std::min<size_t>(std::max<size_t>(index->nprobe, 1), index->nlist));
+        for (size_t l = 0; l < index->nlist; l++) {
+            const size_t n = index->invlists->list_size(l);
+            if (n == 0) {
+                continue;
+            }
+            const uint8_t *codes = index->invlists->get_codes(l);
+            const idx_t *ids = index->invlists->get_ids(l);
+            const int rc = ivfpq_add_codes(h_, (int64_t)l, (int64_t)n, codes, reinterpret_cast<const int64_t *>(ids));
+            index->invlists->release_codes(l, codes);
+            index->invlists->release_ids(l, ids);
+            ixaThrowIfError(rc);
+        }
+        syncTotal();
     }
-    virtual uint32_t getListLength(int listId) const
+
+    // Copy ourselves to the given CPU index; will overwrite all data (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:453-508)
+    void copyTo(faiss::IndexIVFPQ *index) const
     {
-        int64_t v = 0;
-        ixaThrowIfError(ivfpq_list_length(h_, listId, &v));
-        return (uint32_t)v;
+        if (index == nullptr) {
+            throw FaissException("index is nullptr.");
+        }
+        if (!is_trained) {
+            throw FaissException("Index is not trained");
+        }
+        if (index->ntotal > 0) {
+            index->reset();
+        }
+        index->d = d;
+        index->metric_type = metric_type;
+        index->is_trained = true;
+        index->nlist = (size_t)nlist;
+        index->nprobe = (size_t)getNumProbes();
+        index->by_residual = false;
+        index->cp = ivfConfig.cp;
+        index->pq.d = (size_t)d;
+        index->pq.M = (size_t)msubs_;
+        index->pq.nbits = 8;
+        index->pq.set_derived_values();
+        std::vector<float> centroids((size_t)nlist * d);
+        ixaThrowIfError(ivfpq_get_trained(h_, centroids.data(), index->pq.centroids.data()));
+        faiss::IndexFlat *quantizer = metric_type == faiss::METRIC_INNER_PRODUCT
+                                          ? static_cast<faiss::IndexFlat *>(new faiss::IndexFlatIP(d))
+                                          : static_cast<faiss::IndexFlat *>(new faiss::IndexFlatL2(d));
+        quantizer->add(nlist, centroids.data());
+        if (index->own_fields) {
+            delete index->quantizer;
+        }
+        index->quantizer = quantizer;
+        index->own_fields = true;
+        index->code_size = (size_t)msubs_;
+        faiss::InvertedLists *ivf = new faiss::ArrayInvertedLists((size_t)nlist, index->code_size);
+        index->replace_invlists(ivf, true);
+        std::vector<uint8_t> codes;
+        std::vector<ascend_idx_t> ids;
+        index->ntotal = 0;
+        for (int l = 0; l < nlist; l++) {
+            getListCodesAndIds(l, codes, ids);
+            if (!ids.empty()) {
+                ivf->add_entries((size_t)l, ids.size(), reinterpret_cast<const idx_t *>(ids.data()), codes.data());
+                index->ntotal += (idx_t)ids.size();
+            }
+        }
     }
-    virtual void getListCodesAndIds(int listId, std::vector<uint8_t> &codes, std::vector<ascend_idx_t> &ids) const
-    {
-        const uint32_t len = getListLength(listId);
-        codes.resize((size_t)len * msubs_);
-        ids.resize(len);
-        ixaThrowIfError(ivfpq_get_list(h_, listId, codes.data(), reinterpret_cast<int64_t *>(ids.data())));
-    }
-    // Quantizer exchange: the part of copyFrom / copyTo (faiss::IndexIVFPQ with by_residual = false)
-    // that does not need faiss types.  centroids[nlist*d], codebook[msubs*256*(d/msubs)].
+
+    // ---- additions of this build -----------------------------------------------------------------------------
+    // Quantizer exchange without faiss types: centroids[nlist*d], codebook[msubs*256*(d/msubs)].
     void copyFromTrained(const float *centroids, const float *codebook)
     {
         ixaThrowIfError(ivfpq_set_trained(h_, centroids, codebook));
@@ -149,14 +183,15 @@ public:
     {
         ixaThrowIfError(ivfpq_get_trained(h_, centroids, codebook));
     }
+    // ascend::IndexIVFPQ::addPQCodes (FR/ascenddaemon/impl/IndexIVFPQ.cpp:210-235)
     void addPQCodes(int listId, size_t n, const uint8_t *codes, const idx_t *ids)
     {
         ixaThrowIfError(ivfpq_add_codes(h_, listId, (int64_t)n, codes, reinterpret_cast<const int64_t *>(ids)));
         syncTotal();
     }
-    // File form of copyTo / copyFrom(faiss::IndexIVFPQ *): the byte layout of faiss::write_index for an
-    // IndexIVFPQ with by_residual = false.  readFaiss replaces this object's index; the file must have the
-    // dims, metric, nlist and msubs this object was constructed with.
+    // File form of copyTo / copyFrom: the byte layout of faiss::write_index for an IndexIVFPQ with
+    // by_residual = false.  readFaiss replaces this object's index; the file must have the dims, metric,
+    // nlist and msubs this object was constructed with.
     void writeFaiss(const char *path) const { ixaThrowIfError(ivfpq_write_faiss(h_, path)); }
     void readFaiss(const char *path)
     {
@@ -165,7 +200,7 @@ public:
         int fd = 0, fm = 0, fM = 0;
         int64_t fl = 0;
         ivfpq_get_shape(loaded, &fd, &fm, &fl, &fM);
-        if (fd != d || fm != (int)metric_type || fl != nlist_ || fM != msubs_) {
+        if (fd != d || fm != (int)metric_type || fl != nlist || fM != msubs_) {
             ivfpq_destroy(loaded);
             throw FaissException("the file's dims / metric / nlist / msubs differ from this index");
         }
@@ -174,17 +209,27 @@ public:
         is_trained = true;
         syncTotal();
     }
-    ivfpq_index_t *handle() const { return h_; }
 
 protected:
-    void syncTotal()
+    void create(int dims, faiss::MetricType metric, int nlist_, int msubs, int nbits)
     {
-        int64_t v = 0;
-        ixaThrowIfError(ivfpq_ntotal(h_, &v));
-        ntotal = v;
+        ivfpq_config_t c;
+        ivfpq_config_default(&c);
+        c.niter = ivfPQConfig.cp.niter;
+        c.pq_niter = ivfPQConfig.pqNiter;
+        c.spherical = ivfPQConfig.cp.spherical ? 1 : -1;   // -1: on for inner product, as the reference forces it
+        c.train_samples_per_list = ivfPQConfig.trainSamplesPerList;
+        c.max_train_samples = ivfPQConfig.maxTrainSamples;
+        c.lut_fp16 = ivfPQConfig.lutFp16 ? 1 : 0;
+        c.strict_reference_params = ivfPQConfig.strictReferenceParams ? 1 : 0;
+        if (ivfPQConfig.resourceSize > c.scratch_bytes) {
+            c.scratch_bytes = ivfPQConfig.resourceSize;
+        }
+        ixaThrowIfError(ivfpq_create(dims, (int)metric, nlist_, msubs, nbits, &c, &h_));
+        codeSize = msubs;
     }
-    ivfpq_index_t *h_ = nullptr;
-    int nlist_, msubs_;
+    AscendIndexIVFPQConfig ivfPQConfig;
+    int msubs_, nbits_;
 };
 
 // AscendIndexImpl::mergeSearchResult (FR/ascend/impl/AscendIndexImpl.cpp:587-640) for callers that

@@ -1,15 +1,22 @@
-// Minimal stand-in for the faiss types that the reference's public classes derive from
-// (faiss::Index, faiss::MetricType, faiss::FaissException).  faiss itself is not a dependency of
-// this build; a project that already has faiss can define IXA_USE_REAL_FAISS and include the real
-// headers instead.
+// Minimal stand-in for the faiss types that the reference's public classes derive from or exchange data
+// with (faiss::Index, MetricType, FaissException, ClusteringParameters, IndexFlat, ProductQuantizer,
+// ArrayInvertedLists, IndexIVFPQ): the members copyFrom / copyTo and the class hierarchy touch, under
+// faiss 1.10's names.  faiss itself is not a dependency of this build; a project that has faiss defines
+// IXA_USE_REAL_FAISS and gets the real headers instead.
 #pragma once
 #ifdef IXA_USE_REAL_FAISS
+#include <faiss/Clustering.h>
 #include <faiss/Index.h>
+#include <faiss/IndexFlat.h>
+#include <faiss/IndexIVFPQ.h>
 #include <faiss/impl/FaissException.h>
+#include <faiss/invlists/InvertedLists.h>
 #else
+#include <cstddef>
 #include <cstdint>
 #include <exception>
 #include <string>
+#include <vector>
 
 namespace faiss {
 
@@ -26,6 +33,20 @@ public:
 
 struct SearchParameters {
     virtual ~SearchParameters() {}
+};
+
+struct ClusteringParameters {
+    int niter = 25;
+    int nredo = 1;
+    bool verbose = false;
+    bool spherical = false;
+    bool int_centroids = false;
+    bool update_index = false;
+    bool frozen_centroids = false;
+    int min_points_per_centroid = 39;
+    int max_points_per_centroid = 256;
+    int seed = 1234;
+    size_t decode_block_size = 32768;
 };
 
 struct Index {
@@ -45,6 +66,127 @@ struct Index {
     virtual void search(idx_t n, const float *x, idx_t k, float *distances, idx_t *labels,
                         const SearchParameters *params = nullptr) const = 0;
     virtual void reset() = 0;
+};
+
+// The coarse quantizer of an IndexIVFPQ as copyFrom / copyTo see it: a row store.
+struct IndexFlat : Index {
+    std::vector<float> xb;
+    explicit IndexFlat(idx_t d_ = 0, MetricType metric = METRIC_L2) : Index(d_, metric) {}
+    void add(idx_t n, const float *x) override
+    {
+        xb.insert(xb.end(), x, x + (size_t)n * d);
+        ntotal += n;
+    }
+    void search(idx_t, const float *, idx_t, float *, idx_t *, const SearchParameters * = nullptr) const override
+    {
+        throw FaissException("the stand-in IndexFlat only stores rows");
+    }
+    void reset() override
+    {
+        xb.clear();
+        ntotal = 0;
+    }
+    const float *get_xb() const { return xb.data(); }
+};
+struct IndexFlatL2 : IndexFlat {
+    explicit IndexFlatL2(idx_t d_ = 0) : IndexFlat(d_, METRIC_L2) {}
+};
+struct IndexFlatIP : IndexFlat {
+    explicit IndexFlatIP(idx_t d_ = 0) : IndexFlat(d_, METRIC_INNER_PRODUCT) {}
+};
+
+struct ProductQuantizer {
+    size_t d = 0, M = 0, nbits = 0, dsub = 0, code_size = 0, ksub = 0;
+    std::vector<float> centroids;   // [M][ksub][dsub]
+    ProductQuantizer() {}
+    ProductQuantizer(size_t d_, size_t M_, size_t nbits_) : d(d_), M(M_), nbits(nbits_) { set_derived_values(); }
+    void set_derived_values()
+    {
+        dsub = M ? d / M : 0;
+        code_size = (nbits * M + 7) / 8;
+        ksub = (size_t)1 << nbits;
+        centroids.resize(d * ksub);
+    }
+};
+
+struct InvertedLists {
+    size_t nlist, code_size;
+    InvertedLists(size_t nlist_, size_t code_size_) : nlist(nlist_), code_size(code_size_) {}
+    virtual ~InvertedLists() {}
+    virtual size_t list_size(size_t list_no) const = 0;
+    virtual const uint8_t *get_codes(size_t list_no) const = 0;
+    virtual const idx_t *get_ids(size_t list_no) const = 0;
+    virtual void release_codes(size_t, const uint8_t *) const {}
+    virtual void release_ids(size_t, const idx_t *) const {}
+    virtual size_t add_entries(size_t list_no, size_t n_entry, const idx_t *ids, const uint8_t *code) = 0;
+};
+
+struct ArrayInvertedLists : InvertedLists {
+    std::vector<std::vector<uint8_t>> codes;
+    std::vector<std::vector<idx_t>> ids;
+    ArrayInvertedLists(size_t nlist_, size_t code_size_) : InvertedLists(nlist_, code_size_), codes(nlist_), ids(nlist_) {}
+    size_t list_size(size_t l) const override { return ids[l].size(); }
+    const uint8_t *get_codes(size_t l) const override { return codes[l].data(); }
+    const idx_t *get_ids(size_t l) const override { return ids[l].data(); }
+    size_t add_entries(size_t l, size_t n, const idx_t *ids_in, const uint8_t *code) override
+    {
+        const size_t at = ids[l].size();
+        ids[l].insert(ids[l].end(), ids_in, ids_in + n);
+        codes[l].insert(codes[l].end(), code, code + n * code_size);
+        return at;
+    }
+};
+
+// faiss::IndexIVFPQ with the members of IndexIVF / Level1Quantizer that the exchange touches.
+struct IndexIVFPQ : Index {
+    Index *quantizer = nullptr;
+    size_t nlist = 0;
+    bool own_fields = false;
+    ClusteringParameters cp;
+    InvertedLists *invlists = nullptr;
+    bool own_invlists = false;
+    size_t code_size = 0;
+    size_t nprobe = 1;
+    bool by_residual = true;
+    ProductQuantizer pq;
+    IndexIVFPQ() {}
+    IndexIVFPQ(Index *quantizer_, size_t d_, size_t nlist_, size_t M, size_t nbits_per_idx, MetricType metric = METRIC_L2)
+        : Index((idx_t)d_, metric), quantizer(quantizer_), nlist(nlist_), invlists(new ArrayInvertedLists(nlist_, M)),
+          own_invlists(true), code_size(M), pq(d_, M, nbits_per_idx)
+    {
+        is_trained = false;
+    }
+    ~IndexIVFPQ() override
+    {
+        if (own_invlists) {
+            delete invlists;
+        }
+        if (own_fields) {
+            delete quantizer;
+        }
+    }
+    IndexIVFPQ(const IndexIVFPQ &) = delete;
+    IndexIVFPQ &operator=(const IndexIVFPQ &) = delete;
+    void replace_invlists(InvertedLists *il, bool own = false)
+    {
+        if (own_invlists) {
+            delete invlists;
+        }
+        invlists = il;
+        own_invlists = own;
+    }
+    void add(idx_t, const float *) override { throw FaissException("the stand-in IndexIVFPQ only carries data"); }
+    void search(idx_t, const float *, idx_t, float *, idx_t *, const SearchParameters * = nullptr) const override
+    {
+        throw FaissException("the stand-in IndexIVFPQ only carries data");
+    }
+    void reset() override
+    {
+        if (invlists) {
+            replace_invlists(new ArrayInvertedLists(nlist, code_size), true);
+        }
+        ntotal = 0;
+    }
 };
 
 }  // namespace faiss

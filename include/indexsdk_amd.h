@@ -116,8 +116,14 @@ typedef struct ivfpq_index ivfpq_index_t;
 typedef struct ivfpq_config {
     int32_t niter;                  /* cp.niter of the coarse k-means; reference CPU mode uses 25 */
     int32_t pq_niter;               /* pqNiter; -1 = niter */
-    int32_t spherical;              /* cp.spherical for the COARSE quantizer; 0 = plain Lloyd (default here),
-                                       1 = centroids L2-normalised every iteration (reference default) */
+    int32_t spherical;              /* cp.spherical for the COARSE quantizer: 1 = centroids L2-normalised after every
+                                       update, 0 = plain Lloyd, -1 (default) = normalised for inner product only.  The
+                                       reference forces it for inner product and, in its CPU mode, for L2 as well
+                                       (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1159-1171), which suits unit-norm data
+                                       only.  Sub-quantizer codebooks are never normalised here (the reference's CPU
+                                       mode does, :1064-1067).  useKmeansPP of the reference's config selects WHERE it
+                                       trains (its NPU k-means or faiss on the host); this build always trains on the
+                                       device, seeded with random samples, whatever that flag says. */
     int32_t train_samples_per_list; /* trainSamplesPerList */
     int64_t max_train_samples;      /* maxTrainSamples */
     int32_t lut_fp16;               /* 1 = store the per-query LUT as IEEE half (accumulate in fp32) */

@@ -82,7 +82,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
 {
     ixa::IvfpqConfig c;
     if (cfg) {
-        IXA_REQUIRE(cfg->niter >= 0 && cfg->train_samples_per_list >= 1 && cfg->max_train_samples >= 1 &&
+        IXA_REQUIRE(cfg->spherical >= -1 && cfg->spherical <= 1 && cfg->niter >= 0 && cfg->train_samples_per_list >= 1 && cfg->max_train_samples >= 1 &&
                         cfg->scratch_bytes >= (1 << 20) && cfg->code_layout >= -1 && cfg->code_layout <= 2,
                     ixa::kErrInvalidParam, "invalid ivfpq_config_t field");
         c.niter = cfg->niter;

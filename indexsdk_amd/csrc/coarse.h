@@ -106,10 +106,12 @@ void launch_select_rows_i32(const int32_t *scores, int64_t nrows, int64_t ld, in
 
 // Exact best-nout SET from approximately scored, sorted candidates (see refine_boundary_kernel):
 // re-evaluates only the candidates within 2 * err of the rank-nout score; a query whose list
-// cannot be proven to contain every winner is appended to flag[1 + flag[0]++] (flag: 1 + nq ints).  out_ids: [nq][nout], unordered.
+// cannot be proven to contain every winner is appended to flag[1 + flag[0]++] (flag: 1 + nq ints); complete = the
+// candidates are ALL base rows, so nothing is left to prove.  out_ids: [nq][nout], unordered.
 void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                             int metric, const unsigned long long *running, int ncand, int nout, float cmax,
-                            float err_scale, float round_scale, int32_t *out_ids, int *flag, hipStream_t s);
+                            float err_scale, float round_scale, int32_t *out_ids, int *flag, bool complete,
+                            hipStream_t s);
 
 // Canonical scores of all nc centroids for every row (one lane per score; the exact plan of last resort).
 void launch_canonical_scores(const float *Q, int64_t nq, const float *C, int64_t nc, int d, const float *qn,

@@ -1098,7 +1098,8 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
                                                               const float *__restrict__ cn, int metric,
                                                               const key_t *__restrict__ running, int ncand, int nout,
                                                               float cmax, float err_scale, float round_scale,
-                                                              int32_t *__restrict__ out_ids, int *__restrict__ flag)
+                                                              int32_t *__restrict__ out_ids, int *__restrict__ flag,
+                                                              int complete)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1125,7 +1126,7 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
     const float err = err_scale * qlen * cmax + round_scale * (qlen + cmax) * (qlen + cmax);
     const float lo = T - 2.0f * err, hi = T + 2.0f * err;
     const key_t last = run[ncand - 1];
-    if (lane == 0 && last != kEmptyKey && !(key_score(last) > hi)) {
+    if (lane == 0 && !complete && last != kEmptyKey && !(key_score(last) > hi)) {   // a list of all rows is complete
         flag[1 + atomicAdd(flag, 1)] = (int)row;   // the list of queries that need another plan
     }
     int n_in = 0, n_amb = 0;
@@ -1196,7 +1197,8 @@ __global__ __launch_bounds__(256) void refine_boundary_kernel(const float *__res
 
 void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                             int metric, const unsigned long long *running, int ncand, int nout, float cmax,
-                            float err_scale, float round_scale, int32_t *out_ids, int *flag, hipStream_t s)
+                            float err_scale, float round_scale, int32_t *out_ids, int *flag, bool complete,
+                            hipStream_t s)
 {
     if (nq == 0) {
         return;
@@ -1212,7 +1214,7 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
                                     (int)smem));
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
-                       ncand, nout, cmax, err_scale, round_scale, out_ids, flag);
+                       ncand, nout, cmax, err_scale, round_scale, out_ids, flag, complete ? 1 : 0);
 }
 
 // The boundary refinement above straight from the records of a record-mode score launch over the whole

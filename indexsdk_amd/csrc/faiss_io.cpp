@@ -172,10 +172,20 @@ void write_faiss_ivfpq(const IvfpqIndex &idx, const char *path)
 std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig &cfg)
 {
     File f(path, "rb");
+    // every size the file states is held against the index's limits and against the file's own length before
+    // anything is allocated, cast or divided by it
+    IXA_REQUIRE(std::fseek(f.f, 0, SEEK_END) == 0, kErrInvalidParam, "%s: can not seek", path);
+    const long file_len = std::ftell(f.f);
+    IXA_REQUIRE(file_len >= 0 && std::fseek(f.f, 0, SEEK_SET) == 0, kErrInvalidParam, "%s: can not seek", path);
+    const uint64_t file_bytes = (uint64_t)file_len;
     IXA_REQUIRE(f.get1<uint32_t>() == fourcc("IwPQ"), kErrInvalidParam, "%s is not a faiss IndexIVFPQ file (IwPQ)", path);
     const Header h = get_header(f);
     const uint64_t nlist = f.get1<uint64_t>(), nprobe = f.get1<uint64_t>();
-    IXA_REQUIRE(h.d > 0 && nlist > 0 && nlist <= ((uint64_t)1 << 24), kErrInvalidParam, "%s: bad d or nlist", path);
+    IXA_REQUIRE(h.d >= 1 && h.d <= 4096 && nlist >= 1 && nlist <= ((uint64_t)1 << 20) && h.ntotal >= 0 &&
+                    (h.metric == kMetricL2 || h.metric == kMetricInnerProduct),
+                kErrInvalidParam, "%s: d = %d, nlist = %lu, ntotal = %ld or metric = %d is outside what an index holds", path,
+                h.d, (unsigned long)nlist, (long)h.ntotal, h.metric);
+    IXA_REQUIRE(nlist * (uint64_t)h.d * 4 <= file_bytes, kErrInvalidParam, "%s is shorter than its coarse quantizer", path);
     const uint32_t q4 = f.get1<uint32_t>();
     IXA_REQUIRE(q4 == fourcc("IxF2") || q4 == fourcc("IxFI"), kErrInvalidParam,
                 "%s: the coarse quantizer must be an IndexFlat (IxF2 / IxFI)", path);
@@ -190,14 +200,16 @@ std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig
     const uint64_t map_n = f.get1<uint64_t>();
     IXA_REQUIRE(map_type != 2, kErrInvalidParam, "%s: hashtable direct maps are not supported", path);
     if (map_n) {
-        IXA_REQUIRE(std::fseek(f.f, (long)(map_n * 8), SEEK_CUR) == 0, kErrInvalidParam, "%s is truncated", path);
+        IXA_REQUIRE(map_n <= file_bytes / 8 && std::fseek(f.f, (long)(map_n * 8), SEEK_CUR) == 0, kErrInvalidParam,
+                    "%s is truncated (direct map of %lu entries)", path, (unsigned long)map_n);
     }
     const uint8_t by_residual = f.get1<uint8_t>();
     IXA_REQUIRE(by_residual == 0, kErrInvalidParam,
                 "%s was built with by_residual = true: its codes encode residuals and cannot be searched here", path);
     const uint64_t code_size = f.get1<uint64_t>();
     const uint64_t pq_d = f.get1<uint64_t>(), M = f.get1<uint64_t>(), nbits = f.get1<uint64_t>();
-    IXA_REQUIRE(pq_d == (uint64_t)h.d && nbits == 8 && M >= 1 && code_size == M && h.d % (int)M == 0, kErrInvalidParam,
+    IXA_REQUIRE(pq_d == (uint64_t)h.d && nbits == 8 && M >= 1 && M <= 128 && code_size == M &&
+                    (uint64_t)h.d % M == 0, kErrInvalidParam,
                 "%s: product quantizer d=%lu M=%lu nbits=%lu code_size=%lu is not supported", path, (unsigned long)pq_d,
                 (unsigned long)M, (unsigned long)nbits, (unsigned long)code_size);
     const uint64_t ncb = f.get1<uint64_t>();
@@ -251,7 +263,8 @@ std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig
         if (n == 0) {
             continue;
         }
-        IXA_REQUIRE(n < ((uint64_t)1 << 31), kErrInvalidParam, "%s: list %lu is too long", path, (unsigned long)l);
+        IXA_REQUIRE(n < ((uint64_t)1 << 31) && (uint64_t)n * (M + 8) <= file_bytes, kErrInvalidParam,
+                    "%s: list %lu is longer than the file", path, (unsigned long)l);
         const size_t at = list_no.size();
         list_no.resize(at + n, (int32_t)l);
         codes.resize((at + n) * M);

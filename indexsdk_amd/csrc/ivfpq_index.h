@@ -14,7 +14,9 @@ namespace ixa {
 struct IvfpqConfig {
     int niter = 25;                   // coarse k-means iterations (reference CPU mode: 25)
     int pq_niter = -1;                // sub-quantizer k-means iterations; -1 = niter (pqNiter)
-    int spherical = 0;                // 1 = L2-normalise centroids after every update (reference default)
+    int spherical = -1;               // coarse centroids L2-normalised after every update: 1 yes, 0 no, -1 = for inner
+                                      // product only (the reference forces it there, AscendIndexIVFPQImpl.cpp:1159-1163;
+                                      // its CPU mode also does it for L2, which suits unit-norm data only)
     int train_samples_per_list = 256; // rows sampled per coarse centroid (trainSamplesPerList)
     int64_t max_train_samples = 10000000;  // maxTrainSamples
     int lut_fp16 = 0;                 // LUT entries stored as IEEE half

@@ -632,7 +632,7 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
         // cannot decide are re-evaluated
         launch_refine_boundary(x_dev, n, centroids_.data(), d_, ws_qn_.data(), cnorm_.data(), select_metric,
                                ws_running_.data(), ncand, nout, cmax_, err_scale, round_scale, out_ids,
-                               ws_flag_.data(), stream_);
+                               ws_flag_.data(), ncand >= nlist_, stream_);
     } else {
         float *dist = out_dist;
         if (!dist) {
@@ -1604,7 +1604,7 @@ void IvfpqIndex::kmeans_coarse(const std::vector<float> &sample, int64_t ns)
                            stream_, xs.data(), d_, order_dev.data(), seg_dev.data(), centroids_.data(), mean_dev.data());
         mean_dev.download(cent.data(), cent.size(), stream_);
         split_empty(cent, cnt, nlist_, d_);
-        if (cfg_.spherical) {
+        if (cfg_.spherical < 0 ? metric_ == kMetricInnerProduct : cfg_.spherical != 0) {
             normalise_rows(cent, nlist_, d_);
         }
     }

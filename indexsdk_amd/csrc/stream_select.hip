@@ -161,8 +161,15 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     // when the whole score matrix of a query block fits the scratch, one materialised pass is the
     // cheapest plan (measured on the IVFPQ coarse stage: 16384 centroids); the filtered plan is for
     // long bases
-    const bool can_fuse = nb_total > nb && nb_total >= 4 * seed_rows &&
-                          pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    bool can_fuse = nb_total > nb && nb_total >= 4 * seed_rows && pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    if (can_fuse && qb * (int64_t)cap * (int64_t)sizeof(key_t) > scratch_bytes) {
+        // the candidate buffers of a query block count against the scratch budget too: a narrower block
+        qb = std::max<int64_t>(128, scratch_bytes / ((int64_t)cap * (int64_t)sizeof(key_t)) / 128 * 128);
+        nb = scratch_bytes / (qb * (int64_t)sizeof(S));
+        nb = std::max<int64_t>(128, nb / 128 * 128);
+        nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(nb_total, 1), 128));
+        can_fuse = nb_total > nb;
+    }
     // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query; keep
     // that expectation below a quarter of the candidate buffer
     const int64_t growth = std::max<int64_t>(2, cap / (4 * (int64_t)ncand));

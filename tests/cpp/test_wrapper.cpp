@@ -25,6 +25,7 @@ static std::string construct_msg(int dim, int nlist, int msub, int nbit)
 {
     try {
         AscendIndexIVFPQConfig conf({0});
+        conf.strictReferenceParams = true;   // the reference's whitelists and messages
         AscendIndexIVFPQ index(dim, faiss::METRIC_L2, nlist, msub, nbit, conf);
     } catch (std::exception &e) {
         return e.what();
@@ -62,13 +63,21 @@ int main(int argc, char **argv)
             v = nd(gen);
         }
         AscendIndexIVFPQConfig conf({0});
-        conf.niter = 3;
+        conf.cp.niter = 3;                       // ClusteringParameters of the coarse quantizer (AscendIndexIVFConfig)
+        conf.useKmeansPP = true;                 // accepted, changes nothing here
         AscendIndexIVFPQ index(d, faiss::METRIC_L2, nlist, M, 8, conf);
         EXPECT(!index.is_trained);
         index.train(n, x.data());
-        index.add(n, x.data());
-        EXPECT(index.ntotal == n);
-        index.setNumProbes(32);
+        // the levels of the hierarchy: AscendIndexIVFPQ -> AscendIndexIVF -> AscendIndex -> faiss::Index
+        AscendIndexIVF *ivf = &index;
+        AscendIndex *base = ivf;
+        faiss::Index *root = base;
+        base->reserveMemory((size_t)n);
+        root->add(n, x.data());
+        EXPECT(index.ntotal == n && ivf->getNumLists() == nlist && base->getDeviceList().size() == 1);
+        EXPECT(base->reclaimMemory() > 0);
+        ivf->setNumProbes(32);
+        EXPECT(ivf->getNumProbes() == 32);
         std::vector<float> D((size_t)nq * k);
         std::vector<faiss::idx_t> I((size_t)nq * k);
         index.search(nq, x.data(), k, D.data(), I.data());
@@ -103,11 +112,66 @@ int main(int argc, char **argv)
         }
         EXPECT(threw);
         std::remove(path.c_str());
+        {
+            // copyTo / copyFrom through faiss::IndexIVFPQ (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:392-508)
+            faiss::IndexIVFPQ cpu;
+            index.copyTo(&cpu);
+            EXPECT(cpu.ntotal == n && cpu.nlist == (size_t)nlist && cpu.nprobe == 32 && !cpu.by_residual);
+            EXPECT(cpu.pq.M == (size_t)M && cpu.pq.dsub == (size_t)(d / M) && cpu.quantizer->ntotal == nlist);
+            size_t in_lists = 0;
+            for (size_t l = 0; l < cpu.nlist; l++) {
+                in_lists += cpu.invlists->list_size(l);
+            }
+            EXPECT(in_lists == (size_t)n);
+            AscendIndexIVFPQConfig other_conf({0});
+            AscendIndexIVFPQ from_cpu(d, faiss::METRIC_L2, 2048, 8, 8, other_conf);   // another shape: overwritten
+            from_cpu.copyFrom(&cpu);
+            EXPECT(from_cpu.is_trained && from_cpu.ntotal == n && from_cpu.getNumLists() == nlist &&
+                   from_cpu.getNumProbes() == 32);
+            std::vector<float> D3((size_t)nq * k);
+            std::vector<faiss::idx_t> I3((size_t)nq * k);
+            from_cpu.search(nq, x.data(), k, D3.data(), I3.data());
+            EXPECT(I3 == I && D3 == D);
+            std::vector<uint8_t> ca, cb2;
+            std::vector<ascend_idx_t> ia, ib;
+            index.getListCodesAndIds(5, ca, ia);
+            from_cpu.getListCodesAndIds(5, cb2, ib);
+            EXPECT(ca == cb2 && ia == ib);
+            cpu.by_residual = true;   // codes of residuals can not be searched against raw queries: refused
+            bool refused = false;
+            try {
+                from_cpu.copyFrom(&cpu);
+            } catch (const faiss::FaissException &e) {
+                refused = std::string(e.what()).find("by_residual") != std::string::npos;
+            }
+            EXPECT(refused && from_cpu.ntotal == n);
+        }
         AscendIndexFlatL2 flat(d);
+        AscendIndex *flat_base = &flat;
+        EXPECT(flat_base->reclaimMemory() == 0);
         flat.add(n, x.data());
         flat.search(nq, x.data(), k, D.data(), I.data());
         for (int i = 0; i < nq; i++) {
             EXPECT(I[(size_t)i * k] == i);
+        }
+        faiss::IndexFlatL2 cpu_flat(d);
+        flat.copyTo(&cpu_flat);
+        EXPECT(cpu_flat.ntotal == n && std::memcmp(cpu_flat.get_xb(), x.data(), x.size() * sizeof(float)) == 0);
+        AscendIndexFlat flat2(&cpu_flat);
+        EXPECT(flat2.ntotal == n);
+        // int8: AscendIndexInt8Flat -> AscendIndexInt8
+        std::vector<int8_t> b((size_t)4096 * 64);
+        for (auto &v : b) {
+            v = (int8_t)((int)(gen() % 255) - 127);
+        }
+        AscendIndexInt8Flat i8(64);
+        AscendIndexInt8 *i8_base = &i8;
+        i8_base->add(4096, b.data());
+        std::vector<float> Di((size_t)4 * 3);
+        std::vector<faiss::idx_t> Ii((size_t)4 * 3);
+        i8_base->search(4, b.data(), 3, Di.data(), Ii.data());
+        for (int i = 0; i < 4; i++) {
+            EXPECT(Ii[(size_t)i * 3] == i && Di[(size_t)i * 3] == 0.f);
         }
     }
     std::printf(failures ? "wrapper test FAILED\n" : "wrapper test ok\n");

@@ -208,3 +208,47 @@ def test_scan_lds_plan_keeps_every_region_inside_the_allocation(capi):
                                 assert a1 <= b0, (an, bn, M, k, nprobe, W, sh)
                             checked += 1
     assert checked > 5000
+
+
+def _faiss_file(tmp_path, name, d=4, nlist=1, ntotal=0, M=2, code_size=None, nbits=8, map_n=0, cent_floats=None,
+                metric=1):
+    """The leading part of a faiss IndexIVFPQ file (fourcc IwPQ, IndexFlat quantizer, product quantizer), as
+    faiss 1.10's write_index lays it out, with the given -- possibly absurd -- sizes."""
+    import struct
+    hdr = lambda dd, nt: struct.pack("<iqqqBi", dd, nt, 1 << 20, 1 << 20, 1, metric)
+    n_cent = nlist * d if cent_floats is None else cent_floats
+    out = b"IwPQ" + hdr(d, ntotal) + struct.pack("<QQ", nlist, 1)
+    out += (b"IxF2" if metric == 1 else b"IxFI") + hdr(d, nlist) + struct.pack("<Q", nlist * d)
+    out += b"\0" * (4 * min(n_cent, 1 << 16))
+    out += struct.pack("<BQ", 0, map_n) + struct.pack("<B", 0)
+    out += struct.pack("<QQQQ", M if code_size is None else code_size, d, M, nbits)
+    out += struct.pack("<Q", 256 * d) + b"\0" * (4 * 256 * min(d, 64))
+    p = tmp_path / name
+    p.write_bytes(out)
+    return str(p).encode()
+
+
+@pytest.mark.parametrize("kw,needle", [
+    (dict(d=100000), "outside what an index holds"),
+    (dict(d=0), "outside what an index holds"),
+    (dict(nlist=1 << 21), "outside what an index holds"),
+    (dict(nlist=0), "outside what an index holds"),
+    (dict(ntotal=-5), "outside what an index holds"),
+    (dict(d=4096, nlist=1 << 20), "shorter than its coarse quantizer"),
+    (dict(M=1 << 32, code_size=1 << 32), "product quantizer"),          # d % (int)M would divide by zero
+    (dict(M=3), "product quantizer"),                                    # 3 does not divide 4
+    (dict(M=2, code_size=3), "product quantizer"),
+    (dict(M=256, d=256, code_size=256), "product quantizer"),            # more sub-quantizers than the index takes
+    (dict(nbits=4), "product quantizer"),
+    (dict(map_n=1 << 61), "truncated"),
+])
+def test_reader_of_faiss_files_rejects_absurd_headers_before_using_them(capi, tmp_path, kw, needle):
+    """Sizes a file states are checked against the index's limits and the file's own length before they are
+    allocated, cast or divided by: every one of these comes back as an error message (no crash, no GPU needed,
+    no huge allocation)."""
+    lib = capi.load()
+    path = _faiss_file(tmp_path, "bad.index", **kw)
+    h = ctypes.c_void_p()
+    rc = lib.ivfpq_read_faiss(path, None, ctypes.byref(h))
+    msg = lib.ixa_last_error().decode()
+    assert rc == 2001 and needle in msg and not h.value, (rc, msg)

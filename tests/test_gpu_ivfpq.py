@@ -731,3 +731,50 @@ def test_search_in_query_pages_equals_one_batch(ix, oracle):
     Dr, Ir = ref.search(q, 20, 8)
     assert paged["scanned_codes"] == ref.last_scanned
     assert_topk_parity(oracle, ref, q, Dp, Ip, Dr, Ir, TOL_FP32)
+
+
+@pytest.mark.parametrize("spherical,metric_name", [(0, "L2"), (1, "L2"), (-1, "IP")])
+def test_coarse_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, spherical, metric_name):
+    """Centroids after n + 1 iterations = one Lloyd update of the centroids after n: nearest-centroid
+    assignment under L2 (the add path's rule), float64 sums in sample order for the means, a cluster without
+    members re-seeded by splitting the most populated one (its centroid times 1 -+ 1/1024, the sign
+    alternating over the components, members shared out evenly), rows normalised when spherical (which
+    inner product switches on by default).  The data leave some of the 96 clusters empty."""
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    d, nlist, n = 32, 96, 5000
+    rng = np.random.default_rng(17 + spherical)
+    centres = rng.standard_normal((6, d)).astype(np.float32) * 4
+    x = (centres[rng.integers(0, 6, n)] + 0.05 * rng.standard_normal((n, d))).astype(np.float32)
+    x[100:] = centres[rng.integers(0, 6, n - 100)]        # 4900 rows are exact copies of six points: of the
+    #                                                       centroids that coincide on one, all but the first stay empty
+    if metric == ix.METRIC_INNER_PRODUCT:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    cents = []
+    for niter in (2, 3):
+        cfg = ix.AscendIndexIVFPQConfig(niter=niter, pq_niter=0, spherical=spherical, train_samples_per_list=1 << 20)
+        gpu = ix.AscendIndexIVFPQ(d, metric, nlist, 8, 8, cfg)
+        gpu.train(x)
+        cents.append(gpu.get_trained()[0])
+    before, after = cents
+    asg = oracle.assign(x, before)
+    cnt = np.bincount(asg, minlength=nlist).astype(np.int64)
+    want = before.copy()
+    for c in range(nlist):
+        if cnt[c]:
+            rows = x[asg == c].astype(np.float64)
+            want[c] = (np.cumsum(rows, axis=0)[-1] / cnt[c]).astype(np.float32)
+    empties = int((cnt == 0).sum())
+    eps = np.where(np.arange(d) % 2 == 1, np.float32(1 / 1024), np.float32(-1 / 1024)).astype(np.float32)
+    for c in range(nlist):
+        if cnt[c] == 0:
+            big = int(np.argmax(cnt))
+            v = want[big].copy()
+            want[c] = v * (np.float32(1) + eps)
+            want[big] = v * (np.float32(1) - eps)
+            cnt[c] = cnt[big] // 2
+            cnt[big] -= cnt[c]
+    if spherical == 1 or (spherical < 0 and metric == ix.METRIC_INNER_PRODUCT):
+        norm = np.sqrt(np.cumsum(want.astype(np.float64) ** 2, axis=1)[:, -1])      # summed left to right
+        want = (want.astype(np.float64) / norm[:, None]).astype(np.float32)
+    assert empties >= 1, "the data should leave clusters empty"
+    assert np.array_equal(want.view(np.uint32), after.view(np.uint32))
