@@ -127,7 +127,9 @@ typedef struct ivfpq_config {
     int32_t train_samples_per_list; /* trainSamplesPerList */
     int64_t max_train_samples;      /* maxTrainSamples */
     int32_t lut_fp16;               /* 1 = store the per-query LUT as IEEE half (accumulate in fp32) */
-    int32_t code_layout;            /* -1 = choose, 0 = row-major codes, 1 = bank-rotated (M in {32,64,96}),
+    int32_t code_layout;            /* -1 = choose (by measurement: rotated for 64 and 96 sub-quantizers and for 32
+                                       with a half LUT, xor-rotated for 48 with an fp32 LUT, else row-major),
+                                       0 = row-major codes, 1 = bank-rotated (M in {32,64,96}),
                                        2 = xor-rotated (M = 48, fp32 LUT) */
     int64_t scratch_bytes;          /* resourceSize: bound of the coarse-score scratch in HBM */
     uint64_t seed;                  /* sampling / initialisation seed */
@@ -178,6 +180,8 @@ int ivfpq_read_faiss(const char *path, const ivfpq_config_t *cfg, ivfpq_index_t 
 /* Shape of an index (the public members d, metric_type, nlist and pq.M of the reference class); any output
  * may be NULL. */
 int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int64_t *nlist, int *msubs);
+/* The code layout in use (the values of ivfpq_config_t.code_layout, never -1). */
+int ivfpq_get_code_layout(const ivfpq_index_t *h, int *layout);
 
 /* AscendIndex::add / add_with_ids  FR/ascend/AscendIndex.h:66-71, AscendIndexIVFPQImpl.cpp:694-864.
  * ids == NULL numbers the vectors ntotal, ntotal+1, ... */

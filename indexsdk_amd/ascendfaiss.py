@@ -198,6 +198,12 @@ class AscendIndexIVFPQ:
     def reset(self):
         _capi.check(self._lib.ivfpq_reset(self._h))
 
+    def code_layout(self):
+        """0 = row-major codes, 1 = bank-rotated, 2 = xor-rotated (what the index chose, or was told)."""
+        out = ctypes.c_int()
+        _capi.check(self._lib.ivfpq_get_code_layout(self._h, ctypes.byref(out)))
+        return out.value
+
     def reserveMemory(self, num_vecs):
         """AscendIndexIVF::reserveMemory: room for num_vecs more vectors without replacing the code arena."""
         _capi.check(self._lib.ivfpq_reserve_memory(self._h, int(num_vecs)))

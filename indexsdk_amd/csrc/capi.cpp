@@ -184,6 +184,15 @@ IXA_EXPORT int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int6
     });
 }
 
+IXA_EXPORT int ivfpq_get_code_layout(const ivfpq_index_t *h, int *layout)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        IXA_REQUIRE(layout, ixa::kErrInvalidParam, "layout can not be nullptr.");
+        *layout = h->impl.code_layout();
+    });
+}
+
 IXA_EXPORT int ivfpq_destroy(ivfpq_index_t *h)
 {
     return guarded([&] { delete h; });

@@ -68,8 +68,9 @@ def test_random_write_sequences_at_a_million_vectors(oracle):
     train = draw(40_000)
     cent, _ = oracle.kmeans(train, nlist, niter=3, seed=5)
     cb = oracle.train_pq(train[:8000], M, niter=2, seed=5)
-    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(code_layout=1))
     gpu.set_trained(cent, cb)
+    assert gpu.code_layout() == 1
     model = ListModel(nlist, M)
     next_id = [0]
 
