@@ -86,6 +86,34 @@ struct GroupRef {
 // choice for k so large that private pools would leave room for only a few waves per CU.
 // The half-LUT rot32 variants are held to 128 registers (4 waves per SIMD): their LDS plan admits
 // two 8-wave workgroups per CU and the register allocator would otherwise trade that away.
+// Byte j of a 32-bit word times 2^SH as one instruction: a left shift whose shifted operand is selected by
+// byte (sub-dword addressing), so no separate extraction is needed.
+template <int SH>
+__device__ __forceinline__ uint32_t byte_times_pow2(uint32_t w, int j)
+{
+    uint32_t r;
+    const uint32_t sh = SH;
+    switch (j) {
+        case 0:
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+                : "=v"(r) : "s"(sh), "v"(w));
+            break;
+        case 1:
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1"
+                : "=v"(r) : "s"(sh), "v"(w));
+            break;
+        case 2:
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2"
+                : "=v"(r) : "s"(sh), "v"(w));
+            break;
+        default:
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3"
+                : "=v"(r) : "s"(sh), "v"(w));
+            break;
+    }
+    return r;
+}
+
 template <int MT, typename LutT, int LAYOUT, int W, bool SHARED>
 __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARED) ? 4 : 1) void ivfpq_scan_kernel(
     ScanParams p)
@@ -291,6 +319,11 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     };
 
     constexpr int NW = MT > 0 ? (MT + 3) / 4 : 1;
+    // Lanes past the end of a list load nothing when a code is long: with 96-byte codes the padding of the last
+    // group is 5 % of the bytes of a 600-code list, and the launch is bound by the bytes it fetches (20M x 96 B,
+    // 4096 queries x 128 lists: 5.2 -> 4.95 ms).  With short codes the exec-mask bookkeeping costs more than the bytes
+    // (10M x 32 B, 10000 queries x 64 lists: 1.59 -> 1.61 ms), so those kernels load whole groups.
+    constexpr bool kSkipPadding = MT >= 64;
     auto load_codes = [&](uint32_t slot, uint32_t (&w)[NW]) {
         if (MT == 0) {
             return;
@@ -402,12 +435,25 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             }
             return (acc[0] + acc[1]) + (acc[2] + acc[3]);
         }
-        // row layout: m = 0..M-1 in sequence, the accumulation order of the reference's scalar path
+        // row layout: m = 0..M-1 in sequence, the accumulation order of the reference's scalar path.  The byte
+        // offset of the entry inside its 256-entry row is ONE instruction (a shift whose operand is byte m % 4 of
+        // the code word) and the row's start is the load's immediate offset: two VALU instructions per lookup
+        // with the addition, where extract, scale and add are three -- the scan loop is bound by VALU issue.
+        // The LUT is the first thing in the workgroup's LDS and the kernel has no static LDS (the host checks
+        // that before the first launch), so its LDS address is 0 and needs no addition either.
+        typedef __attribute__((address_space(3))) const float lds_f32_t;
         float s = 0.f;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            const uint32_t code = (w[(m >> 2) % NW] >> (8 * (m & 3))) & 0xffu;
-            s = __fadd_rn(s, from_lut(lut[m * 256 + code]));
+            const uint32_t off = byte_times_pow2<sizeof(LutT) == 4 ? 2 : 1>(w[(m >> 2) % NW], m & 3);
+            const uint32_t addr = (uint32_t)(m * 256 * sizeof(LutT)) + off;
+            float v;
+            if constexpr (sizeof(LutT) == 4) {
+                v = *(lds_f32_t *)(size_t)addr;
+            } else {
+                v = __half2float(__ushort_as_half(*(lds_half_t *)(size_t)addr));
+            }
+            s = __fadd_rn(s, v);
         }
         return s;
     };
@@ -431,7 +477,9 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     do {                                                                                              \
         if ((G) + W < total) {                                                                        \
             NXT = locate((G) + W);                                                                    \
-            load_codes(NXT.slot, WNXT); /* in flight while the current group is evaluated */          \
+            if (!kSkipPadding || NXT.valid) { /* lanes past the list's end fetch nothing */           \
+                load_codes(NXT.slot, WNXT); /* in flight while the current group is evaluated */      \
+            }                                                                                         \
         }                                                                                             \
         const float s_ = adc(CUR.slot, WCUR);                                                         \
         const bool compacted_ =                                                                       \
@@ -446,7 +494,9 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     do {                                                                                              \
         if ((G) + W < total) {                                                                        \
             NXT = locate((G) + W);                                                                    \
-            load_codes(NXT.slot, WNXT);                                                               \
+            if (!kSkipPadding || NXT.valid) {                                                         \
+                load_codes(NXT.slot, WNXT);                                                           \
+            }                                                                                         \
         }                                                                                             \
         if (bpool.poll()) {                                                                           \
             bpool.rendezvous(tid);                                                                    \
@@ -459,9 +509,11 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     int total_keys;
     if constexpr (SHARED) {
         if (wave < total) {
-            uint32_t wa[NW], wb[NW];
+            uint32_t wa[NW] = {}, wb[NW] = {};
             GroupRef ga = locate(wave), gb = ga;
-            load_codes(ga.slot, wa);
+            if (!kSkipPadding || ga.valid) {
+                load_codes(ga.slot, wa);
+            }
             for (int G = wave; G < total; G += 2 * W) {
                 IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb);
                 if (G + W < total) {
@@ -475,9 +527,11 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
         total_keys = bpool.sort_all(tid);
     } else {
         if (wave < total) {
-            uint32_t wa[NW], wb[NW];
+            uint32_t wa[NW] = {}, wb[NW] = {};
             GroupRef ga = locate(wave), gb = ga;
-            load_codes(ga.slot, wa);
+            if (!kSkipPadding || ga.valid) {
+                load_codes(ga.slot, wa);
+            }
             for (int G = wave; G < total; G += 2 * W) {
                 IXA_SCAN_STEP(G, ga, wa, gb, wb);
                 if (G + W < total) {
@@ -726,12 +780,29 @@ void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const i
     hipLaunchKernelGGL(scatter_order_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, cls, nq, cursor, order);
 }
 
+// The row-layout lookups address the LUT from LDS address 0: true while the kernel declares no static LDS, which
+// is asked of the loaded code object once per kernel and refused loudly otherwise.
+static void require_no_static_lds(const void *kern, bool &checked)
+{
+    if (checked) {
+        return;
+    }
+    hipFuncAttributes attr{};
+    IXA_HIP(hipFuncGetAttributes(&attr, kern));
+    IXA_REQUIRE(attr.sharedSizeBytes == 0, kErrInner,
+                "the scan kernel has %zu bytes of static LDS: its LUT would not start at LDS address 0",
+                (size_t)attr.sharedSizeBytes);
+    checked = true;
+}
+
 template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
     const int64_t slots = p.xcd_chunks ? (nq + 7) / 8 * 8 : nq;
+    static bool lds_checked[4] = {false, false, false, false};
     if (p.shared_pool && p.waves == 16) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 16, true>;
+        require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[0]);
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -739,6 +810,7 @@ static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(1024), smem, s, p);
     } else if (p.shared_pool) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, true>;
+        require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[1]);
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -746,6 +818,7 @@ static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else if (p.waves == 8) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, false>;
+        require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[2]);
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -753,6 +826,7 @@ static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4, false>;
+        require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[3]);
         if (smem > 48 * 1024) {
             IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
