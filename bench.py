@@ -103,6 +103,11 @@ WORKLOADS = {
                metric="L2", lut_fp16=0, ntrain=500_000, seed=1236),
     "C3": dict(n=20_000_000, nq=4096, d=768, comp=4096, sigma=0.05, nlist=32768, M=96, nprobe=128, k=100,
                metric="IP", lut_fp16=1, ntrain=1_310_720, seed=1237, unit=True),
+    # the shape the reference's design document states its latency targets on (10M x 128, nlist 1024, M 4, k 300,
+    # batches of 1..64, nprobe 32 / 64 / 128: 880 / 1350 / 2340 us on its hardware,
+    # docs/rfc/26.1.0/IVFPQ...RFC.md:84-93); `--latency-sweep` reports those cells
+    "RFC": dict(n=10_000_000, nq=64, d=128, comp=1024, sigma=0.25, nlist=1024, M=4, nprobe=64, k=300,
+                metric="L2", lut_fp16=0, ntrain=500_000, seed=1240),
     "C5": dict(n=100_000_000, nq=1024, d=96, comp=256, sigma=0.25, nlist=65536, M=48, nprobe=256, k=1024,
                metric="L2", lut_fp16=0, ntrain=2_621_440, seed=1239, zipf=1.1),
 }
@@ -182,7 +187,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"],
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "RFC"],
                     help="benchmark configuration; C2 (default) is the one the metric is quoted on")
     ap.add_argument("--n", type=int, default=0, help="override the number of base vectors")
     ap.add_argument("--nq", type=int, default=0)
@@ -205,6 +210,9 @@ def main():
     ap.add_argument("--same-queries", action="store_true",
                     help="diagnostic: every query is a copy of the first, so the scanned lists stay in L2 "
                          "(the scan kernel's own ceiling, without HBM); not the benchmark")
+    ap.add_argument("--latency-sweep", action="store_true",
+                    help="also report the median latency of one search call for batches of 1..64 queries at "
+                         "nprobe 32 / 64 / 128 (device-resident queries and results, and through host pointers)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB plain copy kernel (yardstick for rocprofv3 traffic counters)")
     args = ap.parse_args()
@@ -380,6 +388,39 @@ def main():
     result["host_io"] = {"ms_per_step": host_io_ms, "queries_per_s": nq / (host_io_ms * 1e-3),
                          "note": "ivfpq_search with host pointers: H2D of the queries and D2H of the results included"}
     log(f"host-pointer search: {host_io_ms:.3f} ms per batch, {nq / (host_io_ms * 1e-3):.0f} QPS")
+
+    if args.latency_sweep:
+        # one search call per cell, synchronised, 40 calls after 5 warm-up calls: the median wall time of a call
+        sweep = {}
+        for np_ in (32, 64, 128):
+            if np_ > nlist:
+                continue
+            index.setNumProbes(np_)
+            for b in (1, 2, 4, 8, 16, 32, 64):
+                if b > nq:
+                    continue
+                qd = queries[:b].contiguous()
+                qh_b = qd.cpu().numpy()
+                cell = {}
+                for kind in ("device", "host"):
+                    ts = []
+                    for it in range(45):
+                        torch.cuda.synchronize()
+                        t1 = time.perf_counter()
+                        if kind == "device":
+                            _capi.check(lib.ivfpq_search_device(index._h, b, ctypes.c_void_p(qd.data_ptr()), k,
+                                                                ctypes.c_void_p(D.data_ptr()), ctypes.c_void_p(I.data_ptr())))
+                        else:
+                            index.search(qh_b, k)
+                        ts.append((time.perf_counter() - t1) * 1e6)
+                    cell[kind + "_us"] = float(np.median(ts[5:]))
+                st = index.last_search_stats()
+                cell["nsplit"] = int(st.get("nsplit", 0))
+                sweep[f"nprobe{np_}_batch{b}"] = cell
+                log(f"latency nprobe {np_:4d} batch {b:3d}: device {cell['device_us']:8.1f} us, host pointers "
+                    f"{cell['host_us']:8.1f} us (nsplit {cell['nsplit']})")
+        index.setNumProbes(nprobe)
+        result["latency_sweep"] = sweep
 
     if not args.no_cpu:
         from oracle import oracle as orc

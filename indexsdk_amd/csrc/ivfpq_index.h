@@ -124,7 +124,7 @@ private:
                       std::vector<int32_t> *redone = nullptr);
     ScanParams scan_params(const float *xd, int64_t n, const int32_t *probes, int nprobe, int64_t k, float *dd,
                            int64_t *ld, const ScanScratch *ext = nullptr);
-    static int scan_nsplit(int64_t n, int nprobe, int64_t k);
+    static int scan_nsplit(int64_t n, int nprobe, int64_t k, int64_t codes_per_query);
     void coarse_exact_rows(const float *x_dev, const std::vector<int64_t> &rows, int nout, int select_metric,
                            int32_t *out_ids, float *out_dist);
     void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev,

@@ -1185,16 +1185,22 @@ void IvfpqIndex::reset()
     sync_list_tables();
 }
 
-// Workgroups per query of the scan.  Small batches are split over several workgroups per query, about 384
-// workgroups in all and at most eight per query: every workgroup builds the query's whole LUT, so more of
-// them cost more than they balance.  Measured at nlist 16384, nprobe 64: 8 queries 0.31 -> 0.16 ms and 64
-// queries 0.33 -> 0.17 ms against a rule that aimed at 2048 workgroups; from about 400 queries on one
-// workgroup per query is best.
-int IvfpqIndex::scan_nsplit(int64_t n, int nprobe, int64_t k)
+// Workgroups per query of the scan.  Small batches are split over several workgroups per query.  Every workgroup
+// builds the query's whole LUT, so more of them cost more than they balance unless each keeps thousands of codes
+// to scan: up to eight per query and about 384 in all when a query's lists hold few codes (measured at nlist
+// 16384, nprobe 64, 39000 codes per query: 8 queries 0.31 -> 0.16 ms and 64 queries 0.33 -> 0.17 ms against a
+// rule that aimed at 2048 workgroups), up to 64 per query and about 1024 in all while a workgroup keeps 4096
+// codes or more on average (nlist 1024 on 10M vectors, nprobe 32: 312000 codes per query; a single query is
+// bound by the latency of one wave's loads, and 8 workgroups leave 98 % of the GPU idle).  From about 400
+// queries on one workgroup per query is best.  The slices are merged by radix selection, whose cost does not
+// grow with their number.
+int IvfpqIndex::scan_nsplit(int64_t n, int nprobe, int64_t k, int64_t codes_per_query)
 {
-    int nsplit = (int)std::max<int64_t>(1, std::min<int64_t>(8, (384 + n / 2) / n));
-    nsplit = std::min(nsplit, nprobe);
-    return (int)std::min<int64_t>(nsplit, std::max<int64_t>(1, 8192 / pow2_ceil((int)k)));   // one merge pass holds them
+    (void)k;
+    const int64_t cap = std::max<int64_t>(8, std::min<int64_t>(64, codes_per_query / 4096));
+    const int64_t target = cap > 8 ? 1024 : 384;
+    const int64_t nsplit = std::max<int64_t>(1, std::min<int64_t>(cap, (target + n / 2) / n));
+    return (int)std::min<int64_t>(nsplit, nprobe);
 }
 
 // Parameters of the fused LUT + scan + top-k launch for `n` queries and their probe lists.  With `ext` the
@@ -1220,7 +1226,7 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     p.list_len = list_len_dev_.data();
     p.code_layout = layout_;
     p.k = (int)k;
-    const int nsplit = scan_nsplit(n, nprobe, k);
+    const int nsplit = scan_nsplit(n, nprobe, k, nlist_ > 0 ? ntotal_ / nlist_ * nprobe : 0);
     p.nsplit = nsplit;
     if (nsplit > 1) {
         if (ext) {
@@ -1313,7 +1319,7 @@ void IvfpqIndex::search_probes_noalloc(int64_t n, const float *x_dev, const int3
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
     IXA_REQUIRE(nprobe > 0 && nprobe <= nlist_, kErrInvalidParam, "nprobe must be > 0 and <= nlist");
-    const int nsplit = scan_nsplit(n, nprobe, k);
+    const int nsplit = scan_nsplit(n, nprobe, k, nlist_ > 0 ? ntotal_ / nlist_ * nprobe : 0);
     const int64_t hist_bytes = 2 * 1024 * 4, order_bytes = round_up(n * 8, 256),
                   probes_bytes = round_up(n * nprobe * 4, 256), partial_bytes = nsplit > 1 ? n * nsplit * k * 8 : 0;
     const int64_t need = hist_bytes + order_bytes + probes_bytes + partial_bytes;

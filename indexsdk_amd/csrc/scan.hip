@@ -272,6 +272,32 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             build(std::integral_constant<int, 2>{});
         } else if (dsub == 1) {
             build(std::integral_constant<int, 1>{});
+        } else if (dsub % 16 == 0) {
+            // long sub-vectors (128 dimensions in 2, 4 or 8 sub-quantizers): sixteen codeword floats per memory
+            // round trip instead of one, accumulated in the same order
+            for (int m = tid >> 8; m < M; m += NT / 256) {
+                const float *qm = qs + m * dsub;
+                const float4 *cw = reinterpret_cast<const float4 *>(p.codebook + ((int64_t)m * 256 + kk) * dsub);
+                float ip = 0.f, qn = 0.f;
+                for (int t0 = 0; t0 < dsub; t0 += 16) {
+                    float4 c[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        c[u] = cw[(t0 >> 2) + u];
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const float cv[4] = {c[u].x, c[u].y, c[u].z, c[u].w};
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float qv = qm[t0 + 4 * u + j];
+                            ip = __fadd_rn(ip, __fmul_rn(qv, cv[j]));
+                            qn = __fadd_rn(qn, __fmul_rn(qv, qv));
+                        }
+                    }
+                }
+                store_entry(m, ip, qn, l2 ? p.cb_norms[m * 256 + kk] : 0.f);
+            }
         } else {
             for (int m = tid >> 8; m < M; m += NT / 256) {
                 const float *qm = qs + m * dsub;
@@ -568,61 +594,169 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     }
 }
 
-// Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3).
-__global__ __launch_bounds__(256) void ivfpq_merge_kernel(const key_t *__restrict__ partial, int nsplit, int k,
-                                                          int merge_n, int metric, const int64_t *__restrict__ ids,
-                                                          const int32_t *__restrict__ order,
-                                                          float *__restrict__ out_dist,
-                                                          int64_t *__restrict__ out_labels)
+// Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3) by radix selection:
+// the k-th smallest of the nsplit x k keys is found ten key bits at a time, starting below the leading bits that
+// all keys of the query share (a 1024-bin LDS histogram per pass over the keys, which stay in global memory /
+// L2), until the keys at or below the prefix found so far are few; those survivors -- k of them plus the rest
+// of the last histogram bin -- are ranked by counting in LDS (sorted, when there are more than 1024) and the
+// first k written out.  The cost grows with the number of keys, not with keys x slices x log k as a merge that
+// ranks every key in every other slice does (8 slices of 100 keys: 12 us less than that merge; 32 slices of
+// 300 keys: out of its reach), which is what lets a single query be split over more than eight workgroups.
+constexpr int kMergeSelectCap = 4096;
+constexpr int kMergeSelectThreads = 512;
+
+__global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
+    const key_t *__restrict__ partial, int nsplit, int k, int metric, const int64_t *__restrict__ ids,
+    const int32_t *__restrict__ order, float *__restrict__ out_dist, int64_t *__restrict__ out_labels)
 {
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    key_t *lists = reinterpret_cast<key_t *>(smem_raw);   // [nsplit][k], each ascending, empty keys last
-    key_t *merge = lists + merge_n;                        // [k] the result
+    constexpr int NT = kMergeSelectThreads;
+    __shared__ int hist[1024];
+    __shared__ key_t surv[kMergeSelectCap];
+    __shared__ int s_bin, s_below, s_kept;
     const int tid = threadIdx.x;
-    const int64_t q = order ? order[blockIdx.x] : blockIdx.x;   // the scan's own numbering of the queries it served
+    const int64_t q = order ? order[blockIdx.x] : blockIdx.x;
     const int total = nsplit * k;
-    for (int i = tid; i < total; i += 256) {
-        lists[i] = partial[q * total + i];
+    const key_t *src = partial + q * total;
+
+    // the keys of one query share their leading bits (sign, exponent and more): the selection starts below the
+    // common prefix of the smallest and the largest key
+    __shared__ key_t s_min[NT / kWave], s_max[NT / kWave];
+    __shared__ int s_cnt[NT / kWave];
+    key_t mn = kEmptyKey, mx = 0;
+    int nvalid = 0;
+    for (int i = tid; i < total; i += NT) {
+        const key_t key = src[i];
+        if (key != kEmptyKey) {
+            mn = key < mn ? key : mn;
+            mx = key > mx ? key : mx;
+            nvalid++;
+        }
     }
-    for (int i = tid; i < k; i += 256) {
-        merge[i] = kEmptyKey;
+    for (int o = 32; o > 0; o >>= 1) {
+        const key_t omn = __shfl_xor(mn, o), omx = __shfl_xor(mx, o);
+        mn = omn < mn ? omn : mn;
+        mx = omx > mx ? omx : mx;
+        nvalid += __shfl_xor(nvalid, o);
     }
-    __syncthreads();
-    // Every key finds its own rank in the union: its position in its list plus, for every other list,
-    // the number of keys below it (binary search; no barriers, where a sort of the union takes dozens).
-    // Equal keys (one list probed twice) are ordered by split so that ranks stay distinct.
-    for (int e = tid; e < total; e += 256) {
-        const int sp = e / k, pos = e - sp * k;
-        const key_t mine = lists[e];
-        if (mine == kEmptyKey) {
-            continue;
-        }
-        int rank = pos;
-        for (int o = 0; o < nsplit && rank < k; o++) {
-            if (o == sp) {
-                continue;
-            }
-            const key_t *other = lists + o * k;
-            int lo = 0, hi = k;   // first index whose key is not below `mine` (o > sp) / above it (o < sp)
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                const key_t v = other[mid];
-                const bool below = o < sp ? v <= mine : v < mine;
-                lo = below ? mid + 1 : lo;
-                hi = below ? hi : mid;
-            }
-            rank += lo;
-        }
-        if (rank < k) {
-            merge[rank] = mine;
-        }
+    if ((tid & (kWave - 1)) == 0) {
+        s_min[tid / kWave] = mn;
+        s_max[tid / kWave] = mx;
+        s_cnt[tid / kWave] = nvalid;
     }
     __syncthreads();
-    for (int i = tid; i < k; i += 256) {
-        const key_t kk = merge[i];
+    nvalid = 0;
+    for (int w = 0; w < NT / kWave; w++) {
+        mn = s_min[w] < mn ? s_min[w] : mn;
+        mx = s_max[w] > mx ? s_max[w] : mx;
+        nvalid += s_cnt[w];
+    }
+
+    bool all = nvalid <= k;   // no more keys than asked for: every one of them survives
+    int shift = (all || mn == mx) ? 0 : 64 - __clzll((long long)(mn ^ mx));   // the keys differ below this bit
+    key_t prefix = shift >= 64 ? 0 : mn >> shift;   // the bits above `shift` of the k-th smallest key
+    int need = k;                                    // rank of that key among the keys that share the prefix
+    while (!all && shift > 0) {
+        const int bits = shift >= 10 ? 10 : shift;
+        const int upper = shift;   // keys are compared with `prefix` above this bit
+        shift -= bits;
+        for (int i = tid; i < 1024; i += NT) {
+            hist[i] = 0;
+        }
+        __syncthreads();
+        for (int i = tid; i < total; i += NT) {
+            const key_t key = src[i];
+            if (key != kEmptyKey && (upper == 64 || (key >> upper) == prefix)) {
+                atomicAdd(&hist[(uint32_t)(key >> shift) & ((1u << bits) - 1u)], 1);
+            }
+        }
+        __syncthreads();
+        if (tid < kWave) {
+            // first bin whose inclusive count reaches `need`: 16 bins per lane, a wave scan over the lanes
+            int part = 0;
+            for (int j = 0; j < 16; j++) {
+                part += hist[tid * 16 + j];
+            }
+            int incl = part;
+#pragma unroll
+            for (int o = 1; o < kWave; o <<= 1) {
+                const int up = __shfl_up(incl, o);
+                if (tid >= o) {
+                    incl += up;
+                }
+            }
+            const unsigned long long reach = __ballot(incl >= need);   // never empty: nvalid > k >= need
+            const int owner = reach ? __ffsll((long long)reach) - 1 : kWave - 1;
+            if (tid == owner) {
+                int below = incl - part, bin = tid * 16;
+                while (bin < tid * 16 + 15 && below + hist[bin] < need) {
+                    below += hist[bin];
+                    bin++;
+                }
+                s_bin = bin;
+                s_below = below;
+                s_kept = hist[bin];
+            }
+        }
+        __syncthreads();
+        prefix = (prefix << bits) | (key_t)(uint32_t)s_bin;
+        need -= s_below;
+        const int survivors = (k - need) + s_kept;   // keys below the prefix class + the class itself
+        __syncthreads();
+        // few enough to rank by counting (a pass costs about what counting 300 survivors does)
+        if (survivors <= kMergeSelectCap && (survivors <= k + 64 || survivors <= 320)) {
+            break;
+        }
+    }
+    if (tid == 0) {
+        s_kept = 0;
+    }
+    __syncthreads();
+    for (int i = tid; i < total; i += NT) {
+        const key_t key = src[i];
+        const bool keep = key != kEmptyKey && (all || shift >= 64 || (key >> shift) <= prefix);
+        if (keep) {
+            const int at = atomicAdd(&s_kept, 1);
+            if (at < kMergeSelectCap) {
+                surv[at] = key;
+            }
+        }
+    }
+    __syncthreads();
+    const int kept = s_kept < kMergeSelectCap ? s_kept : kMergeSelectCap;
+    const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
+    if (kept <= 1024) {
+        // rank by counting: every thread reads the same survivor at a time (an LDS broadcast)
+        for (int e = tid; e < kept; e += NT) {
+            const key_t mine = surv[e];
+            int rank = 0;
+            for (int j = 0; j < kept; j++) {
+                const key_t v = surv[j];
+                rank += (v < mine || (v == mine && j < e)) ? 1 : 0;
+            }
+            if (rank < k) {
+                const float v = key_score(mine);
+                out_dist[q * k + rank] = metric == kMetricL2 ? v : -v;
+                out_labels[q * k + rank] = ids[key_index(mine)];
+            }
+        }
+        for (int i = kept + tid; i < k; i += NT) {
+            out_dist[q * k + i] = pad;
+            out_labels[q * k + i] = -1;
+        }
+        return;
+    }
+    int n2 = 2048;
+    while (n2 < kept) {
+        n2 <<= 1;
+    }
+    for (int i = kept + tid; i < n2; i += NT) {
+        surv[i] = kEmptyKey;
+    }
+    block_bitonic_sort(surv, n2, tid, NT);
+    for (int i = tid; i < k; i += NT) {
+        const key_t kk = i < kept ? surv[i] : kEmptyKey;
         const bool ok = kk != kEmptyKey;
         const float v = key_score(kk);
-        const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
         out_dist[q * k + i] = ok ? (metric == kMetricL2 ? v : -v) : pad;
         out_labels[q * k + i] = ok ? ids[key_index(kk)] : -1;
     }
@@ -985,16 +1119,10 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
     } else {
         dispatch_m<float>(p, nq, smem, s);
     }
+    IXA_REQUIRE(p.nsplit == 1 || p.partial != nullptr, kErrInner, "a split scan needs a buffer for its partial lists");
     if (p.nsplit > 1) {
-        const int merge_n = p.nsplit * p.k;
-        const size_t msmem = (size_t)(merge_n + p.k) * sizeof(key_t);
-        IXA_REQUIRE(msmem <= 160 * 1024, kErrInner, "merge of %d x %d candidates exceeds LDS", p.nsplit, p.k);
-        if (msmem > 48 * 1024) {
-            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(ivfpq_merge_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem));
-        }
-        hipLaunchKernelGGL(ivfpq_merge_kernel, dim3((unsigned)nq), dim3(256), msmem, s, p.partial, p.nsplit, p.k,
-                           merge_n, p.metric, p.ids, p.order, p.out_dist, p.out_labels);
+        hipLaunchKernelGGL(ivfpq_merge_kernel, dim3((unsigned)nq), dim3(kMergeSelectThreads), 0, s, p.partial,
+                           p.nsplit, p.k, p.metric, p.ids, p.order, p.out_dist, p.out_labels);
     }
 }
 

@@ -65,6 +65,12 @@ __device__ __forceinline__ float wave_uniform(float v)
     return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(v)));
 }
 __device__ __forceinline__ int32_t wave_uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ key_t wave_uniform_key(key_t v)
+{
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return ((key_t)hi << 32) | lo;
+}
 
 template <typename S>
 __device__ __forceinline__ key_t make_key(S score, uint32_t idx)
@@ -136,6 +142,10 @@ struct WavePool {
     int k;
     int count;    // wave-uniform
     S bound;      // wave-uniform: a candidate enters iff score <= bound
+    // Wave-uniform; set once so many candidates TIE at the k-th score that a bound on scores alone keeps
+    // admitting them (coarse quantizers give whole lists one code): from then on a candidate must also be
+    // below this key, the k-th smallest (score, index) seen, so ties are decided by index as in the result.
+    key_t bound_key;
 
     __device__ __forceinline__ void init(key_t *b, int cap_, int k_)
     {
@@ -144,6 +154,7 @@ struct WavePool {
         k = k_;
         count = 0;
         bound = ScoreOps<S>::worst();
+        bound_key = kEmptyKey;
     }
 
     // Smallest kSelectBits-bit prefix P such that at least `rank` pool entries have a score prefix
@@ -236,8 +247,10 @@ struct WavePool {
             }
             wave_bitonic_sort(buf, cap, lane);
             count = k;
-            const S b = wave_uniform(key_score_as<S>(buf[k - 1]));
+            const key_t kth = wave_uniform_key(buf[k - 1]);
+            const S b = key_score_as<S>(kth);
             bound = b < bound ? b : bound;
+            bound_key = kth;   // keys are distinct: a later key that belongs to the k best is below this one
         }
     }
 
@@ -259,6 +272,13 @@ struct WavePool {
         unsigned long long mask = __ballot(pass);
         if (mask == 0) {
             return false;
+        }
+        if (bound_key != kEmptyKey) {
+            pass = pass && make_key(score, idx) < bound_key;
+            mask = __ballot(pass);
+            if (mask == 0) {
+                return false;
+            }
         }
         int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
         if (pass) {
@@ -346,6 +366,7 @@ struct BlockPoolCtl {
     int bin;        // histogram search result
     int below;      // candidates in bins before `bin`
     float bound;
+    key_t bound_key;   // kEmptyKey, or the k-th smallest key once ties at the k-th score overflowed the pool
 };
 
 template <int W>
@@ -357,6 +378,7 @@ struct BlockPool {
     volatile BlockPoolCtl *ctl;
     int cap, k;
     float bound;               // wave-uniform copy of ctl->bound
+    key_t bound_key;           // wave-uniform copy of ctl->bound_key
 
     // All threads call; a __syncthreads() must follow before the first push.
     __device__ __forceinline__ void init(key_t *b, int cap_, int k_, int *hist_, BlockPoolCtl *c, int tid)
@@ -367,7 +389,9 @@ struct BlockPool {
         hist = hist_;
         ctl = c;
         bound = __builtin_inff();
+        bound_key = kEmptyKey;
         if (tid == 0) {
+            c->bound_key = kEmptyKey;
             c->count = 0;
             c->valid_end = cap_;
             c->flag = 0;
@@ -383,9 +407,16 @@ struct BlockPool {
     // candidates against the new bound and try again.
     __device__ __forceinline__ bool try_push(bool pass, float score, uint32_t idx, int lane)
     {
-        const unsigned long long mask = __ballot(pass);
+        unsigned long long mask = __ballot(pass);
         if (mask == 0) {
             return true;
+        }
+        if (bound_key != kEmptyKey) {
+            pass = pass && make_key(score, idx) < bound_key;
+            mask = __ballot(pass);
+            if (mask == 0) {
+                return true;
+            }
         }
         const int n = __popcll(mask);
         const int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
@@ -533,6 +564,9 @@ struct BlockPool {
             block_bitonic_sort(buf, cap, tid, NT);
             kept = k;
             top = key_score(buf[k - 1]);
+            if (tid == 0) {
+                ctl->bound_key = buf[k - 1];
+            }
         }
         __syncthreads();
         if (tid == 0) {
@@ -555,6 +589,7 @@ struct BlockPool {
             prune(tid);
         }
         bound = wave_uniform(ctl->bound);
+        bound_key = wave_uniform_key(ctl->bound_key);
         return d == W;
     }
 

@@ -427,6 +427,70 @@ def test_large_k_shared_pool_all_scores_tie(ix, oracle):
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
 
 
+@pytest.mark.parametrize("k", [300, 1024])
+def test_whole_lists_tie_and_the_answer_does_not_depend_on_the_plan(ix, oracle, k):
+    """Four sub-quantizers over clustered data: every vector of a cluster gets the same code, so whole lists of
+    thousands of vectors share one distance (the shape of the reference's own latency targets: nlist 1024, M 4,
+    k 300).  Ties are decided by position in the index, so the answer is the same whether a query is served by
+    one workgroup (a batch of 600) or split over eight (a batch of one), with private pools (k = 300) or the
+    shared pool (k = 1024)."""
+    rng = np.random.default_rng(4)
+    d, M, nlist, n = 128, 4, 32, 120_000
+    centres = rng.standard_normal((nlist, d)).astype(np.float32)
+    x = (centres[rng.integers(0, nlist, n)] + 0.05 * rng.standard_normal((n, d))).astype(np.float32)
+    q = (centres[rng.integers(0, nlist, 600)] + 0.05 * rng.standard_normal((600, d))).astype(np.float32)
+    cb = oracle.train_pq(centres + 0.01, M, niter=1, seed=3) if nlist >= 256 else None
+    if cb is None:
+        # 256 codewords per sub-quantizer with only 32 clusters: the cluster centres' blocks plus far-away filler
+        cb = (10.0 + rng.standard_normal((M, 256, d // M))).astype(np.float32)
+        cb[:, :nlist, :] = centres.reshape(nlist, M, d // M).transpose(1, 0, 2)
+    ids = np.arange(n, dtype=np.int64)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(centres, cb)
+    gpu.add_with_ids(x, ids)
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, centres, cb, x, ids)
+    codes0, _ = gpu.getListCodesAndIds(0)
+    assert len(np.unique(codes0, axis=0)) <= 4, "the lists of this test should hold (almost) one code each"
+    gpu.setNumProbes(8)
+    D, I = gpu.search(q, k)
+    assert gpu.last_search_stats()["shared_pool"] == (1 if k > 320 else 0)
+    Dr, Ir = ref.search(q, k, 8)
+    assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
+    for j in (0, 7, 311):
+        D1, I1 = gpu.search(q[j:j + 1], k)
+        assert gpu.last_search_stats()["nsplit"] > 1
+        assert np.array_equal(I1[0], I[j]) and np.array_equal(D1[0].view(np.uint32), D[j].view(np.uint32))
+
+
+@pytest.mark.parametrize("metric_name,k", [("L2", 50), ("L2", 300), ("IP", 300), ("L2", 2048)])
+def test_one_query_split_over_many_workgroups(ix, oracle, metric_name, k):
+    """Long lists (25000 codes each): a small batch is split over sixteen workgroups per query, one per probed
+    list, and the slices are merged by radix selection -- a handful of survivors ranked by counting (k = 50,
+    300), thousands sorted (k = 2048).  The answer is the oracle's, and the one a large batch (one workgroup per
+    query, no merge) gives for the same queries, bit for bit."""
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 17, 400_000, 1500, 32, 16, 8, metric, niter=3)
+    gpu.setNumProbes(16)
+    D, I = gpu.search(q, k)
+    assert gpu.last_search_stats()["nsplit"] == 1
+    D3, I3 = gpu.search(q[:3], k)
+    assert gpu.last_search_stats()["nsplit"] == 16
+    assert np.array_equal(I3, I[:3]) and np.array_equal(D3.view(np.uint32), D[:3].view(np.uint32))
+    D40, I40 = gpu.search(q[100:140], k)
+    assert 8 < gpu.last_search_stats()["nsplit"] <= 16
+    assert np.array_equal(I40, I[100:140]) and np.array_equal(D40.view(np.uint32), D[100:140].view(np.uint32))
+    Dr, Ir = ref.search(q[:3], k, 16)
+    assert_topk_parity(oracle, ref, q[:3], D3, I3, Dr, Ir, TOL_FP32)
+    # fewer vectors than k in the probed lists: padding comes out of the merge
+    gpu.setNumProbes(1)
+    small = ix.AscendIndexIVFPQ(32, metric, 16, 8, 8, ix.AscendIndexIVFPQConfig())
+    small.set_trained(ref.cent, ref.codebook)
+    small.add_with_ids(x[:40], ids[:40])
+    small.setNumProbes(16)
+    Ds, Is = small.search(q[:2], k)
+    assert ((Is >= 0).sum(axis=1) == 40).all() and (Is[:, 40:] == -1).all()
+
+
 @pytest.mark.parametrize("metric_name", ["L2", "IP"])
 def test_search_with_tied_and_nearly_tied_centroids(ix, oracle, metric_name):
     """Half of the centroids are exact or 1e-6-perturbed copies of the other half, so the approximate
@@ -561,9 +625,9 @@ def test_pq_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, d, M):
 def test_few_heavy_workgroups_run_heaviest_first(ix, oracle):
     """Long lists, few queries: the scan orders its queries by decreasing work (a scheduling matter only:
     results are those of the oracle, whatever the order)."""
-    gpu, ref, x, q, ids = build_pair(ix, oracle, 81, 200000, 600, 32, 16, 8, ix.METRIC_L2, niter=3)
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 81, 200000, 1400, 32, 16, 8, ix.METRIC_L2, niter=3)
     gpu.setNumProbes(8)
-    for nq, split in ((600, False), (150, True)):      # one workgroup per query, and several
+    for nq, split in ((1400, False), (300, True)):     # one workgroup per query, and three
         D, I = gpu.search(q[:nq], 20)
         st = gpu.last_search_stats()
         assert st["ordered"] == 1 and (st["nsplit"] > 1) == split
