@@ -445,13 +445,14 @@ def main():
         Dr, Ir = ref.search(qh[:probe_n], k, nprobe, lut_fp16=lut16)
         t_probe = time.perf_counter() - t0
         sample = int(min(nq, max(probe_n, args.cpu_seconds / max(t_probe / probe_n, 1e-9))))
-        # repeat the sample until about cpu_seconds of CPU work have been timed; report the best pass
-        passes = int(max(1, min(20, args.cpu_seconds / max(t_probe / probe_n * sample, 1e-9))))
+        # repeat the sample until about cpu_seconds of CPU work have been timed (the probe above ran cold and
+        # overestimates a pass, so the clock decides, not a count fixed in advance); report the median pass
         times = []
-        for _ in range(passes):
+        while sum(times) < args.cpu_seconds and len(times) < 200:
             t0 = time.perf_counter()
             Dr, Ir = ref.search(qh[:sample], k, nprobe, lut_fp16=lut16)
             times.append(time.perf_counter() - t0)
+        passes = len(times)
         t_cpu = float(np.median(times))
         cpu_qps = sample / t_cpu
         Ih, Dh = I[:sample].cpu().numpy(), D[:sample].cpu().numpy()

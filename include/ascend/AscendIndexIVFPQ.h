@@ -28,6 +28,8 @@ struct AscendIndexIVFPQConfig : public AscendIndexIVFConfig {
     bool enableQueryParallelSearch = false;  // no counterpart on one GPU
     // additions of this build
     bool lutFp16 = false;                // per-query LUT stored as IEEE half (distances within 1e-2)
+    bool pqSpherical = false;            // sub-quantizer codewords L2-normalised after every update, as the reference's
+                                         // host training (useKmeansPP = false) does; its device training does not
     bool strictReferenceParams = false;  // true: enforce the reference's whitelists (dims 128, nlist 1024..16384 /
                                          // 262144 / 524288, msubs 2..32) with its "Unsupported ..." messages
 };
@@ -221,6 +223,7 @@ protected:
         c.train_samples_per_list = ivfPQConfig.trainSamplesPerList;
         c.max_train_samples = ivfPQConfig.maxTrainSamples;
         c.lut_fp16 = ivfPQConfig.lutFp16 ? 1 : 0;
+        c.pq_spherical = ivfPQConfig.pqSpherical ? 1 : 0;
         c.strict_reference_params = ivfPQConfig.strictReferenceParams ? 1 : 0;
         if (ivfPQConfig.resourceSize > c.scratch_bytes) {
             c.scratch_bytes = ivfPQConfig.resourceSize;

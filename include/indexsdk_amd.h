@@ -120,8 +120,7 @@ typedef struct ivfpq_config {
                                        update, 0 = plain Lloyd, -1 (default) = normalised for inner product only.  The
                                        reference forces it for inner product and, in its CPU mode, for L2 as well
                                        (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1159-1171), which suits unit-norm data
-                                       only.  Sub-quantizer codebooks are never normalised here (the reference's CPU
-                                       mode does, :1064-1067).  useKmeansPP of the reference's config selects WHERE it
+                                       only.  Sub-quantizer codebooks: see pq_spherical.  useKmeansPP of the reference's config selects WHERE it
                                        trains (its NPU k-means or faiss on the host); this build always trains on the
                                        device, seeded with random samples, whatever that flag says. */
     int32_t train_samples_per_list; /* trainSamplesPerList */
@@ -145,6 +144,10 @@ typedef struct ivfpq_config {
                                        and every query's candidate list is proven complete by count, so that no
                                        query x centroid score matrix is written; 0 = the score matrix of a query
                                        block is written and selected from */
+    int32_t pq_spherical;           /* 1 = sub-quantizer codewords L2-normalised after every update, as the
+                                       reference's host training does (faiss Clustering with cp.spherical = true,
+                                       FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1064-1067); 0 (default) = plain Lloyd,
+                                       as its device training */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */

@@ -32,6 +32,7 @@ class IvfpqConfig(ctypes.Structure):
         ("coarse_fp32_only", ctypes.c_int32),
         ("scan_locality", ctypes.c_int32),
         ("coarse_sampled_bound", ctypes.c_int32),
+        ("pq_spherical", ctypes.c_int32),
     ]
 
 

@@ -98,6 +98,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.coarse_bf16 = cfg->coarse_fp32_only ? 0 : 1;
         c.scan_locality = cfg->scan_locality;
         c.coarse_sampled_bound = cfg->coarse_sampled_bound;
+        c.pq_spherical = cfg->pq_spherical ? 1 : 0;
     }
     return c;
 }
@@ -131,6 +132,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->coarse_fp32_only = d.coarse_bf16 ? 0 : 1;
     cfg->scan_locality = d.scan_locality;
     cfg->coarse_sampled_bound = d.coarse_sampled_bound;
+    cfg->pq_spherical = d.pq_spherical;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,

@@ -17,6 +17,9 @@ struct IvfpqConfig {
     int spherical = -1;               // coarse centroids L2-normalised after every update: 1 yes, 0 no, -1 = for inner
                                       // product only (the reference forces it there, AscendIndexIVFPQImpl.cpp:1159-1163;
                                       // its CPU mode also does it for L2, which suits unit-norm data only)
+    int pq_spherical = 0;             // 1 = sub-quantizer codewords L2-normalised after every update, as the reference's
+                                      // host training does (AscendIndexIVFPQImpl.cpp:1064-1067; its device training does
+                                      // not): only sensible when every sub-vector has unit norm
     int train_samples_per_list = 256; // rows sampled per coarse centroid (trainSamplesPerList)
     int64_t max_train_samples = 10000000;  // maxTrainSamples
     int lut_fp16 = 0;                 // LUT entries stored as IEEE half
@@ -132,11 +135,10 @@ private:
     int64_t remove_sorted_ids(const std::vector<int64_t> &gone, std::vector<uint8_t> *found);
     void relayout(const std::vector<int32_t> &cap, int64_t min_slots);
     void sync_list_tables();
-    void kmeans_coarse(const std::vector<float> &sample, int64_t ns);
-    void kmeans_pq(const std::vector<float> &sample, int64_t ns);
+    void kmeans_coarse(const float *sample_dev, int64_t ns);
+    void kmeans_pq(const float *sample_dev, int64_t ns);
 
     int d_, M_, dsub_, metric_;
-    int nbits_;  // always 8 (256 codewords per sub-quantizer)
     int64_t nlist_;
     IvfpqConfig cfg_;
     int layout_ = 0;

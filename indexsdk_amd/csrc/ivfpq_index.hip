@@ -396,7 +396,7 @@ inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
 // -------------------------------------------------------------------------------------------------
 
 IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const IvfpqConfig &cfg)
-    : d_(d), M_(M), dsub_(0), metric_(metric), nbits_(nbits), nlist_(nlist), cfg_(cfg)
+    : d_(d), M_(M), dsub_(0), metric_(metric), nlist_(nlist), cfg_(cfg)
 {
     // Messages keep the reference's wording (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:510-525) so that
     // its unit tests' substring checks (FR/ut/TestAscendIndexUTIVFPQ.cpp:77-184) carry over.
@@ -1511,7 +1511,6 @@ void IvfpqIndex::train(int64_t n, const float *x, bool on_device)
                 (long)n);
     int64_t ns = std::min<int64_t>({(int64_t)nlist_ * cfg_.train_samples_per_list, n, cfg_.max_train_samples});
     ns = std::max<int64_t>(ns, std::min<int64_t>(n, std::max<int64_t>(nlist_, 256 * 40)));
-    std::vector<float> sample((size_t)ns * d_);
     std::vector<int64_t> idx((size_t)n);
     std::iota(idx.begin(), idx.end(), 0);
     if (ns < n) {
@@ -1519,20 +1518,25 @@ void IvfpqIndex::train(int64_t n, const float *x, bool on_device)
         std::shuffle(idx.begin(), idx.end(), gen);
         idx.resize((size_t)ns);
     }
+    // the sample lives in device memory from here on: rows of a device-resident training set are gathered on
+    // the device and never visit the host; a host training set is sampled on the host and uploaded once
+    DeviceBuffer<float> sample_dev((size_t)ns * d_);
     if (on_device) {
         DeviceBuffer<int64_t> idx_dev;
-        DeviceBuffer<float> out((size_t)ns * d_);
         idx_dev.upload(idx.data(), (size_t)ns, stream_);
         hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for(ns * d_)), dim3(256), 0, stream_, x, idx_dev.data(), ns,
-                           d_, out.data());
-        out.download(sample.data(), sample.size(), stream_);
+                           d_, sample_dev.data());
+        sync_stream(stream_);   // idx_dev is freed on leaving this block
     } else {
+        std::vector<float> sample((size_t)ns * d_);
         for (int64_t i = 0; i < ns; i++) {
             std::memcpy(&sample[(size_t)i * d_], x + idx[(size_t)i] * d_, sizeof(float) * (size_t)d_);
         }
+        sample_dev.upload(sample.data(), sample.size(), stream_);
+        sync_stream(stream_);   // the host copy is freed on leaving this block
     }
-    kmeans_coarse(sample, ns);
-    kmeans_pq(sample, ns);
+    kmeans_coarse(sample_dev.data(), ns);
+    kmeans_pq(sample_dev.data(), ns);
     trained_ = true;
 }
 
@@ -1575,18 +1579,26 @@ void normalise_rows(std::vector<float> &cent, int64_t k, int dim)
 
 }  // namespace
 
-void IvfpqIndex::kmeans_coarse(const std::vector<float> &sample, int64_t ns)
+void IvfpqIndex::kmeans_coarse(const float *sample_dev, int64_t ns)
 {
     std::vector<int64_t> pick((size_t)ns);
     std::iota(pick.begin(), pick.end(), 0);
     std::mt19937_64 gen(cfg_.seed + 1);
     std::shuffle(pick.begin(), pick.end(), gen);
+    // the first centroids are sample rows: gathered on the device, only nlist rows come to the host
     std::vector<float> cent((size_t)nlist_ * d_);
-    for (int64_t c = 0; c < nlist_; c++) {
-        std::memcpy(&cent[(size_t)c * d_], &sample[(size_t)pick[(size_t)c] * d_], sizeof(float) * (size_t)d_);
+    {
+        DeviceBuffer<int64_t> pick_dev;
+        DeviceBuffer<float> rows((size_t)nlist_ * d_);
+        pick_dev.upload(pick.data(), (size_t)nlist_, stream_);
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for(nlist_ * d_)), dim3(256), 0, stream_, sample_dev,
+                           pick_dev.data(), nlist_, d_, rows.data());
+        rows.download(cent.data(), cent.size(), stream_);
     }
-    DeviceBuffer<float> xs;
-    xs.upload(sample.data(), sample.size(), stream_);
+    struct {
+        const float *p;
+        const float *data() const { return p; }
+    } xs{sample_dev};
     DeviceBuffer<int32_t> asg((size_t)ns);
     std::vector<int32_t> h_asg((size_t)ns);
     std::vector<int64_t> cnt((size_t)nlist_), seg((size_t)nlist_ + 1), order((size_t)ns);
@@ -1623,22 +1635,42 @@ void IvfpqIndex::kmeans_coarse(const std::vector<float> &sample, int64_t ns)
     upload_trained(cent.data(), nullptr);
 }
 
-void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
+void IvfpqIndex::kmeans_pq(const float *sample_dev, int64_t ns)
 {
     const int niter = cfg_.pq_niter >= 0 ? cfg_.pq_niter : cfg_.niter;
+    // the first codewords of sub-quantizer m are the m-th sub-vectors of 256 sample rows: those rows are gathered
+    // on the device (M x 256 rows come to the host, not the sample)
     std::vector<float> cb((size_t)M_ * 256 * dsub_);
     std::mt19937_64 gen(cfg_.seed + 2);
-    for (int m = 0; m < M_; m++) {
-        std::vector<int64_t> pick((size_t)ns);
-        std::iota(pick.begin(), pick.end(), 0);
-        std::shuffle(pick.begin(), pick.end(), gen);
-        for (int k = 0; k < 256; k++) {
-            std::memcpy(&cb[((size_t)m * 256 + k) * dsub_], &sample[(size_t)pick[(size_t)(k % ns)] * d_ + m * dsub_],
-                        sizeof(float) * (size_t)dsub_);
+    {
+        std::vector<int64_t> rows_of((size_t)M_ * 256);
+        for (int m = 0; m < M_; m++) {
+            std::vector<int64_t> pick((size_t)ns);
+            std::iota(pick.begin(), pick.end(), 0);
+            std::shuffle(pick.begin(), pick.end(), gen);
+            for (int k = 0; k < 256; k++) {
+                rows_of[(size_t)m * 256 + k] = pick[(size_t)(k % ns)];
+            }
+        }
+        DeviceBuffer<int64_t> rows_dev;
+        DeviceBuffer<float> picked((size_t)M_ * 256 * d_);
+        std::vector<float> h_picked((size_t)M_ * 256 * d_);
+        rows_dev.upload(rows_of.data(), rows_of.size(), stream_);
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for((int64_t)M_ * 256 * d_)), dim3(256), 0, stream_,
+                           sample_dev, rows_dev.data(), (int64_t)M_ * 256, d_, picked.data());
+        picked.download(h_picked.data(), h_picked.size(), stream_);
+        for (int m = 0; m < M_; m++) {
+            for (int k = 0; k < 256; k++) {
+                std::memcpy(&cb[((size_t)m * 256 + k) * dsub_], &h_picked[((size_t)m * 256 + k) * d_ + m * dsub_],
+                            sizeof(float) * (size_t)dsub_);
+            }
         }
     }
-    DeviceBuffer<float> xs;
-    xs.upload(sample.data(), sample.size(), stream_);
+    struct {
+        const float *p;
+        const float *data() const { return p; }
+    } xs{sample_dev};
+    std::vector<float> sample;   // host copy of the sample: only the host update of long sub-vectors needs it
     DeviceBuffer<uint8_t> codes((size_t)ns * M_);
     std::vector<uint8_t> h_codes((size_t)ns * M_);
     std::vector<double> acc((size_t)M_ * 256 * dsub_);
@@ -1655,6 +1687,12 @@ void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
             acc_dev.download(acc.data(), acc.size(), stream_);
             cnt_dev.download(reinterpret_cast<long long *>(cnt.data()), cnt.size(), stream_);
         } else {
+            if (sample.empty()) {
+                sample.resize((size_t)ns * d_);
+                IXA_HIP(hipMemcpyAsync(sample.data(), sample_dev, sample.size() * sizeof(float), hipMemcpyDeviceToHost,
+                                       stream_));
+                sync_stream(stream_);
+            }
             codes.download(h_codes.data(), h_codes.size(), stream_);
             std::fill(acc.begin(), acc.end(), 0.0);
             std::fill(cnt.begin(), cnt.end(), 0);
@@ -1680,8 +1718,12 @@ void IvfpqIndex::kmeans_pq(const std::vector<float> &sample, int64_t ns)
                 }
             }
             split_empty(sub, sc, 256, dsub_);
-            // cfg_.spherical is NOT applied to the sub-quantizers: the reference does normalise them
-            // (AscendIndexIVFPQImpl.cpp:1064-1067), which only makes sense for unit-norm sub-vectors
+            // cfg_.spherical (the coarse quantizer's flag) is not applied here; the reference's HOST training
+            // normalises the sub-quantizers as well (AscendIndexIVFPQImpl.cpp:1064-1067), its device training does
+            // not: pq_spherical asks for the former
+            if (cfg_.pq_spherical) {
+                normalise_rows(sub, 256, dsub_);
+            }
             std::copy(sub.begin(), sub.end(), cb.begin() + (size_t)m * 256 * dsub_);
         }
     }

@@ -430,7 +430,7 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
                 } else {
                     off = ((code << 6) + r4) + (uint32_t)((NB >> 1) * 32768);
                 }
-                const uint32_t raw = *(lds_half_t *)off;
+                const uint32_t raw = *(lds_half_t *)(size_t)off;
                 asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel_hi:[1,0,0]" : "+v"(acc[m & 3]) : "v"(raw));
             }
             return (acc[0] + acc[1]) + (acc[2] + acc[3]);

@@ -622,6 +622,36 @@ def test_pq_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, d, M):
     assert checked > 100
 
 
+def test_training_from_device_memory_equals_training_from_host_memory_and_pq_spherical(ix, oracle):
+    """A training set in device memory is sampled on the device and never visits the host; the quantizers are the
+    ones the host call produces from the same rows, bit for bit (same sample, same seeds, same arithmetic).
+    pq_spherical normalises the sub-quantizer codewords after every update (the reference's host training,
+    AscendIndexIVFPQImpl.cpp:1064-1067)."""
+    import ctypes
+    import torch
+    from indexsdk_amd import _capi
+    lib = _capi.load()
+    rng = np.random.default_rng(12)
+    d, M, nlist = 64, 8, 32
+    x = (rng.standard_normal((20000, d)) + 3.0 * rng.standard_normal((1, d))).astype(np.float32)
+    kw = dict(niter=3, train_samples_per_list=200)       # 6400 of the 20000 rows are sampled
+    a = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(**kw))
+    a.train(x)
+    b = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(**kw))
+    xd = torch.from_numpy(x).cuda()
+    torch.cuda.synchronize()
+    _capi.check(lib.ivfpq_train_device(b._h, len(x), ctypes.c_void_p(xd.data_ptr())))
+    (ca, ba), (cb, bb) = a.get_trained(), b.get_trained()
+    assert np.array_equal(ca.view(np.uint32), cb.view(np.uint32))
+    assert np.array_equal(ba.view(np.uint32), bb.view(np.uint32))
+    assert not np.allclose(np.linalg.norm(ba, axis=2), 1.0, atol=1e-3)
+    s = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(pq_spherical=1, **kw))
+    s.train(x)
+    cs, bs = s.get_trained()
+    assert np.array_equal(cs.view(np.uint32), ca.view(np.uint32))          # the coarse quantizer is not affected
+    assert np.allclose(np.linalg.norm(bs, axis=2), 1.0, atol=1e-5)
+
+
 def test_few_heavy_workgroups_run_heaviest_first(ix, oracle):
     """Long lists, few queries: the scan orders its queries by decreasing work (a scheduling matter only:
     results are those of the oracle, whatever the order)."""
