@@ -104,6 +104,27 @@ int ixa_op_topk_flat_fp32(const float *dists_dev, int64_t batch, int64_t n, int6
 int ixa_op_ivfpq_subspace_distance(const float *queries_dev, int64_t batch, int d, const float *codebook_dev,
                                    int msubs, int metric, float *lut_dev, void *stream);
 
+/* Operator "AscendcIvfpqSearchDistanceL2" (descriptor FR/ascenddaemon/impl/IndexIVFPQ.cpp:1706-1755, kernel
+ * FR/ops/ascendc/op_kernel/ascendc_ivfpq_search_distance_topk.h:39-93, 556-810) with the reference's operands:
+ * queryPQ = lut [batch][msubs][256] (what ixa_op_ivfpq_subspace_distance wrote); codeBase + codeOffset
+ * [batch][nblocks] (byte offsets of the code blocks a query scans) + codeSize [batch][nblocks] (valid codes of
+ * each, 0 = skip; at most 262144, the reference's block size); labelBase + labelOffset [batch][nblocks]
+ * (element offsets of the blocks' ids).  Codes are row-major, msubs bytes each.  Outputs = the operator's
+ * topkIndexFinal / topkValueFinal: the k best (label, distance) per query, best first, padded with -1 and
+ * FLT_MAX (-FLT_MAX for IXA_METRIC_INNER_PRODUCT, where lut holds inner products and larger is better).  The
+ * operator's per-block intermediates (distResult, topkIndex, topkValue, flag) stay inside the launch.
+ * k <= 384 (the reference: 320), nblocks <= 2048. */
+int ixa_op_ivfpq_search_distance_topk(const float *lut_dev, int64_t batch, int msubs, const uint8_t *code_base_dev,
+                                      const int64_t *code_offset_dev, const int64_t *code_size_dev, int nblocks, int k,
+                                      const int64_t *label_base_dev, const int64_t *label_offset_dev, int metric,
+                                      float *topk_values_dev, int64_t *topk_labels_dev, void *stream);
+/* Operator "TopkIvfpqL3" (descriptor FR/ascenddaemon/impl/IndexIVFPQ.cpp:1844-1877, kernel
+ * FR/ops/cpukernel/impl/topk_ivfpq_l3_cpu_kernel.cpp:176-250): merges the best-first lists of `tiles` launches
+ * of the operator above, in_labels / in_values [tiles][batch][list_k] (label -1 = padding), into the k best per
+ * query.  asc = 1: smaller is better (L2); 0: larger is better.  tiles x list_k <= 16384. */
+int ixa_op_topk_ivfpq_l3(const int64_t *in_labels_dev, const float *in_values_dev, int tiles, int64_t batch, int list_k,
+                         int k, int asc, float *out_values_dev, int64_t *out_labels_dev, void *stream);
+
 /* ---------------------------------------------------------------------------------------------
  * IVFPQ
  * ------------------------------------------------------------------------------------------- */

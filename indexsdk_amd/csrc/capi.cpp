@@ -478,6 +478,25 @@ IXA_EXPORT int ixa_op_ivfpq_subspace_distance(const float *queries_dev, int64_t 
                                         static_cast<hipStream_t>(stream));
     });
 }
+IXA_EXPORT int ixa_op_ivfpq_search_distance_topk(const float *lut_dev, int64_t batch, int msubs, const uint8_t *code_base_dev,
+                                                 const int64_t *code_offset_dev, const int64_t *code_size_dev, int nblocks,
+                                                 int k, const int64_t *label_base_dev, const int64_t *label_offset_dev,
+                                                 int metric, float *topk_values_dev, int64_t *topk_labels_dev, void *stream)
+{
+    return guarded([&] {
+        ixa::op_ivfpq_search_distance_topk(lut_dev, batch, msubs, code_base_dev, code_offset_dev, code_size_dev, nblocks, k,
+                                           label_base_dev, label_offset_dev, metric, topk_values_dev, topk_labels_dev,
+                                           static_cast<hipStream_t>(stream));
+    });
+}
+IXA_EXPORT int ixa_op_topk_ivfpq_l3(const int64_t *in_labels_dev, const float *in_values_dev, int tiles, int64_t batch,
+                                    int list_k, int k, int asc, float *out_values_dev, int64_t *out_labels_dev, void *stream)
+{
+    return guarded([&] {
+        ixa::op_topk_ivfpq_l3(in_labels_dev, in_values_dev, tiles, batch, list_k, k, asc, out_values_dev, out_labels_dev,
+                              static_cast<hipStream_t>(stream));
+    });
+}
 IXA_EXPORT int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev,
                                           int nprobe, int64_t k, float *distances_dev, int64_t *labels_dev)
 {

@@ -197,3 +197,81 @@ def test_read_probe_reports_a_duration_and_rejects_bad_sizes(env):
     assert lib.ixa_read_probe(_p(buf), 24, 3, ctypes.byref(ms)) != 0            # not a multiple of 16
     assert lib.ixa_read_probe(_p(buf), 1 << 20, 0, ctypes.byref(ms)) != 0       # no passes
     assert lib.ixa_read_probe(None, 1 << 20, 1, ctypes.byref(ms)) != 0
+
+
+@pytest.mark.parametrize("metric_name,M,k", [("L2", 16, 100), ("L2", 6, 320), ("IP", 8, 50)])
+def test_scan_topk_operator_with_the_reference_operands_and_the_tile_merge(env, oracle, metric_name, M, k):
+    """AscendcIvfpqSearchDistanceL2 with its own operands -- the LUT of the subspace operator, code and label base
+    pointers with per-(query, block) offsets and sizes -- equals the oracle's search over the same lists (row
+    order arithmetic: distances bit for bit); split over two tiles and merged by TopkIvfpqL3 it gives the same."""
+    from tests.parity import assert_topk_parity
+    hip, ix, _capi, lib = env
+    metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
+    rng = np.random.default_rng(M + k)
+    d, nlist, n, nq, nprobe = 48, 24, 30000, 41, 10
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    cent, _ = oracle.kmeans(x[:2000], nlist, niter=2, seed=1)
+    cb = oracle.train_pq(x[:3000], M, niter=2, seed=1)
+    ids = rng.permutation(10 * n)[:n].astype(np.int64)
+    ref = oracle.CsrIndex.build(d, M, metric, cent, cb, x, ids)
+    probes, _ = oracle.coarse_probe(q, cent, nprobe, metric)
+    probes = probes.astype(np.int64)
+    probes[3, 4] = probes[3, 5]                        # one list twice: scanned twice, as the reference would
+    lens = (ref.list_off[1:] - ref.list_off[:-1]).astype(np.int64)
+    code_off = (ref.list_off[:-1].astype(np.int64) * M)[probes]            # bytes from the code base
+    label_off = ref.list_off[:-1].astype(np.int64)[probes]                 # elements from the label base
+    sizes = lens[probes]
+    sizes[5, 2] = 0                                     # a block the caller marks empty is skipped
+    d_lut = hip.empty((nq, M, 256), np.float32)
+    _capi.check(lib.ixa_op_ivfpq_subspace_distance(_p(hip.put(q)), nq, d, _p(hip.put(cb)), M, metric, _p(d_lut), None))
+    d_codes, d_ids = hip.put(ref.codes), hip.put(ref.ids)
+    out_v, out_l = hip.empty((nq, k), np.float32), hip.empty((nq, k), np.int64)
+    _capi.check(lib.ixa_op_ivfpq_search_distance_topk(_p(d_lut), nq, M, _p(d_codes), _p(hip.put(code_off)),
+                                                      _p(hip.put(sizes)), nprobe, k, _p(d_ids), _p(hip.put(label_off)),
+                                                      metric, _p(out_v), _p(out_l), None))
+    V, L = out_v.get(), out_l.get()
+    # the oracle on the same (query, list) visits: per query, the union of its blocks
+    for j in range(nq):
+        cand_d, cand_i = [], []
+        for b in range(nprobe):
+            l, sz = probes[j, b], sizes[j, b]
+            if sz == 0:
+                continue
+            s, e = ref.list_off[l], ref.list_off[l] + sz
+            lut = oracle.lut(q[j:j + 1], cb, metric)[0]                    # [M][256]
+            acc = np.zeros(e - s, dtype=np.float32)
+            for m in range(M):
+                acc = (acc + lut[m][ref.codes[s:e, m]]).astype(np.float32)
+            cand_d.append(acc)
+            cand_i.append(ref.ids[s:e])
+        cd, ci = np.concatenate(cand_d), np.concatenate(cand_i)
+        order = np.lexsort((np.arange(len(cd)), cd if metric == ix.METRIC_L2 else -cd))[:k]
+        kk = len(order)
+        assert np.array_equal(V[j, :kk].view(np.uint32), cd[order].view(np.uint32)), j
+        same = L[j, :kk] == ci[order]
+        assert same.all() or np.array_equal(np.sort(cd[order][~same]), np.sort(V[j, :kk][~same])), j   # ties only
+        assert (L[j, kk:] == -1).all()
+    # two tiles of five blocks each, merged
+    tv, tl = hip.empty((2, nq, k), np.float32), hip.empty((2, nq, k), np.int64)
+    for t in range(2):
+        sl = slice(5 * t, 5 * t + 5)
+        ov, ol = hip.empty((nq, k), np.float32), hip.empty((nq, k), np.int64)
+        _capi.check(lib.ixa_op_ivfpq_search_distance_topk(
+            _p(d_lut), nq, M, _p(d_codes), _p(hip.put(np.ascontiguousarray(code_off[:, sl]))),
+            _p(hip.put(np.ascontiguousarray(sizes[:, sl]))), 5, k, _p(d_ids),
+            _p(hip.put(np.ascontiguousarray(label_off[:, sl]))), metric, _p(ov), _p(ol), None))
+        hip._ok(hip.rt.hipMemcpy(ctypes.c_void_p(tv.ptr.value + t * nq * k * 4), ov.ptr, nq * k * 4, 3))
+        hip._ok(hip.rt.hipMemcpy(ctypes.c_void_p(tl.ptr.value + t * nq * k * 8), ol.ptr, nq * k * 8, 3))
+    mv, ml = hip.empty((nq, k), np.float32), hip.empty((nq, k), np.int64)
+    _capi.check(lib.ixa_op_topk_ivfpq_l3(_p(tl), _p(tv), 2, nq, k, k, 1 if metric == ix.METRIC_L2 else 0, _p(mv), _p(ml),
+                                         None))
+    MV, ML = mv.get(), ml.get()
+    assert np.array_equal(MV.view(np.uint32), V.view(np.uint32))
+    diff = ML != L
+    assert not diff.any() or np.array_equal(np.sort(MV[diff]), np.sort(V[diff]))
+    # refusals
+    assert lib.ixa_op_ivfpq_search_distance_topk(_p(d_lut), nq, M, _p(d_codes), _p(hip.put(code_off)), _p(hip.put(sizes)),
+                                                 nprobe, 385, _p(d_ids), _p(hip.put(label_off)), metric, _p(out_v),
+                                                 _p(out_l), None) != 0
+    assert lib.ixa_op_topk_ivfpq_l3(_p(tl), _p(tv), 2, nq, k, k + 1, 1, _p(mv), _p(ml), None) != 0
