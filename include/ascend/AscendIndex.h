@@ -70,5 +70,34 @@ protected:
     AscendIndexConfig indexConfig;
 };
 
+// The ids a selector names, for the C ABI's remove calls: a range stays a range (isRange), a batch or an
+// array is listed from its own members, any other selector is asked about every id of `idMap` (the index's
+// ids in storage order, fetched by `fetchIdMap` only in that case).
+template <typename FetchIdMap>
+inline bool ixaSelectorIds(const faiss::IDSelector &sel, FetchIdMap fetchIdMap, std::vector<int64_t> &ids, int64_t &imin,
+                           int64_t &imax)
+{
+    if (auto range = dynamic_cast<const faiss::IDSelectorRange *>(&sel)) {
+        imin = range->imin;
+        imax = range->imax;
+        return true;
+    }
+    ids.clear();
+    if (auto batch = dynamic_cast<const faiss::IDSelectorBatch *>(&sel)) {
+        ids.assign(batch->set.begin(), batch->set.end());
+    } else if (auto array = dynamic_cast<const faiss::IDSelectorArray *>(&sel)) {
+        ids.assign(array->ids, array->ids + array->n);
+    } else {
+        std::vector<faiss::idx_t> idMap;
+        fetchIdMap(idMap);
+        for (faiss::idx_t id : idMap) {
+            if (sel.is_member(id)) {
+                ids.push_back(id);
+            }
+        }
+    }
+    return false;
+}
+
 }  // namespace ascend
 }  // namespace faiss

@@ -113,6 +113,20 @@ public:
             ixaThrowIfError(flat_get_ids(h_, 0, ntotal, reinterpret_cast<int64_t *>(idxMap.data())));
         }
     }
+    // remove_ids (FR/ascend/AscendIndex.h:78): the vectors the selector names leave; every hole, from the
+    // highest position down, is refilled with the vector that is last at that moment, as in the reference
+    size_t remove_ids(const faiss::IDSelector &sel) override
+    {
+        std::vector<int64_t> ids;
+        int64_t imin = 0, imax = 0, removed = 0;
+        if (ixaSelectorIds(sel, [this](std::vector<idx_t> &m) { getIdxMap(0, m); }, ids, imin, imax)) {
+            ixaThrowIfError(flat_remove_range(h_, imin, imax, &removed));
+        } else {
+            ixaThrowIfError(flat_remove_ids(h_, (int64_t)ids.size(), ids.data(), &removed));
+        }
+        syncTotal();
+        return (size_t)removed;
+    }
 
 protected:
     void syncTotal()
@@ -171,6 +185,28 @@ public:
         if (ntotal > 0) {
             ixaThrowIfError(flat_i8_get_base(h_, 0, ntotal, xb.data()));
         }
+    }
+    void getIdxMap(int /*deviceId*/, std::vector<idx_t> &idxMap) const
+    {
+        idxMap.resize((size_t)ntotal);
+        if (ntotal > 0) {
+            ixaThrowIfError(flat_i8_get_ids(h_, 0, ntotal, reinterpret_cast<int64_t *>(idxMap.data())));
+        }
+    }
+    // remove_ids (FR/ascend/AscendIndexInt8.h:88), as AscendIndexFlat::remove_ids
+    size_t remove_ids(const faiss::IDSelector &sel) override
+    {
+        std::vector<int64_t> ids;
+        int64_t imin = 0, imax = 0, removed = 0;
+        if (ixaSelectorIds(sel, [this](std::vector<idx_t> &m) { getIdxMap(0, m); }, ids, imin, imax)) {
+            ixaThrowIfError(flat_i8_remove_range(h_, imin, imax, &removed));
+        } else {
+            ixaThrowIfError(flat_i8_remove_ids(h_, (int64_t)ids.size(), ids.data(), &removed));
+        }
+        int64_t v = 0;
+        ixaThrowIfError(flat_i8_ntotal(h_, &v));
+        ntotal = v;
+        return (size_t)removed;
     }
     void reset()
     {

@@ -50,9 +50,17 @@ public:
     {
         searchImpl(n, reinterpret_cast<const int8_t *>(x), k, distances, labels);
     }
+    virtual size_t remove_ids(const faiss::IDSelector & /*sel*/)
+    {
+        throw faiss::FaissException("remove_ids not implemented for this type of index");
+    }
     virtual void reserveMemory(size_t /*numVecs*/) {}
     virtual size_t reclaimMemory() { return 0; }
     std::vector<int> getDeviceList() { return indexConfig.deviceList; }
+    int getDim() const { return d; }
+    idx_t getNTotal() const { return ntotal; }
+    bool isTrained() const { return is_trained; }
+    faiss::MetricType getMetricType() const { return metric_type; }
 
     int d;
     idx_t ntotal = 0;

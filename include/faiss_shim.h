@@ -10,12 +10,14 @@
 #include <faiss/IndexFlat.h>
 #include <faiss/IndexIVFPQ.h>
 #include <faiss/impl/FaissException.h>
+#include <faiss/impl/IDSelector.h>
 #include <faiss/invlists/InvertedLists.h>
 #else
 #include <cstddef>
 #include <cstdint>
 #include <exception>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 namespace faiss {
@@ -33,6 +35,37 @@ public:
 
 struct SearchParameters {
     virtual ~SearchParameters() {}
+};
+
+// The selectors remove_ids takes (faiss/impl/IDSelector.h): a predicate on ids, with the three concrete
+// kinds the reference's callers use.
+struct IDSelector {
+    virtual bool is_member(idx_t id) const = 0;
+    virtual ~IDSelector() {}
+};
+struct IDSelectorRange : IDSelector {
+    idx_t imin, imax;   // ids in [imin, imax)
+    IDSelectorRange(idx_t imin_, idx_t imax_) : imin(imin_), imax(imax_) {}
+    bool is_member(idx_t id) const override { return id >= imin && id < imax; }
+};
+struct IDSelectorArray : IDSelector {
+    size_t n;
+    const idx_t *ids;
+    IDSelectorArray(size_t n_, const idx_t *ids_) : n(n_), ids(ids_) {}
+    bool is_member(idx_t id) const override
+    {
+        for (size_t i = 0; i < n; i++) {
+            if (ids[i] == id) {
+                return true;
+            }
+        }
+        return false;
+    }
+};
+struct IDSelectorBatch : IDSelector {
+    std::unordered_set<idx_t> set;
+    IDSelectorBatch(size_t n, const idx_t *indices) : set(indices, indices + n) {}
+    bool is_member(idx_t id) const override { return set.count(id) != 0; }
 };
 
 struct ClusteringParameters {
@@ -66,6 +99,10 @@ struct Index {
     virtual void search(idx_t n, const float *x, idx_t k, float *distances, idx_t *labels,
                         const SearchParameters *params = nullptr) const = 0;
     virtual void reset() = 0;
+    virtual size_t remove_ids(const IDSelector & /*sel*/)
+    {
+        throw FaissException("remove_ids not implemented for this type of index");
+    }
 };
 
 // The coarse quantizer of an IndexIVFPQ as copyFrom / copyTo see it: a row store.

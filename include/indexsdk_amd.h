@@ -363,6 +363,14 @@ int flat_search_device(flat_index_t *h, int64_t n, const float *x_dev, int64_t k
 int flat_get_base(const flat_index_t *h, int64_t offset, int64_t n, float *out);
 int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out);
 int flat_ntotal(const flat_index_t *h, int64_t *out);
+/* AscendIndex::remove_ids(const faiss::IDSelector &)  FR/ascend/AscendIndex.h:78 -> AscendIndexImpl::removeImpl
+ * (FR/ascend/impl/AscendIndexImpl.cpp:208-270) + Index::removeIdsBatch (FR/ascenddaemon/impl/Index.cpp:86-113):
+ * the vectors whose id is one of the n ids (IDSelectorBatch; ids the index does not hold and repeats are
+ * ignored) or lies in [imin, imax) (IDSelectorRange) leave the index; *removed (may be NULL) = how many.
+ * As in the reference every removed position, from the highest to the lowest, is refilled with the vector
+ * that is last at that moment, so the order of the remaining vectors (getBase / getIdxMap) is the reference's. */
+int flat_remove_ids(flat_index_t *h, int64_t n, const int64_t *ids, int64_t *removed);
+int flat_remove_range(flat_index_t *h, int64_t imin, int64_t imax, int64_t *removed);
 int flat_reset(flat_index_t *h);
 int flat_last_search_stats(const flat_index_t *h, flat_search_stats_t *out);
 
@@ -380,7 +388,13 @@ int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, in
 int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x_dev, int64_t k, int32_t *distances_dev,
                           int64_t *labels_dev);
 int flat_i8_get_base(const flat_i8_index_t *h, int64_t offset, int64_t n, int8_t *out);
+/* AscendIndexInt8Flat::getIdxMap  FR/ascend/AscendIndexInt8Flat.h:83 */
+int flat_i8_get_ids(const flat_i8_index_t *h, int64_t offset, int64_t n, int64_t *out);
 int flat_i8_ntotal(const flat_i8_index_t *h, int64_t *out);
+/* AscendIndexInt8::remove_ids(const faiss::IDSelector &)  FR/ascend/AscendIndexInt8.h:88 ->
+ * AscendIndexInt8FlatImpl::removeImpl (FR/ascend/impl/AscendIndexInt8FlatImpl.cpp:819-867); as flat_remove_*. */
+int flat_i8_remove_ids(flat_i8_index_t *h, int64_t n, const int64_t *ids, int64_t *removed);
+int flat_i8_remove_range(flat_i8_index_t *h, int64_t imin, int64_t imax, int64_t *removed);
 int flat_i8_reset(flat_i8_index_t *h);
 int flat_i8_last_search_stats(const flat_i8_index_t *h, flat_search_stats_t *out);
 

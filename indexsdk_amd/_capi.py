@@ -134,11 +134,13 @@ for _pfx, _dist in (("flat", ctypes.c_void_p), ("flat_i8", ctypes.c_void_p)):
         f"{_pfx}_search_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, _dist,
                                                  ctypes.c_void_p]),
         f"{_pfx}_get_base": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+        f"{_pfx}_get_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),
+        f"{_pfx}_remove_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
+        f"{_pfx}_remove_range": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
         f"{_pfx}_ntotal": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int64)]),
         f"{_pfx}_reset": (ctypes.c_int, [_H]),
         f"{_pfx}_last_search_stats": (ctypes.c_int, [_H, ctypes.POINTER(FlatSearchStats)]),
     })
-_SIGNATURES["flat_get_ids"] = (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p])
 
 _lib = None
 

@@ -293,6 +293,26 @@ class _FlatCommon:
         _capi.check(self._fn("get_base")(self._h, offset, n, _ptr(out)))
         return out
 
+    def getIdxMap(self, offset=0, n=None):
+        """The id of every stored vector, in storage order (getIdxMap, FR/ascend/AscendIndexFlat.h:76)."""
+        n = self.ntotal - offset if n is None else n
+        out = np.empty(n, dtype=np.int64)
+        _capi.check(self._fn("get_ids")(self._h, offset, n, _ptr(out)))
+        return out
+
+    def remove_ids(self, ids):
+        """remove_ids(IDSelectorBatch(ids)) -- FR/ascend/AscendIndex.h:78; returns the number of vectors removed."""
+        ids = _as(ids, np.int64, 1, "ids")
+        removed = ctypes.c_int64()
+        _capi.check(self._fn("remove_ids")(self._h, ids.shape[0], _ptr(ids), ctypes.byref(removed)))
+        return removed.value
+
+    def remove_range(self, imin, imax):
+        """remove_ids(IDSelectorRange(imin, imax)): the vectors whose id lies in [imin, imax)."""
+        removed = ctypes.c_int64()
+        _capi.check(self._fn("remove_range")(self._h, imin, imax, ctypes.byref(removed)))
+        return removed.value
+
     def reset(self):
         _capi.check(self._fn("reset")(self._h))
 

@@ -388,6 +388,30 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
     {                                                                                                             \
         return guarded([&] { IXA_HANDLE(h); h->impl.get_base(offset, n, out); });                                 \
     }                                                                                                             \
+    IXA_EXPORT int PFX##_get_ids(const HT *h, int64_t offset, int64_t n, int64_t *out)                           \
+    {                                                                                                             \
+        return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });                                  \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_remove_ids(HT *h, int64_t n, const int64_t *ids, int64_t *removed)                      \
+    {                                                                                                             \
+        return guarded([&] {                                                                                      \
+            IXA_HANDLE(h);                                                                                        \
+            const int64_t r = h->impl.remove_ids(n, ids);                                                         \
+            if (removed) {                                                                                        \
+                *removed = r;                                                                                     \
+            }                                                                                                     \
+        });                                                                                                       \
+    }                                                                                                             \
+    IXA_EXPORT int PFX##_remove_range(HT *h, int64_t imin, int64_t imax, int64_t *removed)                       \
+    {                                                                                                             \
+        return guarded([&] {                                                                                      \
+            IXA_HANDLE(h);                                                                                        \
+            const int64_t r = h->impl.remove_range(imin, imax);                                                   \
+            if (removed) {                                                                                        \
+                *removed = r;                                                                                     \
+            }                                                                                                     \
+        });                                                                                                       \
+    }                                                                                                             \
     IXA_EXPORT int PFX##_ntotal(const HT *h, int64_t *out)                                                        \
     {                                                                                                             \
         return guarded([&] {                                                                                      \
@@ -547,10 +571,6 @@ IXA_EXPORT int ixa_read_probe(const void *src_dev, int64_t bytes, int passes, do
         IXA_REQUIRE(ms_per_pass != nullptr, ixa::kErrInvalidParam, "ms_per_pass can not be nullptr.");
         *ms_per_pass = ixa::launch_read_probe(src_dev, bytes, passes);
     });
-}
-IXA_EXPORT int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out)
-{
-    return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });
 }
 IXA_EXPORT int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels)
 {

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <unordered_map>
 #include <vector>
 
 #include "coarse.h"
@@ -303,6 +304,61 @@ __global__ __launch_bounds__(256) void map_labels_kernel(const int32_t *__restri
     }
 }
 
+// Positions of the vectors a removal selects: those whose id is among the sorted `victims` (binary search),
+// or, without a victim list, inside [imin, imax).  Every hit takes a slot of `out` from an atomic counter
+// (positions arrive in no particular order); with out == nullptr the launch only counts.
+__global__ __launch_bounds__(256) void select_positions_kernel(const int64_t *__restrict__ ids, int64_t n,
+                                                               const int64_t *__restrict__ victims, int64_t nv,
+                                                               int64_t imin, int64_t imax, int64_t *__restrict__ out,
+                                                               int64_t cap, unsigned long long *__restrict__ count)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const int64_t id = ids[i];
+    bool hit;
+    if (victims == nullptr) {
+        hit = id >= imin && id < imax;
+    } else {
+        int64_t lo = 0, hi = nv;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (victims[mid] < id) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        hit = lo < nv && victims[lo] == id;
+    }
+    if (hit) {
+        const unsigned long long slot = atomicAdd(count, 1ull);
+        if (out != nullptr && (int64_t)slot < cap) {
+            out[slot] = i;
+        }
+    }
+}
+
+// Move j copies row moves[2 j + 1] (vector, id, norm) over row moves[2 j].  Sources lie past the new end of
+// the base and destinations before it, so no move reads what another writes.
+template <typename T>
+__global__ __launch_bounds__(128) void move_rows_kernel(T *__restrict__ base, int64_t *__restrict__ ids,
+                                                        uint32_t *__restrict__ norms,
+                                                        const int64_t *__restrict__ moves, int d)
+{
+    const int64_t dst = moves[2 * (int64_t)blockIdx.x], src = moves[2 * (int64_t)blockIdx.x + 1];
+    for (int t = threadIdx.x; t < d; t += 128) {
+        base[dst * d + t] = base[src * d + t];
+    }
+    if (threadIdx.x == 0) {
+        ids[dst] = ids[src];
+        if (norms != nullptr) {
+            norms[dst] = norms[src];
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void iota_ids_kernel(int64_t *out, int64_t n, int64_t base)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -477,6 +533,82 @@ void FlatBase<T>::get_ids(int64_t offset, int64_t n, int64_t *out) const
     }
 }
 
+// remove_ids (FR/ascend/impl/AscendIndexImpl.cpp:208-270 picks the positions whose id the selector names,
+// FR/ascenddaemon/impl/Index.cpp:86-113 removes them): the positions are visited from the highest to the
+// lowest and each is overwritten with the vector that is last at that moment, which then leaves the end.
+// The device does the outcome of that sequence in one launch: every removed position below the new end
+// receives the vector the sequence leaves there (always one from at or past the new end), everything else
+// stays where it is.  victims == nullptr selects by range.
+template <typename T>
+int64_t FlatBase<T>::remove_selected(int64_t nv, const int64_t *victims, int64_t imin, int64_t imax, uint32_t *norms)
+{
+    IXA_REQUIRE(nv >= 0 && nv < kMaxN && (nv == 0 || victims), kErrInvalidParam, "ids can not be nullptr.");
+    if (ntotal_ == 0 || (victims == nullptr ? imin >= imax : nv == 0)) {
+        return 0;
+    }
+    DeviceBuffer<int64_t> victims_dev;
+    if (victims) {
+        std::vector<int64_t> sorted(victims, victims + nv);
+        std::sort(sorted.begin(), sorted.end());
+        sorted.erase(std::unique(sorted.begin(), sorted.end()), sorted.end());
+        nv = (int64_t)sorted.size();
+        victims_dev.upload(sorted.data(), sorted.size(), stream_);
+    }
+    DeviceBuffer<unsigned long long> count(1);
+    unsigned long long hits = 0;
+    IXA_HIP(hipMemsetAsync(count.data(), 0, 8, stream_));
+    hipLaunchKernelGGL(select_positions_kernel, dim3(blocks_for(ntotal_)), dim3(256), 0, stream_, ids_.data(), ntotal_,
+                       victims ? victims_dev.data() : nullptr, nv, imin, imax, (int64_t *)nullptr, (int64_t)0,
+                       count.data());
+    count.download(&hits, 1, stream_);
+    if (hits == 0) {
+        return 0;
+    }
+    DeviceBuffer<int64_t> pos_dev((size_t)hits);
+    IXA_HIP(hipMemsetAsync(count.data(), 0, 8, stream_));
+    hipLaunchKernelGGL(select_positions_kernel, dim3(blocks_for(ntotal_)), dim3(256), 0, stream_, ids_.data(), ntotal_,
+                       victims ? victims_dev.data() : nullptr, nv, imin, imax, pos_dev.data(), (int64_t)hits,
+                       count.data());
+    std::vector<int64_t> gone((size_t)hits);
+    pos_dev.download(gone.data(), gone.size(), stream_);
+    std::sort(gone.begin(), gone.end());
+    const int64_t left = ntotal_ - (int64_t)hits;
+    // The sequence is replayed on the host with only the overwritten positions recorded (a vector can move
+    // several times: into a hole of the tail first, on into a lower hole later); what finally matters is
+    // which original vector each hole below the new end holds.  Those vectors all come from positions at
+    // or past the new end, each exactly once.
+    std::unordered_map<int64_t, int64_t> holds;   // position -> original position of the vector now there
+    holds.reserve(gone.size());
+    auto at = [&](int64_t p) {
+        const auto it = holds.find(p);
+        return it == holds.end() ? p : it->second;
+    };
+    int64_t cur = ntotal_;
+    for (int64_t g = (int64_t)gone.size() - 1; g >= 0; g--, cur--) {
+        const int64_t hole = gone[(size_t)g];
+        if (hole != cur - 1) {
+            holds[hole] = at(cur - 1);
+        }
+    }
+    std::vector<int64_t> moves;
+    for (size_t g = 0; g < gone.size() && gone[g] < left; g++) {
+        const int64_t src = holds.at(gone[g]);
+        IXA_REQUIRE(src >= left && src < ntotal_, kErrInner, "remove: hole %ld would be filled from position %ld",
+                    (long)gone[g], (long)src);
+        moves.push_back(gone[g]);
+        moves.push_back(src);
+    }
+    if (!moves.empty()) {
+        DeviceBuffer<int64_t> moves_dev;
+        moves_dev.upload(moves.data(), moves.size(), stream_);
+        hipLaunchKernelGGL((move_rows_kernel<T>), dim3((unsigned)(moves.size() / 2)), dim3(128), 0, stream_, base_.data(),
+                           ids_.data(), norms, moves_dev.data(), d_);
+        sync_stream(stream_);   // moves_dev is freed on return
+    }
+    ntotal_ = left;
+    return (int64_t)hits;
+}
+
 template <typename T>
 void FlatBase<T>::reset()
 {
@@ -559,6 +691,17 @@ void FlatIndex::reset()
 {
     FlatBase<float>::reset();
     norms_.release();
+}
+
+int64_t FlatIndex::remove_ids(int64_t n, const int64_t *ids)
+{
+    IXA_REQUIRE(n >= 0 && (n == 0 || ids), kErrInvalidParam, "ids can not be nullptr.");
+    return remove_selected(n, ids, 0, 0, reinterpret_cast<uint32_t *>(norms_.data()));
+}
+
+int64_t FlatIndex::remove_range(int64_t imin, int64_t imax)
+{
+    return remove_selected(0, nullptr, imin, imax, reinterpret_cast<uint32_t *>(norms_.data()));
 }
 
 // search (FR/ascendhost/src/index/IndexFlatL2Aicpu.cpp:157-306): the base is walked in row chunks;
@@ -657,6 +800,17 @@ void FlatI8Index::add(int64_t n, const int8_t *x, const int64_t *ids, bool on_de
                        base_.data() + before * d_, n, d_, nn.data() + before);
     sync_stream(stream_);
     norms_ = std::move(nn);
+}
+
+int64_t FlatI8Index::remove_ids(int64_t n, const int64_t *ids)
+{
+    IXA_REQUIRE(n >= 0 && (n == 0 || ids), kErrInvalidParam, "ids can not be nullptr.");
+    return remove_selected(n, ids, 0, 0, reinterpret_cast<uint32_t *>(norms_.data()));
+}
+
+int64_t FlatI8Index::remove_range(int64_t imin, int64_t imax)
+{
+    return remove_selected(0, nullptr, imin, imax, reinterpret_cast<uint32_t *>(norms_.data()));
 }
 
 void FlatI8Index::reset()

@@ -41,6 +41,9 @@ public:
 
 protected:
     void reserve(int64_t n);
+    // removes the vectors whose id is one of the nv host ids (victims != nullptr) or lies in [imin, imax);
+    // norms: the derived class's 4-byte norm per vector, moved along; returns the number removed
+    int64_t remove_selected(int64_t nv, const int64_t *victims, int64_t imin, int64_t imax, uint32_t *norms);
     int d_, metric_;
     int64_t scratch_bytes_;
     int64_t ntotal_ = 0, capacity_ = 0;
@@ -58,6 +61,8 @@ public:
     FlatIndex(int d, int metric, int64_t scratch_bytes);
     void add(int64_t n, const float *x, const int64_t *ids, bool on_device);
     void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
+    int64_t remove_ids(int64_t n, const int64_t *ids);       // host ids; returns the number of vectors removed
+    int64_t remove_range(int64_t imin, int64_t imax);        // ids in [imin, imax)
     void reset();
 
 private:
@@ -75,6 +80,8 @@ public:
     FlatI8Index(int d, int metric, int64_t scratch_bytes);
     void add(int64_t n, const int8_t *x, const int64_t *ids, bool on_device);
     void search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device);
+    int64_t remove_ids(int64_t n, const int64_t *ids);
+    int64_t remove_range(int64_t imin, int64_t imax);
     void reset();
 
 private:

@@ -203,6 +203,20 @@ def flat_i8(base, q, k, ids=None):
     return dist, labels
 
 
+def flat_remove_order(ntotal, positions):
+    """Storage order of a Flat index after the reference removes the vectors at ``positions``: original
+    positions of the survivors, in their new order.  The reference's loop as it stands
+    (Index::removeIdsBatch, FR/ascenddaemon/impl/Index.cpp:86-113; the host id map is edited the same way,
+    AscendIndexImpl::removeIdx, FR/ascend/impl/AscendIndexImpl.cpp:253-270): positions outside the index and
+    repeats are dropped, the rest are visited from the highest to the lowest, each is overwritten with the
+    vector that is last at that moment, and the index shrinks by one."""
+    order = list(range(int(ntotal)))
+    for pos in sorted({int(p) for p in positions if 0 <= int(p) < ntotal}, reverse=True):
+        order[pos] = order[-1]
+        order.pop()
+    return np.asarray(order, dtype=np.int64)
+
+
 def merge_results(dist, labels, metric=METRIC_L2):
     """dist/labels: [ndev][n][k] per-device result lists -> merged ([n][k], [n][k])."""
     dist = _f32(dist)

@@ -159,6 +159,24 @@ int main(int argc, char **argv)
         EXPECT(cpu_flat.ntotal == n && std::memcmp(cpu_flat.get_xb(), x.data(), x.size() * sizeof(float)) == 0);
         AscendIndexFlat flat2(&cpu_flat);
         EXPECT(flat2.ntotal == n);
+        // remove_ids through the faiss::Index interface: a range, a batch, and a selector of the caller's own
+        {
+            faiss::Index *as_index = &flat2;
+            EXPECT(as_index->remove_ids(faiss::IDSelectorRange(n - 2, n + 5)) == 2 && flat2.ntotal == n - 2);
+            const faiss::idx_t some[] = {0, 3, 3, n + 7};
+            EXPECT(as_index->remove_ids(faiss::IDSelectorBatch(4, some)) == 2 && flat2.ntotal == n - 4);
+            std::vector<faiss::idx_t> map;
+            flat2.getIdxMap(0, map);
+            // the holes 3 and 0, in that order, took the vectors that were last: n - 3, then n - 4
+            EXPECT((faiss::idx_t)map.size() == n - 4 && map[3] == n - 3 && map[0] == n - 4 && map[1] == 1);
+            struct Multiples : faiss::IDSelector {
+                bool is_member(faiss::idx_t id) const override { return id % 100 == 1; }
+            };
+            const size_t expect = (size_t)((n - 3 - 1) / 100 + 1);   // 1, 101, ... among the ids up to n - 3 that are left
+            EXPECT(as_index->remove_ids(Multiples()) == expect && flat2.ntotal == n - 4 - (faiss::idx_t)expect);
+            flat2.search(1, x.data() + (size_t)5 * d, 1, D.data(), I.data());
+            EXPECT(I[0] == 5);
+        }
         // int8: AscendIndexInt8Flat -> AscendIndexInt8
         std::vector<int8_t> b((size_t)4096 * 64);
         for (auto &v : b) {
@@ -173,6 +191,12 @@ int main(int argc, char **argv)
         for (int i = 0; i < 4; i++) {
             EXPECT(Ii[(size_t)i * 3] == i && Di[(size_t)i * 3] == 0.f);
         }
+        EXPECT(i8_base->remove_ids(faiss::IDSelectorRange(1, 3)) == 2 && i8_base->getNTotal() == 4094);
+        std::vector<faiss::idx_t> map8;
+        i8.getIdxMap(0, map8);
+        EXPECT(map8.size() == 4094 && map8[0] == 0 && map8[2] == 4095 && map8[1] == 4094);
+        i8_base->search(1, b.data() + (size_t)4095 * 64, 3, Di.data(), Ii.data());
+        EXPECT(Ii[0] == 4095 && Di[0] == 0.f);
     }
     std::printf(failures ? "wrapper test FAILED\n" : "wrapper test ok\n");
     return failures ? 1 : 0;

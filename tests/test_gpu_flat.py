@@ -242,3 +242,66 @@ def test_flat_largest_k(ix, oracle, n, nq, scratch):
         Dr, Ir = oracle.flat_f32(base, q, k, metric)
         assert np.array_equal(I, Ir)
         assert np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+
+
+@pytest.mark.parametrize("kind", ["fp32_L2", "fp32_IP", "int8"])
+def test_flat_remove_ids_follows_the_reference_order(ix, oracle, kind):
+    """remove_ids with a batch of ids (some absent, some repeated, some held by two vectors) and with an id
+    range: the count, the storage order afterwards (getIdxMap / getBase: every hole, highest first, is
+    refilled with the vector that is last at that moment; Index.cpp:86-113) and the searches on what is left
+    equal the oracle's, and vectors added afterwards land behind the survivors."""
+    rng = np.random.default_rng(31)
+    d, n = 48, 30000
+    if kind == "int8":
+        index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=4 << 20)
+        base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+        q = rng.integers(-127, 128, size=(40, d), dtype=np.int8)
+    else:
+        metric = ix.METRIC_L2 if kind == "fp32_L2" else ix.METRIC_INNER_PRODUCT
+        index = ix.AscendIndexFlat(d, metric, scratch_bytes=4 << 20)
+        base = rng.standard_normal((n, d)).astype(np.float32)
+        q = rng.standard_normal((40, d)).astype(np.float32)
+    ids = rng.permutation(10 * n)[:n].astype(np.int64)
+    ids[100] = ids[7]                                   # one id held by two vectors: both leave
+    index.add_with_ids(base[:20000], ids[:20000])
+    index.add_with_ids(base[20000:], ids[20000:])
+
+    def check(base, ids, k=12):
+        assert index.ntotal == len(ids)
+        assert np.array_equal(index.getIdxMap(), ids)
+        assert np.array_equal(index.getBase(), base)
+        if kind == "int8":
+            D, I = index.search_int32(q, k)
+            Dr, Ir = oracle.flat_i8(base, q, k, ids=ids)
+            assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+        else:
+            D, I = index.search(q, k)
+            Dr, Ir = oracle.flat_f32(base, q, k, index.metric_type, ids=ids)
+            assert np.array_equal(I, Ir) and np.array_equal(D.view(np.uint32), Dr.view(np.uint32))
+
+    check(base, ids)
+    victims = np.concatenate([rng.choice(ids, 2500, replace=False), ids[-3:], [ids[7]], [-5, 10 * n + 1], ids[:4], ids[:4]])
+    gone = np.nonzero(np.isin(ids, victims))[0]
+    assert index.remove_ids(victims) == len(gone)
+    order = oracle.flat_remove_order(n, gone)
+    base, ids = base[order], ids[order]
+    check(base, ids)
+    assert index.remove_ids(np.array([-5], dtype=np.int64)) == 0 and index.remove_ids(np.empty(0, dtype=np.int64)) == 0
+    lo, hi = 1000, 40000
+    gone = np.nonzero((ids >= lo) & (ids < hi))[0]
+    assert len(gone) > 1000 and index.remove_range(lo, hi) == len(gone)
+    order = oracle.flat_remove_order(len(ids), gone)
+    base, ids = base[order], ids[order]
+    check(base, ids)
+    assert index.remove_range(hi, lo) == 0
+    extra = base[:50][::-1].copy()
+    extra_ids = np.arange(50, dtype=np.int64) + 20 * n
+    index.add_with_ids(extra, extra_ids)
+    base, ids = np.concatenate([base, extra]), np.concatenate([ids, extra_ids])
+    check(base, ids)
+    assert index.remove_range(-1, 30 * n) == len(ids) and index.ntotal == 0      # everything leaves
+    if kind == "int8":
+        D, I = index.search_int32(q[:2], 3)
+    else:
+        D, I = index.search(q[:2], 3)
+    assert (I == -1).all()

@@ -358,3 +358,25 @@ def test_parity_rule_measures_cancelling_sums_against_their_terms(oracle):
     wrong[0, r] += np.float32(1e-3 * scale)
     with pytest.raises(AssertionError):
         assert_topk_parity(oracle, idx, q, wrong, I, D, I, 1e-4)
+
+
+def test_flat_remove_order_worked_examples(oracle):
+    """The removal order of the Flat indexes, against sequences worked by hand from the reference's loop
+    (highest position first, the last vector moves into the hole; Index.cpp:86-113): a vector can move
+    twice, a removed last vector just leaves, repeats and positions past the end are ignored."""
+    assert oracle.flat_remove_order(10, [2, 7]).tolist() == [0, 1, 8, 3, 4, 5, 6, 9]
+    assert oracle.flat_remove_order(10, [8, 2]).tolist() == [0, 1, 9, 3, 4, 5, 6, 7]       # 9 -> 8 -> 2
+    assert oracle.flat_remove_order(10, [1, 2]).tolist() == [0, 8, 9, 3, 4, 5, 6, 7]
+    assert oracle.flat_remove_order(5, [4, 4, 9, -1]).tolist() == [0, 1, 2, 3]
+    assert oracle.flat_remove_order(4, [0, 1, 2, 3]).tolist() == []
+    assert oracle.flat_remove_order(6, [0]).tolist() == [5, 1, 2, 3, 4]
+    assert oracle.flat_remove_order(3, []).tolist() == [0, 1, 2]
+    # survivors are exactly the positions that were not named, each once
+    rng = np.random.default_rng(3)
+    for _ in range(20):
+        n = int(rng.integers(1, 60))
+        gone = rng.integers(0, n, int(rng.integers(0, n + 1)))
+        order = oracle.flat_remove_order(n, gone)
+        assert sorted(order.tolist()) == sorted(set(range(n)) - set(gone.tolist()))
+        stay = [p for p in range(n - len(set(gone.tolist()))) if p not in set(gone.tolist())]
+        assert all(order[p] == p for p in stay)        # a survivor below the new end never moves
