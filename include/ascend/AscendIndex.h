@@ -4,6 +4,7 @@
 // faiss::FaissException on a non-zero status, as the reference's public layer does (FAISS_THROW_IF_NOT_FMT).
 #pragma once
 #include <cstdint>
+#include <cstring>
 #include <initializer_list>
 #include <string>
 #include <vector>
@@ -20,6 +21,32 @@ const idx_t MAX_N = 1000000000;
 const idx_t MAX_K = 4096;
 const int64_t INDEX_DEFAULT_MEM = 0x2000000;   // 32M
 const uint32_t DEFAULT_BLOCK_SIZE = 16384 * 16;
+
+// IEEE binary16 -> binary32, exact (subnormals, infinities and NaNs included).
+inline float ixaHalfToFloat(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu, man = h & 0x3ffu, bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {
+            int shift = 0;
+            while (!(man & 0x400u)) {
+                man <<= 1;
+                shift++;
+            }
+            bits = sign | ((uint32_t)(113 - shift) << 23) | ((man & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 112) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
 
 inline void ixaThrowIfError(int status)
 {
@@ -66,7 +93,39 @@ public:
     virtual size_t reclaimMemory() { return 0; }
     std::vector<int> getDeviceList() { return indexConfig.deviceList; }
 
+    // The reference's calls with IEEE half inputs (FR/ascend/AscendIndex.h:103-107).  Its indexes store and
+    // compare in half precision anyway; this build computes in fp32, so the halves are widened (exactly) first.
+    void add(idx_t n, const uint16_t *x) { add_with_ids(n, x, nullptr); }
+    void add_with_ids(idx_t n, const uint16_t *x, const idx_t *ids)
+    {
+        const std::vector<float> wide = ixaWiden(n, x);
+        if (ids) {
+            add_with_ids(n, wide.data(), ids);
+        } else {
+            add(n, wide.data());
+        }
+    }
+    void search(idx_t n, const uint16_t *x, idx_t k, float *distances, idx_t *labels) const
+    {
+        const std::vector<float> wide = ixaWiden(n, x);
+        search(n, wide.data(), k, distances, labels);
+    }
+    using faiss::Index::add;
+    using faiss::Index::add_with_ids;
+    using faiss::Index::search;
+
 protected:
+    std::vector<float> ixaWiden(idx_t n, const uint16_t *x) const
+    {
+        if (x == nullptr || n < 0) {
+            throw faiss::FaissException("x can not be nullptr.");
+        }
+        std::vector<float> out((size_t)n * d);
+        for (size_t i = 0; i < out.size(); i++) {
+            out[i] = ixaHalfToFloat(x[i]);
+        }
+        return out;
+    }
     AscendIndexConfig indexConfig;
 };
 

@@ -79,6 +79,50 @@ public:
             index->add(ntotal, xb.data());
         }
     }
+    // Initialize ourselves from a CPU index with user ids (FR/ascend/AscendIndexFlat.h:52, 62): its rows must
+    // be an IndexFlat
+    explicit AscendIndexFlat(const faiss::IndexIDMap *index, AscendIndexFlatConfig config = AscendIndexFlatConfig())
+        : AscendIndex(index ? index->d : 0, index ? index->metric_type : faiss::METRIC_L2, config)
+    {
+        if (index == nullptr) {
+            throw FaissException("index is nullptr.");
+        }
+        ixaThrowIfError(flat_create(index->d, (int)index->metric_type, scratchOf(config.resourceSize), &h_));
+        try {
+            copyFrom(index);
+        } catch (...) {
+            flat_destroy(h_);
+            throw;
+        }
+    }
+    void copyFrom(const faiss::IndexIDMap *index)
+    {
+        const faiss::IndexFlat *rows = index ? dynamic_cast<const faiss::IndexFlat *>(index->index) : nullptr;
+        if (rows == nullptr || rows->d != d || rows->metric_type != metric_type ||
+            (idx_t)index->id_map.size() != rows->ntotal) {
+            throw FaissException("copyFrom: the source must be an IndexIDMap over an IndexFlat with this index's "
+                                 "dims and metric");
+        }
+        reset();
+        if (rows->ntotal > 0) {
+            add_with_ids(rows->ntotal, rows->get_xb(), index->id_map.data());
+        }
+    }
+    void copyTo(faiss::IndexIDMap *index) const
+    {
+        faiss::IndexFlat *rows = index ? dynamic_cast<faiss::IndexFlat *>(index->index) : nullptr;
+        if (rows == nullptr) {
+            throw FaissException("copyTo: the target must be an IndexIDMap over an IndexFlat");
+        }
+        copyTo(rows);
+        getIdxMap(0, index->id_map);
+        index->d = d;
+        index->metric_type = metric_type;
+        index->ntotal = ntotal;
+    }
+    using AscendIndex::add;            // the IEEE half overloads
+    using AscendIndex::add_with_ids;
+    using AscendIndex::search;
     void add(idx_t n, const float *x) override { add_with_ids(n, x, nullptr); }
     void add_with_ids(idx_t n, const float *x, const idx_t *ids) override
     {
@@ -213,6 +257,9 @@ public:
         ixaThrowIfError(flat_i8_reset(h_));
         ntotal = 0;
     }
+    // setPageSize (FR/ascend/AscendIndexInt8Flat.h:101) tunes how many base blocks the reference searches
+    // per operator call; the search here streams the whole base through one persistent kernel: accepted, no effect
+    void setPageSize(uint16_t /*pageBlockNum*/) {}
 
 protected:
     void addImpl(idx_t n, const int8_t *x, const idx_t *ids) override

@@ -87,6 +87,9 @@ public:
         ids.resize(len);
         ixaThrowIfError(ivfpq_get_list(h_, listId, codes.data(), reinterpret_cast<int64_t *>(ids.data())));
     }
+    using AscendIndex::add;            // the IEEE half overloads
+    using AscendIndex::add_with_ids;
+    using AscendIndex::search;
     void add(idx_t n, const float *x) override { add_with_ids(n, x, nullptr); }
     void add_with_ids(idx_t n, const float *x, const idx_t *ids) override
     {

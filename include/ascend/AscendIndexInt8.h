@@ -50,6 +50,12 @@ public:
     {
         searchImpl(n, reinterpret_cast<const int8_t *>(x), k, distances, labels);
     }
+    // assign (FR/ascend/AscendIndexInt8.h:90): the labels of a search for the k nearest
+    void assign(idx_t n, const int8_t *x, idx_t *labels, idx_t k = 1)
+    {
+        std::vector<float> distances((size_t)n * k);
+        searchImpl(n, x, k, distances.data(), labels);
+    }
     virtual size_t remove_ids(const faiss::IDSelector & /*sel*/)
     {
         throw faiss::FaissException("remove_ids not implemented for this type of index");

@@ -8,6 +8,7 @@
 #include <faiss/Clustering.h>
 #include <faiss/Index.h>
 #include <faiss/IndexFlat.h>
+#include <faiss/IndexIDMap.h>
 #include <faiss/IndexIVFPQ.h>
 #include <faiss/impl/FaissException.h>
 #include <faiss/impl/IDSelector.h>
@@ -130,6 +131,42 @@ struct IndexFlatL2 : IndexFlat {
 };
 struct IndexFlatIP : IndexFlat {
     explicit IndexFlatIP(idx_t d_ = 0) : IndexFlat(d_, METRIC_INNER_PRODUCT) {}
+};
+
+// faiss::IndexIDMap as copyFrom / copyTo see it: an index plus the user ids of its rows.
+struct IndexIDMap : Index {
+    Index *index = nullptr;
+    bool own_fields = false;
+    std::vector<idx_t> id_map;
+    explicit IndexIDMap(Index *inner = nullptr) : Index(inner ? inner->d : 0, inner ? inner->metric_type : METRIC_L2), index(inner)
+    {
+        if (inner) {
+            ntotal = inner->ntotal;
+        }
+    }
+    ~IndexIDMap() override
+    {
+        if (own_fields) {
+            delete index;
+        }
+    }
+    void add(idx_t, const float *) override { throw FaissException("add does not make sense with IndexIDMap, use add_with_ids"); }
+    void add_with_ids(idx_t n, const float *x, const idx_t *xids) override
+    {
+        index->add(n, x);
+        id_map.insert(id_map.end(), xids, xids + n);
+        ntotal = index->ntotal;
+    }
+    void search(idx_t, const float *, idx_t, float *, idx_t *, const SearchParameters * = nullptr) const override
+    {
+        throw FaissException("the stand-in IndexIDMap only stores rows and ids");
+    }
+    void reset() override
+    {
+        index->reset();
+        id_map.clear();
+        ntotal = 0;
+    }
 };
 
 struct ProductQuantizer {

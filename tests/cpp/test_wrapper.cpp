@@ -177,6 +177,37 @@ int main(int argc, char **argv)
             flat2.search(1, x.data() + (size_t)5 * d, 1, D.data(), I.data());
             EXPECT(I[0] == 5);
         }
+        // user ids in and out through faiss::IndexIDMap, and the calls with IEEE half inputs
+        {
+            faiss::IndexFlatL2 rows(d);
+            faiss::IndexIDMap with_ids(&rows);
+            std::vector<faiss::idx_t> user_ids(100);
+            for (int i = 0; i < 100; i++) {
+                user_ids[(size_t)i] = 7000 + 3 * i;
+            }
+            with_ids.add_with_ids(100, x.data(), user_ids.data());
+            AscendIndexFlat from_map(&with_ids);
+            EXPECT(from_map.ntotal == 100);
+            from_map.search(1, x.data() + (size_t)9 * d, 1, D.data(), I.data());
+            EXPECT(I[0] == 7027);
+            faiss::IndexFlatL2 rows_back(d);
+            faiss::IndexIDMap back(&rows_back);
+            from_map.copyTo(&back);
+            EXPECT(back.ntotal == 100 && back.id_map == user_ids &&
+                   std::memcmp(rows_back.get_xb(), x.data(), (size_t)100 * d * sizeof(float)) == 0);
+            // halves: 1.0, -2.0, 0.5, the smallest subnormal, 65504
+            EXPECT(ixaHalfToFloat(0x3c00) == 1.0f && ixaHalfToFloat(0xc000) == -2.0f && ixaHalfToFloat(0x3800) == 0.5f &&
+                   ixaHalfToFloat(0x0001) == 5.9604644775390625e-08f && ixaHalfToFloat(0x7bff) == 65504.0f);
+            std::vector<uint16_t> halves((size_t)3 * d, 0x3c00);     // three rows of ones ...
+            halves[(size_t)d] = 0xc000;                              // ... the second starts with -2
+            halves[(size_t)2 * d + 1] = 0x3800;                      // ... the third has a 0.5
+            AscendIndexFlat half_index(d, faiss::METRIC_L2);
+            AscendIndex *half_base = &half_index;
+            half_base->add(3, halves.data());
+            EXPECT(half_index.ntotal == 3);
+            half_base->search(1, halves.data() + (size_t)d, 2, D.data(), I.data());
+            EXPECT(I[0] == 1 && D[0] == 0.f && I[1] == 0 && D[1] == 9.f);
+        }
         // int8: AscendIndexInt8Flat -> AscendIndexInt8
         std::vector<int8_t> b((size_t)4096 * 64);
         for (auto &v : b) {
@@ -191,6 +222,10 @@ int main(int argc, char **argv)
         for (int i = 0; i < 4; i++) {
             EXPECT(Ii[(size_t)i * 3] == i && Di[(size_t)i * 3] == 0.f);
         }
+        std::vector<faiss::idx_t> nearest(4);
+        i8_base->assign(4, b.data(), nearest.data());
+        EXPECT(nearest[0] == 0 && nearest[3] == 3);
+        i8.setPageSize(8);
         EXPECT(i8_base->remove_ids(faiss::IDSelectorRange(1, 3)) == 2 && i8_base->getNTotal() == 4094);
         std::vector<faiss::idx_t> map8;
         i8.getIdxMap(0, map8);
