@@ -87,6 +87,30 @@ public:
         ids.resize(len);
         ixaThrowIfError(ivfpq_get_list(h_, listId, codes.data(), reinterpret_cast<int64_t *>(ids.data())));
     }
+    // remove_ids(const IDSelector &) (FR/ascend/AscendIndex.h:78 -> AscendIndexIVFImpl::removeImpl,
+    // FR/ascend/impl/AscendIndexIVFImpl.cpp:413-460): a batch or a range of ids; lists keep their order.  A
+    // selector of another kind (the reference ignores it) is asked about every stored id.
+    size_t remove_ids(const faiss::IDSelector &sel) override
+    {
+        std::vector<int64_t> ids;
+        int64_t imin = 0, imax = 0, removed = 0;
+        auto allIds = [this](std::vector<idx_t> &m) {
+            m.clear();
+            std::vector<uint8_t> codes;
+            std::vector<ascend_idx_t> listIds;
+            for (int l = 0; l < nlist; l++) {
+                getListCodesAndIds(l, codes, listIds);
+                m.insert(m.end(), listIds.begin(), listIds.end());
+            }
+        };
+        if (ixaSelectorIds(sel, allIds, ids, imin, imax)) {
+            ixaThrowIfError(ivfpq_remove_range(h_, imin, imax, &removed));
+        } else {
+            ixaThrowIfError(ivfpq_remove_ids(h_, (int64_t)ids.size(), ids.data(), &removed));
+        }
+        syncTotal();
+        return (size_t)removed;
+    }
     using AscendIndex::add;            // the IEEE half overloads
     using AscendIndex::add_with_ids;
     using AscendIndex::search;

@@ -52,6 +52,7 @@ public:
         ixaThrowIfError(ivfpq_train(h_, n, x));
         is_trained = true;
     }
+    using AscendIndexIVF::remove_ids;   // by selector
     void remove_ids(size_t n, const idx_t *ids)
     {
         ixaThrowIfError(ivfpq_remove_ids(h_, (int64_t)n, reinterpret_cast<const int64_t *>(ids), nullptr));

@@ -266,6 +266,10 @@ int ivfpq_get_list(const ivfpq_index_t *h, int64_t list, uint8_t *codes, int64_t
 
 /* AscendIndexIVFPQ::remove_ids(n, ids)  FR/ascend/AscendIndexIVFPQ.h:90; *removed may be NULL. */
 int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *removed);
+/* AscendIndex::remove_ids(IDSelectorRange)  FR/ascend/AscendIndex.h:78 -> AscendIndexIVFImpl::removeImpl
+ * (FR/ascend/impl/AscendIndexIVFImpl.cpp:432-440): the vectors whose id lies in [imin, imax) leave; lists keep
+ * the order of their survivors, as with ivfpq_remove_ids. */
+int ivfpq_remove_range(ivfpq_index_t *h, int64_t imin, int64_t imax, int64_t *removed);
 /* AscendIndexIVFPQ::update(n, x, ids)  FR/ascend/AscendIndexIVFPQ.h:92, AscendIndexIVFPQImpl.cpp:540-601:
  * vectors whose id exists are replaced (delete + add); ids that do not exist are written to
  * missing_ids (room for n entries, may be NULL) and counted in *n_missing (may be NULL). */

@@ -115,6 +115,7 @@ _SIGNATURES = {
     "ivfpq_list_length": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
     "ivfpq_get_list": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_remove_ids": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
+    "ivfpq_remove_range": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]),
     "ivfpq_update": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                     ctypes.POINTER(ctypes.c_int64)]),
     "ivfpq_reset": (ctypes.c_int, [_H]),

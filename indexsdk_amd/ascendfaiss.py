@@ -185,6 +185,12 @@ class AscendIndexIVFPQ:
         _capi.check(self._lib.ivfpq_remove_ids(self._h, ids.shape[0], _ptr(ids), ctypes.byref(out)))
         return out.value
 
+    def remove_range(self, imin, imax):
+        """remove_ids(IDSelectorRange(imin, imax)): the vectors whose id lies in [imin, imax); returns how many."""
+        removed = ctypes.c_int64()
+        _capi.check(self._lib.ivfpq_remove_range(self._h, imin, imax, ctypes.byref(removed)))
+        return removed.value
+
     def update(self, x, ids):
         """Replaces the vectors of existing ids; returns the ids that were not found."""
         x = _as(x, np.float32, 2, "x")

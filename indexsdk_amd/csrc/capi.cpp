@@ -279,6 +279,16 @@ IXA_EXPORT int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids,
         }
     });
 }
+IXA_EXPORT int ivfpq_remove_range(ivfpq_index_t *h, int64_t imin, int64_t imax, int64_t *removed)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        const int64_t r = h->impl.remove_range(imin, imax);
+        if (removed) {
+            *removed = r;
+        }
+    });
+}
 IXA_EXPORT int ivfpq_update(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids, int64_t *missing_ids,
                             int64_t *n_missing)
 {

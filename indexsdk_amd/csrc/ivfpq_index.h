@@ -99,6 +99,7 @@ public:
     int64_t list_length(int64_t list) const;
     void get_list(int64_t list, uint8_t *codes, int64_t *ids) const;                    // host pointers
     int64_t remove_ids(int64_t n, const int64_t *ids);
+    int64_t remove_range(int64_t imin, int64_t imax);   // the ids in [imin, imax)
     void reserve_memory(int64_t num_vecs);   // AscendIndexIVF::reserveMemory
     int64_t reclaim_memory();                // AscendIndexIVF::reclaimMemory: bytes released
     // slots allocated / handed out / abandoned by lists that moved (the arena's fill state)
@@ -133,6 +134,8 @@ private:
     void append(int64_t n, const int32_t *list_no_dev, const uint8_t *codes_dev, const int64_t *ids_dev,
                 const float *assigned_from = nullptr);
     int64_t remove_sorted_ids(const std::vector<int64_t> &gone, std::vector<uint8_t> *found);
+    int64_t remove_selected(const std::vector<int64_t> *gone_ids, int64_t imin, int64_t imax,
+                            std::vector<uint8_t> *found);
     void relayout(const std::vector<int32_t> &cap, int64_t min_slots);
     void sync_list_tables();
     void kmeans_coarse(const float *sample_dev, int64_t ns);

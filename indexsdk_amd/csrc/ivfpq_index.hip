@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void remove_ids_kernel(uint8_t *__restrict__ c
                                                          const int64_t *__restrict__ list_off,
                                                          int32_t *__restrict__ list_len, int M, int layout,
                                                          const int64_t *__restrict__ gone, int64_t n_gone,
-                                                         uint8_t *__restrict__ found,
+                                                         int64_t imin, int64_t imax, uint8_t *__restrict__ found,
                                                          unsigned long long *__restrict__ removed)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -155,18 +155,22 @@ __global__ __launch_bounds__(256) void remove_ids_kernel(uint8_t *__restrict__ c
         bool drop = false;
         if (valid) {
             id = ids[off + p];
-            int64_t lo = 0, hi = n_gone;   // first element not below id
-            while (lo < hi) {
-                const int64_t mid = (lo + hi) >> 1;
-                if (gone[mid] < id) {
-                    lo = mid + 1;
-                } else {
-                    hi = mid;
+            if (gone == nullptr) {
+                drop = id >= imin && id < imax;   // removal by id range
+            } else {
+                int64_t lo = 0, hi = n_gone;   // first element not below id
+                while (lo < hi) {
+                    const int64_t mid = (lo + hi) >> 1;
+                    if (gone[mid] < id) {
+                        lo = mid + 1;
+                    } else {
+                        hi = mid;
+                    }
                 }
-            }
-            drop = lo < n_gone && gone[lo] == id;
-            if (drop && found) {
-                found[lo] = 1;
+                drop = lo < n_gone && gone[lo] == id;
+                if (drop && found) {
+                    found[lo] = 1;
+                }
             }
         }
         const bool keep = valid && !drop;
@@ -1093,7 +1097,16 @@ void IvfpqIndex::get_list(int64_t list, uint8_t *codes, int64_t *ids) const
 // UNIQUE id list whether the index held it.
 int64_t IvfpqIndex::remove_sorted_ids(const std::vector<int64_t> &gone, std::vector<uint8_t> *found)
 {
-    if (gone.empty() || ntotal_ == 0) {
+    return remove_selected(&gone, 0, 0, found);
+}
+
+// gone != nullptr: the sorted unique ids to remove; otherwise the ids in [imin, imax) leave.
+int64_t IvfpqIndex::remove_selected(const std::vector<int64_t> *gone_ids, int64_t imin, int64_t imax,
+                                    std::vector<uint8_t> *found)
+{
+    static const std::vector<int64_t> none;
+    const std::vector<int64_t> &gone = gone_ids ? *gone_ids : none;
+    if ((gone_ids ? gone.empty() : imin >= imax) || ntotal_ == 0) {
         if (found) {
             found->assign(gone.size(), 0);
         }
@@ -1102,7 +1115,9 @@ int64_t IvfpqIndex::remove_sorted_ids(const std::vector<int64_t> &gone, std::vec
     DeviceBuffer<int64_t> gone_dev;
     DeviceBuffer<uint8_t> found_dev;
     DeviceBuffer<unsigned long long> removed_dev(1);
-    gone_dev.upload(gone.data(), gone.size(), stream_);
+    if (gone_ids) {
+        gone_dev.upload(gone.data(), gone.size(), stream_);
+    }
     if (found) {
         found_dev.resize(gone.size());
         IXA_HIP(hipMemsetAsync(found_dev.data(), 0, found_dev.bytes(), stream_));
@@ -1110,7 +1125,8 @@ int64_t IvfpqIndex::remove_sorted_ids(const std::vector<int64_t> &gone, std::vec
     IXA_HIP(hipMemsetAsync(removed_dev.data(), 0, 8, stream_));
     const size_t smem = (size_t)256 * M_ + 64;
     hipLaunchKernelGGL(remove_ids_kernel, dim3((unsigned)nlist_), dim3(256), smem, stream_, codes_.data(), ids_.data(),
-                       list_off_dev_.data(), list_len_dev_.data(), M_, layout_, gone_dev.data(), (int64_t)gone.size(),
+                       list_off_dev_.data(), list_len_dev_.data(), M_, layout_,
+                       gone_ids ? gone_dev.data() : (const int64_t *)nullptr, (int64_t)gone.size(), imin, imax,
                        found ? found_dev.data() : nullptr, removed_dev.data());
     unsigned long long removed = 0;
     removed_dev.download(&removed, 1, stream_);
@@ -1137,6 +1153,13 @@ int64_t IvfpqIndex::remove_ids(int64_t n, const int64_t *ids)
     std::sort(gone.begin(), gone.end());
     gone.erase(std::unique(gone.begin(), gone.end()), gone.end());
     return remove_sorted_ids(gone, nullptr);
+}
+
+// remove_ids(IDSelectorRange) (FR/ascend/impl/AscendIndexIVFImpl.cpp:432-440): the ids in [imin, imax) leave
+int64_t IvfpqIndex::remove_range(int64_t imin, int64_t imax)
+{
+    flush_stats();
+    return remove_selected(nullptr, imin, imax, nullptr);
 }
 
 // update (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:540-601): ids that exist are deleted and re-added with

@@ -102,6 +102,24 @@ int main(int argc, char **argv)
         other.search(nq, x.data(), k, D2.data(), I2.data());
         EXPECT(I2 == I && D2 == D);
         std::remove(path.c_str());
+        {
+            // remove_ids(const IDSelector &) on the second object, through the root of the hierarchy
+            faiss::Index *other_root = &other;
+            EXPECT(other_root->remove_ids(faiss::IDSelectorRange(10, 20)) == 10 && other.ntotal == n - 10);
+            const faiss::idx_t some[] = {0, 5, 15, 5};      // 15 has left already
+            EXPECT(other_root->remove_ids(faiss::IDSelectorBatch(4, some)) == 2 && other.ntotal == n - 12);
+            struct EndsIn77 : faiss::IDSelector {
+                bool is_member(faiss::idx_t id) const override { return id % 100 == 77; }
+            };
+            EXPECT(other_root->remove_ids(EndsIn77()) == (size_t)((n - 78) / 100 + 1));
+            other.search(nq, x.data(), k, D2.data(), I2.data());
+            bool none_left = true;
+            for (size_t i = 0; i < I2.size(); i++) {
+                const faiss::idx_t id = I2[i];
+                none_left = none_left && !(id >= 10 && id < 20) && id != 0 && id != 5 && id % 100 != 77;
+            }
+            EXPECT(none_left && I2[0] >= 0);
+        }
         AscendIndexIVFPQ wrong(d, faiss::METRIC_L2, 2048, M, 8, conf);
         bool threw = false;
         try {

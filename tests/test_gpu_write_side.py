@@ -166,3 +166,30 @@ def test_many_small_adds_extend_lists_in_place(oracle):
     assert released > 0
     _check(gpu, model, range(0, nlist, 7))
     assert gpu.arena_state()[2] == 0
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_remove_by_id_range_equals_removing_those_ids(oracle, layout):
+    """remove_ids(IDSelectorRange) (FR/ascend/impl/AscendIndexIVFImpl.cpp:432-440): the vectors whose id lies in
+    [imin, imax) leave, every list keeps the order of its survivors, with a position-dependent code layout too;
+    an empty or inverted range removes nothing."""
+    import indexsdk_amd as ix
+    d, M, nlist, n = 64, 32, 64, 60000
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    cent, _ = oracle.kmeans(x[:8000], nlist, niter=3, seed=3)
+    cb = oracle.train_pq(x[:4000], M, niter=2, seed=3)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(code_layout=layout))
+    gpu.set_trained(cent, cb)
+    ids = rng.permutation(4 * n)[:n].astype(np.int64)
+    gpu.add_with_ids(x, ids)
+    model = ListModel(nlist, M)
+    model.add(oracle.assign(x, cent), oracle.pq_encode(x, cb), ids)
+    assert gpu.remove_range(500, 500) == 0 and gpu.remove_range(900, 100) == 0
+    lo, hi = 30000, 90000
+    victims = ids[(ids >= lo) & (ids < hi)]
+    assert len(victims) > 10000
+    assert gpu.remove_range(lo, hi) == model.remove(victims) == len(victims)
+    _check(gpu, model, range(nlist))
+    assert gpu.remove_range(lo, hi) == 0
+    assert gpu.remove_range(-10, 10 * n) == model.ntotal and gpu.ntotal == 0
