@@ -3,10 +3,12 @@
 // tiny train/add/search through the class interface.
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <random>
 #include <string>
 #include <vector>
 
+#include "ascend/AscendCloner.h"
 #include "ascend/AscendIndexFlat.h"
 #include "ascend/AscendIndexIVFPQ.h"
 
@@ -225,6 +227,42 @@ int main(int argc, char **argv)
             EXPECT(half_index.ntotal == 3);
             half_base->search(1, halves.data() + (size_t)d, 2, D.data(), I.data());
             EXPECT(I[0] == 1 && D[0] == 0.f && I[1] == 0 && D[1] == 9.f);
+        }
+        // the cloner: device -> CPU -> device, Flat (ids travel in an IndexIDMap) and IVFPQ
+        {
+            std::unique_ptr<faiss::Index> cpu_copy(index_ascend_to_cpu(&flat));
+            auto *as_map = dynamic_cast<faiss::IndexIDMap *>(cpu_copy.get());
+            EXPECT(as_map != nullptr && as_map->ntotal == n && as_map->own_fields && (faiss::idx_t)as_map->id_map.size() == n &&
+                   as_map->id_map[7] == 7);
+            std::unique_ptr<faiss::Index> device_copy(index_cpu_to_ascend({0}, cpu_copy.get()));
+            EXPECT(dynamic_cast<AscendIndexFlat *>(device_copy.get()) != nullptr && device_copy->ntotal == n);
+            device_copy->search(nq, x.data(), k, D.data(), I.data());
+            for (int i = 0; i < nq; i++) {
+                EXPECT(I[(size_t)i * k] == i);
+            }
+            std::unique_ptr<faiss::Index> pq_cpu(index_ascend_to_cpu(&index));
+            EXPECT(dynamic_cast<faiss::IndexIVFPQ *>(pq_cpu.get()) != nullptr && pq_cpu->ntotal == n);
+            AscendClonerOptions options;
+            options.reserveVecs = 1000;
+            std::unique_ptr<faiss::Index> pq_device(index_cpu_to_ascend(std::vector<int>{0}, pq_cpu.get(), &options));
+            auto *pq_again = dynamic_cast<AscendIndexIVFPQ *>(pq_device.get());
+            EXPECT(pq_again != nullptr && pq_again->ntotal == n && pq_again->getNumProbes() == 32);
+            std::vector<float> Dc((size_t)nq * k);
+            std::vector<faiss::idx_t> Ic((size_t)nq * k);
+            index.search(nq, x.data(), k, D.data(), I.data());
+            pq_again->search(nq, x.data(), k, Dc.data(), Ic.data());
+            EXPECT(Ic == I && Dc == D);
+            bool refused = false;
+            try {
+                AscendIndexInt8Flat not_cloneable(64);
+                faiss::IndexFlatL2 other_kind(8);
+                faiss::IndexIDMap map_over_map(&other_kind);
+                faiss::IndexIDMap outer(&map_over_map);
+                index_cpu_to_ascend({0}, &outer);
+            } catch (const faiss::FaissException &e) {
+                refused = std::string(e.what()).find("not supported") != std::string::npos;
+            }
+            EXPECT(refused);
         }
         // int8: AscendIndexInt8Flat -> AscendIndexInt8
         std::vector<int8_t> b((size_t)4096 * 64);
