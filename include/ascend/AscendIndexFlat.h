@@ -134,6 +134,18 @@ public:
     {
         ixaThrowIfError(flat_search(h_, n, x, k, distances, reinterpret_cast<int64_t *>(labels)));
     }
+    // search_with_masks (FR/ascend/AscendIndexFlat.h:78-82): query i may only return the vectors whose bit
+    // is set in row i of the mask (n rows of ceil(ntotal / 8) bytes; storage position p = bit p % 8 of byte p / 8)
+    void search_with_masks(idx_t n, const float *x, idx_t k, float *distances, idx_t *labels, const void *mask) const
+    {
+        ixaThrowIfError(flat_search_with_masks(h_, n, x, k, static_cast<const uint8_t *>(mask), distances,
+                                               reinterpret_cast<int64_t *>(labels)));
+    }
+    void search_with_masks(idx_t n, const uint16_t *x, idx_t k, float *distances, idx_t *labels, const void *mask) const
+    {
+        const std::vector<float> wide = ixaWiden(n, x);
+        search_with_masks(n, wide.data(), k, distances, labels, mask);
+    }
     void reset() override
     {
         ixaThrowIfError(flat_reset(h_));
@@ -221,6 +233,16 @@ public:
     void searchInt32(idx_t n, const int8_t *x, idx_t k, int32_t *distances, idx_t *labels) const
     {
         ixaThrowIfError(flat_i8_search(h_, n, x, k, distances, reinterpret_cast<int64_t *>(labels)));
+    }
+    // search_with_masks (FR/ascend/AscendIndexInt8Flat.h:98-99), float distances like search()
+    void search_with_masks(idx_t n, const int8_t *x, idx_t k, float *distances, idx_t *labels, const void *mask) const
+    {
+        std::vector<int32_t> tmp((size_t)n * k);
+        ixaThrowIfError(flat_i8_search_with_masks(h_, n, x, k, static_cast<const uint8_t *>(mask), tmp.data(),
+                                                  reinterpret_cast<int64_t *>(labels)));
+        for (size_t i = 0; i < tmp.size(); i++) {
+            distances[i] = labels[i] < 0 ? FLT_MAX : (float)tmp[i];
+        }
     }
     size_t getBaseSize(int /*deviceId*/ = 0) const { return (size_t)ntotal; }
     void getBase(int /*deviceId*/, std::vector<int8_t> &xb) const

@@ -363,6 +363,13 @@ int flat_add_with_ids_device(flat_index_t *h, int64_t n, const float *x_dev, con
 int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels);
 int flat_search_device(flat_index_t *h, int64_t n, const float *x_dev, int64_t k, float *distances_dev,
                        int64_t *labels_dev);
+/* AscendIndexFlat::search_with_masks  FR/ascend/AscendIndexFlat.h:78-82 (FR/ascend/impl/AscendIndexFlatImpl.cpp:461-511):
+ * mask = n rows of ceil(ntotal / 8) bytes in host memory; query i may only return the vectors whose bit is
+ * set in row i (the vector at storage position p: bit p % 8 of byte p / 8).  Results as flat_search on the
+ * vectors that take part; fewer than k of them leave (FLT_MAX | -FLT_MAX, -1).  Every stretch of the score
+ * matrix is written and masked before the selection reads it, so this is slower than flat_search. */
+int flat_search_with_masks(flat_index_t *h, int64_t n, const float *x, int64_t k, const uint8_t *mask, float *distances,
+                           int64_t *labels);
 /* AscendIndexFlat::getBase / getBaseSize  FR/ascend/AscendIndexFlat.h; rows [offset, offset + n). */
 int flat_get_base(const flat_index_t *h, int64_t offset, int64_t n, float *out);
 int flat_get_ids(const flat_index_t *h, int64_t offset, int64_t n, int64_t *out);
@@ -391,6 +398,10 @@ int flat_i8_add_with_ids_device(flat_i8_index_t *h, int64_t n, const int8_t *x_d
 int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances, int64_t *labels);
 int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x_dev, int64_t k, int32_t *distances_dev,
                           int64_t *labels_dev);
+/* AscendIndexInt8Flat::search_with_masks  FR/ascend/AscendIndexInt8Flat.h:98-99; as flat_search_with_masks
+ * (missing results: distance INT32_MAX, label -1). */
+int flat_i8_search_with_masks(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, const uint8_t *mask,
+                              int32_t *distances, int64_t *labels);
 int flat_i8_get_base(const flat_i8_index_t *h, int64_t offset, int64_t n, int8_t *out);
 /* AscendIndexInt8Flat::getIdxMap  FR/ascend/AscendIndexInt8Flat.h:83 */
 int flat_i8_get_ids(const flat_i8_index_t *h, int64_t offset, int64_t n, int64_t *out);

@@ -132,6 +132,8 @@ for _pfx, _dist in (("flat", ctypes.c_void_p), ("flat_i8", ctypes.c_void_p)):
         f"{_pfx}_add_with_ids_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
         f"{_pfx}_search": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, _dist,
                                           ctypes.c_void_p]),
+        f"{_pfx}_search_with_masks": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                                     _dist, ctypes.c_void_p]),
         f"{_pfx}_search_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, _dist,
                                                  ctypes.c_void_p]),
         f"{_pfx}_get_base": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]),

@@ -342,6 +342,18 @@ class AscendIndexFlat(_FlatCommon):
         return D, I
 
 
+    def search_with_masks(self, x, k, mask):
+        """search_with_masks (FR/ascend/AscendIndexFlat.h:78-82): mask uint8 [n, ceil(ntotal / 8)], bit p % 8 of
+        byte p / 8 of row i set = query i may return the vector at storage position p."""
+        x = _as(x, np.float32, 2, "x")
+        mask = _as(mask, np.uint8, 2, "mask")
+        assert x.shape[1] == self.d and mask.shape == (x.shape[0], (self.ntotal + 7) // 8)
+        D = np.empty((x.shape[0], k), dtype=np.float32)
+        I = np.empty((x.shape[0], k), dtype=np.int64)
+        _capi.check(self._lib.flat_search_with_masks(self._h, x.shape[0], _ptr(x), k, _ptr(mask), _ptr(D), _ptr(I)))
+        return D, I
+
+
 class AscendIndexFlatL2(AscendIndexFlat):
     def __init__(self, dims, scratch_bytes=0):
         super().__init__(dims, METRIC_L2, scratch_bytes)
@@ -360,6 +372,16 @@ class AscendIndexInt8Flat(_FlatCommon):
         D = np.empty((x.shape[0], k), dtype=np.int32)
         I = np.empty((x.shape[0], k), dtype=np.int64)
         _capi.check(self._lib.flat_i8_search(self._h, x.shape[0], _ptr(x), k, _ptr(D), _ptr(I)))
+        return D, I
+
+    def search_with_masks_int32(self, x, k, mask):
+        """search_with_masks (FR/ascend/AscendIndexInt8Flat.h:98-99) with the exact int32 distances."""
+        x = _as(x, np.int8, 2, "x")
+        mask = _as(mask, np.uint8, 2, "mask")
+        assert x.shape[1] == self.d and mask.shape == (x.shape[0], (self.ntotal + 7) // 8)
+        D = np.empty((x.shape[0], k), dtype=np.int32)
+        I = np.empty((x.shape[0], k), dtype=np.int64)
+        _capi.check(self._lib.flat_i8_search_with_masks(self._h, x.shape[0], _ptr(x), k, _ptr(mask), _ptr(D), _ptr(I)))
         return D, I
 
     def search(self, x, k):

@@ -586,6 +586,11 @@ IXA_EXPORT int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
 }
+IXA_EXPORT int flat_search_with_masks(flat_index_t *h, int64_t n, const float *x, int64_t k, const uint8_t *mask,
+                                      float *distances, int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search_with_masks(n, x, k, mask, distances, labels); });
+}
 IXA_EXPORT int flat_search_device(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances,
                                   int64_t *labels)
 {
@@ -595,6 +600,11 @@ IXA_EXPORT int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, in
                               int64_t *labels)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+}
+IXA_EXPORT int flat_i8_search_with_masks(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, const uint8_t *mask,
+                                         int32_t *distances, int64_t *labels)
+{
+    return guarded([&] { IXA_HANDLE(h); h->impl.search_with_masks(n, x, k, mask, distances, labels); });
 }
 IXA_EXPORT int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances,
                                      int64_t *labels)

@@ -651,7 +651,7 @@ void FlatIndex::add(int64_t n, const float *x, const int64_t *ids, bool on_devic
 // Exact plan of last resort (queries whose candidate list cannot be proven complete): canonical scores
 // of the whole base, chunk by chunk, with an exact running selection.
 void FlatIndex::exact_rows(const float *xd, const std::vector<int64_t> &rows, int64_t k, float *dist_dev,
-                           int64_t *labels_dev)
+                           int64_t *labels_dev, const uint8_t *mask_dev, int64_t mask_stride)
 {
     const int64_t total_rows = (int64_t)rows.size();
     DeviceBuffer<int64_t> rows_dev;
@@ -676,7 +676,13 @@ void FlatIndex::exact_rows(const float *xd, const std::vector<int64_t> &rows, in
             const int64_t nc = std::min(cols, ntotal_ - c0);
             launch_canonical_scores(xsub.data(), m, base_.data() + c0 * d_, nc, d_, qn.data(), norms_.data() + c0, metric_,
                                     scores.data(), nc, stream_);
+            if (mask_dev) {
+                launch_apply_mask(scores.data(), m, nc, nc, mask_dev, mask_stride, rows_dev.data() + r0, c0, stream_);
+            }
             launch_select_rows(scores.data(), m, nc, nc, (int)k, nullptr, c0, running.data(), stream_);
+        }
+        if (mask_dev) {
+            launch_drop_worst_keys_f32(running.data(), m * k, stream_);
         }
         const float pad = metric_ == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
         hipLaunchKernelGGL((finish_keys_kernel<float, float>), dim3(blocks_for(m * k)), dim3(256), 0, stream_,
@@ -709,6 +715,35 @@ int64_t FlatIndex::remove_range(int64_t imin, int64_t imax)
 // are re-evaluated in the canonical scalar arithmetic before the final top-k is written.
 void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
 {
+    search_masked(n, x, k, dist, labels, on_device, nullptr, 0);
+}
+
+// search_with_masks (FR/ascend/AscendIndexFlat.h:78-82; FR/ascend/impl/AscendIndexFlatImpl.cpp:461-511): row i of
+// the mask (ceil(ntotal / 8) bytes, host memory) says which base vectors query i may return: bit p % 8 of
+// byte p / 8 set = the vector at position p takes part.  Queries go in pages whose masks fit a bounded
+// device buffer.
+void FlatIndex::search_with_masks(int64_t n, const float *x, int64_t k, const uint8_t *mask, float *dist, int64_t *labels)
+{
+    IXA_REQUIRE(mask, kErrInvalidParam, "mask cannot be nullptr.");
+    IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    const int64_t stride = (ntotal_ + 7) / 8;
+    if (stride == 0) {
+        search_masked(n, x, k, dist, labels, false, nullptr, 0);
+        return;
+    }
+    const int64_t page = std::max<int64_t>(1, std::min<int64_t>(n, kMaskPageBytes / stride));
+    DeviceBuffer<uint8_t> mask_dev;
+    for (int64_t q0 = 0; q0 < n; q0 += page) {
+        const int64_t nq = std::min(page, n - q0);
+        mask_dev.upload(mask + q0 * stride, (size_t)(nq * stride), stream_);
+        search_masked(nq, x + q0 * d_, k, dist + q0 * k, labels + q0 * k, false, mask_dev.data(), stride);
+    }
+}
+
+void FlatIndex::search_masked(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device,
+                              const uint8_t *mask_dev, int64_t mask_stride)
+{
     IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
@@ -733,7 +768,11 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
     IXA_HIP(hipEventRecord(ev_[0], stream_));
     launch_sqnorm_rows(xd, n, d_, ws_qn_.data(), stream_);
     const int launches = stream_select_f32(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), metric_,
-                                           ncand, ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
+                                           ncand, ws_running_.data(), ws_sel_, scratch_bytes_, stream_, mask_dev,
+                                           mask_stride);
+    if (mask_dev) {
+        launch_drop_worst_keys_f32(ws_running_.data(), n * ncand, stream_);   // vectors the query leaves out
+    }
     IXA_HIP(hipEventRecord(ev_[1], stream_));
     launch_keys_to_idx(ws_running_.data(), n * ncand, ws_cand_.data(), stream_);
     launch_refine(xd, n, base_.data(), d_, ws_qn_.data(), norms_.data(), metric_, ws_cand_.data(), ncand,
@@ -761,7 +800,7 @@ void FlatIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64_
             IXA_HIP(hipMemcpyAsync(rows32.data(), ws_flag_.data() + 1, (size_t)nfail * 4, hipMemcpyDeviceToHost, stream_));
             sync_stream(stream_);
             std::sort(rows32.begin(), rows32.end());
-            exact_rows(xd, std::vector<int64_t>(rows32.begin(), rows32.end()), k, dd, ld);
+            exact_rows(xd, std::vector<int64_t>(rows32.begin(), rows32.end()), k, dd, ld, mask_dev, mask_stride);
             stats_.exact_reruns = nfail;
         }
     }
@@ -821,6 +860,33 @@ void FlatI8Index::reset()
 
 void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device)
 {
+    search_masked(n, x, k, dist, labels, on_device, nullptr, 0);
+}
+
+// search_with_masks (FR/ascend/AscendIndexInt8Flat.h:98-99): as FlatIndex::search_with_masks
+void FlatI8Index::search_with_masks(int64_t n, const int8_t *x, int64_t k, const uint8_t *mask, int32_t *dist,
+                                    int64_t *labels)
+{
+    IXA_REQUIRE(mask, kErrInvalidParam, "mask cannot be nullptr.");
+    IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
+    IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
+    const int64_t stride = (ntotal_ + 7) / 8;
+    if (stride == 0) {
+        search_masked(n, x, k, dist, labels, false, nullptr, 0);
+        return;
+    }
+    const int64_t page = std::max<int64_t>(1, std::min<int64_t>(n, kMaskPageBytes / stride));
+    DeviceBuffer<uint8_t> mask_dev;
+    for (int64_t q0 = 0; q0 < n; q0 += page) {
+        const int64_t nq = std::min(page, n - q0);
+        mask_dev.upload(mask + q0 * stride, (size_t)(nq * stride), stream_);
+        search_masked(nq, x + q0 * d_, k, dist + q0 * k, labels + q0 * k, false, mask_dev.data(), stride);
+    }
+}
+
+void FlatI8Index::search_masked(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device,
+                                const uint8_t *mask_dev, int64_t mask_stride)
+{
     IXA_REQUIRE(x && dist && labels, kErrInvalidParam, "x, distances and labels can not be nullptr.");
     IXA_REQUIRE(n > 0 && n < kMaxN, kErrInvalidParam, "n must be > 0 and < %ld", (long)kMaxN);
     IXA_REQUIRE(k > 0 && k <= kMaxK, kErrInvalidParam, "k must be > 0 and <= %ld", (long)kMaxK);
@@ -843,7 +909,10 @@ void FlatI8Index::search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, i
     hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_, xd, n, d_,
                        ws_qn_.data());
     const int launches = stream_select_i8(xd, n, base_.data(), ntotal_, d_, ws_qn_.data(), norms_.data(), (int)k,
-                                          ws_running_.data(), ws_sel_, scratch_bytes_, stream_);
+                                          ws_running_.data(), ws_sel_, scratch_bytes_, stream_, mask_dev, mask_stride);
+    if (mask_dev) {
+        launch_drop_worst_keys_i32(ws_running_.data(), n * k, stream_);   // vectors the query leaves out
+    }
     hipLaunchKernelGGL((finish_keys_kernel<int32_t, int32_t>), dim3(blocks_for(n * k)), dim3(256), 0, stream_,
                        ws_running_.data(), n * k, kMetricL2, ids_.data(), (int32_t)0x7fffffff, dd, ld);
     IXA_HIP(hipEventRecord(ev_[1], stream_));

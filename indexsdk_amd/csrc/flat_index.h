@@ -14,6 +14,8 @@
 
 namespace ixa {
 
+constexpr int64_t kMaskPageBytes = (int64_t)256 << 20;   // masks of one query page of a masked search
+
 struct FlatStats {
     double ms_score = 0;        // all score-tile launches of the last search
     double ms_select = 0;       // all selection launches (+ refine / finalisation)
@@ -61,13 +63,18 @@ public:
     FlatIndex(int d, int metric, int64_t scratch_bytes);
     void add(int64_t n, const float *x, const int64_t *ids, bool on_device);
     void search(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
+    // host pointers; mask: n rows of ceil(ntotal / 8) bytes, bit set = the vector at that position takes part
+    void search_with_masks(int64_t n, const float *x, int64_t k, const uint8_t *mask, float *dist, int64_t *labels);
     int64_t remove_ids(int64_t n, const int64_t *ids);       // host ids; returns the number of vectors removed
     int64_t remove_range(int64_t imin, int64_t imax);        // ids in [imin, imax)
     void reset();
 
 private:
     // exact results for the listed query rows, from canonical scores of the whole base
-    void exact_rows(const float *xd, const std::vector<int64_t> &rows, int64_t k, float *dist_dev, int64_t *labels_dev);
+    void exact_rows(const float *xd, const std::vector<int64_t> &rows, int64_t k, float *dist_dev, int64_t *labels_dev,
+                    const uint8_t *mask_dev, int64_t mask_stride);
+    void search_masked(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device,
+                       const uint8_t *mask_dev, int64_t mask_stride);
     DeviceBuffer<float> norms_, ws_qn_, ws_dist_;
     StreamSelectWorkspace<float> ws_sel_;
     DeviceBuffer<int32_t> ws_cand_, ws_idx_, ws_flag_;
@@ -80,11 +87,14 @@ public:
     FlatI8Index(int d, int metric, int64_t scratch_bytes);
     void add(int64_t n, const int8_t *x, const int64_t *ids, bool on_device);
     void search(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device);
+    void search_with_masks(int64_t n, const int8_t *x, int64_t k, const uint8_t *mask, int32_t *dist, int64_t *labels);
     int64_t remove_ids(int64_t n, const int64_t *ids);
     int64_t remove_range(int64_t imin, int64_t imax);
     void reset();
 
 private:
+    void search_masked(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device,
+                       const uint8_t *mask_dev, int64_t mask_stride);
     DeviceBuffer<int32_t> norms_, ws_qn_, ws_dist_;
     StreamSelectWorkspace<int32_t> ws_sel_;
     DeviceBuffer<int64_t> ws_labels_;

@@ -21,9 +21,14 @@ struct StreamSelectWorkspace {
 // ncand-th score and the admitted keys are merged.  If a query ever admits more keys than its
 // buffer holds (adversarial base order), the whole selection is redone through the scratch.
 // Returns the number of score launches.
+// With a mask (device memory, one row of mask_stride bytes per query row, bit b % 8 of byte b / 8 set = base row b
+// takes part; AscendIndexFlat::search_with_masks, FR/ascend/AscendIndexFlat.h:78-82) every stretch of the
+// score matrix is materialised and the scores of the rows a query leaves out are overwritten with the
+// worst score before the selection reads them; keys with that score may come back when fewer than ncand
+// rows take part (the caller drops them).
 int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn, const float *bn,
                       int metric, int ncand, unsigned long long *running, StreamSelectWorkspace<float> &ws,
-                      int64_t scratch_bytes, hipStream_t s);
+                      int64_t scratch_bytes, hipStream_t s, const uint8_t *mask = nullptr, int64_t mask_stride = 0);
 // Same selection with approximate scores: Qs / Bs are the bf16 x 3 splits of the operands (rows of d3
 // bf16 elements, see launch_split_bf16x3), qn / bn the exact fp32 norms.  Returns -1 without doing
 // anything when the shape does not qualify for the bf16 matrix-core kernel.
@@ -51,7 +56,17 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq, const uint16_t 
                                  const BoundaryRefine *refine, hipStream_t s);
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
-                     int64_t scratch_bytes, hipStream_t s);
+                     int64_t scratch_bytes, hipStream_t s, const uint8_t *mask = nullptr, int64_t mask_stride = 0);
+
+// scores[r][c] (nq rows of ld, columns [0, nc) standing for base rows col0 + c) = the worst score wherever bit
+// col0 + c of the row's mask is clear; the mask row of score row r is row_map[r], or r without a map.
+void launch_apply_mask(float *scores, int64_t nq, int64_t ld, int64_t nc, const uint8_t *mask, int64_t mask_stride,
+                       const int64_t *row_map, int64_t col0, hipStream_t s);
+void launch_apply_mask(int32_t *scores, int64_t nq, int64_t ld, int64_t nc, const uint8_t *mask, int64_t mask_stride,
+                       const int64_t *row_map, int64_t col0, hipStream_t s);
+// keys[i] = kEmptyKey where its score is the worst score of S (float: +inf, int32: INT32_MAX)
+void launch_drop_worst_keys_f32(unsigned long long *keys, int64_t n, hipStream_t s);
+void launch_drop_worst_keys_i32(unsigned long long *keys, int64_t n, hipStream_t s);
 
 // idx[i] = row index of keys[i], or -1 for an empty key.
 void launch_keys_to_idx(const unsigned long long *keys, int64_t n, int32_t *idx, hipStream_t s);

@@ -44,6 +44,57 @@ __global__ __launch_bounds__(256) void threshold_i32_kernel(const int32_t *__res
     }
 }
 
+// One thread per (score row, mask byte): the eight base rows of the byte, those inside the stretch.
+template <typename S>
+__global__ __launch_bounds__(256) void apply_mask_kernel(S *__restrict__ scores, int64_t nq, int64_t ld, int64_t nc,
+                                                         const uint8_t *__restrict__ mask, int64_t stride,
+                                                         const int64_t *__restrict__ row_map, int64_t col0,
+                                                         int64_t first_byte, int64_t nbytes)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= nq * nbytes) {
+        return;
+    }
+    const int64_t r = i / nbytes, b = first_byte + i % nbytes;
+    const uint8_t m = mask[(row_map ? row_map[r] : r) * stride + b];
+    if (m == 0xff) {
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        const int64_t c = (b << 3) + t - col0;
+        if (c >= 0 && c < nc && !((m >> t) & 1)) {
+            scores[r * ld + c] = ScoreOps<S>::worst();
+        }
+    }
+}
+
+template <typename S>
+void apply_mask(S *scores, int64_t nq, int64_t ld, int64_t nc, const uint8_t *mask, int64_t stride,
+                const int64_t *row_map, int64_t col0, hipStream_t s)
+{
+    if (nq <= 0 || nc <= 0) {
+        return;
+    }
+    const int64_t first_byte = col0 >> 3, nbytes = ((col0 + nc + 7) >> 3) - first_byte;
+    IXA_REQUIRE(mask != nullptr && ((col0 + nc + 7) >> 3) <= stride, kErrInner,
+                "mask rows of %ld bytes do not cover base rows up to %ld", (long)stride, (long)(col0 + nc));
+    hipLaunchKernelGGL(apply_mask_kernel<S>, dim3(blocks_for(nq * nbytes)), dim3(256), 0, s, scores, nq, ld, nc, mask,
+                       stride, row_map, col0, first_byte, nbytes);
+}
+
+template <typename S>
+__global__ __launch_bounds__(256) void drop_worst_keys_kernel(key_t *__restrict__ keys, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const key_t kk = keys[i];
+        if (kk != kEmptyKey && key_score_as<S>(kk) == ScoreOps<S>::worst()) {
+            keys[i] = kEmptyKey;
+        }
+    }
+}
+
 struct F32Ops {
     using T = float;
     using S = float;
@@ -138,7 +189,7 @@ struct I8Ops {
 template <typename Ops>
 int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, const typename Ops::T *B, int64_t nb_total,
                   int d, int ncand, key_t *running, StreamSelectWorkspace<typename Ops::S> &ws, int64_t scratch_bytes,
-                  hipStream_t s)
+                  hipStream_t s, const uint8_t *mask = nullptr, int64_t mask_stride = 0)
 {
     using S = typename Ops::S;
     if (nq_total == 0) {
@@ -161,7 +212,9 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     // when the whole score matrix of a query block fits the scratch, one materialised pass is the
     // cheapest plan (measured on the IVFPQ coarse stage: 16384 centroids); the filtered plan is for
     // long bases
-    bool can_fuse = nb_total > nb && nb_total >= 4 * seed_rows && pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
+    // (a masked search materialises every stretch: the mask is applied to the stored scores)
+    bool can_fuse = mask == nullptr && nb_total > nb && nb_total >= 4 * seed_rows &&
+                    pow2_ceil(ncand + cap) * sizeof(key_t) <= 160 * 1024;
     if (can_fuse && qb * (int64_t)cap * (int64_t)sizeof(key_t) > scratch_bytes) {
         // the candidate buffers of a query block count against the scratch budget too: a narrower block
         qb = std::max<int64_t>(128, scratch_bytes / ((int64_t)cap * (int64_t)sizeof(key_t)) / 128 * 128);
@@ -224,6 +277,9 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             for (int64_t b0 = 0; b0 < head; b0 += ldo) {
                 const int64_t nbc = std::min(ldo, head - b0);
                 ops.scores(Q + q0 * d, nq, q0, B + b0 * d, nbc, b0, d, ws.scores.data(), ldo, s);
+                if (mask) {
+                    apply_mask(ws.scores.data(), nq, ldo, nbc, mask + q0 * mask_stride, mask_stride, nullptr, b0, s);
+                }
                 // the first chunk of a query block starts its running keys (whatever `running` held)
                 ops.select(ws.scores.data(), nq, ldo, nbc, ncand, b0, running + q0 * ncand, b0 == 0, s);
                 launches++;
@@ -262,9 +318,33 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
 
 int stream_select_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn, const float *bn,
                       int metric, int ncand, unsigned long long *running, StreamSelectWorkspace<float> &ws,
-                      int64_t scratch_bytes, hipStream_t s)
+                      int64_t scratch_bytes, hipStream_t s, const uint8_t *mask, int64_t mask_stride)
 {
-    return stream_select(F32Ops{qn, bn, metric}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s);
+    return stream_select(F32Ops{qn, bn, metric}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s, mask,
+                         mask_stride);
+}
+
+void launch_apply_mask(float *scores, int64_t nq, int64_t ld, int64_t nc, const uint8_t *mask, int64_t mask_stride,
+                       const int64_t *row_map, int64_t col0, hipStream_t s)
+{
+    apply_mask(scores, nq, ld, nc, mask, mask_stride, row_map, col0, s);
+}
+void launch_apply_mask(int32_t *scores, int64_t nq, int64_t ld, int64_t nc, const uint8_t *mask, int64_t mask_stride,
+                       const int64_t *row_map, int64_t col0, hipStream_t s)
+{
+    apply_mask(scores, nq, ld, nc, mask, mask_stride, row_map, col0, s);
+}
+void launch_drop_worst_keys_f32(unsigned long long *keys, int64_t n, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(drop_worst_keys_kernel<float>, dim3(blocks_for(n)), dim3(256), 0, s, keys, n);
+    }
+}
+void launch_drop_worst_keys_i32(unsigned long long *keys, int64_t n, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(drop_worst_keys_kernel<int32_t>, dim3(blocks_for(n)), dim3(256), 0, s, keys, n);
+    }
 }
 
 int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3, const float *qn,
@@ -367,9 +447,9 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uin
 
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
-                     int64_t scratch_bytes, hipStream_t s)
+                     int64_t scratch_bytes, hipStream_t s, const uint8_t *mask, int64_t mask_stride)
 {
-    return stream_select(I8Ops{qn, bn}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s);
+    return stream_select(I8Ops{qn, bn}, Q, nq, B, nb, d, ncand, running, ws, scratch_bytes, s, mask, mask_stride);
 }
 
 void launch_keys_to_idx(const unsigned long long *keys, int64_t n, int32_t *idx, hipStream_t s)

@@ -1,6 +1,7 @@
 // Host-side check of the C++ wrappers: constructor validation messages as in
 // FR/ut/TestAscendIndexUTIVFPQ.cpp:77-184.  With a GPU present (argv[1] == "gpu") it also runs a
 // tiny train/add/search through the class interface.
+#include <cfloat>
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -277,6 +278,20 @@ int main(int argc, char **argv)
         i8_base->search(4, b.data(), 3, Di.data(), Ii.data());
         for (int i = 0; i < 4; i++) {
             EXPECT(Ii[(size_t)i * 3] == i && Di[(size_t)i * 3] == 0.f);
+        }
+        {
+            // masks: the query that is base vector 0 may only see vectors 8..15 -> its nearest comes from there
+            std::vector<uint8_t> mask((size_t)4096 / 8, 0);
+            mask[1] = 0xff;
+            i8.search_with_masks(1, b.data(), 3, Di.data(), Ii.data(), mask.data());
+            EXPECT(Ii[0] >= 8 && Ii[0] < 16 && Ii[1] >= 8 && Ii[1] < 16 && Di[0] > 0.f && Di[0] <= Di[1]);
+            mask[0] = 0x01;
+            i8.search_with_masks(1, b.data(), 3, Di.data(), Ii.data(), mask.data());
+            EXPECT(Ii[0] == 0 && Di[0] == 0.f);
+            std::vector<uint8_t> fmask((size_t)(n + 7) / 8, 0);
+            fmask[0] = 0x04;                                  // only vector 2
+            flat.search_with_masks(1, x.data(), 2, D.data(), I.data(), fmask.data());
+            EXPECT(I[0] == 2 && I[1] == -1 && D[1] == FLT_MAX);
         }
         std::vector<faiss::idx_t> nearest(4);
         i8_base->assign(4, b.data(), nearest.data());

@@ -305,3 +305,64 @@ def test_flat_remove_ids_follows_the_reference_order(ix, oracle, kind):
     else:
         D, I = index.search(q[:2], 3)
     assert (I == -1).all()
+
+
+@pytest.mark.parametrize("kind", ["fp32_L2", "fp32_IP", "int8"])
+def test_flat_search_with_masks(ix, oracle, kind):
+    """search_with_masks: every query has its own bit mask over the storage positions (bit p % 8 of byte p / 8;
+    FR/test/DTascendhost/TestAscendIndexInt8Flat.cpp:230-240 reads it that way); the answer is the oracle's
+    brute force over the vectors that take part, bit for bit, with sentinels when fewer than k do.  A full
+    mask gives the plain search; the base has a length that is no multiple of eight and spans several
+    stretches of the score scratch."""
+    rng = np.random.default_rng(61)
+    d, n, nq, k = 40, 20003, 24, 30
+    if kind == "int8":
+        index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=1 << 20)
+        base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+        q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+        base[101] = base[7]                              # a tie across the mask
+    else:
+        metric = ix.METRIC_L2 if kind == "fp32_L2" else ix.METRIC_INNER_PRODUCT
+        index = ix.AscendIndexFlat(d, metric, scratch_bytes=1 << 20)
+        base = rng.standard_normal((n, d)).astype(np.float32)
+        q = rng.standard_normal((nq, d)).astype(np.float32)
+    ids = rng.permutation(5 * n)[:n].astype(np.int64)
+    index.add_with_ids(base, ids)
+    stride = (n + 7) // 8
+    allowed = rng.random((nq, n)) < 0.5
+    allowed[0] = True                                    # everything takes part
+    allowed[1] = False                                   # nothing does
+    allowed[2] = False
+    allowed[2, rng.choice(n, 11, replace=False)] = True  # fewer than k
+    allowed[3] = False
+    allowed[3, -1] = True                                # only the last vector (a bit of the last, partial byte)
+    allowed[4, 7] = False                                # of two equal vectors only the later one
+    allowed[4, 101] = True
+    mask = np.packbits(allowed, axis=1, bitorder="little")
+    assert mask.shape == (nq, stride)
+    if kind == "int8":
+        q[4] = base[7]
+        search = lambda qq, m: index.search_with_masks_int32(qq, k, m)
+        plain = index.search_int32(q, k)
+        brute = lambda sel, qq: oracle.flat_i8(base[sel], qq, k, ids=ids[sel])
+    else:
+        search = lambda qq, m: index.search_with_masks(qq, k, m)
+        plain = index.search(q, k)
+        brute = lambda sel, qq: oracle.flat_f32(base[sel], qq, k, index.metric_type, ids=ids[sel])
+    D, I = search(q, mask)
+    assert np.array_equal(I[0], plain[1][0]) and np.array_equal(D[0], plain[0][0])
+    for i in range(nq):
+        sel = np.nonzero(allowed[i])[0]
+        if len(sel) == 0:
+            assert (I[i] == -1).all()
+            continue
+        Dr, Ir = brute(sel, q[i:i + 1])
+        assert np.array_equal(I[i], Ir[0]), i
+        assert np.array_equal(D[i].view(np.uint32), Dr[0].view(np.uint32)), i
+    assert (I[2, 11:] == -1).all() and (I[2, :11] >= 0).all()
+    assert I[3, 0] == ids[-1] and (I[3, 1:] == -1).all()
+    if kind == "int8":
+        assert I[4, 0] == ids[101] and D[4, 0] == 0
+    # the index answers plain searches as before
+    again = index.search_int32(q, k) if kind == "int8" else index.search(q, k)
+    assert np.array_equal(again[1], plain[1]) and np.array_equal(again[0], plain[0])
