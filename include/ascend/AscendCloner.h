@@ -4,6 +4,8 @@
 //                         AscendIndexIVFPQ   -> IndexIVFPQ with by_residual = false (copyTo)
 //   index_cpu_to_ascend:  IndexFlat, IndexIDMap over IndexFlat -> AscendIndexFlat (FR/ascend/AscendCloner.cpp:133-165)
 //                         IndexIVFPQ (by_residual = false)     -> AscendIndexIVFPQ (copyFrom)
+//   index_int8_ascend_to_cpu / index_int8_cpu_to_ascend: AscendIndexInt8Flat <-> IndexIDMap over
+//                         IndexScalarQuantizer (one int8 per dimension in its codes)
 // The reference's cloner does not know its IVFPQ index; the two IVFPQ directions are this build's addition, on
 // top of the copyFrom / copyTo the reference does have.  The caller owns what is returned.  Header-only.
 #pragma once
@@ -77,6 +79,48 @@ inline faiss::Index *index_cpu_to_ascend(std::initializer_list<int> devices, con
                                          const AscendClonerOptions *options = nullptr)
 {
     return index_cpu_to_ascend(std::vector<int>(devices), index, options);
+}
+
+// int8 indexes (FR/ascend/AscendCloner.h:42-47; FR/ascend/AscendCloner.cpp:97-113, 205-230): AscendIndexInt8Flat
+// <-> IndexIDMap over an IndexScalarQuantizer whose codes are the int8 vectors
+inline faiss::Index *index_int8_ascend_to_cpu(const AscendIndexInt8 *index)
+{
+    if (auto flat = dynamic_cast<const AscendIndexInt8Flat *>(index)) {
+        std::unique_ptr<faiss::IndexScalarQuantizer> codes(new faiss::IndexScalarQuantizer());
+        std::unique_ptr<faiss::IndexIDMap> res(new faiss::IndexIDMap(codes.get()));
+        res->own_fields = true;
+        codes.release();
+        flat->copyTo(res.get());
+        return res.release();
+    }
+    throw faiss::FaissException("clone from ascend to cpu not supported for this type of Index");
+}
+
+inline AscendIndexInt8 *index_int8_cpu_to_ascend(std::vector<int> devices, const faiss::Index *index,
+                                                 const AscendClonerOptions *options = nullptr)
+{
+    if (devices.empty()) {
+        throw faiss::FaissException("device list can not be empty!");
+    }
+    const AscendClonerOptions opt = options ? *options : AscendClonerOptions();
+    AscendIndexInt8FlatConfig config;
+    config.deviceList = devices;
+    config.resourceSize = opt.resourceSize;
+    if (auto sq = dynamic_cast<const faiss::IndexScalarQuantizer *>(index)) {
+        return new AscendIndexInt8Flat(sq, config);
+    }
+    if (auto idm = dynamic_cast<const faiss::IndexIDMap *>(index)) {
+        if (dynamic_cast<const faiss::IndexScalarQuantizer *>(idm->index)) {
+            return new AscendIndexInt8Flat(idm, config);
+        }
+    }
+    throw faiss::FaissException("clone from cpu to ascend not supported for this type of Index");
+}
+
+inline AscendIndexInt8 *index_int8_cpu_to_ascend(std::initializer_list<int> devices, const faiss::Index *index,
+                                                 const AscendClonerOptions *options = nullptr)
+{
+    return index_int8_cpu_to_ascend(std::vector<int>(devices), index, options);
 }
 
 }  // namespace ascend

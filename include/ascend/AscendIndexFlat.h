@@ -229,7 +229,85 @@ public:
     {
         ixaThrowIfError(flat_i8_create(dims, (int)metric, scratchOf(config.resourceSize), &h_));
     }
+    // Construct from a CPU index that holds int8 codes (FR/ascend/AscendIndexInt8Flat.h:60-66)
+    explicit AscendIndexInt8Flat(const faiss::IndexScalarQuantizer *index,
+                                 AscendIndexInt8FlatConfig config = AscendIndexInt8FlatConfig())
+        : AscendIndexInt8(index ? index->d : 0, index ? index->metric_type : faiss::METRIC_L2, config)
+    {
+        if (index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        ixaThrowIfError(flat_i8_create(index->d, (int)index->metric_type, scratchOf(config.resourceSize), &h_));
+        try {
+            copyFrom(index);
+        } catch (...) {
+            flat_i8_destroy(h_);
+            throw;
+        }
+    }
+    explicit AscendIndexInt8Flat(const faiss::IndexIDMap *index,
+                                 AscendIndexInt8FlatConfig config = AscendIndexInt8FlatConfig())
+        : AscendIndexInt8(index && index->index ? index->index->d : 0,
+                          index && index->index ? index->index->metric_type : faiss::METRIC_L2, config)
+    {
+        if (index == nullptr || index->index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        ixaThrowIfError(flat_i8_create(d, (int)metric_type, scratchOf(config.resourceSize), &h_));
+        try {
+            copyFrom(index);
+        } catch (...) {
+            flat_i8_destroy(h_);
+            throw;
+        }
+    }
     virtual ~AscendIndexInt8Flat() { flat_i8_destroy(h_); }
+    // copyFrom / copyTo (FR/ascend/AscendIndexInt8Flat.h:90-96; FR/ascend/impl/AscendIndexInt8FlatImpl.cpp:327-431,
+    // 580-626): the bytes of IndexScalarQuantizer::codes are the int8 vectors; an IndexIDMap carries the ids
+    void copyFrom(const faiss::IndexScalarQuantizer *index) { copyCodes(index, nullptr, 0); }
+    void copyFrom(const faiss::IndexIDMap *index)
+    {
+        if (index == nullptr || index->index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        const auto *sq = dynamic_cast<const faiss::IndexScalarQuantizer *>(index->index);
+        if (sq == nullptr) {
+            throw FaissException("Invalid sqIndex nullptr.");
+        }
+        if (!index->id_map.empty() && index->id_map.size() != (size_t)sq->ntotal) {
+            throw FaissException("The size of id_map must be equal to ntotal.\n");
+        }
+        copyCodes(sq, index->id_map.empty() ? nullptr : index->id_map.data(), index->id_map.size());
+    }
+    void copyTo(faiss::IndexScalarQuantizer *index) const
+    {
+        if (index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        index->reset();
+        index->metric_type = metric_type;
+        index->d = d;
+        index->code_size = (size_t)d;
+        index->is_trained = is_trained;
+        if (ntotal > 0) {
+            std::vector<int8_t> xb;
+            getBase(0, xb);
+            index->codes.assign(reinterpret_cast<const uint8_t *>(xb.data()),
+                                reinterpret_cast<const uint8_t *>(xb.data()) + xb.size());
+        }
+        index->ntotal = ntotal;
+    }
+    void copyTo(faiss::IndexIDMap *index) const
+    {
+        if (index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        copyTo(dynamic_cast<faiss::IndexScalarQuantizer *>(index->index));
+        getIdxMap(0, index->id_map);
+        index->d = d;
+        index->metric_type = metric_type;
+        index->ntotal = ntotal;
+    }
     void searchInt32(idx_t n, const int8_t *x, idx_t k, int32_t *distances, idx_t *labels) const
     {
         ixaThrowIfError(flat_i8_search(h_, n, x, k, distances, reinterpret_cast<int64_t *>(labels)));
@@ -284,6 +362,25 @@ public:
     void setPageSize(uint16_t /*pageBlockNum*/) {}
 
 protected:
+    void copyCodes(const faiss::IndexScalarQuantizer *index, const idx_t *ids, size_t nids)
+    {
+        if (index == nullptr) {
+            throw FaissException("Invalid index nullptr.");
+        }
+        if (index->d != d || index->metric_type != metric_type) {
+            throw FaissException("copyFrom: the source index must have this index's dims and metric");
+        }
+        (void)nids;
+        reset();
+        is_trained = index->is_trained;
+        if (!index->is_trained || index->codes.empty()) {
+            return;
+        }
+        if (index->codes.size() != (size_t)index->ntotal * (size_t)d) {
+            throw FaissException("The size of codes must be equal to ntotal * dim.\n");
+        }
+        addImpl(index->ntotal, reinterpret_cast<const int8_t *>(index->codes.data()), ids);
+    }
     void addImpl(idx_t n, const int8_t *x, const idx_t *ids) override
     {
         ixaThrowIfError(flat_i8_add_with_ids(h_, n, x, reinterpret_cast<const int64_t *>(ids)));

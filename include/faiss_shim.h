@@ -10,6 +10,7 @@
 #include <faiss/IndexFlat.h>
 #include <faiss/IndexIDMap.h>
 #include <faiss/IndexIVFPQ.h>
+#include <faiss/IndexScalarQuantizer.h>
 #include <faiss/impl/FaissException.h>
 #include <faiss/impl/IDSelector.h>
 #include <faiss/invlists/InvertedLists.h>
@@ -131,6 +132,24 @@ struct IndexFlatL2 : IndexFlat {
 };
 struct IndexFlatIP : IndexFlat {
     explicit IndexFlatIP(idx_t d_ = 0) : IndexFlat(d_, METRIC_INNER_PRODUCT) {}
+};
+
+// faiss::IndexScalarQuantizer as the int8 exchange sees it: one byte per dimension in `codes`
+// (the reference reads and writes them as int8, FR/ascend/impl/AscendIndexInt8FlatImpl.cpp:414-431, 580-607).
+struct IndexScalarQuantizer : Index {
+    std::vector<uint8_t> codes;
+    size_t code_size = 0;
+    explicit IndexScalarQuantizer(idx_t d_ = 0, MetricType metric = METRIC_L2) : Index(d_, metric), code_size((size_t)d_) {}
+    void add(idx_t, const float *) override { throw FaissException("the stand-in IndexScalarQuantizer only carries codes"); }
+    void search(idx_t, const float *, idx_t, float *, idx_t *, const SearchParameters * = nullptr) const override
+    {
+        throw FaissException("the stand-in IndexScalarQuantizer only carries codes");
+    }
+    void reset() override
+    {
+        codes.clear();
+        ntotal = 0;
+    }
 };
 
 // faiss::IndexIDMap as copyFrom / copyTo see it: an index plus the user ids of its rows.

@@ -293,6 +293,24 @@ int main(int argc, char **argv)
             flat.search_with_masks(1, x.data(), 2, D.data(), I.data(), fmask.data());
             EXPECT(I[0] == 2 && I[1] == -1 && D[1] == FLT_MAX);
         }
+        {
+            // int8 cloner: device -> IndexIDMap over IndexScalarQuantizer -> device
+            std::unique_ptr<faiss::Index> cpu8(index_int8_ascend_to_cpu(i8_base));
+            auto *map8c = dynamic_cast<faiss::IndexIDMap *>(cpu8.get());
+            auto *sq8 = map8c ? dynamic_cast<faiss::IndexScalarQuantizer *>(map8c->index) : nullptr;
+            EXPECT(sq8 != nullptr && map8c->ntotal == 4096 && sq8->codes.size() == b.size() &&
+                   std::memcmp(sq8->codes.data(), b.data(), b.size()) == 0 && map8c->id_map[4095] == 4095);
+            for (auto &id : map8c->id_map) {
+                id += 100000;
+            }
+            std::unique_ptr<AscendIndexInt8> back8(index_int8_cpu_to_ascend({0}, cpu8.get()));
+            EXPECT(back8->getNTotal() == 4096 && back8->getDim() == 64);
+            back8->search(2, b.data() + (size_t)17 * 64, 1, Di.data(), Ii.data());
+            EXPECT(Ii[0] == 100017 && Ii[1] == 100018 && Di[0] == 0.f);
+            AscendIndexInt8Flat from_codes(sq8);          // without ids: numbered from 0
+            from_codes.search(1, b.data() + (size_t)5 * 64, 1, Di.data(), Ii.data());
+            EXPECT(from_codes.getNTotal() == 4096 && Ii[0] == 5);
+        }
         std::vector<faiss::idx_t> nearest(4);
         i8_base->assign(4, b.data(), nearest.data());
         EXPECT(nearest[0] == 0 && nearest[3] == 3);
