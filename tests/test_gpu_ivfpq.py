@@ -427,13 +427,13 @@ def test_large_k_shared_pool_all_scores_tie(ix, oracle):
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
 
 
-@pytest.mark.parametrize("k", [300, 1024])
+@pytest.mark.parametrize("k", [100, 300, 1024])
 def test_whole_lists_tie_and_the_answer_does_not_depend_on_the_plan(ix, oracle, k):
     """Four sub-quantizers over clustered data: every vector of a cluster gets the same code, so whole lists of
     thousands of vectors share one distance (the shape of the reference's own latency targets: nlist 1024, M 4,
     k 300).  Ties are decided by position in the index, so the answer is the same whether a query is served by
-    one workgroup (a batch of 600) or split over eight (a batch of one), with private pools (k = 300) or the
-    shared pool (k = 1024)."""
+    one workgroup (a batch of 600) or split over eight (a batch of one), with private pools (k = 100: pools of
+    256 keys) or the shared pool (k = 300, k = 1024)."""
     rng = np.random.default_rng(4)
     d, M, nlist, n = 128, 4, 32, 120_000
     centres = rng.standard_normal((nlist, d)).astype(np.float32)
@@ -453,7 +453,7 @@ def test_whole_lists_tie_and_the_answer_does_not_depend_on_the_plan(ix, oracle, 
     assert len(np.unique(codes0, axis=0)) <= 4, "the lists of this test should hold (almost) one code each"
     gpu.setNumProbes(8)
     D, I = gpu.search(q, k)
-    assert gpu.last_search_stats()["shared_pool"] == (1 if k > 320 else 0)
+    assert gpu.last_search_stats()["shared_pool"] == (1 if k > 128 else 0)
     Dr, Ir = ref.search(q, k, 8)
     assert_topk_parity(oracle, ref, q, D, I, Dr, Ir, TOL_FP32)
     for j in (0, 7, 311):
