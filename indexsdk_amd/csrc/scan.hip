@@ -622,16 +622,30 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
     // common prefix of the smallest and the largest key
     __shared__ key_t s_min[NT / kWave], s_max[NT / kWave];
     __shared__ int s_cnt[NT / kWave];
+    // every pass over the keys (they stay in global memory / L2) keeps eight loads per thread in flight
+    auto for_each_key = [&](auto &&fn) {
+        for (int base = tid; base < total; base += NT * 8) {
+            key_t kk[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int i = base + j * NT;
+                kk[j] = i < total ? src[i] : kEmptyKey;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (kk[j] != kEmptyKey) {
+                    fn(kk[j]);
+                }
+            }
+        }
+    };
     key_t mn = kEmptyKey, mx = 0;
     int nvalid = 0;
-    for (int i = tid; i < total; i += NT) {
-        const key_t key = src[i];
-        if (key != kEmptyKey) {
-            mn = key < mn ? key : mn;
-            mx = key > mx ? key : mx;
-            nvalid++;
-        }
-    }
+    for_each_key([&](key_t key) {
+        mn = key < mn ? key : mn;
+        mx = key > mx ? key : mx;
+        nvalid++;
+    });
     for (int o = 32; o > 0; o >>= 1) {
         const key_t omn = __shfl_xor(mn, o), omx = __shfl_xor(mx, o);
         mn = omn < mn ? omn : mn;
@@ -663,12 +677,11 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
             hist[i] = 0;
         }
         __syncthreads();
-        for (int i = tid; i < total; i += NT) {
-            const key_t key = src[i];
-            if (key != kEmptyKey && (upper == 64 || (key >> upper) == prefix)) {
+        for_each_key([&](key_t key) {
+            if (upper == 64 || (key >> upper) == prefix) {
                 atomicAdd(&hist[(uint32_t)(key >> shift) & ((1u << bits) - 1u)], 1);
             }
-        }
+        });
         __syncthreads();
         if (tid < kWave) {
             // first bin whose inclusive count reaches `need`: 16 bins per lane, a wave scan over the lanes
@@ -711,16 +724,14 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         s_kept = 0;
     }
     __syncthreads();
-    for (int i = tid; i < total; i += NT) {
-        const key_t key = src[i];
-        const bool keep = key != kEmptyKey && (all || shift >= 64 || (key >> shift) <= prefix);
-        if (keep) {
+    for_each_key([&](key_t key) {
+        if (all || shift >= 64 || (key >> shift) <= prefix) {
             const int at = atomicAdd(&s_kept, 1);
             if (at < kMergeSelectCap) {
                 surv[at] = key;
             }
         }
-    }
+    });
     __syncthreads();
     const int kept = s_kept < kMergeSelectCap ? s_kept : kMergeSelectCap;
     const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
