@@ -169,6 +169,11 @@ typedef struct ivfpq_config {
                                        reference's host training does (faiss Clustering with cp.spherical = true,
                                        FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1064-1067); 0 (default) = plain Lloyd,
                                        as its device training */
+    int32_t coarse_exact_small;     /* coarse stage of a handful of queries (queries x centroids x dims <= 2^27;
+                                       results do not depend on it): 1 or -1 = the probed lists are selected from
+                                       canonical scores of every centroid (three small launches, exact by
+                                       construction), 0 = such batches go through the matrix-core plans and their
+                                       proof as well */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */

@@ -33,6 +33,7 @@ class IvfpqConfig(ctypes.Structure):
         ("scan_locality", ctypes.c_int32),
         ("coarse_sampled_bound", ctypes.c_int32),
         ("pq_spherical", ctypes.c_int32),
+        ("coarse_exact_small", ctypes.c_int32),
     ]
 
 

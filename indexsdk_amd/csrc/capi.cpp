@@ -99,6 +99,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.scan_locality = cfg->scan_locality;
         c.coarse_sampled_bound = cfg->coarse_sampled_bound;
         c.pq_spherical = cfg->pq_spherical ? 1 : 0;
+        c.coarse_exact_small = cfg->coarse_exact_small;
     }
     return c;
 }
@@ -133,6 +134,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->scan_locality = d.scan_locality;
     cfg->coarse_sampled_bound = d.coarse_sampled_bound;
     cfg->pq_spherical = d.pq_spherical;
+    cfg->coarse_exact_small = d.coarse_exact_small;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,

@@ -31,6 +31,9 @@ struct IvfpqConfig {
     int coarse_sampled_bound = -1;    // coarse stage of large batches: 1 / -1 = admission bound from a seed stretch of
                                       // the centroids and a proof by count (no score matrix is written), 0 = the
                                       // whole score matrix of a query block is written and selected from
+    int coarse_exact_small = -1;      // a handful of queries (queries x centroids x dims <= 2^27) selects its lists from
+                                      // canonical scores of every centroid (three launches, nothing to prove): 1 / -1
+                                      // yes, 0 = such batches take the matrix-core plans too
     int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
                                       // stay exact: candidates are re-evaluated in fp32 and the superset
                                       // property is verified, with an fp32 rerun if it cannot be proven)
@@ -160,6 +163,7 @@ private:
     int32_t max_list_len_ = 0;
     int last_coarse_reruns_ = 0;
     int last_coarse_plan_ = 0;        // plan of the last coarse_select(): 0 materialised, 1 sampled bound
+    bool last_coarse_exact_ = false;  // the last coarse_select() selected from canonical scores: nothing to verify
     int64_t last_coarse_n_ = 0;       // its number of queries
     bool sampled_bound_ok_ = true;    // cleared when the sampled bound failed too many proofs on this index
     bool flag_pending_ = true;   // ws_flag_[0] may be non-zero: clear it before the next coarse stage

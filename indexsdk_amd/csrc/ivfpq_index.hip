@@ -77,6 +77,7 @@ constexpr int64_t kMaxN = 1000000000;   // MAX_N, FR/ascend/AscendIndex.h
 constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this build (reference device limit: 320)
 constexpr int kMaxNprobe = 2048;        // probed lists per query (the reference's L3 operator takes 128 per tile)
 constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
+constexpr int64_t kCoarseExactMaxMacs = (int64_t)1 << 27;   // queries x centroids x dims up to which a search selects its lists exactly
 
 // ---- arena kernels ------------------------------------------------------------------------------
 
@@ -575,6 +576,22 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     }
     ws_qn_.resize((size_t)n);
     launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
+    // A handful of queries (a search that only needs the probed SET): canonical scores of every centroid and an
+    // exact selection from them, the plan coarse_exact_rows() uses for rows without proof.  Three small launches,
+    // nothing to prove and no verdict for the host to read, where the matrix-core plans queue seven and a round
+    // trip; worth it while the work is small (the canonical kernel reads every centroid once per query: 10M x 128
+    // in 16384 lists, 32 queries: 106 us per search against 133; 20M x 768 in 32768 lists, 4 queries: 166 / 224).
+    last_coarse_exact_ = cfg_.coarse_exact_small != 0 && set_only && !out_dist && n * nlist_ * d_ <= kCoarseExactMaxMacs &&
+                         n <= 65535;
+    if (last_coarse_exact_) {
+        last_coarse_plan_ = 0;
+        last_coarse_n_ = n;
+        ws_exact_.resize((size_t)n * nlist_);
+        launch_canonical_scores(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
+                                ws_exact_.data(), nlist_, stream_);
+        launch_select_rows(ws_exact_.data(), n, nlist_, nlist_, nout, out_ids, 0, nullptr, stream_);
+        return;
+    }
     int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 16 + nout / 8);
     // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
     // when it was not, so the common case needs no fill in front of the kernels that append to it
@@ -677,6 +694,9 @@ float IvfpqIndex::bf16x3_err_scale(int select_metric) const
 int IvfpqIndex::coarse_finish(const float *x_dev, int nout, int select_metric, int32_t *out_ids, float *out_dist,
                               std::vector<int32_t> *redone)
 {
+    if (last_coarse_exact_) {
+        return 0;   // exact by construction: no list of rows without proof exists
+    }
     int32_t nfail = 0;
     ws_flag_.download(&nfail, 1, stream_);
     if (nfail == 0) {

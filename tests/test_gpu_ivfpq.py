@@ -536,7 +536,9 @@ def test_search_redoes_only_the_queries_whose_coarse_proof_fails(ix, oracle):
     cb = oracle.train_pq(x[:4000], M, niter=3, seed=3)
     ids = np.arange(40000, dtype=np.int64)
     ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, ids)
-    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    # (batches this small would select their lists from canonical scores: switched off, the matrix-core plans
+    # and their proof are what this test is about)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(coarse_exact_small=0))
     gpu.set_trained(cent, cb)
     gpu.add_with_ids(x, ids)
     gpu.setNumProbes(nprobe)
@@ -551,13 +553,23 @@ def test_search_redoes_only_the_queries_whose_coarse_proof_fails(ix, oracle):
     assert np.array_equal(pi, oi) and np.array_equal(pd.view(np.uint32), od.view(np.uint32))
     # a small batch: every query is split over eight workgroups, and the second scan (of the redone queries
     # only) goes through the split merge under its own numbering
-    q2 = np.ascontiguousarray(np.concatenate([near[:20], far[:10]]))
+    q2 = np.ascontiguousarray(np.concatenate([near[:25], far[:15]]))
     D2, I2 = gpu.search(q2, 20)
     st = gpu.last_search_stats()
-    assert st["nsplit"] == 8 and 1 <= st["coarse_reruns"] <= 20, st
+    assert st["nsplit"] == 8 and 1 <= st["coarse_reruns"] <= 25, st
     Dr2, Ir2 = ref.search(q2, 20, nprobe)
     assert st["scanned_codes"] == ref.last_scanned
     assert_topk_parity(oracle, ref, q2, D2, I2, Dr2, Ir2, TOL_FP32)
+    # by default a batch of this size (queries x centroids x dims <= 2^27) selects its lists from canonical
+    # scores of every centroid: exact by construction, so the tied centroids cost no rerun, same answers
+    exact = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    exact.set_trained(cent, cb)
+    exact.add_with_ids(x, ids)
+    exact.setNumProbes(nprobe)
+    for batch, ref_D, ref_I in ((q, D, I), (q2, D2, I2)):
+        D3, I3 = exact.search(batch, 20)
+        assert exact.last_search_stats()["coarse_reruns"] == 0
+        assert np.array_equal(I3, ref_I) and np.array_equal(D3.view(np.uint32), ref_D.view(np.uint32))
 
 
 def test_reset_keeps_quantizers_and_readd_reproduces_codes(ix, oracle):
