@@ -547,8 +547,9 @@ int64_t FlatBase<T>::remove_selected(int64_t nv, const int64_t *victims, int64_t
         return 0;
     }
     DeviceBuffer<int64_t> victims_dev;
+    std::vector<int64_t> sorted;   // source of an asynchronous copy: lives until the stream has been waited for
     if (victims) {
-        std::vector<int64_t> sorted(victims, victims + nv);
+        sorted.assign(victims, victims + nv);
         std::sort(sorted.begin(), sorted.end());
         sorted.erase(std::unique(sorted.begin(), sorted.end()), sorted.end());
         nv = (int64_t)sorted.size();
