@@ -582,7 +582,7 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     // trip; worth it while the work is small (the canonical kernel reads every centroid once per query: 10M x 128
     // in 16384 lists, 32 queries: 106 us per search against 133; 20M x 768 in 32768 lists, 4 queries: 166 / 224).
     last_coarse_exact_ = cfg_.coarse_exact_small != 0 && set_only && !out_dist && n * nlist_ * d_ <= kCoarseExactMaxMacs &&
-                         n <= 65535;
+                         n <= 65535 && n * nlist_ * (int64_t)sizeof(float) <= cfg_.scratch_bytes;
     if (last_coarse_exact_) {
         last_coarse_plan_ = 0;
         last_coarse_n_ = n;
