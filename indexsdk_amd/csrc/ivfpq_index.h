@@ -190,6 +190,7 @@ private:
     std::vector<int32_t> touch_mark_; // scratch of append(): -1, or the list's place among the touched lists
     std::vector<int32_t> add_pos_;    // scratch of append(): position of every new vector inside its list
     PinnedBuffer add_stage_, add_pack_;   // append(): assignments coming down, kernel inputs going up
+    PinnedBuffer io_stage_;               // small host searches: queries going up, results coming down
     DeviceBuffer<int64_t> ws_add_pack_, ws_add_ids_;
     DeviceBuffer<int32_t> ws_add_lists_;
     DeviceBuffer<uint8_t> ws_add_codes_;

@@ -77,6 +77,7 @@ constexpr int64_t kMaxN = 1000000000;   // MAX_N, FR/ascend/AscendIndex.h
 constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this build (reference device limit: 320)
 constexpr int kMaxNprobe = 2048;        // probed lists per query (the reference's L3 operator takes 128 per tile)
 constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
+constexpr size_t kStagedIoBytes = (size_t)1 << 20;   // host searches whose queries and results fit go through pinned staging
 constexpr int64_t kCoarseExactMaxMacs = (int64_t)1 << 27;   // queries x centroids x dims up to which a search selects its lists exactly
 
 // ---- arena kernels ------------------------------------------------------------------------------
@@ -1432,7 +1433,21 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
 void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
 {
     const float *xd = x;
-    if (!on_device) {
+    // A small batch in host memory goes through one page-locked staging buffer (queries | distances | labels): a
+    // copy to or from pageable memory costs about 45 us each on its own, whatever its size, and the results
+    // then come down behind a single wait.
+    const size_t in_bytes = (size_t)n * d_ * sizeof(float), dist_bytes = (size_t)n * k * sizeof(float),
+                 label_bytes = (size_t)n * k * sizeof(int64_t);
+    const size_t dist_at = (in_bytes + 255) / 256 * 256, label_at = dist_at + (dist_bytes + 255) / 256 * 256;
+    const bool staged_io = !on_device && label_at + label_bytes <= kStagedIoBytes;
+    unsigned char *io = nullptr;
+    if (staged_io) {
+        io = static_cast<unsigned char *>(io_stage_.reserve(label_at + label_bytes));
+        std::memcpy(io, x, in_bytes);
+        ws_x_.resize((size_t)n * d_);
+        IXA_HIP(hipMemcpyAsync(ws_x_.data(), io, in_bytes, hipMemcpyHostToDevice, stream_));
+        xd = ws_x_.data();
+    } else if (!on_device) {
         ws_x_.upload(x, (size_t)n * d_, stream_);
         xd = ws_x_.data();
     }
@@ -1477,7 +1492,13 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     }
     IXA_HIP(hipEventRecord(ev_[2], stream_));
 
-    if (!on_device) {
+    if (staged_io) {
+        IXA_HIP(hipMemcpyAsync(io + dist_at, ws_dist_.data(), dist_bytes, hipMemcpyDeviceToHost, stream_));
+        IXA_HIP(hipMemcpyAsync(io + label_at, ws_labels_.data(), label_bytes, hipMemcpyDeviceToHost, stream_));
+        sync_stream(stream_);
+        std::memcpy(dist, io + dist_at, dist_bytes);
+        std::memcpy(labels, io + label_at, label_bytes);
+    } else if (!on_device) {
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);
     } else {
