@@ -366,3 +366,33 @@ def test_flat_search_with_masks(ix, oracle, kind):
     # the index answers plain searches as before
     again = index.search_int32(q, k) if kind == "int8" else index.search(q, k)
     assert np.array_equal(again[1], plain[1]) and np.array_equal(again[0], plain[0])
+
+
+def test_flat_int8_mask_precision_recipe(ix, oracle):
+    """The reference's own mask test (testMaskPrecision, FR/test/DTascendhost/TestAscendIndexInt8Flat.cpp:287-325):
+    300000 vectors of 384 int8 (more than one 262144-row block of the reference), top 100, every second mask
+    byte 255 and the others 0, for 1, 32 and 128 queries taken from the base.  Its check -- every label of the
+    plain search that passes the mask is among the masked results with the same distance -- and the stricter
+    one here: the masked results are the brute-force answer over the vectors that pass, bit for bit."""
+    rng = np.random.default_rng(2024)
+    n, d, k = 300_000, 384, 100
+    base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2)
+    index.add(base)
+    stride = (n + 7) // 8
+    row = np.zeros(stride, dtype=np.uint8)
+    row[1::2] = 255
+    passes = np.unpackbits(row, bitorder="little")[:n].astype(bool)
+    sel = np.nonzero(passes)[0]
+    for nq in (1, 32, 128):
+        q = base[:nq]
+        mask = np.ascontiguousarray(np.broadcast_to(row, (nq, stride)))
+        D, I = index.search_int32(q, k)
+        Dm, Im = index.search_with_masks_int32(q, k, mask)
+        for i in range(nq):
+            keep = passes[I[i]]
+            found = {int(l): int(v) for l, v in zip(Im[i], Dm[i])}
+            assert all(found.get(int(l)) == int(v) for l, v in zip(I[i][keep], D[i][keep])), i
+        Dr, Ir = oracle.flat_i8(base[sel], q, k, ids=sel.astype(np.int64))
+        assert np.array_equal(Im, Ir) and np.array_equal(Dm, Dr)
+        assert passes[Im].all()
