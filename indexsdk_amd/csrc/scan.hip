@@ -677,11 +677,33 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
             hist[i] = 0;
         }
         __syncthreads();
-        for_each_key([&](key_t key) {
-            if (upper == 64 || (key >> upper) == prefix) {
-                atomicAdd(&hist[(uint32_t)(key >> shift) & ((1u << bits) - 1u)], 1);
+        // (tied scores put most keys of a pass into one bin: the lanes that share the first counted lane's bin
+        // add once for all of them, the others one by one)
+        for (int base = 0; base < total; base += NT * 8) {
+            key_t kk[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int i = base + j * NT + tid;
+                kk[j] = i < total ? src[i] : kEmptyKey;
             }
-        });
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const key_t key = kk[j];
+                const bool counted = key != kEmptyKey && (upper == 64 || (key >> upper) == prefix);
+                const uint32_t bin = (uint32_t)(key >> shift) & ((1u << bits) - 1u);
+                const unsigned long long any = __ballot(counted);
+                if (any) {
+                    const int leader = __ffsll((long long)any) - 1;
+                    const uint32_t leader_bin = (uint32_t)__shfl((int)bin, leader);
+                    const unsigned long long same = __ballot(counted && bin == leader_bin);
+                    if ((tid & (kWave - 1)) == leader) {
+                        atomicAdd(&hist[leader_bin], __popcll(same));
+                    } else if (counted && bin != leader_bin) {
+                        atomicAdd(&hist[bin], 1);
+                    }
+                }
+            }
+        }
         __syncthreads();
         if (tid < kWave) {
             // first bin whose inclusive count reaches `need`: 16 bins per lane, a wave scan over the lanes
