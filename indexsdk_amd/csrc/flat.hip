@@ -565,6 +565,10 @@ int64_t FlatBase<T>::remove_selected(int64_t nv, const int64_t *victims, int64_t
     if (hits == 0) {
         return 0;
     }
+    if ((int64_t)hits == ntotal_) {   // everything leaves: nothing to move
+        ntotal_ = 0;
+        return (int64_t)hits;
+    }
     DeviceBuffer<int64_t> pos_dev((size_t)hits);
     IXA_HIP(hipMemsetAsync(count.data(), 0, 8, stream_));
     hipLaunchKernelGGL(select_positions_kernel, dim3(blocks_for(ntotal_)), dim3(256), 0, stream_, ids_.data(), ntotal_,
