@@ -593,15 +593,20 @@ struct BlockPool {
         return d == W;
     }
 
-    // After the last rendezvous: sorts the pool ascending in place, returns the number of keys.
+    // After the last rendezvous: sorts the pool ascending in place, returns the number of keys.  Only the
+    // smallest power of two that holds them is sorted (a pool pruned to little more than k is far from full).
     __device__ inline int sort_all(int tid)
     {
         const int n = size();
+        int n2 = 2;
+        while (n2 < n) {
+            n2 <<= 1;
+        }
         __syncthreads();
-        for (int i = n + tid; i < cap; i += NT) {
+        for (int i = n + tid; i < n2; i += NT) {
             buf[i] = kEmptyKey;
         }
-        block_bitonic_sort(buf, cap, tid, NT);
+        block_bitonic_sort(buf, n2, tid, NT);
         return n;
     }
 };
