@@ -1224,7 +1224,7 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
 // the undecided as above.  The records hold EVERY centroid whose approximate score is at or below tau,
 // so the set is proven complete when tau > T + 2 err -- whatever tau was derived from.  A query without
 // proof (that, dropped records, more scores than the wave's 64 E places, more undecided candidates than
-// amb_cap) is appended to flag[1 + flag[0]++] for the caller's exact plan.
+// amb_cap) is appended to flag[1 + flag[0]++] for the caller's exact plan, and its nout ids are all -1.
 template <bool VEC4, int E>
 __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
     const float *__restrict__ Q, int64_t nq, const float *__restrict__ C, int d, const float *__restrict__ qn,
@@ -1346,6 +1346,11 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
         fail = n_amb > amb_cap;
     }
     if (fail) {
+        // the row's ids must not stay what the memory happened to hold: work queued behind this launch (the scan
+        // of a search) may read them before the caller's exact plan has replaced them, and -1 is "no list" there
+        for (int i = lane; i < nout; i += kWave) {
+            out[i] = -1;
+        }
         if (lane == 0) {
             flag[1 + atomicAdd(flag, 1)] = (int)(row_base + row);   // the list of queries that need another plan
         }
@@ -1438,6 +1443,8 @@ void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int
 // Canonical scores of whole rows: out[row * ldo + col] for every centroid, one lane per score, in the
 // arithmetic of the refinement kernels (dot product left to right, no FMA).  The plan of last resort
 // for queries whose approximate candidate lists cannot be proven complete: slow, exact by construction.
+// Without row norms (qn == nullptr, L2) every lane adds up its row's squares beside the dot product, in the
+// order of sqnorm_rows_kernel, so the scores are the same bits and a small search saves that launch.
 template <bool VEC4>
 __global__ __launch_bounds__(256) void canonical_scores_kernel(const float *__restrict__ Q, int64_t nq,
                                                                const float *__restrict__ C, int64_t nc, int d,
@@ -1451,7 +1458,8 @@ __global__ __launch_bounds__(256) void canonical_scores_kernel(const float *__re
     }
     const float *q = Q + row * d;
     const float *cv = C + col * d;
-    float g = 0.f;
+    const bool own_norm = qn == nullptr && metric == kMetricL2;
+    float g = 0.f, qq = 0.f;
     if (VEC4) {
 #pragma unroll 4
         for (int t = 0; t < d; t += 4) {
@@ -1461,15 +1469,24 @@ __global__ __launch_bounds__(256) void canonical_scores_kernel(const float *__re
             g = __fadd_rn(g, __fmul_rn(a.y, b.y));
             g = __fadd_rn(g, __fmul_rn(a.z, b.z));
             g = __fadd_rn(g, __fmul_rn(a.w, b.w));
+            if (own_norm) {
+                qq = __fadd_rn(qq, __fmul_rn(a.x, a.x));
+                qq = __fadd_rn(qq, __fmul_rn(a.y, a.y));
+                qq = __fadd_rn(qq, __fmul_rn(a.z, a.z));
+                qq = __fadd_rn(qq, __fmul_rn(a.w, a.w));
+            }
         }
     } else {
         for (int t = 0; t < d; t++) {
             g = __fadd_rn(g, __fmul_rn(q[t], cv[t]));
+            if (own_norm) {
+                qq = __fadd_rn(qq, __fmul_rn(q[t], q[t]));
+            }
         }
     }
     float v;
     if (metric == kMetricL2) {
-        v = __fadd_rn(qn[row], cn[col]);
+        v = __fadd_rn(own_norm ? qq : qn[row], cn[col]);
         v = __fsub_rn(v, g);
         v = __fsub_rn(v, g);
     } else {

@@ -575,10 +575,8 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     if (n == 0) {
         return;
     }
-    ws_qn_.resize((size_t)n);
-    launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
     // A handful of queries (a search that only needs the probed SET): canonical scores of every centroid and an
-    // exact selection from them, the plan coarse_exact_rows() uses for rows without proof.  Three small launches,
+    // exact selection from them, the plan coarse_exact_rows() uses for rows without proof.  Two small launches,
     // nothing to prove and no verdict for the host to read, where the matrix-core plans queue seven and a round
     // trip; worth it while the work is small (the canonical kernel reads every centroid once per query: 10M x 128
     // in 16384 lists, 32 queries: 106 us per search against 133; 20M x 768 in 32768 lists, 4 queries: 166 / 224).
@@ -588,11 +586,13 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
         last_coarse_plan_ = 0;
         last_coarse_n_ = n;
         ws_exact_.resize((size_t)n * nlist_);
-        launch_canonical_scores(x_dev, n, centroids_.data(), nlist_, d_, ws_qn_.data(), cnorm_.data(), select_metric,
-                                ws_exact_.data(), nlist_, stream_);
+        launch_canonical_scores(x_dev, n, centroids_.data(), nlist_, d_, nullptr, cnorm_.data(), select_metric,
+                                ws_exact_.data(), nlist_, stream_);   // without row norms: the kernel adds them up itself
         launch_select_rows(ws_exact_.data(), n, nlist_, nlist_, nout, out_ids, 0, nullptr, stream_);
         return;
     }
+    ws_qn_.resize((size_t)n);
+    launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
     int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 16 + nout / 8);
     // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
     // when it was not, so the common case needs no fill in front of the kernels that append to it
