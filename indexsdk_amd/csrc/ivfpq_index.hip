@@ -1268,6 +1268,7 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     p.ids = ids_.data();
     p.list_off = list_off_dev_.data();
     p.list_len = list_len_dev_.data();
+    p.nlist = nlist_;
     p.code_layout = layout_;
     p.k = (int)k;
     const int nsplit = scan_nsplit(n, nprobe, k, nlist_ > 0 ? ntotal_ / nlist_ * nprobe : 0);
@@ -1303,7 +1304,7 @@ ScanParams IvfpqIndex::scan_params(const float *xd, int64_t n, const int32_t *pr
     };
     if (n * nsplit <= 8192 && n >= 64 && codes_per_group >= 16384) {
         own_order_buffers();
-        launch_order_by_work(probes, n, nprobe, list_len_dev_.data(), (long long)nprobe * max_list_len_, order + n, hist,
+        launch_order_by_work(probes, n, nprobe, list_len_dev_.data(), nlist_, (long long)nprobe * max_list_len_, order + n, hist,
                              hist + 1024, order, stream_);
         p.order = order;
     }
@@ -1538,7 +1539,8 @@ const SearchStats &IvfpqIndex::stats()
     if (stats_pending_) {
         ws_counter_.resize(1);
         IXA_HIP(hipMemsetAsync(ws_counter_.data(), 0, 8, stream_));
-        launch_count_scanned(ws_probes_.data(), stats_rows_ * stats_nprobe_, list_len_dev_.data(), ws_counter_.data(), stream_);
+        launch_count_scanned(ws_probes_.data(), stats_rows_ * stats_nprobe_, list_len_dev_.data(), nlist_, ws_counter_.data(),
+                             stream_);
         unsigned long long scanned = 0;
         ws_counter_.download(&scanned, 1, stream_);
         float ms01 = 0, ms12 = 0;

@@ -16,7 +16,7 @@ __host__ __device__ inline int xor48_byte_of_sq(int m, int p) { return m < 32 ? 
 struct ScanParams {
     // query side
     const float *queries;      // [nq][d]
-    const int32_t *probes;     // [nq][nprobe] list ids, best first, -1 = none
+    const int32_t *probes;     // [nq][nprobe] list ids, best first; an id outside [0, nlist) (-1 by convention) = none
     int nprobe;
     // trained state
     const float *codebook;     // [M][256][dsub]
@@ -28,6 +28,7 @@ struct ScanParams {
     const int64_t *ids;
     const int64_t *list_off;   // first slot of each list
     const int32_t *list_len;   // valid entries of each list
+    int nlist;                 // number of lists
     int code_layout;           // 0 = row, 1 = rot32, 2 = xor48
     // selection
     int k;
@@ -62,11 +63,11 @@ void launch_order_by_locality(const int32_t *probes, int64_t nq, int nprobe, int
 // order[0 .. nq) = the queries by descending work class (work = sum of the probed lists' lengths, at most
 // max_work).  cls: nq ints; hist: 1024 ints that are ZERO on entry and zero again afterwards;
 // cursor: 1024 ints (scratch).
-void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, long long max_work,
+void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, int nlist, long long max_work,
                           int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s);
 
-// *out += sum over probes of list_len[probe]  (probe < 0 contributes nothing).
-void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, unsigned long long *out,
+// *out += sum over probes of list_len[probe]  (a probe outside [0, nlist) contributes nothing).
+void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, int nlist, unsigned long long *out,
                           hipStream_t s);
 
 }  // namespace ixa

@@ -158,9 +158,10 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     }
     for (int i = tid; i < nlocal; i += NT) {
         const int l = p.probes[q * p.nprobe + split + i * p.nsplit];
-        const int len = l >= 0 ? p.list_len[l] : 0;
+        const bool has = (uint32_t)l < (uint32_t)p.nlist;   // anything else is "no list", whatever the caller left there
+        const int len = has ? p.list_len[l] : 0;
         t_len[i] = len;
-        t_off[i] = l >= 0 ? (uint32_t)p.list_off[l] : 0u;
+        t_off[i] = has ? (uint32_t)p.list_off[l] : 0u;
     }
     __syncthreads();
     if (wave == 0) {
@@ -798,14 +799,14 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
 // Sum of the lengths of all probed lists (the number of codes the scan visits): grid-stride
 // partial sums, one atomic per workgroup.
 __global__ __launch_bounds__(256) void count_scanned_kernel(const int32_t *__restrict__ probes, int64_t n,
-                                                            const int32_t *__restrict__ list_len,
+                                                            const int32_t *__restrict__ list_len, int nlist,
                                                             unsigned long long *__restrict__ out)
 {
     __shared__ unsigned long long part[4];
     unsigned long long v = 0;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
         const int l = probes[i];
-        v += l >= 0 ? (unsigned long long)list_len[l] : 0ull;
+        v += (uint32_t)l < (uint32_t)nlist ? (unsigned long long)list_len[l] : 0ull;
     }
     for (int o = 32; o > 0; o >>= 1) {
         v += __shfl_down(v, o);
@@ -819,14 +820,14 @@ __global__ __launch_bounds__(256) void count_scanned_kernel(const int32_t *__res
     }
 }
 
-void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, unsigned long long *out,
+void launch_count_scanned(const int32_t *probes, int64_t n, const int32_t *list_len, int nlist, unsigned long long *out,
                           hipStream_t s)
 {
     if (n == 0) {
         return;
     }
     const unsigned grid = (unsigned)std::min<int64_t>(64, (n + 255) / 256);
-    hipLaunchKernelGGL(count_scanned_kernel, dim3(grid), dim3(256), 0, s, probes, n, list_len, out);
+    hipLaunchKernelGGL(count_scanned_kernel, dim3(grid), dim3(256), 0, s, probes, n, list_len, nlist, out);
 }
 
 // ---- execution order: heaviest queries first ------------------------------------------------------
@@ -838,8 +839,9 @@ constexpr int kWorkClasses = 1024;
 
 // one wavefront per query: cls[q] and the class histogram
 __global__ __launch_bounds__(256) void work_class_kernel(const int32_t *__restrict__ probes, int64_t nq, int nprobe,
-                                                         const int32_t *__restrict__ list_len, long long max_work,
-                                                         int32_t *__restrict__ cls, int32_t *__restrict__ hist)
+                                                         const int32_t *__restrict__ list_len, int nlist,
+                                                         long long max_work, int32_t *__restrict__ cls,
+                                                         int32_t *__restrict__ hist)
 {
     const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -849,7 +851,7 @@ __global__ __launch_bounds__(256) void work_class_kernel(const int32_t *__restri
     long long w = 0;
     for (int j = lane; j < nprobe; j += 64) {
         const int l = probes[q * nprobe + j];
-        w += l >= 0 ? list_len[l] : 0;
+        w += (uint32_t)l < (uint32_t)nlist ? list_len[l] : 0;
     }
     for (int o = 32; o > 0; o >>= 1) {
         w += __shfl_xor(w, o);
@@ -935,14 +937,14 @@ void launch_order_by_locality(const int32_t *probes, int64_t nq, int nprobe, int
     hipLaunchKernelGGL(scatter_order_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, cls, nq, cursor, order);
 }
 
-void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, long long max_work,
-                          int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s)
+void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const int32_t *list_len, int nlist,
+                          long long max_work, int32_t *cls, int32_t *hist, int32_t *cursor, int32_t *order, hipStream_t s)
 {
     if (nq == 0) {
         return;
     }
     hipLaunchKernelGGL(work_class_kernel, dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, s, probes, nq, nprobe, list_len,
-                       max_work, cls, hist);
+                       nlist, max_work, cls, hist);
     hipLaunchKernelGGL(class_offsets_kernel, dim3(1), dim3(kWorkClasses), 0, s, hist, cursor);
     hipLaunchKernelGGL(scatter_order_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, cls, nq, cursor, order);
 }
