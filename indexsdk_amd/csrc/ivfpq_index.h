@@ -203,6 +203,7 @@ private:
     DeviceBuffer<unsigned long long> ws_running_;
     DeviceBuffer<int32_t> ws_cand_, ws_probes_;
     DeviceBuffer<int64_t> ws_labels_;
+    DeviceBuffer<unsigned char> ws_results_;   // distances | labels of a small host search (one copy down)
     DeviceBuffer<unsigned long long> ws_partial_, ws_counter_;
     SearchStats stats_;
 };

@@ -1454,7 +1454,12 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     }
     float *dd = dist;
     int64_t *ld = labels;
-    if (!on_device) {
+    if (staged_io) {
+        // distances and labels lie in one device buffer as they lie in the staging buffer: one copy brings both down
+        ws_results_.resize(label_at - dist_at + label_bytes);
+        dd = reinterpret_cast<float *>(ws_results_.data());
+        ld = reinterpret_cast<int64_t *>(ws_results_.data() + (label_at - dist_at));
+    } else if (!on_device) {
         ws_dist_.resize((size_t)n * k);
         ws_labels_.resize((size_t)n * k);
         dd = ws_dist_.data();
@@ -1494,8 +1499,8 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     IXA_HIP(hipEventRecord(ev_[2], stream_));
 
     if (staged_io) {
-        IXA_HIP(hipMemcpyAsync(io + dist_at, ws_dist_.data(), dist_bytes, hipMemcpyDeviceToHost, stream_));
-        IXA_HIP(hipMemcpyAsync(io + label_at, ws_labels_.data(), label_bytes, hipMemcpyDeviceToHost, stream_));
+        IXA_HIP(hipMemcpyAsync(io + dist_at, ws_results_.data(), label_at - dist_at + label_bytes, hipMemcpyDeviceToHost,
+                               stream_));
         sync_stream(stream_);
         std::memcpy(dist, io + dist_at, dist_bytes);
         std::memcpy(labels, io + label_at, label_bytes);
