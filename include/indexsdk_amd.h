@@ -246,7 +246,7 @@ int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, 
  * arguments, same results bit for bit; it calls no hipMalloc / hipFree: the intermediates of the launch
  * (sanitised probe lists, execution order, split partials) lie in a static device array of
  * IVFPQ_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.  A call that
- * needs more (8192 + 8 n + 4 n nprobe + 8 n nsplit k bytes, each term rounded up to 256; nsplit <= 8 is
+ * needs more (8192 + 8 n + 4 n nprobe + 8 n nsplit k bytes, each term rounded up to 256; nsplit <= 64 is
  * the number of workgroups a query of a small batch is split over) fails with IXA_ERR_INVALID_PARAM and a
  * message that names the need and the limit.  All calls on one GPU share the array; inside one process
  * they take turns (a lock), and the array's contents mean nothing between calls.  It leaves
