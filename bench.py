@@ -277,6 +277,7 @@ def main():
     del buf
     torch.cuda.empty_cache()
     index.setNumProbes(nprobe)
+    index.set_stage_timings(1)   # the steps below report their coarse / scan split, whatever the batch size
 
     D = torch.empty(nq, k, device="cuda", dtype=torch.float32)
     I = torch.empty(nq, k, device="cuda", dtype=torch.int64)
@@ -392,6 +393,7 @@ def main():
     if args.latency_sweep:
         # one search call per cell, synchronised, 40 calls after 5 warm-up calls: the median wall time of a call
         sweep = {}
+        index.set_stage_timings(-1)   # the library's default: small batches record no stage events
         for np_ in (32, 64, 128):
             if np_ > nlist:
                 continue
@@ -420,6 +422,7 @@ def main():
                 log(f"latency nprobe {np_:4d} batch {b:3d}: device {cell['device_us']:8.1f} us, host pointers "
                     f"{cell['host_us']:8.1f} us (nsplit {cell['nsplit']})")
         index.setNumProbes(nprobe)
+        index.set_stage_timings(1)
         result["latency_sweep"] = sweep
 
     if not args.no_cpu:

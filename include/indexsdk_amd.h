@@ -171,9 +171,13 @@ typedef struct ivfpq_config {
                                        as its device training */
     int32_t coarse_exact_small;     /* coarse stage of a handful of queries (queries x centroids x dims <= 2^27;
                                        results do not depend on it): 1 or -1 = the probed lists are selected from
-                                       canonical scores of every centroid (three small launches, exact by
+                                       canonical scores of every centroid (two small launches, exact by
                                        construction), 0 = such batches go through the matrix-core plans and their
                                        proof as well */
+    int32_t stage_timings;          /* HIP events around the stages of a search, which ms_coarse / ms_scan / ms_total
+                                       of ivfpq_last_search_stats come from: 1 = always, 0 = never, -1 (default) =
+                                       for pages of 256 queries or more (recording them costs a small batch 5-10 us
+                                       per call); a search without them reports 0 ms */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */
@@ -224,6 +228,9 @@ int ivfpq_add_codes(ivfpq_index_t *h, int64_t list, int64_t n, const uint8_t *co
  * the number of lists is clamped to it; more than 2048 probed lists are refused. */
 int ivfpq_set_nprobe(ivfpq_index_t *h, int nprobe);
 int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out);
+/* config.stage_timings of an existing index, from its next search on (-1, 0 or 1).  No counterpart in the
+ * reference: a serving loop of small batches switches the stage events off, a measurement switches them on. */
+int ivfpq_set_stage_timings(ivfpq_index_t *h, int mode);
 
 /* AscendIndex::search(n, x, k, distances, labels)  FR/ascend/AscendIndex.h:79-80 ->
  * ascend::IndexIVFPQ::searchImpl  FR/ascenddaemon/impl/IndexIVFPQ.cpp:2373-2411.  0 < n < 1e9, 0 < k <= 2048
@@ -311,8 +318,9 @@ typedef struct ivfpq_scan_lds_plan {
 int ivfpq_plan_scan_lds(int d, int msubs, int lut_fp16, int code_layout, int nprobe, int nsplit, int k, int waves,
                         int shared_pool, ivfpq_scan_lds_plan_t *out);
 
-/* Device timings of the last ivfpq_search* call, measured with HIP events on the index's stream.
- * No counterpart in the reference (it prints std::chrono timers when verbose). */
+/* Device timings of the last ivfpq_search* call, measured with HIP events on the index's stream (0 for a
+ * search that recorded none: config.stage_timings).  No counterpart in the reference (it prints std::chrono
+ * timers when verbose). */
 typedef struct ivfpq_search_stats {
     double scanned_codes; /* sum of the lengths of all probed lists */
     double ms_coarse;     /* stage 1: scores + selection + refine */
@@ -332,7 +340,8 @@ typedef struct ivfpq_search_stats {
                              scanned codes and reruns are reported; the plan fields are the last page's) */
 } ivfpq_search_stats_t;
 int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out);
-/* Device times of the last search only (HIP events on the index's stream, in ms); either output may be NULL.
+/* Device times of the last search only (HIP events on the index's stream, in ms; 0 for a search that recorded
+ * none: config.stage_timings); either output may be NULL.
  * Unlike ivfpq_last_search_stats, which counts the scanned codes with a kernel launch and a host
  * synchronisation the first time it is called after a search, this call does no device work, so it can sit
  * inside a timed loop.  No counterpart in the reference: a measurement aid. */

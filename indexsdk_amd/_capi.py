@@ -34,6 +34,7 @@ class IvfpqConfig(ctypes.Structure):
         ("coarse_sampled_bound", ctypes.c_int32),
         ("pq_spherical", ctypes.c_int32),
         ("coarse_exact_small", ctypes.c_int32),
+        ("stage_timings", ctypes.c_int32),
     ]
 
 
@@ -101,6 +102,7 @@ _SIGNATURES = {
     "ivfpq_add_with_ids_device": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_add_codes": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]),
     "ivfpq_set_nprobe": (ctypes.c_int, [_H, ctypes.c_int]),
+    "ivfpq_set_stage_timings": (ctypes.c_int, [_H, ctypes.c_int]),
     "ivfpq_get_nprobe": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int)]),
     "ivfpq_search": (ctypes.c_int, [_H, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
                                     ctypes.c_void_p]),

@@ -226,8 +226,13 @@ class AscendIndexIVFPQ:
         _capi.check(self._lib.ivfpq_arena_state(self._h, ctypes.byref(a), ctypes.byref(u), ctypes.byref(h)))
         return a.value, u.value, h.value
 
+    def set_stage_timings(self, mode):
+        """Stage events of a search (ms_coarse / ms_scan): 1 always, 0 never, -1 for pages of >= 256 queries."""
+        _capi.check(self._lib.ivfpq_set_stage_timings(self._h, mode))
+
     def last_search_timings(self):
-        """(ms_coarse, ms_scan) of the last search; no device work, usable inside a timed loop."""
+        """(ms_coarse, ms_scan) of the last search (0, 0 when it recorded no stage events); no device work, usable
+        inside a timed loop."""
         a, b = ctypes.c_double(), ctypes.c_double()
         _capi.check(self._lib.ivfpq_last_search_timings(self._h, ctypes.byref(a), ctypes.byref(b)))
         return a.value, b.value

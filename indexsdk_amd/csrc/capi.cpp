@@ -100,6 +100,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.coarse_sampled_bound = cfg->coarse_sampled_bound;
         c.pq_spherical = cfg->pq_spherical ? 1 : 0;
         c.coarse_exact_small = cfg->coarse_exact_small;
+        c.stage_timings = cfg->stage_timings;
     }
     return c;
 }
@@ -135,6 +136,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->coarse_sampled_bound = d.coarse_sampled_bound;
     cfg->pq_spherical = d.pq_spherical;
     cfg->coarse_exact_small = d.coarse_exact_small;
+    cfg->stage_timings = d.stage_timings;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,
@@ -237,6 +239,14 @@ IXA_EXPORT int ivfpq_add_codes(ivfpq_index_t *h, int64_t list, int64_t n, const 
 IXA_EXPORT int ivfpq_set_nprobe(ivfpq_index_t *h, int nprobe)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.set_nprobe(nprobe); });
+}
+IXA_EXPORT int ivfpq_set_stage_timings(ivfpq_index_t *h, int mode)
+{
+    return guarded([&] {
+        IXA_HANDLE(h);
+        IXA_REQUIRE(mode >= -1 && mode <= 1, ixa::kErrInvalidParam, "stage_timings must be -1, 0 or 1");
+        h->impl.set_stage_timings(mode);
+    });
 }
 IXA_EXPORT int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out)
 {

@@ -32,8 +32,11 @@ struct IvfpqConfig {
                                       // the centroids and a proof by count (no score matrix is written), 0 = the
                                       // whole score matrix of a query block is written and selected from
     int coarse_exact_small = -1;      // a handful of queries (queries x centroids x dims <= 2^27) selects its lists from
-                                      // canonical scores of every centroid (three launches, nothing to prove): 1 / -1
+                                      // canonical scores of every centroid (two launches, nothing to prove): 1 / -1
                                       // yes, 0 = such batches take the matrix-core plans too
+    int stage_timings = -1;           // events around the stages of a search (ms_coarse / ms_scan of the statistics):
+                                      // 1 = always, 0 = never, -1 = for pages of 256 queries or more (the three
+                                      // event records cost a small batch 5-10 us per call); untimed stages report 0
     int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
                                       // stay exact: candidates are re-evaluated in fp32 and the superset
                                       // property is verified, with an fp32 rerun if it cannot be proven)
@@ -76,6 +79,7 @@ public:
     bool is_trained() const { return trained_; }
     int nprobe() const { return nprobe_; }
     void set_nprobe(int nprobe);
+    void set_stage_timings(int mode) { cfg_.stage_timings = mode; }   // as IvfpqConfig::stage_timings, from the next search on
     int code_layout() const { return layout_; }
     hipStream_t stream() const { return stream_; }
 
@@ -168,6 +172,7 @@ private:
     bool sampled_bound_ok_ = true;    // cleared when the sampled bound failed too many proofs on this index
     bool flag_pending_ = true;   // ws_flag_[0] may be non-zero: clear it before the next coarse stage
     bool stats_pending_ = false;
+    bool stats_timed_ = false;   // the last search recorded its stage events
     int64_t stats_rows_ = 0;
     int stats_nprobe_ = 0;
     // the probe lists and list lengths the pending statistics refer to are about to change

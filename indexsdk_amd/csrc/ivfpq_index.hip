@@ -1468,10 +1468,15 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     ws_probes_.resize((size_t)n * nprobe_);
     ws_counter_.resize(1);
 
-    IXA_HIP(hipEventRecord(ev_[0], stream_));
+    const bool timed = cfg_.stage_timings > 0 || (cfg_.stage_timings < 0 && n >= 256);
+    if (timed) {
+        IXA_HIP(hipEventRecord(ev_[0], stream_));
+    }
     last_coarse_reruns_ = 0;
     coarse_select(xd, n, nprobe_, metric_, ws_probes_.data(), nullptr, true, true);
-    IXA_HIP(hipEventRecord(ev_[1], stream_));
+    if (timed) {
+        IXA_HIP(hipEventRecord(ev_[1], stream_));
+    }
 
     ScanParams p = scan_params(xd, n, ws_probes_.data(), nprobe_, k, dd, ld);
     const int nsplit = p.nsplit;
@@ -1496,7 +1501,10 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
         stats_.scan_waves = planned.waves;
         stats_.shared_pool = planned.shared_pool;
     }
-    IXA_HIP(hipEventRecord(ev_[2], stream_));
+    if (timed) {
+        IXA_HIP(hipEventRecord(ev_[2], stream_));
+    }
+    stats_timed_ = timed;
 
     if (staged_io) {
         IXA_HIP(hipMemcpyAsync(io + dist_at, ws_results_.data(), label_at - dist_at + label_bytes, hipMemcpyDeviceToHost,
@@ -1525,8 +1533,10 @@ void IvfpqIndex::last_timings(double *ms_coarse, double *ms_scan)
 {
     float ms01 = 0, ms12 = 0;
     if (stats_pending_) {   // the events of the last search have completed: search() synchronises its stream
-        IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
-        IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+        if (stats_timed_) {
+            IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
+            IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+        }
     } else {
         ms01 = (float)stats_.ms_coarse;
         ms12 = (float)stats_.ms_scan;
@@ -1549,8 +1559,10 @@ const SearchStats &IvfpqIndex::stats()
         unsigned long long scanned = 0;
         ws_counter_.download(&scanned, 1, stream_);
         float ms01 = 0, ms12 = 0;
-        IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
-        IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+        if (stats_timed_) {
+            IXA_HIP(hipEventElapsedTime(&ms01, ev_[0], ev_[1]));
+            IXA_HIP(hipEventElapsedTime(&ms12, ev_[1], ev_[2]));
+        }
         stats_.scanned_codes = (double)scanned;
         stats_.ms_coarse = ms01;
         stats_.ms_scan = ms12;

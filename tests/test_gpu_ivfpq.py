@@ -170,6 +170,35 @@ def test_search_empty_index_and_single_query(ix, oracle):
     assert np.all(I == -1) and np.all(D == FLT_MAX)
 
 
+def test_stage_timings_are_recorded_for_large_pages_or_on_request(ix, oracle):
+    """ms_coarse / ms_scan come from events around the stages: recorded for pages of 256 queries or more, for
+    smaller ones only on request (they cost a small batch several microseconds); results never depend on it."""
+    gpu, ref, x, q, ids = build_pair(ix, oracle, 29, 6000, 300, 32, 16, 4, ix.METRIC_L2)
+    gpu.setNumProbes(4)
+    D8, I8 = gpu.search(q[:8], 5)
+    assert gpu.last_search_timings() == (0.0, 0.0)
+    st = gpu.last_search_stats()
+    assert st["ms_total"] == 0.0 and st["scanned_codes"] > 0
+    gpu.search(q, 5)
+    c, s = gpu.last_search_timings()
+    assert c > 0 and s > 0 and gpu.last_search_stats()["ms_scan"] > 0
+    gpu.set_stage_timings(1)
+    D8t, I8t = gpu.search(q[:8], 5)
+    assert min(gpu.last_search_timings()) > 0
+    assert np.array_equal(I8, I8t) and np.array_equal(D8.view(np.uint32), D8t.view(np.uint32))
+    gpu.set_stage_timings(0)
+    gpu.search(q, 5)
+    assert gpu.last_search_timings() == (0.0, 0.0)
+    with pytest.raises(ix.IndexSdkError):
+        gpu.set_stage_timings(2)
+    never = ix.AscendIndexIVFPQ(32, ix.METRIC_L2, 16, 4, 8, ix.AscendIndexIVFPQConfig(stage_timings=1))
+    never.set_trained(ref.cent, ref.codebook)
+    never.add_with_ids(x, ids)
+    never.setNumProbes(4)
+    never.search(q[:2], 5)
+    assert min(never.last_search_timings()) > 0
+
+
 def test_large_k(ix, oracle):
     gpu, ref, x, q, ids = build_pair(ix, oracle, 27, 30000, 40, 96, 32, 48, ix.METRIC_L2)
     gpu.setNumProbes(16)
