@@ -595,57 +595,155 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     }
 }
 
-// Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3) by radix selection:
-// the k-th smallest of the nsplit x k keys is found ten key bits at a time, starting below the leading bits that
-// all keys of the query share (a 1024-bin LDS histogram per pass over the keys, which stay in global memory /
-// L2), until the keys at or below the prefix found so far are few; those survivors -- k of them plus the rest
-// of the last histogram bin -- are ranked by counting in LDS (sorted, when there are more than 1024) and the
-// first k written out.  The cost grows with the number of keys, not with keys x slices x log k as a merge that
-// ranks every key in every other slice does (8 slices of 100 keys: 12 us less than that merge; 32 slices of
-// 300 keys: out of its reach), which is what lets a single query be split over more than eight workgroups.
+// Merges the nsplit sorted partial lists of a query (tile merge, the role of op TopkIvfpqL3).
+//
+// 1. A bound from the slices' own order.  Every slice is sorted, so two of its keys bound the k-th smallest key
+//    of the query from above: the last key of a slice that is full (that slice alone has k keys at or below it),
+//    and the largest of the slices' keys at rank r = ceil(k / nsplit) (r keys of every slice lie at or below
+//    it).  ONE pass over the nsplit x k keys (global memory / L2) keeps those at or below the smaller of the
+//    two: they contain the k smallest, and they are few -- k when one slice holds the best, two to five times k
+//    when the slices are alike.
+// 2. Radix selection among them: the k-th smallest is found ten key bits at a time, starting below the leading
+//    bits that all of them share (a 1024-bin LDS histogram per pass), until the keys at or below the prefix
+//    found so far are few.  The kept keys sit in registers (at most four per thread), so a pass reads no
+//    memory.  A query whose bound keeps more keys than the survivor array holds (short slices, say) runs the
+//    same passes over the keys in global memory instead.
+// 3. The survivors -- k of them plus the rest of the last histogram bin -- are ranked by counting in LDS
+//    (sorted, when there are more than 384) and the first k written out.
+// The cost grows with the number of keys, not with keys x slices x log k as a merge that ranks every key in every
+// other slice does (8 slices of 100 keys: 12 us less than that merge; 32 slices of 300 keys: out of its reach),
+// which is what lets a single query be split over more than eight workgroups.  Against radix passes over all
+// keys in global memory, without the bound: 32 slices of 300 tied keys 21.6 -> 14.1 us, 19 slices of 1000 keys
+// 85 -> 42 us, 9 slices of 100 keys 9.2 -> 8.9 us.
 constexpr int kMergeSelectCap = 4096;
-constexpr int kMergeSelectThreads = 512;
+constexpr int kMergeSelectThreads = 1024;
+constexpr int kMergeCountMax = 384;   // survivors ranked by counting; more are sorted
 
 __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
     const key_t *__restrict__ partial, int nsplit, int k, int metric, const int64_t *__restrict__ ids,
     const int32_t *__restrict__ order, float *__restrict__ out_dist, int64_t *__restrict__ out_labels)
 {
     constexpr int NT = kMergeSelectThreads;
+    constexpr int kPer = kMergeSelectCap / NT;   // keys of the survivor array per thread
+    static_assert(kMergeSelectCap == kPer * NT, "a thread holds its share of the survivor array in registers");
     __shared__ int hist[1024];
-    __shared__ key_t surv[kMergeSelectCap];
+    __shared__ __align__(16) key_t surv[kMergeSelectCap];
     __shared__ int s_bin, s_below, s_kept;
+    __shared__ key_t s_bound;
+    __shared__ key_t s_min[NT / kWave], s_max[NT / kWave];
+    __shared__ int s_cnt[NT / kWave];
     const int tid = threadIdx.x;
     const int64_t q = order ? order[blockIdx.x] : blockIdx.x;
     const int total = nsplit * k;
     const key_t *src = partial + q * total;
 
-    // the keys of one query share their leading bits (sign, exponent and more): the selection starts below the
-    // common prefix of the smallest and the largest key
-    __shared__ key_t s_min[NT / kWave], s_max[NT / kWave];
-    __shared__ int s_cnt[NT / kWave];
-    // every pass over the keys (they stay in global memory / L2) keeps eight loads per thread in flight
-    auto for_each_key = [&](auto &&fn) {
-        for (int base = tid; base < total; base += NT * 8) {
-            key_t kk[8];
+    // ---- 1. the bound, and the keys at or below it.  A query with no more keys than the survivor array holds
+    // takes them into registers at once, while the first wavefront fetches the bound: one memory round trip.
+    const bool small = total <= kMergeSelectCap;
+    key_t mine[kPer];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int i = base + j * NT;
+    for (int j = 0; j < kPer; j++) {
+        const int i = j * NT + tid;
+        mine[j] = (small && i < total) ? src[i] : kEmptyKey;
+    }
+    if (tid < kWave) {
+        // (the rank is taken as if every slice were full: a slice with fewer keys than that has kEmptyKey there,
+        // which leaves the first bound alone)
+        const int r = (k + nsplit - 1) / nsplit;
+        key_t full_min = kEmptyKey, rank_max = 0;
+        for (int j = tid; j < nsplit; j += kWave) {
+            const key_t last = src[(int64_t)j * k + (k - 1)], at_r = src[(int64_t)j * k + (r - 1)];
+            full_min = last < full_min ? last : full_min;
+            rank_max = at_r > rank_max ? at_r : rank_max;
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const key_t a = __shfl_xor(full_min, o), b = __shfl_xor(rank_max, o);
+            full_min = a < full_min ? a : full_min;
+            rank_max = b > rank_max ? b : rank_max;
+        }
+        if (tid == 0) {
+            s_bound = full_min < rank_max ? full_min : rank_max;
+            s_kept = 0;
+        }
+    }
+    __syncthreads();
+    // every pass over the keys in global memory keeps four loads per thread in flight; fn sees every key,
+    // kEmptyKey included, and is called the same number of times by every thread (it may hold ballots)
+    auto visit_global = [&](auto &&fn) {
+        for (int base = 0; base < total; base += NT * kPer) {
+            key_t kk[kPer];
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                const int i = base + j * NT + tid;
                 kk[j] = i < total ? src[i] : kEmptyKey;
             }
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                if (kk[j] != kEmptyKey) {
-                    fn(kk[j]);
-                }
+            for (int j = 0; j < kPer; j++) {
+                fn(kk[j]);
             }
         }
     };
+    // appends the keys that a wavefront keeps to the survivor array: one LDS atomic per wavefront and call
+    // (every lane calls, the same number of times)
+    auto append = [&](bool keep, key_t key) {
+        const unsigned long long m = __ballot(keep);
+        if (m == 0) {
+            return;
+        }
+        const int lane = tid & (kWave - 1), leader = __ffsll((long long)m) - 1;
+        int base = 0;
+        if (lane == leader) {
+            base = atomicAdd(&s_kept, __popcll(m));
+        }
+        base = __shfl(base, leader);
+        const int at = base + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+        if (keep && at < kMergeSelectCap) {
+            surv[at] = key;
+        }
+    };
+    bool in_regs = small;   // uniform over the workgroup: the rest of the selection never reads global memory
+    {
+        const key_t bound = s_bound;
+        if (small) {
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                mine[j] = mine[j] <= bound ? mine[j] : kEmptyKey;
+            }
+        } else {
+            visit_global([&](key_t key) { append(key != kEmptyKey && key <= bound, key); });
+            __syncthreads();
+            const int bounded = s_kept;
+            in_regs = bounded <= kMergeSelectCap;
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                const int i = j * NT + tid;
+                mine[j] = (in_regs && i < bounded) ? surv[i] : kEmptyKey;
+            }
+        }
+    }
+    auto visit = [&](auto &&fn) {
+        if (in_regs) {
+#pragma unroll
+            for (int j = 0; j < kPer; j++) {
+                fn(mine[j]);
+            }
+        } else {
+            visit_global(fn);
+        }
+    };
+    __syncthreads();   // the survivor array is free again: every thread has its keys
+
+    // ---- 2. radix selection among the kept keys (all keys of the query, when the bound kept too many).  They
+    // share their leading bits (sign, exponent and more): the selection starts below the common prefix of the
+    // smallest and the largest
     key_t mn = kEmptyKey, mx = 0;
     int nvalid = 0;
-    for_each_key([&](key_t key) {
-        mn = key < mn ? key : mn;
-        mx = key > mx ? key : mx;
-        nvalid++;
+    visit([&](key_t key) {
+        if (key != kEmptyKey) {
+            mn = key < mn ? key : mn;
+            mx = key > mx ? key : mx;
+            nvalid++;
+        }
     });
     for (int o = 32; o > 0; o >>= 1) {
         const key_t omn = __shfl_xor(mn, o), omx = __shfl_xor(mx, o);
@@ -666,7 +764,10 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         nvalid += s_cnt[w];
     }
 
-    bool all = nvalid <= k;   // no more keys than asked for: every one of them survives
+    // Few enough to rank at once: every one of them survives.  A pass over keys in registers costs about what
+    // ranking 64 more survivors does, a pass over global memory three times that.
+    const int few = in_regs ? k + 64 : (k + 64 > 320 ? k + 64 : 320);
+    bool all = nvalid <= k || (nvalid <= kMergeSelectCap && nvalid <= few);
     int shift = (all || mn == mx) ? 0 : 64 - __clzll((long long)(mn ^ mx));   // the keys differ below this bit
     key_t prefix = shift >= 64 ? 0 : mn >> shift;   // the bits above `shift` of the k-th smallest key
     int need = k;                                    // rank of that key among the keys that share the prefix
@@ -680,31 +781,21 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         __syncthreads();
         // (tied scores put most keys of a pass into one bin: the lanes that share the first counted lane's bin
         // add once for all of them, the others one by one)
-        for (int base = 0; base < total; base += NT * 8) {
-            key_t kk[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int i = base + j * NT + tid;
-                kk[j] = i < total ? src[i] : kEmptyKey;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const key_t key = kk[j];
-                const bool counted = key != kEmptyKey && (upper == 64 || (key >> upper) == prefix);
-                const uint32_t bin = (uint32_t)(key >> shift) & ((1u << bits) - 1u);
-                const unsigned long long any = __ballot(counted);
-                if (any) {
-                    const int leader = __ffsll((long long)any) - 1;
-                    const uint32_t leader_bin = (uint32_t)__shfl((int)bin, leader);
-                    const unsigned long long same = __ballot(counted && bin == leader_bin);
-                    if ((tid & (kWave - 1)) == leader) {
-                        atomicAdd(&hist[leader_bin], __popcll(same));
-                    } else if (counted && bin != leader_bin) {
-                        atomicAdd(&hist[bin], 1);
-                    }
+        visit([&](key_t key) {
+            const bool counted = key != kEmptyKey && (upper == 64 || (key >> upper) == prefix);
+            const uint32_t bin = (uint32_t)(key >> shift) & ((1u << bits) - 1u);
+            const unsigned long long any = __ballot(counted);
+            if (any) {
+                const int leader = __ffsll((long long)any) - 1;
+                const uint32_t leader_bin = (uint32_t)__shfl((int)bin, leader);
+                const unsigned long long same = __ballot(counted && bin == leader_bin);
+                if ((tid & (kWave - 1)) == leader) {
+                    atomicAdd(&hist[leader_bin], __popcll(same));
+                } else if (counted && bin != leader_bin) {
+                    atomicAdd(&hist[bin], 1);
                 }
             }
-        }
+        });
         __syncthreads();
         if (tid < kWave) {
             // first bin whose inclusive count reaches `need`: 16 bins per lane, a wave scan over the lanes
@@ -738,8 +829,7 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         need -= s_below;
         const int survivors = (k - need) + s_kept;   // keys below the prefix class + the class itself
         __syncthreads();
-        // few enough to rank by counting (a pass costs about what counting 300 survivors does)
-        if (survivors <= kMergeSelectCap && (survivors <= k + 64 || survivors <= 320)) {
+        if (survivors <= kMergeSelectCap && survivors <= few) {
             break;
         }
     }
@@ -747,30 +837,43 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         s_kept = 0;
     }
     __syncthreads();
-    for_each_key([&](key_t key) {
-        if (all || shift >= 64 || (key >> shift) <= prefix) {
-            const int at = atomicAdd(&s_kept, 1);
-            if (at < kMergeSelectCap) {
-                surv[at] = key;
-            }
-        }
-    });
+    visit([&](key_t key) { append(key != kEmptyKey && (all || shift >= 64 || (key >> shift) <= prefix), key); });
     __syncthreads();
+
+    // ---- 3. rank the survivors
     const int kept = s_kept < kMergeSelectCap ? s_kept : kMergeSelectCap;
     const float pad = metric == kMetricL2 ? 3.402823466e+38f : -3.402823466e+38f;
-    if (kept <= 1024) {
-        // rank by counting: every thread reads the same survivor at a time (an LDS broadcast)
-        for (int e = tid; e < kept; e += NT) {
-            const key_t mine = surv[e];
-            int rank = 0;
-            for (int j = 0; j < kept; j++) {
-                const key_t v = surv[j];
-                rank += (v < mine || (v == mine && j < e)) ? 1 : 0;
+    if (kept <= kMergeCountMax) {
+        // rank by counting (work grows with the square of the survivors: beyond a few hundred the sort below wins).  With fewer survivors than threads, `parts` threads share a survivor: each counts over
+        // its stretch of the array (neighbouring lanes read the same keys: LDS broadcasts) and adds to the
+        // survivor's rank in LDS.
+        const int parts = kept > 0 ? (NT / kept < 8 ? (NT / kept < 1 ? 1 : NT / kept) : 8) : 1;
+        const int stretch = (kept + parts - 1) / parts;
+        for (int i = tid; i < kept; i += NT) {
+            hist[i] = 0;
+        }
+        __syncthreads();
+        {
+            const int e = tid / parts, part = tid - e * parts;
+            if (e < kept) {
+                const key_t me = surv[e];
+                const int j0 = part * stretch, j1 = j0 + stretch < kept ? j0 + stretch : kept;
+                int rank = 0;
+                for (int j = j0; j < j1; j++) {
+                    const key_t v = surv[j];
+                    rank += (v < me || (v == me && j < e)) ? 1 : 0;
+                }
+                atomicAdd(&hist[e], rank);
             }
+        }
+        __syncthreads();
+        for (int e = tid; e < kept; e += NT) {
+            const int rank = hist[e];
             if (rank < k) {
-                const float v = key_score(mine);
+                const key_t me = surv[e];
+                const float v = key_score(me);
                 out_dist[q * k + rank] = metric == kMetricL2 ? v : -v;
-                out_labels[q * k + rank] = ids[key_index(mine)];
+                out_labels[q * k + rank] = ids[key_index(me)];
             }
         }
         for (int i = kept + tid; i < k; i += NT) {
@@ -779,7 +882,7 @@ __global__ __launch_bounds__(kMergeSelectThreads) void ivfpq_merge_kernel(
         }
         return;
     }
-    int n2 = 2048;
+    int n2 = 512;
     while (n2 < kept) {
         n2 <<= 1;
     }
