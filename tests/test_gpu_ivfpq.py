@@ -491,11 +491,43 @@ def test_whole_lists_tie_and_the_answer_does_not_depend_on_the_plan(ix, oracle, 
         assert np.array_equal(I1[0], I[j]) and np.array_equal(D1[0].view(np.uint32), D[j].view(np.uint32))
 
 
+@pytest.mark.parametrize("k", [2048, 700])
+def test_merge_of_slices_that_give_no_bound(ix, oracle, k):
+    """Eight probed lists, one per workgroup of a split query: seven of 1500 vectors (fewer than k = 2048, so no
+    slice is full) and one of 50 (fewer than the rank the merge samples in every slice), so the slices' own order
+    bounds nothing and all 10550 keys -- more than the merge keeps in registers -- go through the radix
+    selection in global memory.  With k = 700 the seven slices are full and the bound keeps a few thousand keys
+    in registers.  Either way the answer is the oracle's and the one a large batch (no split, no merge) gives."""
+    rng = np.random.default_rng(91)
+    d, M, nlist = 32, 4, 8
+    cent = (4.0 * rng.standard_normal((nlist, d))).astype(np.float32)
+    sizes = [1500] * 7 + [50]
+    owner = np.repeat(np.arange(nlist), sizes)
+    x = (cent[owner] + 0.5 * rng.standard_normal((len(owner), d))).astype(np.float32)
+    q = (cent[rng.integers(0, nlist, 500)] + 0.5 * rng.standard_normal((500, d))).astype(np.float32)
+    cb = oracle.train_pq(x[::3], M, niter=4, seed=5)
+    ids = rng.permutation(10 * len(x))[: len(x)].astype(np.int64)
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, ids)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig())
+    gpu.set_trained(cent, cb)
+    gpu.add_with_ids(x, ids)
+    assert sorted(gpu.getListLength(l) for l in range(nlist)) == sorted(sizes)
+    gpu.setNumProbes(nlist)
+    D, I = gpu.search(q, k)
+    assert gpu.last_search_stats()["nsplit"] == 1
+    Dr, Ir = ref.search(q[:4], k, nlist)
+    assert_topk_parity(oracle, ref, q[:4], D[:4], I[:4], Dr, Ir, TOL_FP32)
+    for j in (0, 1, 2, 3, 77):
+        D1, I1 = gpu.search(q[j:j + 1], k)
+        assert gpu.last_search_stats()["nsplit"] == 8
+        assert np.array_equal(I1[0], I[j]) and np.array_equal(D1[0].view(np.uint32), D[j].view(np.uint32))
+
+
 @pytest.mark.parametrize("metric_name,k", [("L2", 50), ("L2", 300), ("IP", 300), ("L2", 2048)])
 def test_one_query_split_over_many_workgroups(ix, oracle, metric_name, k):
     """Long lists (25000 codes each): a small batch is split over sixteen workgroups per query, one per probed
-    list, and the slices are merged by radix selection -- a handful of survivors ranked by counting (k = 50,
-    300), thousands sorted (k = 2048).  The answer is the oracle's, and the one a large batch (one workgroup per
+    list, and the slices are merged (a bound from their own order, then radix selection) -- a few hundred
+    survivors ranked by counting (k = 50, 300), thousands sorted (k = 2048).  The answer is the oracle's, and the one a large batch (one workgroup per
     query, no merge) gives for the same queries, bit for bit."""
     metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
     gpu, ref, x, q, ids = build_pair(ix, oracle, 17, 400_000, 1500, 32, 16, 8, metric, niter=3)
