@@ -196,6 +196,8 @@ def main():
     ap.add_argument("--nprobe", type=int, default=0)
     ap.add_argument("--k", type=int, default=0)
     ap.add_argument("--m", type=int, default=0, help="override the number of sub-quantizers")
+    ap.add_argument("--sigma", type=float, default=0.0,
+                    help="override the within-cluster standard deviation of the synthetic mixture (centres are N(0, 1))")
     ap.add_argument("--min-seconds", type=float, default=0.5,
                     help="after the K timed steps, keep stepping until this much time has been measured in all "
                          "(reported under 'sustained'; 'value' stays the K steps)")
@@ -239,7 +241,7 @@ def main():
             w[key] = getattr(args, key)
     if args.m:
         w["M"] = args.m
-    d, M, comp, sigma = w["d"], w["M"], w["comp"], w["sigma"]
+    d, M, comp, sigma = w["d"], w["M"], w["comp"], args.sigma or w["sigma"]
     n, nq, k, nprobe, nlist = w["n"], w["nq"], w["k"], w["nprobe"], w["nlist"]
     metric = ix.METRIC_L2 if w["metric"] == "L2" else ix.METRIC_INNER_PRODUCT
     unit = bool(w.get("unit"))

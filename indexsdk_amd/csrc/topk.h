@@ -373,21 +373,33 @@ template <int W>
 struct BlockPool {
     static constexpr int NT = W * kWave;
     static constexpr int kMaxPerThread = W >= 16 ? 4 : 8;   // cap <= kMaxPerThread * NT
-    key_t *buf;
-    int *hist;                 // 1024 ints
-    volatile BlockPoolCtl *ctl;
+    // Every pointer SAYS that it is an LDS address.  Through generic pointers the compiler emits flat
+    // instructions, which count as vector-memory operations as well: with one anywhere in the scan loop (the
+    // poll of `flag`, a prune) it can no longer tell a pending flat access from the codes of the next group that
+    // were requested a moment ago, waits for everything before it evaluates the current group, and the scan runs
+    // at one memory latency per group.
+    typedef __attribute__((address_space(3))) key_t lds_key_t;
+    typedef __attribute__((address_space(3))) int lds_int_t;
+    typedef __attribute__((address_space(3))) BlockPoolCtl lds_ctl_t;
+    lds_key_t *buf;
+    lds_int_t *hist;           // 1024 ints
+    volatile lds_ctl_t *ctl;
     int cap, k;
+    static __device__ __forceinline__ int lds_add(volatile lds_int_t *p, int v)
+    {
+        return __hip_atomic_fetch_add((lds_int_t *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     float bound;               // wave-uniform copy of ctl->bound
     key_t bound_key;           // wave-uniform copy of ctl->bound_key
 
     // All threads call; a __syncthreads() must follow before the first push.
     __device__ __forceinline__ void init(key_t *b, int cap_, int k_, int *hist_, BlockPoolCtl *c, int tid)
     {
-        buf = b;
+        buf = (lds_key_t *)b;
         cap = cap_;
         k = k_;
-        hist = hist_;
-        ctl = c;
+        hist = (lds_int_t *)hist_;
+        ctl = (volatile lds_ctl_t *)c;
         bound = __builtin_inff();
         bound_key = kEmptyKey;
         if (tid == 0) {
@@ -401,7 +413,7 @@ struct BlockPool {
         }
     }
 
-    __device__ __forceinline__ bool poll() const { return __builtin_amdgcn_readfirstlane(ctl->flag) != 0; }
+    __device__ __forceinline__ bool poll() const { return __builtin_amdgcn_readfirstlane(ctl->flag) != 0; }   // ds_read
 
     // All lanes of the wave call.  False: the pool is full -- call rendezvous(), re-test the
     // candidates against the new bound and try again.
@@ -422,7 +434,7 @@ struct BlockPool {
         const int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
         int base = 0;
         if (lane == 0) {
-            base = atomicAdd(const_cast<int *>(&ctl->count), n);
+            base = lds_add(&ctl->count, n);
         }
         base = __builtin_amdgcn_readfirstlane(base);
         if (base + n <= cap) {
@@ -443,7 +455,7 @@ struct BlockPool {
     __device__ __forceinline__ void finish_wave(int lane)
     {
         if (lane == 0) {
-            atomicAdd(const_cast<int *>(&ctl->done), 1);
+            lds_add(&ctl->done, 1);
         }
     }
 
@@ -507,7 +519,7 @@ struct BlockPool {
 #pragma unroll
             for (int j = 0; j < kMaxPerThread; j++) {
                 if (e[j] != kEmptyKey) {
-                    atomicAdd(&hist[(uint32_t)(e[j] >> (32 + SH + 10))], 1);
+                    lds_add(&hist[(uint32_t)(e[j] >> (32 + SH + 10))], 1);
                 }
             }
             __syncthreads();
@@ -524,7 +536,7 @@ struct BlockPool {
             for (int j = 0; j < kMaxPerThread; j++) {
                 const uint32_t pre = (uint32_t)(e[j] >> (32 + SH));
                 if (e[j] != kEmptyKey && (pre >> 10) == b1) {
-                    atomicAdd(&hist[pre & 1023u], 1);
+                    lds_add(&hist[pre & 1023u], 1);
                 }
             }
             __syncthreads();
@@ -545,7 +557,7 @@ struct BlockPool {
                     __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
                 int base = 0;
                 if (lane == 0) {
-                    base = atomicAdd(const_cast<int *>(&ctl->kept), __popcll(mask));
+                    base = lds_add(&ctl->kept, __popcll(mask));
                 }
                 base = __builtin_amdgcn_readfirstlane(base);
                 if (keep) {
@@ -561,7 +573,7 @@ struct BlockPool {
             for (int i = kept + tid; i < cap; i += NT) {
                 buf[i] = kEmptyKey;
             }
-            block_bitonic_sort(buf, cap, tid, NT);
+            block_bitonic_sort((key_t *)buf, cap, tid, NT);
             kept = k;
             top = key_score(buf[k - 1]);
             if (tid == 0) {
@@ -606,7 +618,7 @@ struct BlockPool {
         for (int i = n + tid; i < n2; i += NT) {
             buf[i] = kEmptyKey;
         }
-        block_bitonic_sort(buf, n2, tid, NT);
+        block_bitonic_sort((key_t *)buf, n2, tid, NT);
         return n;
     }
 };
