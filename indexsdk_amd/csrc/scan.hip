@@ -500,9 +500,13 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     // One step: start the loads of the group after next, evaluate the current group, offer it to
     // the pool.  Two register sets (a, b) alternate so that no code registers are ever copied; the
     // step is a macro so that both sets stay in registers (no address of either is ever taken).
-#define IXA_SCAN_STEP(G, CUR, WCUR, NXT, WNXT)                                                        \
+    // PF: the step starts the next group's loads.  The loops below start them unconditionally (PF a literal) and
+    // leave the last groups to a tail without them: behind a load that is issued under a condition the compiler
+    // waits for EVERY outstanding load before it evaluates the current group, the one just requested included,
+    // and a wavefront then walks its groups at one memory round trip each.
+#define IXA_SCAN_STEP(G, CUR, WCUR, NXT, WNXT, PF)                                                    \
     do {                                                                                              \
-        if ((G) + W < total) {                                                                        \
+        if (PF) {                                                                                     \
             NXT = locate((G) + W);                                                                    \
             if (!kSkipPadding || NXT.valid) { /* lanes past the list's end fetch nothing */           \
                 load_codes(NXT.slot, WNXT); /* in flight while the current group is evaluated */      \
@@ -517,9 +521,9 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
     } while (0)
     // The same step for the shared pool: poll for a pending prune, evaluate, reserve-and-append;
     // a failed reservation is retried after the workgroup has pruned the pool.
-#define IXA_SCAN_STEP_SHARED(G, CUR, WCUR, NXT, WNXT)                                                 \
+#define IXA_SCAN_STEP_SHARED(G, CUR, WCUR, NXT, WNXT, PF)                                             \
     do {                                                                                              \
-        if ((G) + W < total) {                                                                        \
+        if (PF) {                                                                                     \
             NXT = locate((G) + W);                                                                    \
             if (!kSkipPadding || NXT.valid) {                                                         \
                 load_codes(NXT.slot, WNXT);                                                           \
@@ -541,10 +545,26 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             if (!kSkipPadding || ga.valid) {
                 load_codes(ga.slot, wa);
             }
-            for (int G = wave; G < total; G += 2 * W) {
-                IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb);
-                if (G + W < total) {
-                    IXA_SCAN_STEP_SHARED(G + W, gb, wb, ga, wa);
+            if constexpr (W == 16) {
+                // sixteen wavefronts hide the latency by themselves, and the plain loop measured 2.5 % faster
+                // there (100M x 96, nprobe 256, k 1024: scan 4.34 against 4.44 ms)
+                for (int G = wave; G < total; G += 2 * W) {
+                    IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb, G + W < total);
+                    if (G + W < total) {
+                        IXA_SCAN_STEP_SHARED(G + W, gb, wb, ga, wa, G + 2 * W < total);
+                    }
+                }
+            } else {
+                int G = wave;
+                for (; G + 2 * W < total; G += 2 * W) {   // the groups G, G + W and G + 2 W exist
+                    IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb, 1);
+                    IXA_SCAN_STEP_SHARED(G + W, gb, wb, ga, wa, 1);
+                }
+                if (G + W < total) {   // two groups left (the first is in set a), or one
+                    IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb, 1);
+                    IXA_SCAN_STEP_SHARED(G + W, gb, wb, ga, wa, 0);
+                } else {
+                    IXA_SCAN_STEP_SHARED(G, ga, wa, gb, wb, 0);
                 }
             }
         }
@@ -559,11 +579,16 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             if (!kSkipPadding || ga.valid) {
                 load_codes(ga.slot, wa);
             }
-            for (int G = wave; G < total; G += 2 * W) {
-                IXA_SCAN_STEP(G, ga, wa, gb, wb);
-                if (G + W < total) {
-                    IXA_SCAN_STEP(G + W, gb, wb, ga, wa);
-                }
+            int G = wave;
+            for (; G + 2 * W < total; G += 2 * W) {   // the groups G, G + W and G + 2 W exist
+                IXA_SCAN_STEP(G, ga, wa, gb, wb, 1);
+                IXA_SCAN_STEP(G + W, gb, wb, ga, wa, 1);
+            }
+            if (G + W < total) {   // two groups left (the first is in set a), or one
+                IXA_SCAN_STEP(G, ga, wa, gb, wb, 1);
+                IXA_SCAN_STEP(G + W, gb, wb, ga, wa, 0);
+            } else {
+                IXA_SCAN_STEP(G, ga, wa, gb, wb, 0);
             }
         }
         __syncthreads();  // every wave has published its last value; the LUT is no longer needed
