@@ -38,9 +38,6 @@ void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter
 // Persistent ring kernels (score_ring.hip): same results as the tile kernels, at a much higher
 // matrix-core rate.  Return false when the shape does not qualify (d not a multiple of one K-step,
 // fewer than 1024 base rows, unaligned operands); nothing has been launched then.
-bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
-                          const int32_t *bn, int32_t *out, int64_t ldo, bool filter, ScoreFilter<int32_t> flt,
-                          hipStream_t s);
 bool launch_score_ring_f32(const float *Q, int64_t nq, const float *B, int64_t nb, int d, const float *qn,
                            const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                            hipStream_t s);
@@ -125,11 +122,5 @@ void launch_gather_scores(const float *scores, int64_t ld, const int32_t *idx, i
 void launch_refine(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn, int metric,
                    const int32_t *cand, int ncand, int nout, int out_stride, int32_t *out_ids, float *out_dist,
                    hipStream_t s);
-
-// Exact int32 L2 scores on the int8 matrix cores: out[row * ldo + col] = |q|^2 + |b|^2 - 2 q.b.
-void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
-                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s);
-void launch_score_tiles_i8_filtered(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
-                                    const int32_t *qn, const int32_t *bn, ScoreFilter<int32_t> flt, hipStream_t s);
 
 }  // namespace ixa

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "coarse.h"
+#include "flat_i8.h"
 #include "flat_index.h"
 #include "stream_select.h"
 #include "topk.h"
@@ -47,189 +48,7 @@ __global__ __launch_bounds__(256) void sqnorm_rows_i8_kernel(const int8_t *__res
     }
 }
 
-// Exact int32 L2 score tile: out[row][col] = |q|^2 + |b|^2 - 2 q.b   (integer part of
-// FR/ops/ascendc/op_kernel/ascendc_dist_int8_flat_l2.cpp:201-203, 485-500).
-// 128 x 128 tile per workgroup, 64 x 64 per wavefront as 2 x 2 blocks of v_mfma_i32_32x32x32_i8;
-// K-steps of 64 bytes staged in LDS with an 80-byte row stride (conflict-free 128-bit reads).
-constexpr int kTile = 128;
-constexpr int kKBytes = 64;
-constexpr int kRowStride = 80;
-
-template <bool VEC16>
-__device__ __forceinline__ uint4 load_k16(const int8_t *row, int k, int d)
-{
-    if (VEC16) {
-        if (k < d) {
-            return *reinterpret_cast<const uint4 *>(row + k);
-        }
-        return make_uint4(0, 0, 0, 0);
-    }
-    uint32_t w[4] = {0, 0, 0, 0};
-    for (int t = 0; t < 16; t++) {
-        if (k + t < d) {
-            w[t >> 2] |= (uint32_t)(uint8_t)row[k + t] << (8 * (t & 3));
-        }
-    }
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
-template <bool VEC16, bool FILTER>
-__global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__restrict__ Q, int64_t nq,
-                                                            const int8_t *__restrict__ B, int64_t nb, int d,
-                                                            const int32_t *__restrict__ qn,
-                                                            const int32_t *__restrict__ bn, int32_t *__restrict__ out,
-                                                            int64_t ldo, int tiles_m, int tiles_n,
-                                                            ScoreFilter<int32_t> flt)
-{
-    __shared__ __align__(16) unsigned char As[2][kTile * kRowStride];
-    __shared__ __align__(16) unsigned char Bs[2][kTile * kRowStride];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wr = wave >> 1, wc = wave & 1;
-    const int half = lane >> 5, l32 = lane & 31;
-    // 8 consecutive workgroups (one per XCD) take 8 different base tiles; each XCD then walks all
-    // query tiles of its base tile, so a base tile is fetched from HBM once and re-used from L2
-    const int64_t gs = (int64_t)8 * tiles_m;
-    const int64_t grp = blockIdx.x / gs, rem = blockIdx.x % gs;
-    const int64_t tile_n = grp * 8 + (rem & 7), tile_m = rem >> 3;
-    if (tile_n >= tiles_n) {
-        return;
-    }
-    const int64_t i0 = tile_m * kTile, j0 = tile_n * kTile;
-
-    const int lrow0 = tid >> 2, lrow1 = (tid + 256) >> 2, lk = (tid & 3) * 16;
-    const int64_t qa0 = i0 + lrow0 < nq ? i0 + lrow0 : nq - 1, qa1 = i0 + lrow1 < nq ? i0 + lrow1 : nq - 1;
-    const int64_t ba0 = j0 + lrow0 < nb ? j0 + lrow0 : nb - 1, ba1 = j0 + lrow1 < nb ? j0 + lrow1 : nb - 1;
-    const int8_t *qrow0 = Q + qa0 * d, *qrow1 = Q + qa1 * d;
-    const int8_t *brow0 = B + ba0 * d, *brow1 = B + ba1 * d;
-
-    v16i acc[2][2];
-#pragma unroll
-    for (int a = 0; a < 2; a++) {
-#pragma unroll
-        for (int b = 0; b < 2; b++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[a][b][r] = 0;
-            }
-        }
-    }
-    const int nk = (d + kKBytes - 1) / kKBytes;
-    uint4 ra0 = load_k16<VEC16>(qrow0, lk, d), ra1 = load_k16<VEC16>(qrow1, lk, d);
-    uint4 rb0 = load_k16<VEC16>(brow0, lk, d), rb1 = load_k16<VEC16>(brow1, lk, d);
-    *reinterpret_cast<uint4 *>(&As[0][lrow0 * kRowStride + lk]) = ra0;
-    *reinterpret_cast<uint4 *>(&As[0][lrow1 * kRowStride + lk]) = ra1;
-    *reinterpret_cast<uint4 *>(&Bs[0][lrow0 * kRowStride + lk]) = rb0;
-    *reinterpret_cast<uint4 *>(&Bs[0][lrow1 * kRowStride + lk]) = rb1;
-    __syncthreads();
-    for (int ks = 0; ks < nk; ks++) {
-        const int buf = ks & 1;
-        if (ks + 1 < nk) {
-            const int k = (ks + 1) * kKBytes + lk;
-            ra0 = load_k16<VEC16>(qrow0, k, d);
-            ra1 = load_k16<VEC16>(qrow1, k, d);
-            rb0 = load_k16<VEC16>(brow0, k, d);
-            rb1 = load_k16<VEC16>(brow1, k, d);
-        }
-        v4i a[2][2], b[2][2];
-#pragma unroll
-        for (int blk = 0; blk < 2; blk++) {
-#pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
-                // the k index of an operand byte is a function of (lane half, byte position) that is
-                // the same for both operands, and integer sums are order-free, so any such
-                // assignment gives the exact dot product
-                a[blk][kk] = *reinterpret_cast<const v4i *>(
-                    &As[buf][(wr * 64 + blk * 32 + l32) * kRowStride + kk * 32 + half * 16]);
-                b[blk][kk] = *reinterpret_cast<const v4i *>(
-                    &Bs[buf][(wc * 64 + blk * 32 + l32) * kRowStride + kk * 32 + half * 16]);
-            }
-        }
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-#pragma unroll
-            for (int ra = 0; ra < 2; ra++) {
-#pragma unroll
-                for (int rb = 0; rb < 2; rb++) {
-                    acc[ra][rb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ra][kk], b[rb][kk], acc[ra][rb], 0, 0, 0);
-                }
-            }
-        }
-        if (ks + 1 < nk) {
-            const int nbuf = buf ^ 1;
-            *reinterpret_cast<uint4 *>(&As[nbuf][lrow0 * kRowStride + lk]) = ra0;
-            *reinterpret_cast<uint4 *>(&As[nbuf][lrow1 * kRowStride + lk]) = ra1;
-            *reinterpret_cast<uint4 *>(&Bs[nbuf][lrow0 * kRowStride + lk]) = rb0;
-            *reinterpret_cast<uint4 *>(&Bs[nbuf][lrow1 * kRowStride + lk]) = rb1;
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int rb = 0; rb < 2; rb++) {
-        const int64_t col = j0 + wc * 64 + rb * 32 + l32;
-        const int32_t bnv = col < nb ? bn[col] : 0;
-#pragma unroll
-        for (int ra = 0; ra < 2; ra++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int64_t row = i0 + wr * 64 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (row < nq && col < nb) {
-                    const int32_t v = qn[row] + bnv - 2 * acc[ra][rb][r];
-                    if (FILTER) {
-                        if (v <= flt.tau[row]) {
-                            const int pos = atomicAdd(&flt.cnt[row], 1);
-                            if (pos < flt.cap) {
-                                flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
-                            }
-                        }
-                    } else {
-                        out[row * ldo + col] = v;
-                    }
-                }
-            }
-        }
-    }
-}
-
 }  // namespace
-
-template <bool FILTER>
-static void launch_score_tiles_i8_t(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
-                                    const int32_t *qn, const int32_t *bn, int32_t *out, int64_t ldo,
-                                    ScoreFilter<int32_t> flt, hipStream_t s)
-{
-    if (nq == 0 || nb == 0) {
-        return;
-    }
-    const bool vec = (d % 16 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
-                     (reinterpret_cast<uintptr_t>(B) % 16 == 0);
-    if (vec && launch_score_ring_i8(Q, nq, B, nb, d, qn, bn, out, ldo, FILTER, flt, s)) {
-        return;
-    }
-    const int64_t tiles_m = (nq + kTile - 1) / kTile, tiles_n = (nb + kTile - 1) / kTile;
-    const int64_t nblocks = (tiles_n + 7) / 8 * 8 * tiles_m;
-    IXA_REQUIRE(nblocks < (int64_t)1 << 31, kErrInvalidParam, "score tile grid too large");
-    dim3 grid((unsigned)nblocks), block(256);
-    if (vec) {
-        hipLaunchKernelGGL((score_tile_i8_kernel<true, FILTER>), grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
-                           (int)tiles_m, (int)tiles_n, flt);
-    } else {
-        hipLaunchKernelGGL((score_tile_i8_kernel<false, FILTER>), grid, block, 0, s, Q, nq, B, nb, d, qn, bn, out, ldo,
-                           (int)tiles_m, (int)tiles_n, flt);
-    }
-}
-
-void launch_score_tiles_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
-                           const int32_t *bn, int32_t *out, int64_t ldo, hipStream_t s)
-{
-    launch_score_tiles_i8_t<false>(Q, nq, B, nb, d, qn, bn, out, ldo, ScoreFilter<int32_t>{}, s);
-}
-
-void launch_score_tiles_i8_filtered(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d,
-                                    const int32_t *qn, const int32_t *bn, ScoreFilter<int32_t> flt, hipStream_t s)
-{
-    launch_score_tiles_i8_t<true>(Q, nq, B, nb, d, qn, bn, nullptr, 0, flt, s);
-}
 
 namespace {
 
@@ -477,17 +296,39 @@ void FlatBase<T>::reserve(int64_t n)
         return;
     }
     const int64_t cap = std::max<int64_t>(n, capacity_ + capacity_ / 2);
-    DeviceBuffer<T> nb((size_t)cap * d_);
     DeviceBuffer<int64_t> ni((size_t)cap);
+    if (ntotal_ > 0) {
+        IXA_HIP(hipMemcpyAsync(ni.data(), ids_.data(), (size_t)ntotal_ * 8, hipMemcpyDeviceToDevice, stream_));
+    }
+    grow_base(cap);   // waits for the stream before it releases the old base
+    ids_ = std::move(ni);
+    capacity_ = cap;
+}
+
+template <typename T>
+void FlatBase<T>::grow_base(int64_t cap)
+{
+    DeviceBuffer<T> nb((size_t)cap * d_);
     if (ntotal_ > 0) {
         IXA_HIP(hipMemcpyAsync(nb.data(), base_.data(), (size_t)ntotal_ * d_ * sizeof(T), hipMemcpyDeviceToDevice,
                                stream_));
-        IXA_HIP(hipMemcpyAsync(ni.data(), ids_.data(), (size_t)ntotal_ * 8, hipMemcpyDeviceToDevice, stream_));
-        sync_stream(stream_);
     }
+    sync_stream(stream_);
     base_ = std::move(nb);
-    ids_ = std::move(ni);
-    capacity_ = cap;
+}
+
+template <typename T>
+void FlatBase<T>::store_rows(int64_t first, int64_t n, const T *x, bool on_device)
+{
+    IXA_HIP(hipMemcpyAsync(base_.data() + first * d_, x, (size_t)n * d_ * sizeof(T),
+                           on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice, stream_));
+}
+
+template <typename T>
+void FlatBase<T>::fetch_rows(int64_t offset, int64_t n, T *out) const
+{
+    IXA_HIP(hipMemcpyAsync(out, base_.data() + offset * d_, (size_t)n * d_ * sizeof(T), hipMemcpyDeviceToHost, stream_));
+    sync_stream(stream_);
 }
 
 // add / add_with_ids (FR/ascend/AscendIndex.h:66-71); ids default to ntotal + i.
@@ -499,7 +340,7 @@ void FlatBase<T>::add(int64_t n, const T *x, const int64_t *ids, bool on_device)
     IXA_REQUIRE(ntotal_ + n < ((int64_t)1 << 32) - 1, kErrInvalidParam, "index would exceed the 32-bit row space");
     reserve(ntotal_ + n);
     const hipMemcpyKind kind = on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
-    IXA_HIP(hipMemcpyAsync(base_.data() + ntotal_ * d_, x, (size_t)n * d_ * sizeof(T), kind, stream_));
+    store_rows(ntotal_, n, x, on_device);
     if (ids) {
         IXA_HIP(hipMemcpyAsync(ids_.data() + ntotal_, ids, (size_t)n * 8, kind, stream_));
     } else {
@@ -516,9 +357,7 @@ void FlatBase<T>::get_base(int64_t offset, int64_t n, T *out) const
     IXA_REQUIRE(offset >= 0 && n >= 0 && offset + n <= ntotal_ && (n == 0 || out), kErrInvalidParam,
                 "range [%ld, %ld) is outside the index (ntotal %ld)", (long)offset, (long)(offset + n), (long)ntotal_);
     if (n) {
-        IXA_HIP(hipMemcpyAsync(out, base_.data() + offset * d_, (size_t)n * d_ * sizeof(T), hipMemcpyDeviceToHost,
-                               stream_));
-        sync_stream(stream_);
+        fetch_rows(offset, n, out);
     }
 }
 
@@ -606,12 +445,18 @@ int64_t FlatBase<T>::remove_selected(int64_t nv, const int64_t *victims, int64_t
     if (!moves.empty()) {
         DeviceBuffer<int64_t> moves_dev;
         moves_dev.upload(moves.data(), moves.size(), stream_);
-        hipLaunchKernelGGL((move_rows_kernel<T>), dim3((unsigned)(moves.size() / 2)), dim3(128), 0, stream_, base_.data(),
-                           ids_.data(), norms, moves_dev.data(), d_);
+        move_rows(moves_dev.data(), (int64_t)(moves.size() / 2), norms);
         sync_stream(stream_);   // moves_dev is freed on return
     }
     ntotal_ = left;
     return (int64_t)hits;
+}
+
+template <typename T>
+void FlatBase<T>::move_rows(const int64_t *moves, int64_t nmoves, uint32_t *norms)
+{
+    hipLaunchKernelGGL((move_rows_kernel<T>), dim3((unsigned)nmoves), dim3(128), 0, stream_, base_.data(), ids_.data(),
+                       norms, moves, d_);
 }
 
 template <typename T>
@@ -832,29 +677,88 @@ FlatI8Index::FlatI8Index(int d, int metric, int64_t scratch_bytes) : FlatBase<in
     IXA_REQUIRE(metric == kMetricL2, kErrInvalidParam, "Unsupported metric type");
 }
 
+// The base lives in matrix-core order (flat_i8.h); vectors come in and go out row-major through ws_rows_.
+void FlatI8Index::grow_base(int64_t cap)
+{
+    DeviceBuffer<int8_t> nb(i8_tiled_bytes(cap, d_));
+    DeviceBuffer<int32_t> nn((size_t)round_up(cap, kI8TileRows));
+    if (ntotal_ > 0) {
+        // blocks of 32 vectors are contiguous: the blocks that hold the first ntotal_ vectors
+        IXA_HIP(hipMemcpyAsync(nb.data(), base_.data(), (size_t)round_up(ntotal_, kI8BlockRows) * i8_padded_dim(d_),
+                               hipMemcpyDeviceToDevice, stream_));
+        IXA_HIP(hipMemcpyAsync(nn.data(), norms_.data(), (size_t)ntotal_ * 4, hipMemcpyDeviceToDevice, stream_));
+    }
+    sync_stream(stream_);
+    base_ = std::move(nb);
+    norms_ = std::move(nn);
+}
+
+void FlatI8Index::store_rows(int64_t first, int64_t n, const int8_t *x, bool on_device)
+{
+    // host vectors pass through a bounded staging buffer, piece by piece
+    const int64_t piece = on_device ? n : std::max<int64_t>(1, ((int64_t)256 << 20) / d_);
+    for (int64_t o = 0; o < n; o += piece) {
+        const int64_t m = std::min(piece, n - o);
+        const int8_t *xd = x + o * d_;
+        if (!on_device) {
+            if (o > 0) {
+                sync_stream(stream_);   // the kernels that read the previous piece
+            }
+            ws_rows_.upload(xd, (size_t)m * d_, stream_);
+            xd = ws_rows_.data();
+        }
+        launch_i8_tile_rows(xd, m, d_, base_.data(), first + o, stream_);
+        hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((m + 3) / 4)), dim3(256), 0, stream_, xd, m, d_,
+                           norms_.data() + first + o);
+    }
+}
+
+void FlatI8Index::fetch_rows(int64_t offset, int64_t n, int8_t *out) const
+{
+    // in pieces, so that the staging buffer stays small whatever the caller asks for
+    const int64_t piece = std::max<int64_t>(1, ((int64_t)64 << 20) / d_);
+    for (int64_t o = 0; o < n; o += piece) {
+        const int64_t m = std::min(piece, n - o);
+        ws_rows_.resize((size_t)m * d_);
+        launch_i8_untile_rows(base_.data(), offset + o, m, d_, ws_rows_.data(), stream_);
+        ws_rows_.download(out + o * d_, (size_t)m * d_, stream_);
+    }
+}
+
+void FlatI8Index::move_rows(const int64_t *moves, int64_t nmoves, uint32_t *norms)
+{
+    launch_i8_move_rows(base_.data(), d_, ids_.data(), reinterpret_cast<int32_t *>(norms), moves, nmoves, stream_);
+}
+
+void FlatI8Index::pad_norms()
+{
+    if (capacity_ > 0) {
+        launch_i8_pad_norms(norms_.data(), ntotal_, round_up(std::max<int64_t>(ntotal_, 1), kI8TileRows), stream_);
+    }
+}
+
 void FlatI8Index::add(int64_t n, const int8_t *x, const int64_t *ids, bool on_device)
 {
-    const int64_t before = ntotal_;
-    FlatBase<int8_t>::add(n, x, ids, on_device);
-    DeviceBuffer<int32_t> nn((size_t)capacity_);
-    if (before > 0) {
-        IXA_HIP(hipMemcpyAsync(nn.data(), norms_.data(), (size_t)before * 4, hipMemcpyDeviceToDevice, stream_));
-    }
-    hipLaunchKernelGGL(sqnorm_rows_i8_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, stream_,
-                       base_.data() + before * d_, n, d_, nn.data() + before);
+    FlatBase<int8_t>::add(n, x, ids, on_device);   // store_rows computes the norms of what it stores
+    pad_norms();
     sync_stream(stream_);
-    norms_ = std::move(nn);
 }
 
 int64_t FlatI8Index::remove_ids(int64_t n, const int64_t *ids)
 {
     IXA_REQUIRE(n >= 0 && (n == 0 || ids), kErrInvalidParam, "ids can not be nullptr.");
-    return remove_selected(n, ids, 0, 0, reinterpret_cast<uint32_t *>(norms_.data()));
+    const int64_t gone = remove_selected(n, ids, 0, 0, reinterpret_cast<uint32_t *>(norms_.data()));
+    pad_norms();
+    sync_stream(stream_);
+    return gone;
 }
 
 int64_t FlatI8Index::remove_range(int64_t imin, int64_t imax)
 {
-    return remove_selected(0, nullptr, imin, imax, reinterpret_cast<uint32_t *>(norms_.data()));
+    const int64_t gone = remove_selected(0, nullptr, imin, imax, reinterpret_cast<uint32_t *>(norms_.data()));
+    pad_norms();
+    sync_stream(stream_);
+    return gone;
 }
 
 void FlatI8Index::reset()

@@ -28,7 +28,7 @@ template <typename T>
 class FlatBase {
 public:
     FlatBase(int d, int metric, int64_t scratch_bytes);
-    ~FlatBase();
+    virtual ~FlatBase();
     FlatBase(const FlatBase &) = delete;
     FlatBase &operator=(const FlatBase &) = delete;
 
@@ -43,6 +43,15 @@ public:
 
 protected:
     void reserve(int64_t n);
+    // How the vectors lie in base_: row-major here; FlatI8Index keeps them in matrix-core order (flat_i8.h).
+    // new_base <- the first ntotal_ vectors of base_, with room for cap
+    virtual void grow_base(int64_t cap);
+    // vectors [first, first + n) <- n row-major vectors (host or device memory); queued on stream_
+    virtual void store_rows(int64_t first, int64_t n, const T *x, bool on_device);
+    // n row-major vectors in host memory <- vectors [offset, offset + n)
+    virtual void fetch_rows(int64_t offset, int64_t n, T *out) const;
+    // move j: vector moves[2 j + 1] (with id and norm) over vector moves[2 j]; device array of nmoves pairs
+    virtual void move_rows(const int64_t *moves, int64_t nmoves, uint32_t *norms);
     // removes the vectors whose id is one of the nv host ids (victims != nullptr) or lies in [imin, imax);
     // norms: the derived class's 4-byte norm per vector, moved along; returns the number removed
     int64_t remove_selected(int64_t nv, const int64_t *victims, int64_t imin, int64_t imax, uint32_t *norms);
@@ -95,7 +104,14 @@ public:
 private:
     void search_masked(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device,
                        const uint8_t *mask_dev, int64_t mask_stride);
+    void grow_base(int64_t cap) override;
+    void store_rows(int64_t first, int64_t n, const int8_t *x, bool on_device) override;
+    void fetch_rows(int64_t offset, int64_t n, int8_t *out) const override;
+    void move_rows(const int64_t *moves, int64_t nmoves, uint32_t *norms) override;
+    void pad_norms();   // INT32_MAX behind the last vector, up to the end of its tile of 256
+    // norms_: one per vector, allocated in whole tiles of 256 vectors like the tiled base
     DeviceBuffer<int32_t> norms_, ws_qn_, ws_dist_;
+    mutable DeviceBuffer<int8_t> ws_rows_;   // row-major staging of vectors on their way in or out
     StreamSelectWorkspace<int32_t> ws_sel_;
     DeviceBuffer<int64_t> ws_labels_;
 };

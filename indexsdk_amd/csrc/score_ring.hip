@@ -1,12 +1,12 @@
 // Persistent "ring" score kernels: query x base score tiles at matrix-core rate.
 //
-// A K-step of MFMAs lasts a few hundred (int8) to a few thousand (fp32) cycles, and a tile of the
+// A K-step of MFMAs lasts a few hundred (bf16) to a few thousand (fp32) cycles, and a tile of the
 // headline shapes has only 8 K-steps, so a kernel that starts and drains a pipeline per tile spends
 // a large share of its time waiting for the first operands.  Here instead
 //   * a workgroup of 8 wavefronts is persistent (one per CU) and walks a list of 256 x 256 tiles; the
 //     stream of K-steps (64 bytes of every operand row each) runs continuously across tile
 //     boundaries.  The square tile stages 512 rows for 65536 products per K-element: the L2 -> LDS
-//     traffic, which bounds the int8 and bf16 variants, is 2/3 of what a 256 x 128 tile needs;
+//     traffic, which bounds the bf16 variant, is 2/3 of what a 256 x 128 tile needs;
 //   * operands go from global memory straight into LDS (global_load_lds_dwordx4, no VGPR staging)
 //     into a ring of kRingStages buffers, two to three steps ahead of the MFMAs; completion is
 //     tracked with s_waitcnt vmcnt + s_barrier, without the full memory fence of __syncthreads();
@@ -21,11 +21,12 @@
 //     16 different bank groups;
 //   * tiles are dealt so that all workgroups of an XCD work on the same base tile at the same time
 //     (it is fetched from HBM once and re-used out of that XCD's L2).
-// Scores: int8 -> exact int32 |q|^2 + |b|^2 - 2 q.b (v_mfma_i32_32x32x32_i8);
-//         bf16 -> fp32 accumulation (v_mfma_f32_32x32x16_bf16);
+// Scores: bf16 -> fp32 accumulation (v_mfma_f32_32x32x16_bf16);
 //         fp32 -> (|q|^2 + |b|^2) - g - g or -g (v_mfma_f32_32x32x2_f32).
-// The sum over k is order-free for integers, and for floating point any fixed k-assignment that is
-// the same for both operands is a valid accumulation order, so each lane half owns half of a K-step.
+// Any fixed k-assignment that is the same for both operands is a valid accumulation order, so each lane
+// half owns half of a K-step.  (int8 Flat has a kernel of its own: flat_i8.hip.)
+#include <type_traits>
+
 #include "coarse.h"
 #include "topk.h"
 
@@ -78,29 +79,6 @@ __device__ __forceinline__ void ring_wait_frag(RingFrag<V> &f)
                  : "+v"(f.a[0]), "+v"(f.a[1]), "+v"(f.a[2]), "+v"(f.a[3]), "+v"(f.b[0]), "+v"(f.b[1])
                  : "n"(N));
 }
-
-struct I8Traits {
-    using T = int8_t;
-    using S = int32_t;
-    using Acc = v16i;
-    using Frag = RingFrag<v4i>;
-    static constexpr int kElemsPerStep = 64;
-    // half-step hs = 32 bytes of the K-step; a lane half owns 16 of them
-    static __device__ __forceinline__ int chunk(int hs, int half) { return hs * 2 + half; }
-    template <bool SWAP, bool ZERO>
-    static __device__ __forceinline__ void mma(const Frag &f, Acc (&acc)[4][2])
-    {
-#pragma unroll
-        for (int ra = 0; ra < 4; ra++) {
-#pragma unroll
-            for (int rb = 0; rb < 2; rb++) {
-                const Acc c0 = ZERO ? Acc{} : acc[ra][rb];   // a tile's first product starts from zero
-                acc[ra][rb] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(f.b[rb], f.a[ra], c0, 0, 0, 0)
-                                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[ra], f.b[rb], c0, 0, 0, 0);
-            }
-        }
-    }
-};
 
 // bf16 operands, fp32 accumulation (v_mfma_f32_32x32x16_bf16): same data movement as int8.
 struct Bf16Traits {
@@ -175,9 +153,8 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
 {
     using T = typename Tr::T;
     using S = typename Tr::S;
-    constexpr bool kInt = sizeof(T) == 1;
     constexpr bool FILTER = MODE != 0, DUMP = MODE == 2, MINIMA = MODE == 3;
-    static_assert(!(DUMP || MINIMA) || !kInt, "record and group-minima epilogues: floating-point scores only");
+    static_assert(std::is_same<S, float>::value, "floating-point scores");
     extern __shared__ __align__(16) unsigned char ring[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -273,10 +250,10 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
     // these loads (kPrefetchLoads per wave).
     //   aux +   0: 64 base norms      (lanes 0..15, 16 bytes each)
     //   aux + 256: 128 tau or thr     (lanes 16..47)
-    //   aux + 768: 128 query norms    (lanes 0..31 of a second load; fp32 scores only)
-    constexpr int kPrefetchLoads = kInt ? 1 : 2;
+    //   aux + 768: 128 query norms    (lanes 0..31 of a second load)
+    constexpr int kPrefetchLoads = 2;
     unsigned char *aux = ring + kRingStages * kRingStageBytes + wave * kRingAuxBytes;
-    const S *bound = kInt ? flt.thr : flt.tau;
+    const S *bound = flt.tau;
     const bool prefetch = FILTER && nk >= 2 && nb % 4 == 0 && nq % 4 == 0 && bn != nullptr && qn != nullptr &&
                           bound != nullptr && reinterpret_cast<uintptr_t>(bn) % 16 == 0 &&
                           reinterpret_cast<uintptr_t>(qn) % 16 == 0 && reinterpret_cast<uintptr_t>(bound) % 16 == 0;
@@ -302,13 +279,11 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
                                              (__attribute__((address_space(3))) void *)aux, 16, 0, 0);
         }
-        if constexpr (!kInt) {
-            if (lane < 32) {
-                const int64_t first = i0 + wr * 128;
-                const S *p = lane < ((nq - first) >> 2) ? qn + first + lane * 4 : qn;
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
-                                                 (__attribute__((address_space(3))) void *)(aux + 768), 16, 0, 0);
-            }
+        if (lane < 32) {
+            const int64_t first = i0 + wr * 128;
+            const S *p = lane < ((nq - first) >> 2) ? qn + first + lane * 4 : qn;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p,
+                                             (__attribute__((address_space(3))) void *)(aux + 768), 16, 0, 0);
         }
         asm volatile("" ::: "memory");
     };
@@ -405,7 +380,6 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
             const int half = lane >> 5, l32 = lane & 31;
             // The epilogue's operands come out of the wave's staging area: put there one K-step ahead
             // by fetch_epilogue_operands(), or (shapes the staging loads do not serve) filled here.
-            // int8: the norms are negated in place, so that a score's test value is one shift-add.
             if (prefetch) {
                 // the staging loads are older than the K-step loads issued during this K-step
                 if (issued_now) {
@@ -414,23 +388,15 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
                     __builtin_amdgcn_s_waitcnt(ring_vmcnt(0));
                 }
                 asm volatile("" ::: "memory");
-                if constexpr (kInt) {
-                    S *p = reinterpret_cast<S *>(aux) + lane;
-                    *p = -*p;
-                }
             } else {
                 const int64_t col = j0 + wc * 64 + lane;
-                const bool use_bn = kInt || metric == kMetricL2;
-                const S bv = (use_bn && col < nb) ? bn[col] : (S)0;
-                reinterpret_cast<S *>(aux)[lane] = kInt ? -bv : bv;
+                reinterpret_cast<S *>(aux)[lane] = (metric == kMetricL2 && col < nb) ? bn[col] : (S)0;
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const int64_t row = i0 + wr * 128 + t * 64 + lane;
                     const bool ok = row < nq;
                     reinterpret_cast<S *>(aux + 256)[t * 64 + lane] = ok ? bound[row] : (S)0;
-                    if constexpr (!kInt) {
-                        reinterpret_cast<S *>(aux + 768)[t * 64 + lane] = (ok && metric == kMetricL2) ? qn[row] : (S)0;
-                    }
+                    reinterpret_cast<S *>(aux + 768)[t * 64 + lane] = (ok && metric == kMetricL2) ? qn[row] : (S)0;
                 }
             }
             wave_lds_fence();
@@ -543,18 +509,15 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
                 asm volatile("" ::: "memory");   // one query block at a time keeps register pressure low
                 const int64_t row = i0 + (wr * 128 + ra * 32 + l32);
                 const bool row_ok = row < nq;
-                // int8: rowv = tau - |q|^2 (|b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau, exact in
-                // integers); fp32: rowv = |q|^2, tauv = tau
-                const S bv = *reinterpret_cast<const S *>(aux + 256 + (ra * 32 + l32) * 4);
-                const S rowv = kInt ? bv : *reinterpret_cast<const S *>(aux + 768 + (ra * 32 + l32) * 4);
-                const S tauv = kInt ? (S)0 : bv;
+                const S tauv = *reinterpret_cast<const S *>(aux + 256 + (ra * 32 + l32) * 4);
+                const S rowv = *reinterpret_cast<const S *>(aux + 768 + (ra * 32 + l32) * 4);
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
                     // all 16 scores of the block first, then ONE test of their minimum against the
                     // lane's bound: admissions are rare, so the per-score path almost never runs
                     S v[16];
                     S best = ScoreOps<S>::worst();
-                    S bnq[4][4];   // (minus, for int8) the base norms of this lane's 16 columns of the block
+                    S bnq[4][4];   // the base norms of this lane's 16 columns of the block
 #pragma unroll
                     for (int rq = 0; rq < 4; rq++) {
                         const uint4 u = *reinterpret_cast<const uint4 *>(aux + (rb * 32 + 8 * rq + 4 * half) * 4);
@@ -566,27 +529,17 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const S bnv = bnq[r >> 2][r & 3];
-                        if constexpr (kInt) {
-                            // bnq holds -|b|^2: v = -(distance - |q|^2) in one shift-add, largest is best
-                            v[r] = (S)(((uint32_t)acc[ra][rb][r] << 1) + (uint32_t)bnv);
-                            best = (r == 0 || v[r] > best) ? v[r] : best;
-                            continue;
+                        const float g = acc[ra][rb][r];
+                        if (metric == kMetricL2) {
+                            float w = __fadd_rn(rowv, bnv);
+                            w = __fsub_rn(w, g);
+                            v[r] = __fsub_rn(w, g);
                         } else {
-                            const float g = acc[ra][rb][r];
-                            if (metric == kMetricL2) {
-                                float w = __fadd_rn(rowv, bnv);
-                                w = __fsub_rn(w, g);
-                                v[r] = __fsub_rn(w, g);
-                            } else {
-                                v[r] = -g;
-                            }
+                            v[r] = -g;
                         }
                         best = v[r] < best ? v[r] : best;
                     }
-                    const S lane_bound = kInt ? rowv : tauv;
-                    if constexpr (kInt) {
-                        best = -best;
-                    }
+                    const S lane_bound = tauv;
                     if (__ballot(row_ok && best <= lane_bound)) {
                         // opaque to the optimiser here, or it keeps all 32 column offsets of this rare
                         // path in registers across the whole main loop
@@ -595,15 +548,10 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             const int64_t col = j0 + cb + 8 * (r >> 2) + (r & 3);
-                            const S part = kInt ? -v[r] : v[r];
-                            if (row_ok && part <= lane_bound && col < nb) {
-                                S val = part;
-                                if constexpr (kInt) {
-                                    val += qn[row];
-                                }
+                            if (row_ok && v[r] <= lane_bound && col < nb) {
                                 const int pos = atomicAdd(&flt.cnt[row], 1);
                                 if (pos < flt.cap) {
-                                    flt.cand[row * flt.cap + pos] = make_key(val, (uint32_t)(col + flt.col_base));
+                                    flt.cand[row * flt.cap + pos] = make_key(v[r], (uint32_t)(col + flt.col_base));
                                 }
                             }
                         }
@@ -629,24 +577,19 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int rb = 0; rb < 2; rb++) {
                 const int64_t col = j0 + wc * 64 + rb * 32 + l32;
-                bnv[rb] = (col < nb && (kInt || metric == kMetricL2)) ? bn[col] : (S)0;
+                bnv[rb] = (col < nb && metric == kMetricL2) ? bn[col] : (S)0;
             }
 #pragma unroll
             for (int ra = 0; ra < 4; ra++) {
                 // one 32-row block at a time keeps the per-row operands of only 16 rows live
                 asm volatile("" ::: "memory");
-                S rowv[16];   // int8 + FILTER: tau - |q|^2; otherwise |q|^2
-                S tauv[16];   // fp32 + FILTER: tau
+                S rowv[16];   // |q|^2
+                S tauv[16];   // FILTER: tau
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    if (kInt) {
-                        // |b|^2 - 2 q.b <= tau - |q|^2  <=>  distance <= tau (exact in integers)
-                        rowv[r] = row < nq ? (FILTER ? flt.thr[row] : qn[row]) : (FILTER ? (S)0x80000000 : (S)0);
-                    } else {
-                        rowv[r] = (row < nq && metric == kMetricL2) ? qn[row] : (S)0;
-                        tauv[r] = (FILTER && row < nq) ? flt.tau[row] : (S)(-__builtin_inff());
-                    }
+                    rowv[r] = (row < nq && metric == kMetricL2) ? qn[row] : (S)0;
+                    tauv[r] = (FILTER && row < nq) ? flt.tau[row] : (S)(-__builtin_inff());
                 }
 #pragma unroll
                 for (int rb = 0; rb < 2; rb++) {
@@ -655,27 +598,17 @@ __global__ __launch_bounds__(kRingWaves * 64) __attribute__((amdgpu_waves_per_eu
                     for (int r = 0; r < 16; r++) {
                         const int64_t row = i0 + wr * 128 + ra * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                         S v;
-                        bool admit;
-                        if constexpr (kInt) {
-                            const S part = bnv[rb] - 2 * acc[ra][rb][r];
-                            admit = part <= rowv[r];
-                            v = FILTER ? part : part + rowv[r];
+                        const float g = acc[ra][rb][r];
+                        if (metric == kMetricL2) {
+                            v = __fadd_rn(rowv[r], bnv[rb]);
+                            v = __fsub_rn(v, g);
+                            v = __fsub_rn(v, g);
                         } else {
-                            const float g = acc[ra][rb][r];
-                            if (metric == kMetricL2) {
-                                v = __fadd_rn(rowv[r], bnv[rb]);
-                                v = __fsub_rn(v, g);
-                                v = __fsub_rn(v, g);
-                            } else {
-                                v = -g;
-                            }
-                            admit = v <= tauv[r];
+                            v = -g;
                         }
+                        const bool admit = v <= tauv[r];
                         if (FILTER) {
                             if (admit && col < nb) {
-                                if constexpr (kInt) {
-                                    v += qn[row];
-                                }
                                 const int pos = atomicAdd(&flt.cnt[row], 1);
                                 if (pos < flt.cap) {
                                     flt.cand[row * flt.cap + pos] = make_key(v, (uint32_t)(col + flt.col_base));
@@ -754,13 +687,6 @@ bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, i
 }
 
 }  // namespace
-
-bool launch_score_ring_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
-                          const int32_t *bn, int32_t *out, int64_t ldo, bool filter, ScoreFilter<int32_t> flt,
-                          hipStream_t s)
-{
-    return launch_ring<I8Traits>(Q, nq, B, nb, d, qn, bn, kMetricL2, out, ldo, filter ? 1 : 0, flt, s);
-}
 
 bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
                             const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,

@@ -54,6 +54,7 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq, const uint16_t 
                                  const float *qn, const float *bn, int metric, int ncand, unsigned long long *running,
                                  StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, int *flag,
                                  const BoundaryRefine *refine, hipStream_t s);
+// B: the base in matrix-core order and bn its norms padded with kI8PadNorm to whole tiles of 256 rows (flat_i8.h)
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,
                      int64_t scratch_bytes, hipStream_t s, const uint8_t *mask = nullptr, int64_t mask_stride = 0);

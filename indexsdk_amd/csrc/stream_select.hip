@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cmath>
 
+#include "flat_i8.h"
 #include "topk.h"
 
 namespace ixa {
@@ -33,14 +34,15 @@ __global__ __launch_bounds__(256) void keys_to_idx_kernel(const key_t *__restric
     }
 }
 
-// thr[i] = tau[i] - qn[i]
+// thr[i] = min(tau[i], kI8MaxBound) - qn[i]: a bound above every possible distance (a row that is not full yet has
+// the worst score for one) admits every row either way, and the score kernels rely on the smaller number
 __global__ __launch_bounds__(256) void threshold_i32_kernel(const int32_t *__restrict__ tau,
                                                             const int32_t *__restrict__ qn, int64_t n,
                                                             int32_t *__restrict__ thr)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n) {
-        thr[i] = tau[i] - qn[i];   // tau <= INT32_MAX and qn >= 0: no overflow
+        thr[i] = min(tau[i], kI8MaxBound) - qn[i];   // qn >= 0: no overflow
     }
 }
 
@@ -105,12 +107,12 @@ struct F32Ops {
     void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
                 hipStream_t s) const
     {
-        launch_score_tiles(Q, nq, B, nb, d, qn + q0, bn + b0, metric, out, ldo, s);
+        launch_score_tiles(Q, nq, B + b0 * d, nb, d, qn + q0, bn + b0, metric, out, ldo, s);
     }
     void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
                   hipStream_t s) const
     {
-        launch_score_tiles_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, metric, flt, s);
+        launch_score_tiles_filtered(Q, nq, B + b0 * d, nb, d, qn + q0, bn + b0, metric, flt, s);
     }
     void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
                 hipStream_t s) const
@@ -133,14 +135,14 @@ struct Bf16Ops {
     void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
                 hipStream_t s) const
     {
-        const bool ok = launch_score_ring_bf16(Q, nq, B, nb, d, qn + q0, bn + b0, metric, out, ldo, false,
+        const bool ok = launch_score_ring_bf16(Q, nq, B + b0 * d, nb, d, qn + q0, bn + b0, metric, out, ldo, false,
                                                ScoreFilter<float>{}, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
     }
     void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
                   hipStream_t s) const
     {
-        const bool ok = launch_score_ring_bf16(Q, nq, B, nb, d, qn + q0, bn + b0, metric, nullptr, 0, true, flt, s);
+        const bool ok = launch_score_ring_bf16(Q, nq, B + b0 * d, nb, d, qn + q0, bn + b0, metric, nullptr, 0, true, flt, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
     }
     void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
@@ -154,6 +156,8 @@ struct Bf16Ops {
     }
 };
 
+// B is the base in matrix-core order (flat_i8.h) and bn its norms, padded to whole tiles: a stretch of the base is
+// named by its rows, never by a pointer into it
 struct I8Ops {
     using T = int8_t;
     using S = int32_t;
@@ -168,12 +172,12 @@ struct I8Ops {
     void scores(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, S *out, int64_t ldo,
                 hipStream_t s) const
     {
-        launch_score_tiles_i8(Q, nq, B, nb, d, qn + q0, bn + b0, out, ldo, s);
+        launch_i8_scores_stored(Q, nq, B, d, qn + q0, bn, b0, b0 + nb, out, ldo, s);
     }
     void filtered(const T *Q, int64_t nq, int64_t q0, const T *B, int64_t nb, int64_t b0, int d, ScoreFilter<S> flt,
                   hipStream_t s) const
     {
-        launch_score_tiles_i8_filtered(Q, nq, B, nb, d, qn + q0, bn + b0, flt, s);
+        launch_i8_scores_filtered(Q, nq, B, d, qn + q0, bn, b0, b0 + nb, flt, s);
     }
     void select(const S *sc, int64_t nq, int64_t ld, int64_t nc, int k, int64_t base, key_t *run, bool fresh,
                 hipStream_t s) const
@@ -276,7 +280,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             const int64_t head = fused ? seed_rows : nb_total;
             for (int64_t b0 = 0; b0 < head; b0 += ldo) {
                 const int64_t nbc = std::min(ldo, head - b0);
-                ops.scores(Q + q0 * d, nq, q0, B + b0 * d, nbc, b0, d, ws.scores.data(), ldo, s);
+                ops.scores(Q + q0 * d, nq, q0, B, nbc, b0, d, ws.scores.data(), ldo, s);
                 if (mask) {
                     apply_mask(ws.scores.data(), nq, ldo, nbc, mask + q0 * mask_stride, mask_stride, nullptr, b0, s);
                 }
@@ -294,7 +298,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
                 const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * growth, (int64_t)1 << 23});
                 ScoreFilter<S> flt{ws.tau.data() + q0, ops.threshold(ws, q0, nq, s), ws.cnt.data() + q0, ws.filter.data(), cap,
                                    seen};
-                ops.filtered(Q + q0 * d, nq, q0, B + seen * d, nbc, seen, d, flt, s);
+                ops.filtered(Q + q0 * d, nq, q0, B, nbc, seen, d, flt, s);
                 ops.merge(running + q0 * ncand, ncand, flt, ws.tau.data() + q0, nq, overflow, s);
                 launches++;
                 seen += nbc;

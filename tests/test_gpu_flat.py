@@ -69,6 +69,51 @@ def test_flat_i8_golden(ix):
     assert np.array_equal(D, g["flat_i8_D"]) and np.array_equal(I, g["flat_i8_I"])
 
 
+@pytest.mark.parametrize("d", [64, 128, 256, 384, 512, 768, 1024])
+def test_flat_i8_every_dimension_of_the_resident_kernel(ix, oracle, d):
+    """The dimensions of the reference's Int8Flat (AscendIndexInt8FlatImpl.cpp:55), each a kernel instance of its own:
+    a base long enough for the seeded stretch (stored scores) and several bound-filtered launches, queries in more
+    than one query tile with a ragged last block, a base that ends inside a tile of 256 and inside a block of 32."""
+    n, nq, k = 41000 + 77, 300, 20
+    rng = np.random.default_rng(d)
+    base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+    q = rng.integers(-127, 128, size=(nq, d), dtype=np.int8)
+    q[:5] = base[[0, 255, 256, n - 1, 31999]]          # tile edges come back at distance 0
+    base[n - 3] = base[100]                             # a tie across launches: the vector added first wins
+    index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2, scratch_bytes=4 << 20)
+    index.add(base[:1000])
+    index.add(base[1000:1037])                          # adds that start and end inside blocks of 32
+    index.add(base[1037:])
+    D, I = index.search_int32(q, k)
+    Dr, Ir = oracle.flat_i8(base, q, k)
+    assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+    assert index.last_search_stats()["score_launches"] >= 3
+    assert D[:5, 0].tolist() == [0] * 5 and I[:5, 0].tolist() == [0, 255, 256, n - 1, 31999]
+
+
+def test_flat_i8_storage_in_matrix_core_order_round_trips(ix, oracle):
+    """What goes into the tiled base comes back row-major, across blocks of 32 and tiles of 256, for a dimension
+    that is padded (100 -> 128 bytes per row) and one that is not; removal moves vectors inside that layout."""
+    rng = np.random.default_rng(3)
+    for d in (100, 64):
+        n = 3000 + 19
+        base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+        index = ix.AscendIndexInt8Flat(d)
+        for s, e in ((0, 1), (1, 33), (33, 300), (300, n)):
+            index.add(base[s:e])
+        assert np.array_equal(index.getBase(0, n), base)
+        assert np.array_equal(index.getBase(31, 2), base[31:33])
+        assert np.array_equal(index.getBase(250, 600), base[250:850])
+        gone = np.array([0, 31, 32, 255, 256, 1000, n - 1, n - 40], dtype=np.int64)
+        assert index.remove_ids(gone) == len(gone)
+        order = oracle.flat_remove_order(n, np.sort(gone))
+        assert np.array_equal(index.getBase(0, n - len(gone)), base[order])
+        q = rng.integers(-127, 128, size=(9, d), dtype=np.int8)
+        D, I = index.search_int32(q, 7)
+        Dr, Ir = oracle.flat_i8(base[order], q, 7, ids=order.astype(np.int64))
+        assert np.array_equal(D, Dr) and np.array_equal(I, Ir)
+
+
 @pytest.mark.parametrize("metric_name", ["L2", "IP"])
 @pytest.mark.parametrize("d,n,nq,k", [(128, 20000, 100, 10), (96, 7000, 40, 100), (30, 900, 9, 5), (64, 9000, 300, 10)])
 def test_flat_f32_bit_exact(ix, oracle, metric_name, d, n, nq, k):
