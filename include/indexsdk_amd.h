@@ -248,8 +248,9 @@ int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x_dev, int64_t
 int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe,
                                int64_t k, float *distances_dev, int64_t *labels_dev);
 
-/* ivfpq_search_probes_device for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+/* ivfpq_search_probes_device for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference.  It runs on the index's own stream and waits
+ * for the results, so it is not meant to be called under stream capture.  Same
  * arguments, same results bit for bit; it calls no hipMalloc / hipFree: the intermediates of the launch
  * (sanitised probe lists, execution order, split partials) lie in a static device array of
  * IVFPQ_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.  A call that

@@ -156,7 +156,6 @@ private:
     bool trained_ = false;
     int64_t ntotal_ = 0;
     hipStream_t stream_ = nullptr;
-    unsigned char *noalloc_scratch_ = nullptr;   // this device's copy of the static scratch (resolved at construction)
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;

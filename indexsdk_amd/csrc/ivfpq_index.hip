@@ -440,7 +440,6 @@ IvfpqIndex::IvfpqIndex(int d, int metric, int64_t nlist, int M, int nbits, const
     for (auto &ev : ev_) {
         IXA_HIP(hipEventCreate(&ev));
     }
-    noalloc_scratch_ = noalloc_scratch_of_current_device();
     list_off_.assign((size_t)nlist_, 0);
     list_len_.assign((size_t)nlist_, 0);
     list_cap_.assign((size_t)nlist_, 0);
@@ -1351,8 +1350,9 @@ void IvfpqIndex::search_probes(int64_t n, const float *x_dev, const int32_t *pro
     stats_.shared_pool = p.shared_pool;
 }
 
-// The same call with nothing allocated, for callers that cannot call hipMalloc (HIP graph capture, tight
-// serving loops): the sanitised probe lists, the execution order and the split partials lie in the static
+// The same call with nothing allocated, for callers that cannot call hipMalloc (tight serving loops, harnesses
+// that forbid allocation; it launches on the index's own stream and waits for the results, so it is not a call
+// to make under stream capture): the sanitised probe lists, the execution order and the split partials lie in the static
 // device scratch, laid out as [histogram | cursors: 8 KB][order | class: 8 n][probes: 4 n nprobe]
 // [partials: 8 n nsplit k], each part rounded up to 256 bytes.
 void IvfpqIndex::search_probes_noalloc(int64_t n, const float *x_dev, const int32_t *probes_dev, int nprobe, int64_t k,
@@ -1373,14 +1373,15 @@ void IvfpqIndex::search_probes_noalloc(int64_t n, const float *x_dev, const int3
                 "no-allocation entry point holds %zu (use ivfpq_search_probes_device, or fewer queries per call)",
                 (long)n, nprobe, (long)k, (long)need, kNoAllocScratchBytes);
     std::lock_guard<std::mutex> lock(g_noalloc_mu);
-    unsigned char *base = noalloc_scratch_;
+    // resolved on the first call on a device, not when an index is built: a failure here concerns this entry
+    // point only
+    unsigned char *base = noalloc_scratch_of_current_device();
     ScanScratch ext{};
     ext.hist = reinterpret_cast<int32_t *>(base);
     ext.order = reinterpret_cast<int32_t *>(base + hist_bytes);
     int32_t *probes = reinterpret_cast<int32_t *>(base + hist_bytes + order_bytes);
     ext.partial = reinterpret_cast<unsigned long long *>(base + hist_bytes + order_bytes + probes_bytes);
-    // the array keeps what the last call left: the histogram has to start at zero (a fill kernel, not a
-    // memset node, so that the sequence can be captured into a graph)
+    // the array keeps what the last call left: the histogram has to start at zero
     hipLaunchKernelGGL(fill_i32_kernel, dim3(8), dim3(256), 0, stream_, ext.hist, 2 * 1024, 0);
     hipLaunchKernelGGL(sanitize_probes_kernel, dim3(blocks_for(n * nprobe)), dim3(256), 0, stream_, probes_dev,
                        n * nprobe, (int32_t)nlist_, probes);

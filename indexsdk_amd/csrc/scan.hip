@@ -377,6 +377,8 @@ __global__ __launch_bounds__(W * 64, (LAYOUT == 1 && sizeof(LutT) == 2 && !SHARE
             for (int v = 0; v < MT / 4; v++) {
                 w[v % NW] = reinterpret_cast<const uint32_t *>(cp)[v];
             }
+        } else if (MT == 2) {
+            w[0] = *reinterpret_cast<const uint16_t *>(cp);   // slots are 2 bytes apart: always aligned
         } else {
 #pragma unroll
             for (int v = 0; v < NW; v++) {
@@ -1152,6 +1154,9 @@ static void dispatch_m(const ScanParams &p, int64_t nq, size_t smem, hipStream_t
         }
     }
     switch (p.M) {
+        // every sub-quantizer count of the reference's own envelope (2, 4, 8, 16, 32:
+        // FR/ascend/impl/AscendIndexIVFPQImpl.cpp:130-140) has a kernel with compile-time M
+        case 2: return launch_one<2, LutT, 0>(p, nq, smem, s);
         case 4: return launch_one<4, LutT, 0>(p, nq, smem, s);
         case 8: return launch_one<8, LutT, 0>(p, nq, smem, s);
         case 16: return launch_one<16, LutT, 0>(p, nq, smem, s);
@@ -1298,12 +1303,12 @@ void launch_scan(ScanParams p, int64_t nq, hipStream_t s)
                 "IVFPQ scan needs at least %zu bytes of LDS (M=%d, k=%d, %s LUT); the limit is 163840", smem, p.M, p.k,
                 p.lut_fp16 ? "fp16" : "fp32");
     IXA_REQUIRE(nq * p.nsplit < ((int64_t)1 << 31), kErrInvalidParam, "scan grid too large");
+    IXA_REQUIRE(p.nsplit == 1 || p.partial != nullptr, kErrInner, "a split scan needs a buffer for its partial lists");
     if (p.lut_fp16) {
         dispatch_m<__half>(p, nq, smem, s);
     } else {
         dispatch_m<float>(p, nq, smem, s);
     }
-    IXA_REQUIRE(p.nsplit == 1 || p.partial != nullptr, kErrInner, "a split scan needs a buffer for its partial lists");
     if (p.nsplit > 1) {
         hipLaunchKernelGGL(ivfpq_merge_kernel, dim3((unsigned)nq), dim3(kMergeSelectThreads), 0, s, p.partial,
                            p.nsplit, p.k, p.metric, p.ids, p.order, p.out_dist, p.out_labels);
