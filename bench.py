@@ -228,6 +228,12 @@ def run_flat_i8(args, torch, ix, _capi, lib, steps, warmup, cpu_leg):
         log(f"CPU oracle flat int8: {t_cpu:.2f}s for {sample_q}x{sample_n}; GPU bit-exact on the sample: {exact}")
         del sub
     log(f"C4 step {ms:.2f} ms, {result['value']:.0f} QPS, {result['roofline']['achieved']:.1f} TOP/s")
+    if args.copy_probe:
+        src = torch.zeros(1 << 28, device="cuda", dtype=torch.float32)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        _capi.check(lib.ixa_copy_probe(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), 1 << 30))
+        del src, dst
     del index, queries, D, I
     torch.cuda.empty_cache()
     return result

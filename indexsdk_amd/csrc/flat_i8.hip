@@ -320,9 +320,35 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
 
     const int xcd = blockIdx.x & 7, wi = blockIdx.x >> 3, wpx = gridDim.x >> 3;
     const int own_n = ntiles > xcd ? (ntiles - xcd + 7) / 8 : 0;
-    const int nseg = (own_n + seg_tiles - 1) / seg_tiles;
+    // Items: (query tile, segment), query tile fastest, dealt round-robin to the XCD's workgroups.  The S = wpx /
+    // tiles_m segments that are in flight together INTERLEAVE tile by tile inside a group of S * seg_tiles tiles
+    // (segment `sub` of group g takes tiles g * S * seg_tiles + sub, + S, + 2 S, ...): all workgroups of the XCD then
+    // read the same few tiles at any moment, and its L2 (4 MB; a tile is 256 x D bytes) holds them for every
+    // reader however the workgroups drift.  Side by side, the S segments would span S * seg_tiles tiles at once.
+    const int S = wpx / tiles_m > 1 ? wpx / tiles_m : 1;
+    const int group_tiles = S * seg_tiles;
+    const int nseg = (own_n + group_tiles - 1) / group_tiles * S;
     const int items = tiles_m * nseg;
-    if (wi >= items) {
+    // first tile, tile after the last, and query tile of an item; an item of the last group may be empty
+    auto item_range = [&](int it, int &tmv, int &j0, int &j1) {
+        tmv = it % tiles_m;
+        const int seg = it / tiles_m, g = seg / S, sub = seg % S;
+        j0 = g * group_tiles + sub;
+        j1 = min(own_n, (g + 1) * group_tiles);
+    };
+    // the first item at or after `it` (in this workgroup's sequence it, it + wpx, ...) that has a tile, or -1
+    auto next_item = [&](int it) {
+        for (; it < items; it += wpx) {
+            int tmv, j0, j1;
+            item_range(it, tmv, j0, j1);
+            if (j0 < j1) {
+                return it;
+            }
+        }
+        return -1;
+    };
+    const int first_item = next_item(wi);
+    if (first_item < 0) {
         return;
     }
     const uint32_t lds_base = (uint32_t)reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)lds);
@@ -359,9 +385,9 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
         qcount = 0;
     };
 
-    int it_t = wi;   // item = (query tile, segment of this XCD's base tiles), query tile fastest
-    int tm = it_t % tiles_m;
-    int j = (it_t / tiles_m) * seg_tiles, jend = min(own_n, j + seg_tiles);
+    int it_t = first_item;
+    int tm, j, jend;
+    item_range(it_t, tm, j, jend);
     const unsigned char *cur = block_ptr(j);
     // Loads are issued in the same order here and in the loop -- norms of a tile before its fragments -- so that the
     // wait for the norms at a tile's start leaves the PF fragment loads behind them in flight.
@@ -377,6 +403,7 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
     for (int p = 0; p < PF; p++) {
         breg[p] = *reinterpret_cast<const v4i *>(cur + p * 1024);
     }
+    bool staggered = false;
     while (true) {
         if (tm != cur_tm) {
             // the query tile: LDS [chunk][query][16 B]; rows past the end of the batch repeat its last row
@@ -400,16 +427,24 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
             }
             cur_tm = tm;
             __syncthreads();
+            // The two wavefronts of a SIMD (w and w + 4) would otherwise reach the end of every tile together and
+            // leave the matrix cores idle while both test their accumulators: the second one starts half a tile
+            // late, once, and from then on each one's epilogue runs under the other's matrix instructions.
+            if (!staggered && wave >= kResidentWaves / 2) {
+                // a wavefront's tile is NHS * RA matrix instructions of 32 cycles, and two wavefronts share the
+                // matrix core: half a tile of wall time is 32 NHS RA cycles, s_sleep counts in units of 64
+                constexpr int kHalfTile = NHS * RA / 2;
+                __builtin_amdgcn_s_sleep(kHalfTile < 127 ? kHalfTile : 127);
+            }
+            staggered = true;
         }
         // the tile after this one (the last tile names itself: its loads are harmless repeats)
-        int n_it = it_t, n_tm = tm, n_j = j + 1, n_jend = jend;
+        int n_it = it_t, n_tm = tm, n_j = j + S, n_jend = jend;
         bool has_next = true;
         if (n_j >= jend) {
-            n_it = it_t + wpx;
-            if (n_it < items) {
-                n_tm = n_it % tiles_m;
-                n_j = (n_it / tiles_m) * seg_tiles;
-                n_jend = min(own_n, n_j + seg_tiles);
+            n_it = next_item(it_t + wpx);
+            if (n_it >= 0) {
+                item_range(n_it, n_tm, n_j, n_jend);
             } else {
                 has_next = false;
                 n_it = it_t;
@@ -482,40 +517,45 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
         // a lane owns query (block ra, l32) and base rows row0 + 8 g + 4 half + t of the wave's block
         const int64_t col0 = block_row0(j) + 4 * half;
         if constexpr (FILTER) {
-            int T[RA];
+            // per block: {thr, |q|^2, test value} of the lane's query and ONE compare of the block's largest
+            // accumulator with the test value; the lane masks stay in scalar registers
+            int4 mt[RA];
+            unsigned long long hit[RA], any = 0;
 #pragma unroll
             for (int ra = 0; ra < RA; ra++) {
-                T[ra] = meta[ra * 32 + l32].z;
+                mt[ra] = meta[ra * 32 + l32];
             }
-            int over = (int)0x80000000;
 #pragma unroll
             for (int ra = 0; ra < RA; ra++) {
-                over = max(over, max16(acc[ra]) - T[ra]);
+                hit[ra] = __builtin_amdgcn_ballot_w64(max16(acc[ra]) >= mt[ra].z);
+                any |= hit[ra];
             }
-            if (__builtin_amdgcn_ballot_w64(over >= 0) != 0) {
+            if (any != 0) {
                 const uint32_t colv = (uint32_t)col0;
 #pragma unroll
                 for (int ra = 0; ra < RA; ra++) {
-                    if (__builtin_amdgcn_ballot_w64(max16(acc[ra]) >= T[ra]) != 0) {
-                        // exact: |b|^2 - 2 q.b = -(2 acc + parity) <= thr  <=>  2 acc + parity >= -thr
-                        const int4 m = meta[ra * 32 + l32];
-                        const int nthr = -m.x;   // thr <= 2^28 by the caller's clamp, > INT32_MIN
+                    if (hit[ra] != 0) {
+                        const int nthr = -mt[ra].x;   // thr <= 2^28 by the caller's clamp, > INT32_MIN
                         const uint32_t row = (uint32_t)(tm * QT + ra * 32 + l32);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
-                            const int t2 = (acc[ra][r] << 1) + (int)((par >> (16 + r)) & 1u);
-                            const bool pass = t2 >= nthr;
-                            const unsigned long long mask = __builtin_amdgcn_ballot_w64(pass);
-                            if (mask != 0) {
-                                const int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
-                                                                          __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-                                if (pass) {
-                                    const uint32_t score = (uint32_t)(m.y - t2) ^ 0x80000000u;   // ordered int32
-                                    queue[qcount + pre] = make_uint4(colv + 8 * (r >> 2) + (r & 3), score, row, 0u);
-                                }
-                                qcount += __builtin_popcountll(mask);
-                                if (qcount > kQueueKeys - 64) {
-                                    flush_queue();
+                            // the test value again, register by register (a superset test), then in exact integers:
+                            // |b|^2 - 2 q.b = -(2 acc + parity) <= thr  <=>  2 acc + parity >= -thr
+                            if (__builtin_amdgcn_ballot_w64(acc[ra][r] >= mt[ra].z) != 0) {
+                                const int t2 = (acc[ra][r] << 1) + (int)((par >> (16 + r)) & 1u);
+                                const bool pass = t2 >= nthr;
+                                const unsigned long long mask = __builtin_amdgcn_ballot_w64(pass);
+                                if (mask != 0) {
+                                    const int pre = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                                              __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+                                    if (pass) {
+                                        const uint32_t score = (uint32_t)(mt[ra].y - t2) ^ 0x80000000u;   // ordered int32
+                                        queue[qcount + pre] = make_uint4(colv + 8 * (r >> 2) + (r & 3), score, row, 0u);
+                                    }
+                                    qcount += __builtin_popcountll(mask);
+                                    if (qcount > kQueueKeys - 64) {
+                                        flush_queue();
+                                    }
                                 }
                             }
                         }

@@ -101,6 +101,7 @@ struct F32Ops {
     using T = float;
     using S = float;
     static constexpr int64_t kMinChunk = 1;   // its score launchers serve any chunk of base rows
+    static constexpr int64_t kSeedRows = 2048, kMaxGrowth = 1 << 20;
     const float *qn, *bn;
     int metric;
     const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
@@ -129,6 +130,7 @@ struct Bf16Ops {
     using T = uint16_t;
     using S = float;
     static constexpr int64_t kMinChunk = 2048;   // the ring kernel is the only one for split operands
+    static constexpr int64_t kSeedRows = 2048, kMaxGrowth = 1 << 20;
     const float *qn, *bn;
     int metric;
     const S *threshold(StreamSelectWorkspace<S> &, int64_t, int64_t, hipStream_t) const { return nullptr; }
@@ -162,6 +164,11 @@ struct I8Ops {
     using T = int8_t;
     using S = int32_t;
     static constexpr int64_t kMinChunk = 1;
+    // A launch of the resident-query kernel costs little and its bound-filtered epilogue is cheapest when few scores
+    // pass, so the bound is tightened often: a longer seed stretch (a bound from 8192 rows admits a quarter of what
+    // one from 2048 does) and chunks that only double what has been seen (10M x 512, 2048 queries, k 100, same box:
+    // seed 2048 and chunks of 5 x seen 8.91 ms per search; 8192 and 5 x: 8.80; 8192 and 3 x: 8.54; 8192 and 2 x: 8.47)
+    static constexpr int64_t kSeedRows = 8192, kMaxGrowth = 2;
     const int32_t *qn, *bn;
     const S *threshold(StreamSelectWorkspace<S> &ws, int64_t q0, int64_t nq, hipStream_t s) const
     {
@@ -212,7 +219,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     nb = std::max<int64_t>(128, nb / 128 * 128);
     nb = std::min<int64_t>(nb, round_up(std::max<int64_t>(nb_total, 1), 128));
     const int cap = pow2_ceil((int)std::max<int64_t>(1024, 16 * (int64_t)ncand));
-    const int64_t seed_rows = std::min<int64_t>(nb_total, std::max<int64_t>(2048, 16 * (int64_t)ncand));
+    const int64_t seed_rows = std::min<int64_t>(nb_total, std::max<int64_t>(Ops::kSeedRows, 16 * (int64_t)ncand));
     // when the whole score matrix of a query block fits the scratch, one materialised pass is the
     // cheapest plan (measured on the IVFPQ coarse stage: 16384 centroids); the filtered plan is for
     // long bases
@@ -229,7 +236,7 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
     }
     // tau is fixed during a chunk, so a chunk admits about ncand * chunk / seen keys per query; keep
     // that expectation below a quarter of the candidate buffer
-    const int64_t growth = std::max<int64_t>(2, cap / (4 * (int64_t)ncand));
+    const int64_t growth = std::max<int64_t>(2, std::min<int64_t>(Ops::kMaxGrowth, cap / (4 * (int64_t)ncand)));
     if (Ops::kMinChunk > 1) {
         // Dry run of the chunking below (the filtered plan and the materialised one it falls back to): every
         // chunk must be one the score kernel serves, or the caller takes another route.
