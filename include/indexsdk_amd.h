@@ -178,6 +178,10 @@ typedef struct ivfpq_config {
                                        of ivfpq_last_search_stats come from: 1 = always, 0 = never, -1 (default) =
                                        for pages of 256 queries or more (recording them costs a small batch 5-10 us
                                        per call); a search without them reports 0 ms */
+    int32_t coarse_resident;        /* score launches of the sampled-bound coarse plan (results do not depend on it):
+                                       1 (default) = by the kernel that keeps a tile of queries resident in LDS and
+                                       reads the centroids from matrix-core order, where it has an instance (64, 96
+                                       and 128 dimensions); 0 = by the ring kernel that streams both operands */
 } ivfpq_config_t;
 
 /* Fills *cfg with the defaults. */

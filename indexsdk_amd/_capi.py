@@ -35,6 +35,7 @@ class IvfpqConfig(ctypes.Structure):
         ("pq_spherical", ctypes.c_int32),
         ("coarse_exact_small", ctypes.c_int32),
         ("stage_timings", ctypes.c_int32),
+        ("coarse_resident", ctypes.c_int32),
     ]
 
 

@@ -8,7 +8,7 @@ FLAGS=(-O3 --offload-arch=gfx950 -std=c++17 -fPIC -ffp-contract=off -fvisibility
 OBJ="${HERE}/.obj"
 mkdir -p "${OBJ}"
 pids=()
-for src in coarse.hip score_ring.hip pq.hip scan.hip flat.hip flat_i8.hip stream_select.hip ivfpq_index.hip ops.hip; do
+for src in coarse.hip coarse_resident.hip score_ring.hip pq.hip scan.hip flat.hip flat_i8.hip stream_select.hip ivfpq_index.hip ops.hip; do
   [ -f "${HERE}/${src}" ] || continue
   ( /opt/rocm/bin/hipcc "${FLAGS[@]}" -c "${HERE}/${src}" -o "${OBJ}/${src%.hip}.o" 2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) ) &
   pids+=($!)

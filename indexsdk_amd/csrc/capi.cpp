@@ -101,6 +101,7 @@ ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
         c.pq_spherical = cfg->pq_spherical ? 1 : 0;
         c.coarse_exact_small = cfg->coarse_exact_small;
         c.stage_timings = cfg->stage_timings;
+        c.coarse_resident = cfg->coarse_resident ? 1 : 0;
     }
     return c;
 }
@@ -137,6 +138,7 @@ IXA_EXPORT void ivfpq_config_default(ivfpq_config_t *cfg)
     cfg->pq_spherical = d.pq_spherical;
     cfg->coarse_exact_small = d.coarse_exact_small;
     cfg->stage_timings = d.stage_timings;
+    cfg->coarse_resident = d.coarse_resident;
 }
 
 IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbits, const ivfpq_config_t *cfg,

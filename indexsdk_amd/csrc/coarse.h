@@ -46,6 +46,18 @@ bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, in
                             const float *bn, int metric, float *out, int64_t ldo, bool filter, ScoreFilter<float> flt,
                             hipStream_t s);
 
+// The same two launches with the query tile resident in LDS and the split centroids read from matrix-core order
+// (coarse_resident.hip): Bt = the base-side split rows tiled as flat_i8.h describes (rows of 2 d3 bytes, whole tiles of
+// 256 rows, zero rows behind the last), cn_padded = |c|^2 per row (zeros for inner product) padded to whole tiles with
+// +inf.  The records hold DOT PRODUCTS, not scores: the folds below take them with raw = true.  test_scratch: nq
+// floats.  Return false (nothing launched) for split rows they have no instance for.
+bool resident_coarse_serves(int d3);
+bool launch_resident_bf16_minima(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, int64_t nb, int d3, const float *qn,
+                                 const float *cn_padded, int metric, float *out, int64_t ldo, hipStream_t s);
+bool launch_resident_bf16_records(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, int64_t nb, int d3, const float *qn,
+                                  const float *cn_padded, int metric, float cmax, float *test_scratch,
+                                  ScoreFilter<float> flt, hipStream_t s);
+
 // Record mode of the bf16 ring kernel: nothing is stored; every run of four consecutive base rows (first
 // row a multiple of four) whose smallest score is at or below flt.tau[row] is appended to the row's
 // record list: 32 bytes {four fp32 scores, uint32 col_base + first base row, unused} at
@@ -67,14 +79,21 @@ constexpr int kFoldMaxK = 384;
 // kEmptyKey padded; written only), resets cnt[row], and appends every row whose result is not PROVEN to be
 // the k smallest keys of the base (fewer than k scores <= tau[row] on record, or records dropped) to
 // flag[1 + flag[0]++] as row_base + row, marking it by kEmptyKey in its last key.
+// raw (may be null): the records hold dot products (launch_resident_bf16_records); scores are formed from them with
+// these row and column norms (cn 16-byte aligned; unused for inner product)
+struct RawRecords {
+    const float *qn, *cn;
+    int metric;
+};
 void launch_fold_records(unsigned long long *running, int k, ScoreFilter<float> flt, int64_t nq, int *flag,
-                         int64_t row_base, hipStream_t s);
+                         int64_t row_base, hipStream_t s, const RawRecords *raw = nullptr);
 // launch_fold_records and launch_refine_boundary in one launch, without the sort in between: the exact best
 // nout SET of every row; capk = scores <= tau a row may have on record (at most 2048); rows without proof
 // are appended to flag.  Resets cnt[row].
 void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                                  int metric, ScoreFilter<float> flt, int capk, int nout, float cmax, float err_scale,
-                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s);
+                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s,
+                                 bool raw = false);
 
 // out[row] = [hi | hi | lo] (query side) or [hi | lo | hi] (base side) of x[row], each segment
 // zero-padded from d to dp elements of bf16 (stored as uint16_t); out has n * 3 * dp elements.

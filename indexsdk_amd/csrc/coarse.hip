@@ -816,8 +816,34 @@ __global__ __launch_bounds__(256, IXA_SELREG_WAVES) void select_rows_reg_kernel(
 // list they must not judge.  One workgroup per row; k <= kSelRegMaxK.
 constexpr int kFoldCap = 2048;   // scores <= tau the fold ranks at once
 
+// Records of the resident-query launch hold the dot products g of a run, not its scores: the score in the
+// arithmetic of the score kernels, (|q|^2 + |c|^2) - g - g, or -g for inner product.
+__device__ __forceinline__ void record_scores(float (&v)[4], bool raw, int metric, float qnorm,
+                                              const float *__restrict__ cn, uint32_t col)
+{
+    if (!raw) {
+        return;
+    }
+    if (metric == kMetricL2) {
+        const float4 c4 = *reinterpret_cast<const float4 *>(cn + col);   // runs start at multiples of four
+        const float c[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            float w = __fadd_rn(qnorm, c[t]);
+            w = __fsub_rn(w, v[t]);
+            v[t] = __fsub_rn(w, v[t]);
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            v[t] = -v[t];
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void fold_records_kernel(key_t *__restrict__ running, int k, ScoreFilter<float> flt,
-                                                           int *__restrict__ flag, int64_t row_base)
+                                                           int *__restrict__ flag, int64_t row_base, bool raw, int metric,
+                                                           const float *__restrict__ qn, const float *__restrict__ cn)
 {
     __shared__ __align__(16) key_t cand[kFoldCap + 2];
     __shared__ __align__(16) key_t best[kSelRegMaxK];
@@ -839,7 +865,8 @@ __global__ __launch_bounds__(256) void fold_records_kernel(key_t *__restrict__ r
     for (int r = tid; r < nrec; r += 256) {
         const float4 sc = *reinterpret_cast<const float4 *>(records + (int64_t)r * 32);
         const uint32_t col = *reinterpret_cast<const uint32_t *>(records + (int64_t)r * 32 + 16);
-        const float v[4] = {sc.x, sc.y, sc.z, sc.w};
+        float v[4] = {sc.x, sc.y, sc.z, sc.w};
+        record_scores(v, raw, metric, raw ? qn[row] : 0.f, cn, col);
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             if (v[t] <= tau) {
@@ -880,13 +907,14 @@ __global__ __launch_bounds__(256) void fold_records_kernel(key_t *__restrict__ r
 }
 
 void launch_fold_records(unsigned long long *running, int k, ScoreFilter<float> flt, int64_t nq, int *flag,
-                         int64_t row_base, hipStream_t s)
+                         int64_t row_base, hipStream_t s, const RawRecords *raw)
 {
     if (nq == 0) {
         return;
     }
     IXA_REQUIRE(k >= 1 && k <= kSelRegMaxK && k < kFoldCap, kErrInner, "record fold of %d keys", k);
-    hipLaunchKernelGGL(fold_records_kernel, dim3((unsigned)nq), dim3(256), 0, s, running, k, flt, flag, row_base);
+    hipLaunchKernelGGL(fold_records_kernel, dim3((unsigned)nq), dim3(256), 0, s, running, k, flt, flag, row_base,
+                       raw != nullptr, raw ? raw->metric : kMetricL2, raw ? raw->qn : nullptr, raw ? raw->cn : nullptr);
 }
 
 // tau[row] = the `rank`-th smallest (1-based) of the row's G group minima gm[row * G .. + G): an upper bound
@@ -1229,7 +1257,7 @@ template <bool VEC4, int E>
 __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
     const float *__restrict__ Q, int64_t nq, const float *__restrict__ C, int d, const float *__restrict__ qn,
     const float *__restrict__ cn, int metric, ScoreFilter<float> flt, int amb_cap, int nout, float cmax,
-    float err_scale, float round_scale, int32_t *__restrict__ out_ids, int *__restrict__ flag, int64_t row_base)
+    float err_scale, float round_scale, int32_t *__restrict__ out_ids, int *__restrict__ flag, int64_t row_base, bool raw)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     constexpr int capk = 64 * E;
@@ -1273,7 +1301,8 @@ __global__ __launch_bounds__(256) void fold_refine_boundary_kernel(
                 break;   // wave-uniform
             }
             const int r = base + b * kWave + lane;
-            const float v[4] = {sc[b].x, sc[b].y, sc[b].z, sc[b].w};
+            float v[4] = {sc[b].x, sc[b].y, sc[b].z, sc[b].w};
+            record_scores(v, raw, metric, qnorm, cn, col[b]);   // lanes past nrec hold column 0: a valid address
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const bool pass = r < nrec && v[t] <= tau;
@@ -1405,7 +1434,7 @@ template <bool VEC4>
 static void launch_fold_refine_boundary_t(const float *Q, int64_t nq, const float *C, int d, const float *qn,
                                           const float *cn, int metric, ScoreFilter<float> flt, int capk, int nout,
                                           float cmax, float err_scale, float round_scale, int32_t *out_ids, int *flag,
-                                          int64_t row_base, hipStream_t s)
+                                          int64_t row_base, bool raw, hipStream_t s)
 {
     const int amb_cap = 128;
     const int E = capk <= 256 ? 4 : (capk <= 512 ? 8 : (capk <= 1024 ? 16 : 32));
@@ -1418,25 +1447,27 @@ static void launch_fold_refine_boundary_t(const float *Q, int64_t nq, const floa
                                     (int)smem));
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, flt,
-                       amb_cap, nout, cmax, err_scale, round_scale, out_ids, flag, row_base);
+                       amb_cap, nout, cmax, err_scale, round_scale, out_ids, flag, row_base, raw);
 }
 
 void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int d, const float *qn, const float *cn,
                                  int metric, ScoreFilter<float> flt, int capk, int nout, float cmax, float err_scale,
-                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s)
+                                 float round_scale, int32_t *out_ids, int *flag, int64_t row_base, hipStream_t s,
+                                 bool raw)
 {
     if (nq == 0) {
         return;
     }
     IXA_REQUIRE(nout >= 1 && capk >= nout && capk <= 2048, kErrInner, "fold refine of %d from %d keys", nout, capk);
+    IXA_REQUIRE(!raw || reinterpret_cast<uintptr_t>(cn) % 16 == 0, kErrInner, "raw records need aligned norms");
     const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     if (vec4) {
         launch_fold_refine_boundary_t<true>(Q, nq, C, d, qn, cn, metric, flt, capk, nout, cmax, err_scale, round_scale,
-                                            out_ids, flag, row_base, s);
+                                            out_ids, flag, row_base, raw, s);
     } else {
         launch_fold_refine_boundary_t<false>(Q, nq, C, d, qn, cn, metric, flt, capk, nout, cmax, err_scale,
-                                             round_scale, out_ids, flag, row_base, s);
+                                             round_scale, out_ids, flag, row_base, raw, s);
     }
 }
 

@@ -24,9 +24,8 @@
 //   * XCD x owns base tiles x, x + 8, ...; its workgroups take (query tile, segment of base tiles) items with
 //     the query tile fastest, so the workgroups that run together read the same base tiles and the XCD's L2
 //     serves all but the first.
-#include <type_traits>
-
 #include "flat_i8.h"
+#include "resident_tile.h"
 #include "topk.h"
 
 namespace ixa {
@@ -254,33 +253,6 @@ __global__ __launch_bounds__(256) void score_tile_i8_kernel(const int8_t *__rest
 
 // ---- resident-query kernel -----------------------------------------------------------------------------------------
 
-template <int I, int N, typename F>
-__device__ __forceinline__ void static_for(F &&f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-// Four 128-bit LDS reads (query blocks 512 bytes apart) and the wait for them are inline assembly: the compiler's own
-// bookkeeping would wait for a read right after issuing it.  LDS reads complete in order, so "at most 4
-// outstanding" after the 4 reads of the next quad have been issued means that this quad has arrived; the registers
-// pass through the wait statement so that no use of them can be scheduled ahead of it.
-template <int OFF>
-__device__ __forceinline__ void read_quad(uint32_t addr, v4i (&f)[4])
-{
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[0]) : "v"(addr), "n"(OFF));
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[1]) : "v"(addr), "n"(OFF + 512));
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[2]) : "v"(addr), "n"(OFF + 1024));
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f[3]) : "v"(addr), "n"(OFF + 1536));
-}
-template <int N>
-__device__ __forceinline__ void wait_quad(v4i (&f)[4])
-{
-    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]) : "n"(N));
-}
-
 __device__ __forceinline__ int max16(const v16i &a)
 {
     int m0 = max(max(a[0], a[1]), a[2]);
@@ -319,35 +291,9 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
     const int half = lane >> 5, l32 = lane & 31;
 
     const int xcd = blockIdx.x & 7, wi = blockIdx.x >> 3, wpx = gridDim.x >> 3;
-    const int own_n = ntiles > xcd ? (ntiles - xcd + 7) / 8 : 0;
-    // Items: (query tile, segment), query tile fastest, dealt round-robin to the XCD's workgroups.  The S = wpx /
-    // tiles_m segments that are in flight together INTERLEAVE tile by tile inside a group of S * seg_tiles tiles
-    // (segment `sub` of group g takes tiles g * S * seg_tiles + sub, + S, + 2 S, ...): all workgroups of the XCD then
-    // read the same few tiles at any moment, and its L2 (4 MB; a tile is 256 x D bytes) holds them for every
-    // reader however the workgroups drift.  Side by side, the S segments would span S * seg_tiles tiles at once.
-    const int S = wpx / tiles_m > 1 ? wpx / tiles_m : 1;
-    const int group_tiles = S * seg_tiles;
-    const int nseg = (own_n + group_tiles - 1) / group_tiles * S;
-    const int items = tiles_m * nseg;
-    // first tile, tile after the last, and query tile of an item; an item of the last group may be empty
-    auto item_range = [&](int it, int &tmv, int &j0, int &j1) {
-        tmv = it % tiles_m;
-        const int seg = it / tiles_m, g = seg / S, sub = seg % S;
-        j0 = g * group_tiles + sub;
-        j1 = min(own_n, (g + 1) * group_tiles);
-    };
-    // the first item at or after `it` (in this workgroup's sequence it, it + wpx, ...) that has a tile, or -1
-    auto next_item = [&](int it) {
-        for (; it < items; it += wpx) {
-            int tmv, j0, j1;
-            item_range(it, tmv, j0, j1);
-            if (j0 < j1) {
-                return it;
-            }
-        }
-        return -1;
-    };
-    const int first_item = next_item(wi);
+    const ResidentItems sched(tiles_m, ntiles, seg_tiles, xcd, wpx);
+    const int S = sched.S;
+    const int first_item = sched.next(wi);
     if (first_item < 0) {
         return;
     }
@@ -387,7 +333,7 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
 
     int it_t = first_item;
     int tm, j, jend;
-    item_range(it_t, tm, j, jend);
+    sched.range(it_t, tm, j, jend);
     const unsigned char *cur = block_ptr(j);
     // Loads are issued in the same order here and in the loop -- norms of a tile before its fragments -- so that the
     // wait for the norms at a tile's start leaves the PF fragment loads behind them in flight.
@@ -442,9 +388,9 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
         int n_it = it_t, n_tm = tm, n_j = j + S, n_jend = jend;
         bool has_next = true;
         if (n_j >= jend) {
-            n_it = next_item(it_t + wpx);
+            n_it = sched.next(it_t + wpx);
             if (n_it >= 0) {
-                item_range(n_it, n_tm, n_j, n_jend);
+                sched.range(n_it, n_tm, n_j, n_jend);
             } else {
                 has_next = false;
                 n_it = it_t;
@@ -478,20 +424,20 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
             }
         }
         v4i fa[2][4];
-        read_quad<0>(a_lane, fa[0]);
+        lds_read_group<4, 0>(a_lane, fa[0]);
         static_for<0, QPH * NHS>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
             constexpr int hs = u / QPH, p = u % QPH;
             if constexpr (u + 1 < QPH * NHS) {
                 constexpr int off = ((u + 1) / QPH) * kStepLds + ((u + 1) % QPH) * 2048;
                 if constexpr (off >= 65536) {
-                    read_quad<off - 65536>(a_lane_hi, fa[(u + 1) & 1]);
+                    lds_read_group<4, off - 65536>(a_lane_hi, fa[(u + 1) & 1]);
                 } else {
-                    read_quad<off>(a_lane, fa[(u + 1) & 1]);
+                    lds_read_group<4, off>(a_lane, fa[(u + 1) & 1]);
                 }
-                wait_quad<4>(fa[u & 1]);
+                lds_wait_group<4, 4>(fa[u & 1]);
             } else {
-                wait_quad<0>(fa[u & 1]);
+                lds_wait_group<4, 0>(fa[u & 1]);
             }
 #pragma unroll
             for (int t = 0; t < 4; t++) {

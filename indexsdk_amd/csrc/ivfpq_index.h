@@ -37,6 +37,8 @@ struct IvfpqConfig {
     int stage_timings = -1;           // events around the stages of a search (ms_coarse / ms_scan of the statistics):
                                       // 1 = always, 0 = never, -1 = for pages of 256 queries or more (the three
                                       // event records cost a small batch 5-10 us per call); untimed stages report 0
+    int coarse_resident = 1;          // sampled-bound plan: 1 = scores by the resident-query kernel where it has an
+                                      // instance (64, 96, 128 dimensions), 0 = by the ring kernel
     int coarse_bf16 = 1;              // 1 = generate coarse candidates with bf16 x 3 matrix products (results
                                       // stay exact: candidates are re-evaluated in fp32 and the superset
                                       // property is verified, with an fp32 rerun if it cannot be proven)
@@ -160,6 +162,8 @@ private:
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
+    DeviceBuffer<uint8_t> centroids_tiled_;                // centroids_split_ in matrix-core order (flat_i8.h), or empty
+    DeviceBuffer<float> cnorm_pad_;                        // [norms | zeros], each padded to whole tiles with +inf
     DeviceBuffer<int32_t> ws_flag_;
     DeviceBuffer<int32_t> ws_redo_;                    // rows of the queries a search scans a second time
     DeviceBuffer<int32_t> ws_order_, ws_order_hist_;   // execution order of the scan (heaviest queries first)

@@ -11,6 +11,7 @@
 #include <unordered_set>
 
 #include "coarse.h"
+#include "flat_i8.h"
 #include "pq.h"
 #include "scan.h"
 #include "stream_select.h"
@@ -498,6 +499,24 @@ void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
         std::vector<float> cn((size_t)nlist_);
         cnorm_.download(cn.data(), cn.size(), stream_);
         cmax_ = std::sqrt(*std::max_element(cn.begin(), cn.end()));
+        // The split centroids a second time, in matrix-core order, for the resident-query score kernel
+        // (coarse_resident.hip), with their norms padded to whole tiles: +inf behind the last centroid, so that a
+        // padding row never passes a bound; for inner product the kernel wants zeros in their place.
+        centroids_tiled_.release();
+        cnorm_pad_.release();
+        if (resident_coarse_serves(3 * dp_)) {
+            const int row_bytes = 3 * dp_ * 2;
+            const int64_t padded = round_up(nlist_, kI8TileRows);
+            centroids_tiled_.resize(i8_tiled_bytes(nlist_, row_bytes));
+            IXA_HIP(hipMemsetAsync(centroids_tiled_.data(), 0, centroids_tiled_.bytes(), stream_));
+            launch_i8_tile_rows(reinterpret_cast<const int8_t *>(centroids_split_.data()), nlist_, row_bytes,
+                                reinterpret_cast<int8_t *>(centroids_tiled_.data()), 0, stream_);
+            std::vector<float> pad((size_t)2 * padded, std::numeric_limits<float>::infinity());
+            std::copy(cn.begin(), cn.end(), pad.begin());                       // L2: the norms
+            std::fill(pad.begin() + padded, pad.begin() + padded + nlist_, 0.f);   // inner product: zeros
+            cnorm_pad_.upload(pad.data(), pad.size(), stream_);
+            sync_stream(stream_);   // `pad` is the source of an asynchronous copy
+        }
     }
     if (codebook) {
         codebook_.upload(codebook, (size_t)M_ * 256 * dsub_, stream_);
@@ -615,11 +634,13 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
         const bool set_wanted = set_only && !out_dist && ncand > nout;   // search: only the SET of lists matters
         BoundaryRefine br{x_dev, centroids_.data(), d_, nout, cmax_, bf16x3_err_scale(select_metric),
                           select_metric == kMetricL2 ? 4.0f * 5.9604645e-8f : 0.0f, out_ids};
+        const ResidentCoarse rc{reinterpret_cast<const uint16_t *>(centroids_tiled_.data()),
+                                cnorm_pad_.data() + (select_metric == kMetricL2 ? 0 : round_up(nlist_, kI8TileRows)), cmax_};
         if (sampled_bound_ok_ && cfg_.coarse_sampled_bound != 0 &&
             stream_select_bf16x3_sampled(ws_xsplit_.data(), n, centroids_split_.data(), nlist_, 3 * dp_, ws_qn_.data(),
                                          cnorm_.data(), select_metric, ncand, ws_running_.data(), ws_sel_,
-                                         cfg_.scratch_bytes, ws_flag_.data(), set_wanted ? &br : nullptr,
-                                         stream_) >= 0) {
+                                         cfg_.scratch_bytes, ws_flag_.data(), set_wanted ? &br : nullptr, stream_,
+                                         centroids_tiled_.size() && cfg_.coarse_resident != 0 ? &rc : nullptr) >= 0) {
             approx = true;
             last_coarse_plan_ = 1;
             if (set_wanted) {   // the plan has written out_ids itself

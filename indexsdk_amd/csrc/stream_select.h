@@ -50,10 +50,17 @@ struct BoundaryRefine {
     float cmax, err_scale, round_scale;
     int32_t *out_ids;
 };
+// With `resident` (and an instance of the resident-query kernel for d3) the two score launches read the base side
+// from matrix-core order instead (launch_resident_bf16_minima / _records in coarse.h); same plan, same proofs.
+struct ResidentCoarse {
+    const uint16_t *Bt;       // base-side split rows, tiled, zero rows up to a whole tile of 256
+    const float *cn_padded;   // |c|^2 (zeros for inner product), +inf up to a whole tile
+    float cmax;               // largest |c|
+};
 int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int64_t nb, int d3,
                                  const float *qn, const float *bn, int metric, int ncand, unsigned long long *running,
                                  StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, int *flag,
-                                 const BoundaryRefine *refine, hipStream_t s);
+                                 const BoundaryRefine *refine, hipStream_t s, const ResidentCoarse *resident = nullptr);
 // B: the base in matrix-core order and bn its norms padded with kI8PadNorm to whole tiles of 256 rows (flat_i8.h)
 int stream_select_i8(const int8_t *Q, int64_t nq, const int8_t *B, int64_t nb, int d, const int32_t *qn,
                      const int32_t *bn, int ncand, unsigned long long *running, StreamSelectWorkspace<int32_t> &ws,

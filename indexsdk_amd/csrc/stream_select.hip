@@ -392,8 +392,11 @@ int stream_select_bf16x3(const uint16_t *Qs, int64_t nq, const uint16_t *Bs, int
 int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uint16_t *Bs, int64_t nb_total, int d3,
                                  const float *qn, const float *bn, int metric, int ncand, unsigned long long *running,
                                  StreamSelectWorkspace<float> &ws, int64_t scratch_bytes, int *flag,
-                                 const BoundaryRefine *refine, hipStream_t s)
+                                 const BoundaryRefine *refine, hipStream_t s, const ResidentCoarse *resident)
 {
+    if (resident && !resident_coarse_serves(d3)) {
+        resident = nullptr;
+    }
     if (!flag || d3 % 32 != 0 || nb_total % 4 != 0 || ncand > kFoldMaxK || reinterpret_cast<uintptr_t>(Qs) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(Bs) % 16 != 0) {
         return -1;
@@ -426,6 +429,9 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uin
     }
     ws.scores.resize((size_t)qb * G);
     ws.tau.resize((size_t)nq_total);
+    if (resident) {
+        ws.thr.resize((size_t)nq_total);   // the record launch's per-query test values
+    }
     const bool fresh_cnt = ws.cnt.size() < (size_t)nq_total + 1;
     ws.cnt.resize((size_t)nq_total + 1);
     ws.filter.resize((size_t)qb * cap * 4);   // 32-byte records
@@ -436,19 +442,26 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uin
     int launches = 0;
     for (int64_t q0 = 0; q0 < nq_total; q0 += qb) {
         const int64_t nq = std::min(qb, nq_total - q0);
-        bool ok = launch_score_ring_bf16_minima(Qs + q0 * d3, nq, Bs, seed, d3, qn + q0, bn, metric, ws.scores.data(), G, s);
+        bool ok = resident ? launch_resident_bf16_minima(Qs + q0 * d3, nq, resident->Bt, seed, d3, qn + q0,
+                                                         resident->cn_padded, metric, ws.scores.data(), G, s)
+                           : launch_score_ring_bf16_minima(Qs + q0 * d3, nq, Bs, seed, d3, qn + q0, bn, metric,
+                                                           ws.scores.data(), G, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
         launch_tau_from_minima(ws.scores.data(), G, j, nq, ws.tau.data() + q0, s);
         ScoreFilter<float> flt{ws.tau.data() + q0, nullptr, ws.cnt.data() + q0, ws.filter.data(), cap, 0};
-        ok = launch_score_ring_bf16_records(Qs + q0 * d3, nq, Bs, nb_total, d3, qn + q0, bn, metric, flt, s);
+        ok = resident ? launch_resident_bf16_records(Qs + q0 * d3, nq, resident->Bt, nb_total, d3, qn + q0,
+                                                     resident->cn_padded, metric, resident->cmax, ws.thr.data() + q0, flt, s)
+                      : launch_score_ring_bf16_records(Qs + q0 * d3, nq, Bs, nb_total, d3, qn + q0, bn, metric, flt, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
+        // the resident-query launch records dot products; the folds form the scores
+        const RawRecords raw{qn + q0, bn, metric};
         if (refine) {
             // only the exact best-nout SET is wanted: no sorted list in between
             launch_fold_refine_boundary(refine->Q + q0 * refine->d, nq, refine->C, refine->d, qn + q0, bn, metric, flt,
                                         capk, refine->nout, refine->cmax, refine->err_scale, refine->round_scale,
-                                        refine->out_ids + q0 * refine->nout, flag, q0, s);
+                                        refine->out_ids + q0 * refine->nout, flag, q0, s, resident != nullptr);
         } else {
-            launch_fold_records(running + q0 * ncand, ncand, flt, nq, flag, q0, s);
+            launch_fold_records(running + q0 * ncand, ncand, flt, nq, flag, q0, s, resident ? &raw : nullptr);
         }
         launches += 2;
     }

@@ -22,16 +22,25 @@ def _mixture(rng, comp, n, d, sigma, centres=None):
     return (centres[rng.integers(0, len(centres), n)] + sigma * rng.standard_normal((n, d))).astype(np.float32), centres
 
 
-@pytest.mark.parametrize("metric_name,nlist,nprobe,nq,scratch", [
-    ("L2", 8192, 32, 2200, 0),          # the smallest product the plan takes (seed 2048 of 8192 centroids)
-    ("IP", 12000, 64, 2048, 0),         # a last tile of 224 centroids
-    ("L2", 16384, 64, 1500, 0),
-    ("L2", 8192, 32, 2304, 8 << 20),    # a scratch that holds the records of 512 queries: five query blocks
-    ("L2", 32768, 200, 512, 0),         # 241 candidates per query, seed of 4096 centroids, > 1024 scores per fold
+@pytest.mark.parametrize("metric_name,nlist,nprobe,nq,scratch,d,resident", [
+    ("L2", 8192, 32, 2200, 0, 64, 1),          # the smallest product the plan takes (seed 2048 of 8192 centroids)
+    ("IP", 12000, 64, 2048, 0, 64, 1),         # a last tile of 224 centroids
+    ("L2", 16384, 64, 1500, 0, 64, 1),
+    ("L2", 8192, 32, 2304, 8 << 20, 64, 1),    # a scratch that holds the records of 512 queries: five query blocks
+    ("L2", 32768, 200, 512, 0, 64, 1),         # 241 candidates per query, seed of 4096 centroids, > 1024 scores per fold
+    # the other dimensions the resident-query score kernel has instances for, query counts that end inside a tile
+    ("L2", 16384, 64, 1111, 0, 128, 1),
+    ("IP", 9000, 32, 2500, 0, 96, 1),
+    ("L2", 8192, 16, 4000, 0, 96, 1),
+    # the ring kernel (what dimensions without such an instance use), on the shapes above
+    ("L2", 8192, 32, 2200, 0, 64, 0),
+    ("IP", 12000, 64, 2048, 0, 64, 0),
+    ("L2", 16384, 64, 1111, 0, 128, 0),
+    ("L2", 8192, 32, 2200, 0, 160, 1),         # no resident instance for 160 dimensions: the ring kernel serves them
 ])
-def test_sampled_bound_plan_is_bit_exact(ix, oracle, metric_name, nlist, nprobe, nq, scratch):
+def test_sampled_bound_plan_is_bit_exact(ix, oracle, metric_name, nlist, nprobe, nq, scratch, d, resident):
     metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
-    d, M = 64, 8
+    M = 8
     rng = np.random.default_rng(nlist + nprobe)
     cent, centres = _mixture(rng, 48, nlist, d, 0.4)
     q, _ = _mixture(rng, 48, nq, d, 0.4, centres)
@@ -41,7 +50,7 @@ def test_sampled_bound_plan_is_bit_exact(ix, oracle, metric_name, nlist, nprobe,
             a /= np.linalg.norm(a, axis=1, keepdims=True)
     cb = rng.standard_normal((M, 256, d // M)).astype(np.float32)
     kw = {"scratch_bytes": scratch} if scratch else {}
-    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, ix.AscendIndexIVFPQConfig(**kw))
+    gpu = ix.AscendIndexIVFPQ(d, metric, nlist, M, 8, ix.AscendIndexIVFPQConfig(coarse_resident=resident, **kw))
     gpu.set_trained(cent, cb)
     gpu.setNumProbes(nprobe)
     gi, gd = gpu.coarse_probe(q)
@@ -68,13 +77,18 @@ def test_sampled_bound_plan_is_bit_exact(ix, oracle, metric_name, nlist, nprobe,
     assert np.array_equal(I0, I) and np.array_equal(D0.view(np.uint32), D.view(np.uint32))
 
 
-def _group_column(g):
-    """First column of score-kernel group g (32 columns of one 256-column tile that one lane owns)."""
+def _group_column(g, resident):
+    """First column of score-kernel group g, the 32 columns one group minimum of the seed launch covers: 32 consecutive
+    centroids (one wavefront's block) in the resident-query kernel, the 32 columns of a 256-column tile that one lane
+    owns in the ring kernel."""
+    if resident:
+        return 32 * g
     return (g // 8) * 256 + ((g % 8) // 2) * 64 + 4 * (g % 2)
 
 
+@pytest.mark.parametrize("resident", [1, 0])
 @pytest.mark.parametrize("case,scratch", [("farthest_first", 0), ("farthest_first", 8 << 20), ("decoys", 0)])
-def test_sampled_bound_with_centroids_in_an_adverse_order(ix, oracle, case, scratch):
+def test_sampled_bound_with_centroids_in_an_adverse_order(ix, oracle, case, scratch, resident):
     """All queries come from one cluster, and the seed stretch (the first 2048 centroids) says nothing about
     the rest.  farthest_first: the centroids are sorted by decreasing distance to that cluster, so the bound
     admits more than a row's records hold.  decoys: 30 centroids next to the cluster sit in 30 different
@@ -91,13 +105,13 @@ def test_sampled_bound_with_centroids_in_an_adverse_order(ix, oracle, case, scra
         cent = np.ascontiguousarray(cent[np.argsort(dist)[::-1]])
     else:
         for g in range(30):
-            cent[_group_column(g)] = centre + (0.05 * rng.standard_normal(d)).astype(np.float32)
+            cent[_group_column(g, resident)] = centre + (0.05 * rng.standard_normal(d)).astype(np.float32)
     q = (centre + 0.2 * rng.standard_normal((nq, d))).astype(np.float32)
     x = (cent[rng.integers(0, nlist, 20000)] + 0.2 * rng.standard_normal((20000, d))).astype(np.float32)
     cb = rng.standard_normal((M, 256, d // M)).astype(np.float32)
     ids = np.arange(20000, dtype=np.int64)
     kw = {"scratch_bytes": scratch} if scratch else {}
-    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(**kw))
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8, ix.AscendIndexIVFPQConfig(coarse_resident=resident, **kw))
     gpu.set_trained(cent, cb)
     gpu.setNumProbes(nprobe)
     # the first search runs on the empty index, so that nothing but these queries has met the plan yet (adding
