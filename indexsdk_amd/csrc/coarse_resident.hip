@@ -17,8 +17,8 @@
 //            records as {the four DOT PRODUCTS g, first centroid}: the test is made on u = g - |c|^2 / 2 (one fused
 //            multiply-add per score) against a per-query value that lies below (|q|^2 - tau) / 2 by more than the
 //            roundings of both forms can differ, so no run with a score <= tau is missed; the fold that reads the
-//            records turns g into scores (launch_fold_* with raw = true).  A lane counts its passing runs of all RA
-//            blocks first, reserves their places with RA atomics issued back to back, and stores afterwards.
+//            records turns g into scores (launch_fold_* with raw = true).  Records are compacted over the lanes into
+//            a per-wavefront queue in LDS and leave 64 at a time (one atomic and two stores per lane).
 #include <cmath>
 
 #include "coarse.h"
@@ -35,6 +35,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 8;
+constexpr int kQueueRecords = 128;   // per wavefront, 32 bytes each; flushed when fewer than 64 places are left
 enum { kMinima = 0, kRecords = 1 };
 
 template <int NHS, int PF, int RA, int MODE>
@@ -75,6 +76,27 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
     v16f acc[RA];
     bf16x8 breg[PF];
     v4f cnv[4];   // |c|^2 of the lane's 16 centroids of the current tile
+    // RECORDS: the wavefront's queue of records on their way out, 32 bytes each: {four dot products | first centroid,
+    // query row, -, -}
+    uint4 *queue = reinterpret_cast<uint4 *>(lds + QT * D + QT * 4) + wave * (2 * kQueueRecords);
+    int qcount = 0;   // wave-uniform
+    auto flush_queue = [&]() {
+        wave_lds_fence();
+        unsigned char *records = reinterpret_cast<unsigned char *>(flt.cand);
+        for (int i0 = 0; i0 < qcount; i0 += 64) {
+            if (i0 + lane < qcount) {
+                const uint4 sc = queue[2 * (i0 + lane)], id = queue[2 * (i0 + lane) + 1];
+                const int p = atomicAdd(&flt.cnt[id.y], 1);
+                if (p < flt.cap) {
+                    unsigned char *rec = records + ((int64_t)id.y * flt.cap + p) * 32;
+                    *reinterpret_cast<uint4 *>(rec) = sc;
+                    *reinterpret_cast<uint32_t *>(rec + 16) = id.x;
+                }
+            }
+        }
+        wave_lds_fence();
+        qcount = 0;
+    };
     int cur_tm = -1;
     int it_t = first_item;
     int tm, j, jend;
@@ -90,13 +112,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
             if (cur_tm >= 0) {
                 __syncthreads();
             }
-            for (int idx = tid; idx < QT * (D / 16); idx += kWaves * 64) {
-                const int q = idx % QT, c = idx / QT;
-                int64_t row = (int64_t)tm * QT + q;
-                row = row < nq ? row : nq - 1;
-                *reinterpret_cast<uint4 *>(lds + c * (QT * 16) + q * 16) =
-                    *reinterpret_cast<const uint4 *>(Qb + row * D + c * 16);
-            }
+            load_resident_tile<QT, D, kWaves * 64>(lds, Qb, (int64_t)tm * QT, nq, tid);
             if (tid < QT) {
                 const int64_t row = (int64_t)tm * QT + tid;
                 if constexpr (MODE == kRecords) {
@@ -191,13 +207,15 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
                 }
             }
         } else {
-            // pass 1: which runs hold a score that may be <= tau; one counter reservation per block, all in flight
-            uint32_t bits = 0;
-            int pos[RA];
+            // Every run that may hold a score <= tau goes to the wavefront's queue in LDS, compacted over the lanes
+            // (nearly every run has SOME lane that passes -- 64 lanes, 64 queries -- but only one or two do: stored
+            // from their own lanes the records would cost a vector-memory instruction per run for a couple of active
+            // lanes); full batches of 64 leave for the rows' record buffers with one atomic and two stores per lane.
+            const uint32_t colv = (uint32_t)(col0 + flt.col_base);
 #pragma unroll
             for (int ra = 0; ra < RA; ra++) {
                 const float tv = perq[ra * 32 + l32];
-                int npass = 0;
+                const uint32_t row = (uint32_t)(tm * QT + ra * 32 + l32);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     float u[4];
@@ -207,32 +225,19 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
                     }
                     const float m = fmaxf(fmaxf(u[0], u[1]), fmaxf(u[2], u[3]));
                     const bool pass = m >= tv && col0 + 8 * g < nb;
-                    bits |= pass ? 1u << (4 * ra + g) : 0u;
-                    npass += pass ? 1 : 0;
-                }
-                pos[ra] = 0;
-                if (npass > 0) {
-                    pos[ra] = atomicAdd(&flt.cnt[(int64_t)tm * QT + ra * 32 + l32], npass);
-                }
-            }
-            // pass 2: the records
-            if (__builtin_amdgcn_ballot_w64(bits != 0) != 0) {
-                unsigned char *records = reinterpret_cast<unsigned char *>(flt.cand);
-#pragma unroll
-                for (int ra = 0; ra < RA; ra++) {
-                    const int64_t row = (int64_t)tm * QT + ra * 32 + l32;
-                    int p = pos[ra];
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        if ((bits >> (4 * ra + g)) & 1u) {
-                            if (p < flt.cap) {
-                                unsigned char *rec = records + (row * flt.cap + p) * 32;
-                                *reinterpret_cast<float4 *>(rec) = make_float4(acc[ra][4 * g], acc[ra][4 * g + 1],
-                                                                               acc[ra][4 * g + 2], acc[ra][4 * g + 3]);
-                                *reinterpret_cast<uint32_t *>(rec + 16) = (uint32_t)(col0 + 8 * g + flt.col_base);
-                            }
-                            p++;
+                    const unsigned long long mask = __builtin_amdgcn_ballot_w64(pass);
+                    if (mask != 0) {
+                        if (qcount > kQueueRecords - 64) {
+                            flush_queue();
                         }
+                        const int at = qcount + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                                         __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+                        if (pass) {
+                            queue[2 * at] = make_uint4(__float_as_uint(acc[ra][4 * g]), __float_as_uint(acc[ra][4 * g + 1]),
+                                                       __float_as_uint(acc[ra][4 * g + 2]), __float_as_uint(acc[ra][4 * g + 3]));
+                            queue[2 * at + 1] = make_uint4(colv + 8 * g, row, 0u, 0u);
+                        }
+                        qcount += __builtin_popcountll(mask);
                     }
                 }
             }
@@ -245,6 +250,9 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
         j = n_j;
         jend = n_jend;
         cur = nxt;
+    }
+    if constexpr (MODE == kRecords) {
+        flush_queue();
     }
 }
 
@@ -273,8 +281,10 @@ void launch_shape(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const floa
                   const float *test, int metric, float *out, int64_t ldo, ScoreFilter<float> flt, int seg, hipStream_t s)
 {
     constexpr int QT = RA * 32;
-    constexpr size_t smem = (size_t)QT * NHS * 32 + QT * 4;
-    static_assert(smem <= 160 * 1024, "the query tile must fit the LDS of a CU");
+    constexpr size_t smem = (size_t)QT * NHS * 32 + QT * 4 + (MODE == kRecords ? kWaves * kQueueRecords * 32 : 0);
+    if constexpr (smem > 160 * 1024) {
+        fail(kErrInner, "resident coarse kernel: tile of %d queries does not fit LDS", QT);   // the plan never picks it
+    } else {
     auto kern = resident_bf16_kernel<NHS, PF, RA, MODE>;
     static bool configured = false;
     if (!configured) {
@@ -290,6 +300,7 @@ void launch_shape(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const floa
     const unsigned grid = (unsigned)((device_cus() + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), smem, s, Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt,
                        (int)tiles_m, (int)ntiles, seg);
+    }
 }
 
 template <int NHS, int PF, int MODE>
@@ -302,7 +313,7 @@ void launch_ra(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const float *
     int64_t best_seg = 1;
     double best = 1e300;
     for (int ra = 4; ra <= 6; ra++) {
-        if ((size_t)ra * 32 * NHS * 32 + ra * 128 > 160 * 1024) {
+        if ((size_t)ra * 32 * NHS * 32 + ra * 128 + (MODE == kRecords ? kWaves * kQueueRecords * 32 : 0) > 160 * 1024) {
             continue;
         }
         const int64_t tiles_m = (nq + ra * 32 - 1) / (ra * 32);

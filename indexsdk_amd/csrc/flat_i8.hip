@@ -356,13 +356,8 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
             if (cur_tm >= 0) {
                 __syncthreads();
             }
-            for (int idx = tid; idx < QT * (D / 16); idx += kResidentWaves * 64) {
-                const int q = idx % QT, c = idx / QT;
-                int64_t row = (int64_t)tm * QT + q;
-                row = row < nq ? row : nq - 1;
-                *reinterpret_cast<uint4 *>(lds + c * (QT * 16) + q * 16) =
-                    *reinterpret_cast<const uint4 *>(Q + row * D + c * 16);
-            }
+            load_resident_tile<QT, D, kResidentWaves * 64>(lds, reinterpret_cast<const unsigned char *>(Q),
+                                                           (int64_t)tm * QT, nq, tid);
             if constexpr (FILTER) {
                 if (tid < QT) {
                     const int64_t row = (int64_t)tm * QT + tid;

@@ -159,6 +159,8 @@ private:
     int64_t ntotal_ = 0;
     hipStream_t stream_ = nullptr;
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
+    static constexpr int kIoPieces = 4;                               // pieces the results of a large host search come down in
+    hipEvent_t io_ev_[kIoPieces] = {nullptr, nullptr, nullptr, nullptr};   // created on first use
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
@@ -198,7 +200,7 @@ private:
     std::vector<int32_t> touch_mark_; // scratch of append(): -1, or the list's place among the touched lists
     std::vector<int32_t> add_pos_;    // scratch of append(): position of every new vector inside its list
     PinnedBuffer add_stage_, add_pack_;   // append(): assignments coming down, kernel inputs going up
-    PinnedBuffer io_stage_;               // small host searches: queries going up, results coming down
+    PinnedBuffer io_stage_;               // host searches: queries going up, results coming down
     DeviceBuffer<int64_t> ws_add_pack_, ws_add_ids_;
     DeviceBuffer<int32_t> ws_add_lists_;
     DeviceBuffer<uint8_t> ws_add_codes_;

@@ -8,6 +8,7 @@
 #include <mutex>
 #include <numeric>
 #include <random>
+#include <thread>
 #include <unordered_set>
 
 #include "coarse.h"
@@ -79,6 +80,36 @@ constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this 
 constexpr int kMaxNprobe = 2048;        // probed lists per query (the reference's L3 operator takes 128 per tile)
 constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
 constexpr size_t kStagedIoBytes = (size_t)1 << 20;   // host searches whose queries and results fit go through pinned staging
+// Larger host searches up to this size go through the same page-locked buffer with their host-side copies spread over
+// a few threads and the results coming down in pieces (beyond it the runtime's own path for pageable memory serves).
+constexpr size_t kPipelinedIoBytes = (size_t)256 << 20;
+constexpr size_t kParallelCopyBytes = (size_t)2 << 20;   // host copies of at least this much are shared by threads
+
+// memcpy shared by up to four threads (one of them the caller's): a single thread moves a batch's queries and
+// results between pageable and page-locked memory at a few GB/s, which costs a large search more than the DMA does.
+void parallel_memcpy(void *dst, const void *src, size_t bytes)
+{
+    const unsigned hw = std::thread::hardware_concurrency();
+    const int nthreads = bytes < kParallelCopyBytes ? 1 : (int)std::min<unsigned>(4, hw ? hw : 1);
+    if (nthreads <= 1) {
+        std::memcpy(dst, src, bytes);
+        return;
+    }
+    const size_t piece = (bytes / nthreads + 4095) / 4096 * 4096;
+    std::vector<std::thread> workers;
+    for (int t = 1; t < nthreads; t++) {
+        const size_t off = piece * t;
+        if (off < bytes) {
+            workers.emplace_back([=]() {
+                std::memcpy(static_cast<char *>(dst) + off, static_cast<const char *>(src) + off, std::min(piece, bytes - off));
+            });
+        }
+    }
+    std::memcpy(dst, src, std::min(piece, bytes));
+    for (auto &w : workers) {
+        w.join();
+    }
+}
 constexpr int64_t kCoarseExactMaxMacs = (int64_t)1 << 27;   // queries x centroids x dims up to which a search selects its lists exactly
 
 // ---- arena kernels ------------------------------------------------------------------------------
@@ -453,6 +484,11 @@ IvfpqIndex::~IvfpqIndex()
         (void)hipStreamSynchronize(stream_);
     }
     for (auto &ev : ev_) {
+        if (ev) {
+            (void)hipEventDestroy(ev);
+        }
+    }
+    for (auto &ev : io_ev_) {
         if (ev) {
             (void)hipEventDestroy(ev);
         }
@@ -1462,11 +1498,13 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     const size_t in_bytes = (size_t)n * d_ * sizeof(float), dist_bytes = (size_t)n * k * sizeof(float),
                  label_bytes = (size_t)n * k * sizeof(int64_t);
     const size_t dist_at = (in_bytes + 255) / 256 * 256, label_at = dist_at + (dist_bytes + 255) / 256 * 256;
-    const bool staged_io = !on_device && label_at + label_bytes <= kStagedIoBytes;
+    // (larger batches take the same route with their host copies on several threads and the results in pieces)
+    const bool staged_io = !on_device && label_at + label_bytes <= kPipelinedIoBytes;
+    const bool pipelined_io = staged_io && label_at + label_bytes > kStagedIoBytes;
     unsigned char *io = nullptr;
     if (staged_io) {
         io = static_cast<unsigned char *>(io_stage_.reserve(label_at + label_bytes));
-        std::memcpy(io, x, in_bytes);
+        parallel_memcpy(io, x, in_bytes);
         ws_x_.resize((size_t)n * d_);
         IXA_HIP(hipMemcpyAsync(ws_x_.data(), io, in_bytes, hipMemcpyHostToDevice, stream_));
         xd = ws_x_.data();
@@ -1528,7 +1566,53 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     }
     stats_timed_ = timed;
 
-    if (staged_io) {
+    if (pipelined_io) {
+        // The results come down in kIoPieces pieces with an event behind each; a thread per piece waits for its event
+        // and copies its part of the distances and of the labels out of the staging buffer while the next pieces are
+        // still on their way.
+        const size_t total = label_at - dist_at + label_bytes;
+        const size_t piece = (total / kIoPieces + 4095) / 4096 * 4096;
+        for (int c = 0; c < kIoPieces; c++) {
+            if (!io_ev_[c]) {
+                IXA_HIP(hipEventCreateWithFlags(&io_ev_[c], hipEventDisableTiming));
+            }
+            const size_t off = piece * c;
+            if (off < total) {
+                IXA_HIP(hipMemcpyAsync(io + dist_at + off, ws_results_.data() + off, std::min(piece, total - off),
+                                       hipMemcpyDeviceToHost, stream_));
+            }
+            IXA_HIP(hipEventRecord(io_ev_[c], stream_));
+        }
+        hipError_t errs[kIoPieces];
+        auto copy_out = [&](int c) {
+            errs[c] = hipEventSynchronize(io_ev_[c]);
+            if (errs[c] != hipSuccess) {
+                return;
+            }
+            // piece c of the staged [distances | padding | labels]: its overlap with either array
+            const size_t a = dist_at + piece * c, b = std::min(dist_at + total, a + piece);
+            auto part = [&](size_t at, size_t bytes, void *out) {
+                const size_t lo = std::max(a, at), hi = std::min(b, at + bytes);
+                if (lo < hi) {
+                    std::memcpy(static_cast<char *>(out) + (lo - at), io + lo, hi - lo);
+                }
+            };
+            part(dist_at, dist_bytes, dist);
+            part(label_at, label_bytes, labels);
+        };
+        std::vector<std::thread> workers;
+        for (int c = 1; c < kIoPieces; c++) {
+            workers.emplace_back(copy_out, c);
+        }
+        copy_out(0);
+        for (auto &w : workers) {
+            w.join();
+        }
+        for (int c = 0; c < kIoPieces; c++) {
+            IXA_HIP(errs[c]);
+        }
+        sync_stream(stream_);
+    } else if (staged_io) {
         IXA_HIP(hipMemcpyAsync(io + dist_at, ws_results_.data(), label_at - dist_at + label_bytes, hipMemcpyDeviceToHost,
                                stream_));
         sync_stream(stream_);

@@ -45,6 +45,46 @@ __device__ __forceinline__ void lds_wait_group(V (&f)[N])
     }
 }
 
+// The resident tile: rows first .. first + QT - 1 of a row-major array (rows of D bytes; rows past the end of the array
+// repeat its last row) into LDS as [16-byte chunk][row][16 B].  A wavefront moves 16 rows x 4 chunks per step: 64
+// contiguous bytes of every row on the memory side, 256 contiguous bytes per chunk on the LDS side (a four-way bank
+// conflict; row-fastest would read 16 bytes per row, chunk-fastest would put 64 lanes on four banks), and a
+// thread issues eight loads before the first store, so the tile costs a few memory round trips, not one per step.
+template <int QT, int D, int NT>
+__device__ __forceinline__ void load_resident_tile(unsigned char *lds, const unsigned char *__restrict__ rows, int64_t first,
+                                                   int64_t nrows, int tid)
+{
+    static_assert(QT % 16 == 0 && D % 64 == 0, "tile shape");
+    constexpr int kSteps = (QT / 16) * (D / 64);   // wavefront steps of 16 rows x 4 chunks
+    constexpr int kWavesT = NT / 64;
+    constexpr int kPerWave = (kSteps + kWavesT - 1) / kWavesT;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int qq = lane & 15, cc = lane >> 4;
+    constexpr int kBatch = 8;   // loads in flight per thread: registers are scarce where this is called
+#pragma unroll
+    for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
+        uint4 v[kBatch];
+#pragma unroll
+        for (int b = 0; b < kBatch; b++) {
+            const int step = wave + (i0 + b) * kWavesT;
+            const int qb = step % (QT / 16), cb = step / (QT / 16);
+            if (i0 + b < kPerWave && step < kSteps) {
+                int64_t row = first + qb * 16 + qq;
+                row = row < nrows ? row : nrows - 1;
+                v[b] = *reinterpret_cast<const uint4 *>(rows + row * D + (cb * 4 + cc) * 16);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < kBatch; b++) {
+            const int step = wave + (i0 + b) * kWavesT;
+            const int qb = step % (QT / 16), cb = step / (QT / 16);
+            if (i0 + b < kPerWave && step < kSteps) {
+                *reinterpret_cast<uint4 *>(lds + (cb * 4 + cc) * (QT * 16) + (qb * 16 + qq) * 16) = v[b];
+            }
+        }
+    }
+}
+
 // Work items of a persistent launch: XCD x (workgroup b runs on XCD b % 8) owns tiles x, x + 8, ... of the streamed
 // operand; an item is (resident tile, segment of the XCD's tiles), resident tile fastest, dealt round-robin to the
 // XCD's workgroups.  The S = wpx / tiles_m segments that are in flight together INTERLEAVE tile by tile inside a
