@@ -159,8 +159,6 @@ private:
     int64_t ntotal_ = 0;
     hipStream_t stream_ = nullptr;
     hipEvent_t ev_[4] = {nullptr, nullptr, nullptr, nullptr};
-    static constexpr int kIoPieces = 4;                               // pieces the results of a large host search come down in
-    hipEvent_t io_ev_[kIoPieces] = {nullptr, nullptr, nullptr, nullptr};   // created on first use
 
     DeviceBuffer<float> centroids_, cnorm_, codebook_, cbnorm_;
     DeviceBuffer<uint16_t> centroids_split_, ws_xsplit_;   // bf16 x 3 splits (candidate generation only)
@@ -213,7 +211,6 @@ private:
     DeviceBuffer<unsigned long long> ws_running_;
     DeviceBuffer<int32_t> ws_cand_, ws_probes_;
     DeviceBuffer<int64_t> ws_labels_;
-    DeviceBuffer<unsigned char> ws_results_;   // distances | labels of a small host search (one copy down)
     DeviceBuffer<unsigned long long> ws_partial_, ws_counter_;
     SearchStats stats_;
 };

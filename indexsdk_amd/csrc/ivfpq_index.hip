@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <initializer_list>
 #include <mutex>
 #include <numeric>
 #include <random>
@@ -80,32 +81,43 @@ constexpr int64_t kMaxK = 2048;         // LDS-resident selection limit of this 
 constexpr int kMaxNprobe = 2048;        // probed lists per query (the reference's L3 operator takes 128 per tile)
 constexpr int64_t kAddPage = 1 << 20;   // vectors per add page
 constexpr size_t kStagedIoBytes = (size_t)1 << 20;   // host searches whose queries and results fit go through pinned staging
-// Larger host searches up to this size go through the same page-locked buffer with their host-side copies spread over
-// a few threads and the results coming down in pieces (beyond it the runtime's own path for pageable memory serves).
+// Larger host searches up to this size go through the same page-locked buffer with the queries going up in two halves
+// (beyond it the runtime's own path for pageable memory serves).
 constexpr size_t kPipelinedIoBytes = (size_t)256 << 20;
-constexpr size_t kParallelCopyBytes = (size_t)2 << 20;   // host copies of at least this much are shared by threads
+constexpr size_t kParallelCopyBytes = (size_t)4 << 20;   // host copies of at least this much are shared by threads
 
-// memcpy shared by up to four threads (one of them the caller's): a single thread moves a batch's queries and
-// results between pageable and page-locked memory at a few GB/s, which costs a large search more than the DMA does.
-void parallel_memcpy(void *dst, const void *src, size_t bytes)
+// Host copies shared by up to four threads (one of them the caller's) once there is enough to move to pay for
+// starting them (about 80 us for three): results that the GPU has just written into page-locked memory come out of
+// DRAM, not out of the caller's cache, and a single thread moves those at 20-30 GB/s.  Thread t copies the t-th
+// slice of every job.
+struct CopyJob {
+    void *dst;
+    const void *src;
+    size_t bytes;
+};
+
+void parallel_copy(std::initializer_list<CopyJob> jobs)
 {
-    const unsigned hw = std::thread::hardware_concurrency();
-    const int nthreads = bytes < kParallelCopyBytes ? 1 : (int)std::min<unsigned>(4, hw ? hw : 1);
-    if (nthreads <= 1) {
-        std::memcpy(dst, src, bytes);
-        return;
+    size_t total = 0;
+    for (const CopyJob &j : jobs) {
+        total += j.bytes;
     }
-    const size_t piece = (bytes / nthreads + 4095) / 4096 * 4096;
+    const unsigned hw = std::thread::hardware_concurrency();
+    const int nthreads = total < kParallelCopyBytes ? 1 : (int)std::min<unsigned>(4, hw ? hw : 1);
+    auto slice = [&](int t) {
+        for (const CopyJob &j : jobs) {
+            const size_t piece = (j.bytes / nthreads + 4095) / 4096 * 4096, off = piece * t;
+            if (off < j.bytes) {
+                std::memcpy(static_cast<char *>(j.dst) + off, static_cast<const char *>(j.src) + off,
+                            std::min(piece, j.bytes - off));
+            }
+        }
+    };
     std::vector<std::thread> workers;
     for (int t = 1; t < nthreads; t++) {
-        const size_t off = piece * t;
-        if (off < bytes) {
-            workers.emplace_back([=]() {
-                std::memcpy(static_cast<char *>(dst) + off, static_cast<const char *>(src) + off, std::min(piece, bytes - off));
-            });
-        }
+        workers.emplace_back(slice, t);
     }
-    std::memcpy(dst, src, std::min(piece, bytes));
+    slice(0);
     for (auto &w : workers) {
         w.join();
     }
@@ -484,11 +496,6 @@ IvfpqIndex::~IvfpqIndex()
         (void)hipStreamSynchronize(stream_);
     }
     for (auto &ev : ev_) {
-        if (ev) {
-            (void)hipEventDestroy(ev);
-        }
-    }
-    for (auto &ev : io_ev_) {
         if (ev) {
             (void)hipEventDestroy(ev);
         }
@@ -1492,21 +1499,27 @@ void IvfpqIndex::search(int64_t n, const float *x, int64_t k, float *dist, int64
 void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device)
 {
     const float *xd = x;
-    // A small batch in host memory goes through one page-locked staging buffer (queries | distances | labels): a
-    // copy to or from pageable memory costs about 45 us each on its own, whatever its size, and the results
-    // then come down behind a single wait.
+    // A batch in host memory goes through one page-locked staging buffer (queries | distances | labels): a copy to
+    // or from pageable memory costs about 45 us each on its own, whatever its size.
     const size_t in_bytes = (size_t)n * d_ * sizeof(float), dist_bytes = (size_t)n * k * sizeof(float),
                  label_bytes = (size_t)n * k * sizeof(int64_t);
     const size_t dist_at = (in_bytes + 255) / 256 * 256, label_at = dist_at + (dist_bytes + 255) / 256 * 256;
-    // (larger batches take the same route with their host copies on several threads and the results in pieces)
+    // (larger batches take the same route with the queries going up in two halves)
     const bool staged_io = !on_device && label_at + label_bytes <= kPipelinedIoBytes;
     const bool pipelined_io = staged_io && label_at + label_bytes > kStagedIoBytes;
     unsigned char *io = nullptr;
     if (staged_io) {
         io = static_cast<unsigned char *>(io_stage_.reserve(label_at + label_bytes));
-        parallel_memcpy(io, x, in_bytes);
         ws_x_.resize((size_t)n * d_);
-        IXA_HIP(hipMemcpyAsync(ws_x_.data(), io, in_bytes, hipMemcpyHostToDevice, stream_));
+        // the queries go up in two halves when there is much of them: the second half is copied into the staging
+        // buffer while the first is on its way
+        const size_t half = pipelined_io ? (in_bytes / 2 + 4095) / 4096 * 4096 : in_bytes;
+        for (size_t off = 0; off < in_bytes; off += half) {
+            const size_t bytes = std::min(half, in_bytes - off);
+            parallel_copy({{io + off, reinterpret_cast<const unsigned char *>(x) + off, bytes}});
+            IXA_HIP(hipMemcpyAsync(reinterpret_cast<unsigned char *>(ws_x_.data()) + off, io + off, bytes,
+                                   hipMemcpyHostToDevice, stream_));
+        }
         xd = ws_x_.data();
     } else if (!on_device) {
         ws_x_.upload(x, (size_t)n * d_, stream_);
@@ -1515,10 +1528,13 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     float *dd = dist;
     int64_t *ld = labels;
     if (staged_io) {
-        // distances and labels lie in one device buffer as they lie in the staging buffer: one copy brings both down
-        ws_results_.resize(label_at - dist_at + label_bytes);
-        dd = reinterpret_cast<float *>(ws_results_.data());
-        ld = reinterpret_cast<int64_t *>(ws_results_.data() + (label_at - dist_at));
+        // The kernels that finish a query write its distances and labels straight into the page-locked staging buffer,
+        // which the GPU addresses over PCIe: the results travel while other queries are still being scanned, and no
+        // copy engine has to be waited for once the last kernel is done.  (Nothing reads the results back.)
+        void *mapped = nullptr;
+        IXA_HIP(hipHostGetDevicePointer(&mapped, io, 0));
+        dd = reinterpret_cast<float *>(static_cast<unsigned char *>(mapped) + dist_at);
+        ld = reinterpret_cast<int64_t *>(static_cast<unsigned char *>(mapped) + label_at);
     } else if (!on_device) {
         ws_dist_.resize((size_t)n * k);
         ws_labels_.resize((size_t)n * k);
@@ -1566,58 +1582,9 @@ void IvfpqIndex::search_page(int64_t n, const float *x, int64_t k, float *dist, 
     }
     stats_timed_ = timed;
 
-    if (pipelined_io) {
-        // The results come down in kIoPieces pieces with an event behind each; a thread per piece waits for its event
-        // and copies its part of the distances and of the labels out of the staging buffer while the next pieces are
-        // still on their way.
-        const size_t total = label_at - dist_at + label_bytes;
-        const size_t piece = (total / kIoPieces + 4095) / 4096 * 4096;
-        for (int c = 0; c < kIoPieces; c++) {
-            if (!io_ev_[c]) {
-                IXA_HIP(hipEventCreateWithFlags(&io_ev_[c], hipEventDisableTiming));
-            }
-            const size_t off = piece * c;
-            if (off < total) {
-                IXA_HIP(hipMemcpyAsync(io + dist_at + off, ws_results_.data() + off, std::min(piece, total - off),
-                                       hipMemcpyDeviceToHost, stream_));
-            }
-            IXA_HIP(hipEventRecord(io_ev_[c], stream_));
-        }
-        hipError_t errs[kIoPieces];
-        auto copy_out = [&](int c) {
-            errs[c] = hipEventSynchronize(io_ev_[c]);
-            if (errs[c] != hipSuccess) {
-                return;
-            }
-            // piece c of the staged [distances | padding | labels]: its overlap with either array
-            const size_t a = dist_at + piece * c, b = std::min(dist_at + total, a + piece);
-            auto part = [&](size_t at, size_t bytes, void *out) {
-                const size_t lo = std::max(a, at), hi = std::min(b, at + bytes);
-                if (lo < hi) {
-                    std::memcpy(static_cast<char *>(out) + (lo - at), io + lo, hi - lo);
-                }
-            };
-            part(dist_at, dist_bytes, dist);
-            part(label_at, label_bytes, labels);
-        };
-        std::vector<std::thread> workers;
-        for (int c = 1; c < kIoPieces; c++) {
-            workers.emplace_back(copy_out, c);
-        }
-        copy_out(0);
-        for (auto &w : workers) {
-            w.join();
-        }
-        for (int c = 0; c < kIoPieces; c++) {
-            IXA_HIP(errs[c]);
-        }
+    if (staged_io) {
         sync_stream(stream_);
-    } else if (staged_io) {
-        IXA_HIP(hipMemcpyAsync(io + dist_at, ws_results_.data(), label_at - dist_at + label_bytes, hipMemcpyDeviceToHost,
-                               stream_));
-        sync_stream(stream_);
-        std::memcpy(dist, io + dist_at, dist_bytes);
-        std::memcpy(labels, io + label_at, label_bytes);
+        parallel_copy({{dist, io + dist_at, dist_bytes}, {labels, io + label_at, label_bytes}});
     } else if (!on_device) {
         ws_dist_.download(dist, (size_t)n * k, stream_);
         ws_labels_.download(labels, (size_t)n * k, stream_);
