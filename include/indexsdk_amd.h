@@ -18,8 +18,11 @@
  *   - metric: 0 = inner product, 1 = L2 (faiss::MetricType values).
  *   - missing results: label -1, distance FLT_MAX for L2 and -FLT_MAX for inner product
  *     (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2202-2219; FR/ascend/impl/AscendIndexImpl.cpp:587-650).
- *   - one index object may be used by one thread at a time (the reference's default mode,
- *     FR/ascend/impl/AscendIndexImpl.h:215-237 without MX_INDEX_MULTITHREAD).
+ *   - every handle may be used from several threads.  An IVFPQ handle locks as the reference does under
+ *     MX_INDEX_MULTITHREAD (FR/ascend/impl/AscendIndexImpl.h:62, 230; AscendIndexImpl.cpp:204, 508-564):
+ *     ivfpq_search, ivfpq_search_device and ivfpq_search_probes_device take the lock shared and up to four of
+ *     them run side by side, each on a stream and workspaces of its own; every other call takes it
+ *     exclusively.  Calls on one Flat handle are serialised.  Different handles never wait for each other.
  *   - there is no CPU fallback: every entry point fails with IXA_ERR_INDEX_NOT_INIT when no
  *     HIP device is present.
  */
@@ -302,6 +305,10 @@ int ivfpq_reclaim_memory(ivfpq_index_t *h, int64_t *bytes_reclaimed);
  * or abandoned, and abandoned by lists that moved.  Any output may be NULL.  No counterpart in the reference
  * (whose lists are separate device vectors): a diagnostic of the amortised add path. */
 int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocated, int64_t *slots_used, int64_t *slots_holes);
+/* How many search lanes (streams with workspaces of their own) the handle has made so far: 1, plus one for every
+ * further search that was ever in flight at the same time, up to 4.  No counterpart in the reference: a diagnostic of
+ * the shared search lock. */
+int ivfpq_search_lanes(const ivfpq_index_t *h, int *out);
 /* AscendIndexIVF::reset()  FR/ascend/AscendIndexIVF.h:93: drops the lists, keeps the quantizers. */
 int ivfpq_reset(ivfpq_index_t *h);
 int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out);

@@ -88,6 +88,7 @@ _SIGNATURES = {
     "ivfpq_reserve_memory": (ctypes.c_int, [_H, ctypes.c_int64]),
     "ivfpq_reclaim_memory": (ctypes.c_int, [_H, c_i64p]),
     "ivfpq_arena_state": (ctypes.c_int, [_H, c_i64p, c_i64p, c_i64p]),
+    "ivfpq_search_lanes": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int)]),
     "ivfpq_plan_scan_lds": (ctypes.c_int, [ctypes.c_int] * 9 + [ctypes.POINTER(ScanLdsPlan)]),
     "ivfpq_get_code_layout": (ctypes.c_int, [_H, ctypes.POINTER(ctypes.c_int)]),
     "ivfpq_config_default": (None, [ctypes.POINTER(IvfpqConfig)]),

@@ -226,6 +226,12 @@ class AscendIndexIVFPQ:
         _capi.check(self._lib.ivfpq_arena_state(self._h, ctypes.byref(a), ctypes.byref(u), ctypes.byref(h)))
         return a.value, u.value, h.value
 
+    def search_lanes(self):
+        """Streams with workspaces of their own that searches of this index have needed so far (1 to 4)."""
+        out = ctypes.c_int()
+        _capi.check(self._lib.ivfpq_search_lanes(self._h, ctypes.byref(out)))
+        return out.value
+
     def set_stage_timings(self, mode):
         """Stage events of a search (ms_coarse / ms_scan): 1 always, 0 never, -1 for pages of >= 256 queries."""
         _capi.check(self._lib.ivfpq_set_stage_timings(self._h, mode))

@@ -5,7 +5,10 @@
 #include <algorithm>
 #include <cstring>
 #include <memory>
+#include <condition_variable>
 #include <mutex>
+#include <shared_mutex>
+#include <type_traits>
 #include <new>
 #include <string>
 
@@ -20,19 +23,29 @@ std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig
 }  // namespace ixa
 
 // The handle owns the index through a pointer so that a loader can hand over a finished one.
-// Every call on a handle holds the handle's mutex: the reference guards an index with one shared_mutex
-// when MX_INDEX_MULTITHREAD is set (FR/ascend/impl/AscendIndexImpl.h:62, 230); here calls on one index
-// are always serialised (a search uses the index's workspace and stream), calls on different indexes
-// run concurrently.
+// Locking follows the reference's MX_INDEX_MULTITHREAD mode (FR/ascend/impl/AscendIndexImpl.h:62, 230;
+// AscendIndexImpl.cpp:204, 508-564), always on here: a search takes the handle's lock shared, everything that
+// changes the index takes it exclusively.  A search needs a stream and workspaces of its own, so each runs on a
+// lane: lane 0 is the index itself, lanes 1..kSearchViews are views that read the index's trained state and lists
+// in place (IvfpqIndex::borrow_from), made on first need.  A search that finds every lane taken waits for one.
 struct ivfpq_index {
-    mutable std::mutex mu;
+    static constexpr int kSearchViews = 3;
+    mutable std::shared_mutex mu;
     std::unique_ptr<ixa::IvfpqIndex> owned;
     ixa::IvfpqIndex &impl;
+    // lanes (guarded by lane_mu)
+    mutable std::mutex lane_mu;
+    mutable std::condition_variable lane_cv;
+    mutable std::unique_ptr<ixa::IvfpqIndex> views[kSearchViews];
+    mutable uint64_t view_version[kSearchViews] = {0, 0, 0};
+    mutable uint64_t version = 1;       // counts the calls that may have changed the index
+    mutable unsigned busy = 0;          // bit l = lane l is searching
+    mutable ixa::IvfpqIndex *last;      // lane of the search that finished last: "the last search" of the statistics
     ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
-        : owned(new ixa::IvfpqIndex(d, metric, nlist, M, nbits, c)), impl(*owned)
+        : owned(new ixa::IvfpqIndex(d, metric, nlist, M, nbits, c)), impl(*owned), last(owned.get())
     {
     }
-    explicit ivfpq_index(std::unique_ptr<ixa::IvfpqIndex> p) : owned(std::move(p)), impl(*owned) {}
+    explicit ivfpq_index(std::unique_ptr<ixa::IvfpqIndex> p) : owned(std::move(p)), impl(*owned), last(owned.get()) {}
 };
 
 struct flat_index {
@@ -74,9 +87,88 @@ int guarded(F &&f, bool uses_gpu = true)
     }
 }
 
-#define IXA_HANDLE(h)                                                                             \
+// Exclusive use of a handle.  For an IVFPQ handle: the statistics a view still owes refer to lists that the call
+// may move, so they are worked out first; a call that may change the index makes every view borrow again.
+template <typename H>
+struct Exclusive {
+    std::unique_lock<decltype(H::mu)> lock;
+    Exclusive(const H *h, bool) : lock(h->mu) {}
+};
+template <>
+struct Exclusive<ivfpq_index> {
+    std::unique_lock<std::shared_mutex> lock;
+    const ivfpq_index *h;
+    bool changes;
+    Exclusive(const ivfpq_index *handle, bool may_change) : lock(handle->mu), h(handle), changes(may_change)
+    {
+        if (changes) {
+            for (auto &v : h->views) {
+                if (v) {
+                    v->flush_pending_stats();
+                }
+            }
+        }
+    }
+    ~Exclusive()
+    {
+        if (changes) {
+            (void)hipStreamSynchronize(h->impl.stream());   // views read on other streams what this call wrote
+            h->version++;
+        }
+    }
+};
+
+// One search on an IVFPQ handle: the lock shared, and a lane for as long as the search runs.
+class SearchLane {
+public:
+    explicit SearchLane(const ivfpq_index *handle) : shared_(handle->mu), h_(handle)
+    {
+        std::unique_lock<std::mutex> g(h_->lane_mu);
+        const unsigned all = (1u << (1 + ivfpq_index::kSearchViews)) - 1;
+        h_->lane_cv.wait(g, [&] { return (h_->busy & all) != all; });
+        while (h_->busy >> lane_ & 1u) {
+            lane_++;
+        }
+        if (lane_ > 0) {
+            auto &view = h_->views[lane_ - 1];
+            if (!view) {
+                const ixa::IvfpqIndex &o = h_->impl;
+                view.reset(new ixa::IvfpqIndex(o.d(), o.metric(), o.nlist(), o.M(), 8, o.config()));
+            }
+            if (h_->view_version[lane_ - 1] != h_->version) {
+                view->borrow_from(h_->impl);
+                h_->view_version[lane_ - 1] = h_->version;
+            }
+        }
+        h_->busy |= 1u << lane_;
+    }
+    ~SearchLane()
+    {
+        {
+            std::lock_guard<std::mutex> g(h_->lane_mu);
+            h_->busy &= ~(1u << lane_);
+            h_->last = &index();
+        }
+        h_->lane_cv.notify_one();
+    }
+    SearchLane(const SearchLane &) = delete;
+    SearchLane &operator=(const SearchLane &) = delete;
+    ixa::IvfpqIndex &index() const { return lane_ == 0 ? h_->impl : *h_->views[lane_ - 1]; }
+
+private:
+    std::shared_lock<std::shared_mutex> shared_;
+    const ivfpq_index *h_;
+    int lane_ = 0;
+};
+
+#define IXA_HANDLE_AS(h, may_change)                                                              \
     IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.");      \
-    std::lock_guard<std::mutex> ixa_handle_lock((h)->mu)
+    Exclusive<std::remove_cv_t<std::remove_pointer_t<decltype(h)>>> ixa_handle_lock((h), (may_change))
+#define IXA_HANDLE(h) IXA_HANDLE_AS(h, true)        // a call that may change the index
+#define IXA_HANDLE_READS(h) IXA_HANDLE_AS(h, false)  // one that only reads it (but uses its stream or workspaces)
+#define IXA_SEARCH_LANE(h)                                                                        \
+    IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.");      \
+    SearchLane ixa_lane(h)
 
 ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
 {
@@ -154,12 +246,12 @@ IXA_EXPORT int ivfpq_create(int d, int metric, int64_t nlist, int msubs, int nbi
 
 IXA_EXPORT int ivfpq_last_search_timings(const ivfpq_index_t *h, double *ms_coarse, double *ms_scan)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.last_timings(ms_coarse, ms_scan); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->last->last_timings(ms_coarse, ms_scan); });
 }
 
 IXA_EXPORT int ivfpq_write_faiss(const ivfpq_index_t *h, const char *path)
 {
-    return guarded([&] { IXA_HANDLE(h); ixa::write_faiss_ivfpq(h->impl, path); });
+    return guarded([&] { IXA_HANDLE_READS(h); ixa::write_faiss_ivfpq(h->impl, path); });
 }
 
 IXA_EXPORT int ivfpq_read_faiss(const char *path, const ivfpq_config_t *cfg, ivfpq_index_t **out)
@@ -176,7 +268,7 @@ IXA_EXPORT int ivfpq_read_faiss(const char *path, const ivfpq_config_t *cfg, ivf
 IXA_EXPORT int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int64_t *nlist, int *msubs)
 {
     return guarded([&] {
-        IXA_HANDLE(h);
+        IXA_HANDLE_READS(h);
         if (d) {
             *d = h->impl.d();
         }
@@ -195,7 +287,7 @@ IXA_EXPORT int ivfpq_get_shape(const ivfpq_index_t *h, int *d, int *metric, int6
 IXA_EXPORT int ivfpq_get_code_layout(const ivfpq_index_t *h, int *layout)
 {
     return guarded([&] {
-        IXA_HANDLE(h);
+        IXA_HANDLE_READS(h);
         IXA_REQUIRE(layout, ixa::kErrInvalidParam, "layout can not be nullptr.");
         *layout = h->impl.code_layout();
     });
@@ -220,11 +312,11 @@ IXA_EXPORT int ivfpq_set_trained(ivfpq_index_t *h, const float *centroids, const
 }
 IXA_EXPORT int ivfpq_get_trained(const ivfpq_index_t *h, float *centroids, float *codebook)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.get_trained(centroids, codebook); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->impl.get_trained(centroids, codebook); });
 }
 IXA_EXPORT int ivfpq_is_trained(const ivfpq_index_t *h, int *out)
 {
-    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.is_trained(); });
+    return guarded([&] { IXA_HANDLE_READS(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.is_trained(); });
 }
 IXA_EXPORT int ivfpq_add_with_ids(ivfpq_index_t *h, int64_t n, const float *x, const int64_t *ids)
 {
@@ -252,36 +344,36 @@ IXA_EXPORT int ivfpq_set_stage_timings(ivfpq_index_t *h, int mode)
 }
 IXA_EXPORT int ivfpq_get_nprobe(const ivfpq_index_t *h, int *out)
 {
-    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.nprobe(); });
+    return guarded([&] { IXA_HANDLE_READS(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.nprobe(); });
 }
 IXA_EXPORT int ivfpq_search(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, false); });
 }
 IXA_EXPORT int ivfpq_search_device(ivfpq_index_t *h, int64_t n, const float *x, int64_t k, float *distances,
                                    int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, true); });
 }
 IXA_EXPORT int ivfpq_assign(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.assign(n, x, out, false); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->impl.assign(n, x, out, false); });
 }
 IXA_EXPORT int ivfpq_coarse_probe(ivfpq_index_t *h, int64_t n, const float *x, int64_t *out_ids, float *out_dist)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.coarse_probe(n, x, out_ids, out_dist, false); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->impl.coarse_probe(n, x, out_ids, out_dist, false); });
 }
 IXA_EXPORT int ivfpq_encode(ivfpq_index_t *h, int64_t n, const float *x, uint8_t *codes)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.encode(n, x, codes, false); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->impl.encode(n, x, codes, false); });
 }
 IXA_EXPORT int ivfpq_list_length(const ivfpq_index_t *h, int64_t list, int64_t *out)
 {
-    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.list_length(list); });
+    return guarded([&] { IXA_HANDLE_READS(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.list_length(list); });
 }
 IXA_EXPORT int ivfpq_get_list(const ivfpq_index_t *h, int64_t list, uint8_t *codes, int64_t *ids)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.get_list(list, codes, ids); });
+    return guarded([&] { IXA_HANDLE_READS(h); h->impl.get_list(list, codes, ids); });
 }
 IXA_EXPORT int ivfpq_remove_ids(ivfpq_index_t *h, int64_t n, const int64_t *ids, int64_t *removed)
 {
@@ -335,7 +427,7 @@ IXA_EXPORT int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocate
                                  int64_t *slots_holes)
 {
     return guarded([&] {
-        IXA_HANDLE(h);
+        IXA_HANDLE_READS(h);
         int64_t a = 0, u = 0, ho = 0;
         h->impl.arena_state(&a, &u, &ho);
         if (slots_allocated) {
@@ -349,20 +441,31 @@ IXA_EXPORT int ivfpq_arena_state(const ivfpq_index_t *h, int64_t *slots_allocate
         }
     });
 }
+IXA_EXPORT int ivfpq_search_lanes(const ivfpq_index_t *h, int *out)
+{
+    return guarded([&] {
+        IXA_HANDLE_READS(h);
+        IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");
+        *out = 1;
+        for (auto &v : h->views) {
+            *out += v ? 1 : 0;
+        }
+    }, false);
+}
 IXA_EXPORT int ivfpq_reset(ivfpq_index_t *h)
 {
     return guarded([&] { IXA_HANDLE(h); h->impl.reset(); });
 }
 IXA_EXPORT int ivfpq_ntotal(const ivfpq_index_t *h, int64_t *out)
 {
-    return guarded([&] { IXA_HANDLE(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.ntotal(); });
+    return guarded([&] { IXA_HANDLE_READS(h); IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr."); *out = h->impl.ntotal(); });
 }
 IXA_EXPORT int ivfpq_last_search_stats(const ivfpq_index_t *h, ivfpq_search_stats_t *out)
 {
     return guarded([&] {
-        IXA_HANDLE(h);
+        IXA_HANDLE_READS(h);
         IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");
-        const ixa::SearchStats &s = h->impl.stats();
+        const ixa::SearchStats &s = h->last->stats();
         out->scanned_codes = s.scanned_codes;
         out->ms_coarse = s.ms_coarse;
         out->ms_scan = s.ms_scan;
@@ -548,14 +651,17 @@ IXA_EXPORT int ixa_op_topk_ivfpq_l3(const int64_t *in_labels_dev, const float *i
 IXA_EXPORT int ivfpq_search_probes_device(ivfpq_index_t *h, int64_t n, const float *x_dev, const int32_t *probes_dev,
                                           int nprobe, int64_t k, float *distances_dev, int64_t *labels_dev)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search_probes(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev); });
+    return guarded([&] {
+        IXA_SEARCH_LANE(h);
+        ixa_lane.index().search_probes(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev);
+    });
 }
 IXA_EXPORT int ivfpq_search_probes_device_noalloc(ivfpq_index_t *h, int64_t n, const float *x_dev,
                                                   const int32_t *probes_dev, int nprobe, int64_t k,
                                                   float *distances_dev, int64_t *labels_dev)
 {
     return guarded([&] {
-        IXA_HANDLE(h);
+        IXA_HANDLE_READS(h);
         h->impl.search_probes_noalloc(n, x_dev, probes_dev, nprobe, k, distances_dev, labels_dev);
     });
 }

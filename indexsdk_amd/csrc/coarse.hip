@@ -357,10 +357,7 @@ static void launch_merge_candidates_t(key_t *running, int k, ScoreFilter<S> flt,
     }
     const size_t smem = (size_t)pow2_ceil(k + flt.cap) * sizeof(key_t);
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "candidate merge of %d + %d keys exceeds LDS", k, flt.cap);
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(merge_candidates_kernel<S>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(merge_candidates_kernel<S>), smem);
     hipLaunchKernelGGL(merge_candidates_kernel<S>, dim3((unsigned)nq), dim3(256), smem, s, running, k, flt, tau,
                        overflow);
 }
@@ -998,10 +995,7 @@ static void launch_select_rows_t(const S *scores, int64_t nrows, int64_t ld, int
         return;
     }
     auto kern = active == 4 ? select_rows_kernel<S, 4> : (active == 2 ? select_rows_kernel<S, 2> : select_rows_kernel<S, 1>);
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     hipLaunchKernelGGL(kern, dim3((unsigned)nrows), dim3(256), smem, s, scores, ld, nc, ksel, cap, out_idx, col_base,
                        running, fresh);
 }
@@ -1237,10 +1231,7 @@ void launch_refine_boundary(const float *Q, int64_t nq, const float *C, int d, c
     const bool vec4 = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(Q) % 16 == 0) &&
                       (reinterpret_cast<uintptr_t>(C) % 16 == 0);
     auto kern = vec4 ? refine_boundary_kernel<true> : refine_boundary_kernel<false>;
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, running,
                        ncand, nout, cmax, err_scale, round_scale, out_ids, flag, complete ? 1 : 0);
 }
@@ -1442,10 +1433,7 @@ static void launch_fold_refine_boundary_t(const float *Q, int64_t nq, const floa
     auto kern = E == 4 ? fold_refine_boundary_kernel<VEC4, 4>
                        : (E == 8 ? fold_refine_boundary_kernel<VEC4, 8>
                                  : (E == 16 ? fold_refine_boundary_kernel<VEC4, 16> : fold_refine_boundary_kernel<VEC4, 32>));
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     hipLaunchKernelGGL(kern, dim3((unsigned)((nq + 3) / 4)), dim3(256), smem, s, Q, nq, C, d, qn, cn, metric, flt,
                        amb_cap, nout, cmax, err_scale, round_scale, out_ids, flag, row_base, raw);
 }

@@ -258,11 +258,13 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
 
 int device_cus()
 {
-    static int cus = 0;
+    static std::atomic<int> known{0};
+    int cus = known.load(std::memory_order_relaxed);
     if (cus == 0) {
         int dev = 0;
         IXA_HIP(hipGetDevice(&dev));
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        known.store(cus, std::memory_order_relaxed);
     }
     return cus;
 }
@@ -286,7 +288,7 @@ void launch_shape(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const floa
         fail(kErrInner, "resident coarse kernel: tile of %d queries does not fit LDS", QT);   // the plan never picks it
     } else {
     auto kern = resident_bf16_kernel<NHS, PF, RA, MODE>;
-    static bool configured = false;
+    static std::atomic<bool> configured{false};
     if (!configured) {
         hipFuncAttributes attr;
         IXA_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kern)));

@@ -1,6 +1,9 @@
 // Shared host-side plumbing for the MI355X IVFPQ / Flat search library: status codes, error
 // capture, RAII device buffers and the stream every kernel of an index is launched on.
 #pragma once
+#include <atomic>
+#include <mutex>
+#include <unordered_map>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -68,7 +71,26 @@ inline void sync_stream(hipStream_t s)
     IXA_HIP(hipStreamSynchronize(s));
 }
 
-// Owning device allocation.  Grows by reallocation (contents are NOT preserved by reserve()).
+// Raises a kernel's limit of dynamic LDS to at least `bytes` (every kernel starts at 48 KB).  The limit only ever
+// grows: launches from several threads never find it lowered under them, and a launch whose size is covered already
+// costs no runtime call.
+inline void require_dynamic_lds(const void *kern, size_t bytes)
+{
+    if (bytes <= 48 * 1024) {
+        return;
+    }
+    static std::mutex mu;
+    static std::unordered_map<const void *, size_t> limit;
+    std::lock_guard<std::mutex> lock(mu);
+    size_t &have = limit[kern];
+    if (bytes > have) {
+        IXA_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+        have = bytes;
+    }
+}
+
+// Owning device allocation.  Grows by reallocation (contents are NOT preserved by resize()).  borrow() makes it a
+// non-owning window onto another buffer's memory instead (a search view of an index reads the owner's data).
 template <typename T>
 class DeviceBuffer {
 public:
@@ -76,7 +98,12 @@ public:
     explicit DeviceBuffer(size_t n) { resize(n); }
     DeviceBuffer(const DeviceBuffer &) = delete;
     DeviceBuffer &operator=(const DeviceBuffer &) = delete;
-    DeviceBuffer(DeviceBuffer &&o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_) { o.p_ = nullptr; o.n_ = o.cap_ = 0; }
+    DeviceBuffer(DeviceBuffer &&o) noexcept : p_(o.p_), n_(o.n_), cap_(o.cap_), borrowed_(o.borrowed_)
+    {
+        o.p_ = nullptr;
+        o.n_ = o.cap_ = 0;
+        o.borrowed_ = false;
+    }
     DeviceBuffer &operator=(DeviceBuffer &&o) noexcept
     {
         if (this != &o) {
@@ -84,8 +111,10 @@ public:
             p_ = o.p_;
             n_ = o.n_;
             cap_ = o.cap_;
+            borrowed_ = o.borrowed_;
             o.p_ = nullptr;
             o.n_ = o.cap_ = 0;
+            o.borrowed_ = false;
         }
         return *this;
     }
@@ -105,11 +134,20 @@ public:
     }
     void release()
     {
-        if (p_) {
+        if (p_ && !borrowed_) {
             (void)hipFree(p_);
         }
         p_ = nullptr;
         n_ = cap_ = 0;
+        borrowed_ = false;
+    }
+    // This buffer becomes a window onto o's memory: valid until o reallocates or dies.
+    void borrow(const DeviceBuffer &o)
+    {
+        release();
+        p_ = o.p_;
+        n_ = cap_ = o.n_;
+        borrowed_ = p_ != nullptr;
     }
     T *data() const { return p_; }
     size_t size() const { return n_; }
@@ -133,6 +171,7 @@ public:
 private:
     T *p_ = nullptr;
     size_t n_ = 0, cap_ = 0;
+    bool borrowed_ = false;
 };
 
 // Page-locked host memory for the small copies of latency-bound paths (a copy to or from pageable memory

@@ -540,11 +540,13 @@ __global__ __launch_bounds__(kResidentWaves * 64) __attribute__((amdgpu_waves_pe
 
 int device_cus()
 {
-    static int cus = 0;
+    static std::atomic<int> known{0};
+    int cus = known.load(std::memory_order_relaxed);
     if (cus == 0) {
         int dev = 0;
         IXA_HIP(hipGetDevice(&dev));
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        known.store(cus, std::memory_order_relaxed);
     }
     return cus;
 }
@@ -557,7 +559,7 @@ void launch_resident(const int8_t *Q, int64_t nq, const int8_t *tiled, const int
     constexpr size_t smem = (size_t)QT * NHS * 32 + (FILTER ? kResidentExtraLds : 0);
     static_assert(smem <= 160 * 1024, "the query tile must fit the LDS of a CU");
     auto kern = resident_i8_kernel<NHS, PF, RA, FILTER>;
-    static bool configured = false;   // per instantiation
+    static std::atomic<bool> configured{false};   // per instantiation
     if (!configured) {
         hipFuncAttributes attr;
         IXA_HIP(hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kern)));

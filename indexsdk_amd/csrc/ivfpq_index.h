@@ -84,6 +84,14 @@ public:
     void set_stage_timings(int mode) { cfg_.stage_timings = mode; }   // as IvfpqConfig::stage_timings, from the next search on
     int code_layout() const { return layout_; }
     hipStream_t stream() const { return stream_; }
+    const IvfpqConfig &config() const { return cfg_; }
+    // Makes this index a search view of `owner` (same shape and configuration): it reads the owner's trained state
+    // and lists in place and searches them on its own stream with its own workspaces, so that searches on the owner
+    // and on its views run side by side.  The owner must not change (train, add, remove, reset, set_nprobe ...)
+    // while a view is searching, and a view borrows again after every such change before its next search; a view
+    // serves searches only.
+    void borrow_from(const IvfpqIndex &owner);
+    void flush_pending_stats() { flush_stats(); }   // before the lists the statistics refer to change or go away
 
     // x may live on the host or on the device (on_device says which).
     void train(int64_t n, const float *x, bool on_device);

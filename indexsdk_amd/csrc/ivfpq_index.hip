@@ -505,6 +505,38 @@ IvfpqIndex::~IvfpqIndex()
     }
 }
 
+void IvfpqIndex::borrow_from(const IvfpqIndex &o)
+{
+    IXA_REQUIRE(d_ == o.d_ && M_ == o.M_ && metric_ == o.metric_ && nlist_ == o.nlist_, kErrInvalidParam,
+                "a search view needs the shape of the index it borrows from");
+    stats_pending_ = false;   // whatever they referred to is gone
+    cfg_ = o.cfg_;
+    layout_ = o.layout_;
+    nprobe_ = o.nprobe_;
+    trained_ = o.trained_;
+    ntotal_ = o.ntotal_;
+    max_list_len_ = o.max_list_len_;
+    cmax_ = o.cmax_;
+    dp_ = o.dp_;
+    centroids_.borrow(o.centroids_);
+    cnorm_.borrow(o.cnorm_);
+    codebook_.borrow(o.codebook_);
+    cbnorm_.borrow(o.cbnorm_);
+    centroids_split_.borrow(o.centroids_split_);
+    centroids_tiled_.borrow(o.centroids_tiled_);
+    cnorm_pad_.borrow(o.cnorm_pad_);
+    codes_.borrow(o.codes_);
+    ids_.borrow(o.ids_);
+    list_off_dev_.borrow(o.list_off_dev_);
+    list_len_dev_.borrow(o.list_len_dev_);
+    list_off_ = o.list_off_;
+    list_len_ = o.list_len_;
+    list_cap_ = o.list_cap_;
+    arena_slots_ = o.arena_slots_;
+    arena_used_ = o.arena_used_;
+    hole_slots_ = o.hole_slots_;
+}
+
 void IvfpqIndex::set_nprobe(int nprobe)
 {
     flush_stats();

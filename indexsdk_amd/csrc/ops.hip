@@ -335,10 +335,7 @@ void op_ivfpq_search_distance_topk(const float *lut, int64_t batch, int M, const
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam,
                 "AscendcIvfpqSearchDistanceL2: %zu bytes of LDS needed (msubs %d, k %d, %d blocks); the limit is 163840", smem,
                 M, k, nblk);
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(op_ivfpq_scan_topk_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(op_ivfpq_scan_topk_kernel), smem);
     hipLaunchKernelGGL(op_ivfpq_scan_topk_kernel, dim3((unsigned)batch), dim3(kOpScanWaves * 64), smem, s, p);
     IXA_HIP(hipGetLastError());
 }
@@ -355,10 +352,7 @@ void op_topk_ivfpq_l3(const int64_t *in_labels, const float *in_values, int T, i
     }
     const int n2 = pow2_ceil(T * K);
     const size_t smem = (size_t)n2 * sizeof(key_t);
-    if (smem > 48 * 1024) {
-        IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(op_topk_ivfpq_l3_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    }
+    require_dynamic_lds(reinterpret_cast<const void *>(op_topk_ivfpq_l3_kernel), smem);
     hipLaunchKernelGGL(op_topk_ivfpq_l3_kernel, dim3((unsigned)batch), dim3(256), smem, s, in_labels, in_values, T, batch,
                        K, k, asc ? 1 : 0, n2, out_values, out_labels);
     IXA_HIP(hipGetLastError());

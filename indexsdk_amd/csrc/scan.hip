@@ -1081,9 +1081,9 @@ void launch_order_by_work(const int32_t *probes, int64_t nq, int nprobe, const i
 
 // The row-layout lookups address the LUT from LDS address 0: true while the kernel declares no static LDS, which
 // is asked of the loaded code object once per kernel and refused loudly otherwise.
-static void require_no_static_lds(const void *kern, bool &checked)
+static void require_no_static_lds(const void *kern, std::atomic<bool> &checked)
 {
-    if (checked) {
+    if (checked.load(std::memory_order_acquire)) {
         return;
     }
     hipFuncAttributes attr{};
@@ -1091,45 +1091,33 @@ static void require_no_static_lds(const void *kern, bool &checked)
     IXA_REQUIRE(attr.sharedSizeBytes == 0, kErrInner,
                 "the scan kernel has %zu bytes of static LDS: its LUT would not start at LDS address 0",
                 (size_t)attr.sharedSizeBytes);
-    checked = true;
+    checked.store(true, std::memory_order_release);
 }
 
 template <int MT, typename LutT, int LAYOUT>
 static void launch_one(const ScanParams &p, int64_t nq, size_t smem, hipStream_t s)
 {
     const int64_t slots = p.xcd_chunks ? (nq + 7) / 8 * 8 : nq;
-    static bool lds_checked[4] = {false, false, false, false};
+    static std::atomic<bool> lds_checked[4] = {{false}, {false}, {false}, {false}};
     if (p.shared_pool && p.waves == 16) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 16, true>;
         require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[0]);
-        if (smem > 48 * 1024) {
-            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        }
+        require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(1024), smem, s, p);
     } else if (p.shared_pool) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, true>;
         require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[1]);
-        if (smem > 48 * 1024) {
-            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        }
+        require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else if (p.waves == 8) {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 8, false>;
         require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[2]);
-        if (smem > 48 * 1024) {
-            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        }
+        require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(512), smem, s, p);
     } else {
         auto kern = ivfpq_scan_kernel<MT, LutT, LAYOUT, 4, false>;
         require_no_static_lds(reinterpret_cast<const void *>(kern), lds_checked[3]);
-        if (smem > 48 * 1024) {
-            IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        }
+        require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
         hipLaunchKernelGGL(kern, dim3((unsigned)(slots * p.nsplit)), dim3(256), smem, s, p);
     }
 }

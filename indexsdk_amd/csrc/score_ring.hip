@@ -660,11 +660,13 @@ bool launch_ring(const typename Tr::T *Q, int64_t nq, const typename Tr::T *B, i
     if (rt_m * rt_n >= ((int64_t)1 << 31) || rt_m * ((rt_n + 7) / 8) * (d / Tr::kElemsPerStep) >= ((int64_t)1 << 30)) {
         return false;
     }
-    static int cus = 0;
+    static std::atomic<int> known{0};
+    int cus = known.load(std::memory_order_relaxed);
     if (cus == 0) {
         int dev = 0;
         IXA_HIP(hipGetDevice(&dev));
         IXA_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        known.store(cus, std::memory_order_relaxed);
     }
     const unsigned grid = (unsigned)((cus + 7) / 8 * 8);   // one persistent workgroup per CU
     if (mode == 2 || mode == 3) {
