@@ -136,6 +136,7 @@ private:
     void check_trained() const;
     void search_page(int64_t n, const float *x, int64_t k, float *dist, int64_t *labels, bool on_device);
     void upload_trained(const float *centroids, const float *codebook);
+    void derive_from_centroids();
     // best `nout` lists of every row of device matrix x (canonical arithmetic), device outputs
     void coarse_select(const float *x_dev, int64_t n, int nout, int select_metric, int32_t *out_ids,
                        float *out_dist, bool set_only = false, bool defer_check = false);

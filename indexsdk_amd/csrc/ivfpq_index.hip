@@ -328,6 +328,182 @@ __global__ __launch_bounds__(256) void segment_mean_kernel(const float *__restri
     }
 }
 
+// ---- members of every cluster in ascending sample order, built on the device ---------------------------------
+// (a stable counting sort of the samples by their cluster: counts, segment starts, members dropped into their
+// segment in whatever order the hardware runs them, every segment then sorted ascending)
+
+__global__ __launch_bounds__(256) void count_members_kernel(const int32_t *__restrict__ asg, int64_t ns,
+                                                            unsigned long long *__restrict__ cnt)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < ns) {
+        atomicAdd(&cnt[asg[i]], 1ull);
+    }
+}
+
+// seg[c] = number of members of the clusters before c (seg[k] = all of them); cursor[c] = seg[c].  One workgroup.
+__global__ __launch_bounds__(1024) void segment_starts_kernel(const unsigned long long *__restrict__ cnt, int64_t k,
+                                                              int64_t *__restrict__ seg,
+                                                              unsigned long long *__restrict__ cursor)
+{
+    __shared__ unsigned long long part[1024];
+    const int64_t per = (k + 1023) / 1024, b = (int64_t)threadIdx.x * per, e = b + per < k ? b + per : k;
+    unsigned long long sum = 0;
+    for (int64_t c = b; c < e; c++) {
+        sum += cnt[c];
+    }
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const unsigned long long add = threadIdx.x >= (unsigned)off ? part[threadIdx.x - off] : 0;
+        __syncthreads();
+        part[threadIdx.x] += add;
+        __syncthreads();
+    }
+    unsigned long long run = part[threadIdx.x] - sum;
+    for (int64_t c = b; c < e; c++) {
+        seg[c] = (int64_t)run;
+        cursor[c] = run;
+        run += cnt[c];
+    }
+    if (threadIdx.x == 1023) {
+        seg[k] = (int64_t)part[1023];
+    }
+}
+
+__global__ __launch_bounds__(256) void place_members_kernel(const int32_t *__restrict__ asg, int64_t ns,
+                                                            unsigned long long *__restrict__ cursor,
+                                                            int64_t *__restrict__ order)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < ns) {
+        order[atomicAdd(&cursor[asg[i]], 1ull)] = i;
+    }
+}
+
+// One workgroup sorts the members of one segment ascending, in place: a bitonic network whose every exchange puts
+// the smaller value at the lower position, so positions beyond the segment's end count as +infinity and are never
+// touched; segments of any length (the usual one holds a few hundred members and stays in the caches).
+__global__ __launch_bounds__(256) void sort_segments_kernel(int64_t *__restrict__ order, const int64_t *__restrict__ seg)
+{
+    int64_t *a = order + seg[blockIdx.x];
+    const int64_t len = seg[blockIdx.x + 1] - seg[blockIdx.x];
+    if (len < 2) {
+        return;
+    }
+    int64_t n2 = 2;
+    while (n2 < len) {
+        n2 <<= 1;
+    }
+    for (int64_t size = 2; size <= n2; size <<= 1) {
+        for (int64_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int64_t t = threadIdx.x; t < n2 / 2; t += blockDim.x) {
+                // pair t of this step: the first step of a merge mirrors inside blocks of `size`, the others pair
+                // positions `stride` apart
+                const int64_t lo = (t / stride) * (2 * stride) + (t % stride);
+                const int64_t hi = stride == size >> 1 ? (t / stride) * (2 * stride) + (2 * stride - 1 - t % stride)
+                                                       : lo + stride;
+                if (hi < len) {
+                    const int64_t x = a[lo], y = a[hi];
+                    if (x > y) {
+                        a[lo] = y;
+                        a[hi] = x;
+                    }
+                }
+            }
+            __threadfence_block();
+            __syncthreads();
+        }
+    }
+}
+
+// Re-seeds empty clusters by splitting the most populated one (symmetric perturbation), in ascending order of the
+// empty clusters, each split seeing the counts the earlier ones left.  One workgroup.
+__global__ __launch_bounds__(1024) void split_empty_kernel(float *__restrict__ cent, unsigned long long *__restrict__ cnt,
+                                                           int64_t k, int dim)
+{
+    __shared__ long long s_val[1024], s_idx[1024];
+    const int tid = threadIdx.x;
+    long long last = -1;
+    while (true) {
+        long long mine = INT64_MAX;
+        for (long long c = last + 1 + tid; c < k; c += 1024) {
+            if (cnt[c] == 0) {
+                mine = c;
+                break;
+            }
+        }
+        s_idx[tid] = mine;
+        __syncthreads();
+        for (int off = 512; off > 0; off >>= 1) {
+            if (tid < off && s_idx[tid + off] < s_idx[tid]) {
+                s_idx[tid] = s_idx[tid + off];
+            }
+            __syncthreads();
+        }
+        const long long empty = s_idx[0];
+        __syncthreads();
+        if (empty == INT64_MAX) {
+            return;
+        }
+        long long best = -1, at = INT64_MAX;   // the largest count, the first cluster that has it
+        for (long long c = tid; c < k; c += 1024) {
+            const long long v = (long long)cnt[c];
+            if (v > best) {
+                best = v;
+                at = c;
+            }
+        }
+        s_val[tid] = best;
+        s_idx[tid] = at;
+        __syncthreads();
+        for (int off = 512; off > 0; off >>= 1) {
+            if (tid < off) {
+                const long long v = s_val[tid + off], i = s_idx[tid + off];
+                if (v > s_val[tid] || (v == s_val[tid] && i < s_idx[tid])) {
+                    s_val[tid] = v;
+                    s_idx[tid] = i;
+                }
+            }
+            __syncthreads();
+        }
+        const long long big = s_idx[0];
+        __syncthreads();
+        for (int t = tid; t < dim; t += 1024) {
+            const float v = cent[big * dim + t];
+            const float eps = (t & 1) ? 1.0f / 1024 : -1.0f / 1024;
+            cent[empty * dim + t] = v * (1.0f + eps);
+            cent[big * dim + t] = v * (1.0f - eps);
+        }
+        if (tid == 0) {
+            cnt[empty] = cnt[big] / 2;
+            cnt[big] -= cnt[empty];
+        }
+        __threadfence_block();
+        __syncthreads();
+        last = empty;
+    }
+}
+
+// Rows scaled to unit length: the squared length summed in float64 from the first component to the last.
+__global__ __launch_bounds__(256) void normalise_rows_kernel(float *__restrict__ cent, int64_t k, int dim)
+{
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= k) {
+        return;
+    }
+    double nn = 0;
+    for (int t = 0; t < dim; t++) {
+        nn += (double)cent[c * dim + t] * cent[c * dim + t];
+    }
+    nn = sqrt(nn);
+    if (nn > 0) {
+        for (int t = 0; t < dim; t++) {
+            cent[c * dim + t] = (float)(cent[c * dim + t] / nn);
+        }
+    }
+}
+
 // Sub-quantizer update of PQ training: acc[m][k][t] = sum in float64, IN SAMPLE ORDER, of x[i][m*dsub + t]
 // over the samples i whose code for sub-quantizer m is k; cnt[m][k] = their number.  One workgroup
 // per sub-quantizer, thread k owns codeword k: tiles of 256 samples (their sub-vectors and codes) are
@@ -560,38 +736,45 @@ void IvfpqIndex::sync_list_tables()
     sync_stream(stream_);
 }
 
+// Everything the search keeps beside the centroids themselves (norms, bf16 splits, the splits in matrix-core order),
+// from centroids_ as it stands in device memory.
+void IvfpqIndex::derive_from_centroids()
+{
+    cnorm_.resize((size_t)nlist_);
+    launch_sqnorm_rows(centroids_.data(), nlist_, d_, cnorm_.data(), stream_);
+    dp_ = (int)round_up(d_, 32);
+    centroids_split_.resize((size_t)nlist_ * 3 * dp_);
+    launch_split_bf16x3(centroids_.data(), nlist_, d_, dp_, true, centroids_split_.data(), stream_);
+    std::vector<float> cn((size_t)nlist_);
+    cnorm_.download(cn.data(), cn.size(), stream_);
+    cmax_ = std::sqrt(*std::max_element(cn.begin(), cn.end()));
+    // The split centroids a second time, in matrix-core order, for the resident-query score kernel
+    // (coarse_resident.hip), with their norms padded to whole tiles: +inf behind the last centroid, so that a
+    // padding row never passes a bound; for inner product the kernel wants zeros in their place.
+    centroids_tiled_.release();
+    cnorm_pad_.release();
+    if (resident_coarse_serves(3 * dp_)) {
+        const int row_bytes = 3 * dp_ * 2;
+        const int64_t padded = round_up(nlist_, kI8TileRows);
+        centroids_tiled_.resize(i8_tiled_bytes(nlist_, row_bytes));
+        IXA_HIP(hipMemsetAsync(centroids_tiled_.data(), 0, centroids_tiled_.bytes(), stream_));
+        launch_i8_tile_rows(reinterpret_cast<const int8_t *>(centroids_split_.data()), nlist_, row_bytes,
+                            reinterpret_cast<int8_t *>(centroids_tiled_.data()), 0, stream_);
+        std::vector<float> pad((size_t)2 * padded, std::numeric_limits<float>::infinity());
+        std::copy(cn.begin(), cn.end(), pad.begin());                       // L2: the norms
+        std::fill(pad.begin() + padded, pad.begin() + padded + nlist_, 0.f);   // inner product: zeros
+        cnorm_pad_.upload(pad.data(), pad.size(), stream_);
+        sync_stream(stream_);   // `pad` is the source of an asynchronous copy
+    }
+}
+
 // Centroid and codeword norms are produced on the device in the same left-to-right fp32 order the
 // reference uses on the host (FR/ascend/impl/AscendIndexIVFPQImpl.cpp:1114-1126).
 void IvfpqIndex::upload_trained(const float *centroids, const float *codebook)
 {
     if (centroids) {
         centroids_.upload(centroids, (size_t)nlist_ * d_, stream_);
-        cnorm_.resize((size_t)nlist_);
-        launch_sqnorm_rows(centroids_.data(), nlist_, d_, cnorm_.data(), stream_);
-        dp_ = (int)round_up(d_, 32);
-        centroids_split_.resize((size_t)nlist_ * 3 * dp_);
-        launch_split_bf16x3(centroids_.data(), nlist_, d_, dp_, true, centroids_split_.data(), stream_);
-        std::vector<float> cn((size_t)nlist_);
-        cnorm_.download(cn.data(), cn.size(), stream_);
-        cmax_ = std::sqrt(*std::max_element(cn.begin(), cn.end()));
-        // The split centroids a second time, in matrix-core order, for the resident-query score kernel
-        // (coarse_resident.hip), with their norms padded to whole tiles: +inf behind the last centroid, so that a
-        // padding row never passes a bound; for inner product the kernel wants zeros in their place.
-        centroids_tiled_.release();
-        cnorm_pad_.release();
-        if (resident_coarse_serves(3 * dp_)) {
-            const int row_bytes = 3 * dp_ * 2;
-            const int64_t padded = round_up(nlist_, kI8TileRows);
-            centroids_tiled_.resize(i8_tiled_bytes(nlist_, row_bytes));
-            IXA_HIP(hipMemsetAsync(centroids_tiled_.data(), 0, centroids_tiled_.bytes(), stream_));
-            launch_i8_tile_rows(reinterpret_cast<const int8_t *>(centroids_split_.data()), nlist_, row_bytes,
-                                reinterpret_cast<int8_t *>(centroids_tiled_.data()), 0, stream_);
-            std::vector<float> pad((size_t)2 * padded, std::numeric_limits<float>::infinity());
-            std::copy(cn.begin(), cn.end(), pad.begin());                       // L2: the norms
-            std::fill(pad.begin() + padded, pad.begin() + padded + nlist_, 0.f);   // inner product: zeros
-            cnorm_pad_.upload(pad.data(), pad.size(), stream_);
-            sync_stream(stream_);   // `pad` is the source of an asynchronous copy
-        }
+        derive_from_centroids();
     }
     if (codebook) {
         codebook_.upload(codebook, (size_t)M_ * 256 * dsub_, stream_);
@@ -1773,54 +1956,44 @@ void IvfpqIndex::kmeans_coarse(const float *sample_dev, int64_t ns)
     std::iota(pick.begin(), pick.end(), 0);
     std::mt19937_64 gen(cfg_.seed + 1);
     std::shuffle(pick.begin(), pick.end(), gen);
-    // the first centroids are sample rows: gathered on the device, only nlist rows come to the host
-    std::vector<float> cent((size_t)nlist_ * d_);
+    // The first centroids are sample rows, gathered on the device.  From here on an iteration moves nothing of the
+    // sample's size between host and device: assignments, the members of every cluster in sample order, the means
+    // (float64 sums in exactly that order, one workgroup per centroid), the re-seeding of empty clusters and the
+    // normalisation all stay in device memory (only the nlist norms come to the host, for the largest of them).
+    centroids_.resize((size_t)nlist_ * d_);
     {
         DeviceBuffer<int64_t> pick_dev;
-        DeviceBuffer<float> rows((size_t)nlist_ * d_);
         pick_dev.upload(pick.data(), (size_t)nlist_, stream_);
         hipLaunchKernelGGL(gather_rows_kernel, dim3(blocks_for(nlist_ * d_)), dim3(256), 0, stream_, sample_dev,
-                           pick_dev.data(), nlist_, d_, rows.data());
-        rows.download(cent.data(), cent.size(), stream_);
+                           pick_dev.data(), nlist_, d_, centroids_.data());
+        sync_stream(stream_);   // pick_dev is freed on leaving this block
     }
-    struct {
-        const float *p;
-        const float *data() const { return p; }
-    } xs{sample_dev};
     DeviceBuffer<int32_t> asg((size_t)ns);
-    std::vector<int32_t> h_asg((size_t)ns);
-    std::vector<int64_t> cnt((size_t)nlist_), seg((size_t)nlist_ + 1), order((size_t)ns);
-    DeviceBuffer<int64_t> order_dev, seg_dev;
-    DeviceBuffer<float> mean_dev((size_t)nlist_ * d_);
+    DeviceBuffer<unsigned long long> cnt((size_t)nlist_), cursor((size_t)nlist_);
+    DeviceBuffer<int64_t> order((size_t)ns), seg((size_t)nlist_ + 1);
+    DeviceBuffer<float> mean((size_t)nlist_ * d_);
+    const bool spherical = cfg_.spherical < 0 ? metric_ == kMetricInnerProduct : cfg_.spherical != 0;
     for (int it = 0; it < cfg_.niter; it++) {
-        upload_trained(cent.data(), nullptr);
-        coarse_select(xs.data(), ns, 1, kMetricL2, asg.data(), nullptr);
-        asg.download(h_asg.data(), (size_t)ns, stream_);
-        // members of every cluster in sample order (stable counting sort on the host); the means are
-        // then float64 sums in exactly that order, one workgroup per centroid on the device
-        std::fill(cnt.begin(), cnt.end(), 0);
-        for (int64_t i = 0; i < ns; i++) {
-            cnt[(size_t)h_asg[(size_t)i]]++;
-        }
-        seg[0] = 0;
-        for (int64_t c = 0; c < nlist_; c++) {
-            seg[(size_t)c + 1] = seg[(size_t)c] + cnt[(size_t)c];
-        }
-        std::vector<int64_t> fill(seg.begin(), seg.end() - 1);
-        for (int64_t i = 0; i < ns; i++) {
-            order[(size_t)fill[(size_t)h_asg[(size_t)i]]++] = i;
-        }
-        order_dev.upload(order.data(), order.size(), stream_);
-        seg_dev.upload(seg.data(), seg.size(), stream_);
+        derive_from_centroids();
+        coarse_select(sample_dev, ns, 1, kMetricL2, asg.data(), nullptr);
+        IXA_HIP(hipMemsetAsync(cnt.data(), 0, cnt.bytes(), stream_));
+        hipLaunchKernelGGL(count_members_kernel, dim3(blocks_for(ns)), dim3(256), 0, stream_, asg.data(), ns, cnt.data());
+        hipLaunchKernelGGL(segment_starts_kernel, dim3(1), dim3(1024), 0, stream_, cnt.data(), nlist_, seg.data(),
+                           cursor.data());
+        hipLaunchKernelGGL(place_members_kernel, dim3(blocks_for(ns)), dim3(256), 0, stream_, asg.data(), ns,
+                           cursor.data(), order.data());
+        hipLaunchKernelGGL(sort_segments_kernel, dim3((unsigned)nlist_), dim3(256), 0, stream_, order.data(), seg.data());
         hipLaunchKernelGGL(segment_mean_kernel, dim3((unsigned)nlist_), dim3(d_ <= 64 ? 64 : (d_ <= 128 ? 128 : 256)), 0,
-                           stream_, xs.data(), d_, order_dev.data(), seg_dev.data(), centroids_.data(), mean_dev.data());
-        mean_dev.download(cent.data(), cent.size(), stream_);
-        split_empty(cent, cnt, nlist_, d_);
-        if (cfg_.spherical < 0 ? metric_ == kMetricInnerProduct : cfg_.spherical != 0) {
-            normalise_rows(cent, nlist_, d_);
+                           stream_, sample_dev, d_, order.data(), seg.data(), centroids_.data(), mean.data());
+        hipLaunchKernelGGL(split_empty_kernel, dim3(1), dim3(1024), 0, stream_, mean.data(), cnt.data(), nlist_, d_);
+        if (spherical) {
+            hipLaunchKernelGGL(normalise_rows_kernel, dim3(blocks_for(nlist_)), dim3(256), 0, stream_, mean.data(), nlist_,
+                               d_);
         }
+        IXA_HIP(hipMemcpyAsync(centroids_.data(), mean.data(), mean.bytes(), hipMemcpyDeviceToDevice, stream_));
     }
-    upload_trained(cent.data(), nullptr);
+    derive_from_centroids();
+    sync_stream(stream_);
 }
 
 void IvfpqIndex::kmeans_pq(const float *sample_dev, int64_t ns)

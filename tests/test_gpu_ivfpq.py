@@ -900,15 +900,17 @@ def test_search_in_query_pages_equals_one_batch(ix, oracle):
     assert_topk_parity(oracle, ref, q, Dp, Ip, Dr, Ir, TOL_FP32)
 
 
-@pytest.mark.parametrize("spherical,metric_name", [(0, "L2"), (1, "L2"), (-1, "IP")])
-def test_coarse_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, spherical, metric_name):
+@pytest.mark.parametrize("spherical,metric_name,nlist,n", [(0, "L2", 96, 5000), (1, "L2", 96, 5000), (-1, "IP", 96, 5000),
+                                                           (0, "L2", 12, 40000)])
+def test_coarse_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, spherical, metric_name, nlist, n):
     """Centroids after n + 1 iterations = one Lloyd update of the centroids after n: nearest-centroid
     assignment under L2 (the add path's rule), float64 sums in sample order for the means, a cluster without
     members re-seeded by splitting the most populated one (its centroid times 1 -+ 1/1024, the sign
     alternating over the components, members shared out evenly), rows normalised when spherical (which
-    inner product switches on by default).  The data leave some of the 96 clusters empty."""
+    inner product switches on by default).  The data leave some of the clusters empty; the last case has clusters
+    of several thousand members (the member lists are sorted on the device, whatever their length)."""
     metric = ix.METRIC_L2 if metric_name == "L2" else ix.METRIC_INNER_PRODUCT
-    d, nlist, n = 32, 96, 5000
+    d = 32
     rng = np.random.default_rng(17 + spherical)
     centres = rng.standard_normal((6, d)).astype(np.float32) * 4
     x = (centres[rng.integers(0, 6, n)] + 0.05 * rng.standard_normal((n, d))).astype(np.float32)
