@@ -28,7 +28,7 @@ def log(msg):
 
 PROFILES = os.path.join(ROOT, "profiles")
 SCAN_SOURCES = ("scan.hip", "scan.h", "topk.h")
-FLAT_I8_SOURCES = ("flat_i8.hip", "flat_i8.h")
+FLAT_I8_SOURCES = ("flat_i8.hip", "flat_i8.h", "resident_tile.h")
 
 
 def source_hash(names):
@@ -399,7 +399,8 @@ def run_ivfpq(name, args, torch, ix, _capi, lib, steps, warmup, min_seconds, hea
                                f"{'unit-norm ' if unit else ''}mixture sigma {sigma}"
                                f"{' Zipf(%s) sizes' % w['zipf'] if w.get('zipf') else ''}, nlist={nlist}, M={M}x8bit, "
                                f"nq={nq}, nprobe={nprobe}, k={k}, {'fp16' if w['lut_fp16'] else 'fp32'} LUT",
-                   "code_layout": layout_name, "ntrain": int(ntrain), "kmeans_iters": args.niter},
+                   "code_layout": layout_name, "scan_order": {2: "locality", 1: "heaviest first"}.get(int(stats.get("ordered", 0)), "input"),
+                   "ntrain": int(ntrain), "kmeans_iters": args.niter},
         "adc_scan_GBps": achieved, "adc_scan_pct_hbm_peak": 100.0 * achieved / HBM_PEAK_GBPS,
         "ms_coarse": float(np.mean(coarse_ms)), "ms_scan": scan_ms_avg, "scanned_codes_per_step": stats["scanned_codes"],
         "roofline": roofline, "sustained": sustained,
