@@ -45,6 +45,10 @@ constexpr int kRingTM = 256, kRingTN = 256, kRingRows = kRingTM + kRingTN;
 constexpr int kRingStageBytes = kRingRows * 64;
 constexpr int kRingStages = 3;
 constexpr int kRingAuxBytes = 1280;   // per-wave staging of a filtered epilogue's operands
+// The ring lies at the bottom of LDS and the epilogue staging right above it: every destination of a global-to-LDS load
+// stays below 128 KB (a variant that put such destinations higher ended in a memory fault whose cause was never found).
+static_assert(kRingStages * kRingStageBytes + kRingWaves * kRingAuxBytes <= 128 * 1024,
+              "global-to-LDS destinations must stay below 128 KB");
 constexpr int kRingLoadsPerWave = kRingRows / 16 / kRingWaves;  // wave-wide 1 KB loads per stage and wavefront
 
 // Operand fragments of one half-step: 4 query blocks and 2 base blocks of 32 rows, 16 bytes per lane.
@@ -639,8 +643,7 @@ void launch_ring_mode(const typename Tr::T *Q, int64_t nq, const typename Tr::T 
 {
     const size_t smem = (size_t)kRingStages * kRingStageBytes + (MODE != 0 ? kRingWaves * kRingAuxBytes : 0);
     auto kern = score_ring_kernel<Tr, MODE>;
-    IXA_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)smem));
+    require_dynamic_lds(reinterpret_cast<const void *>(kern), smem);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingWaves * 64), smem, s, Q, nq, B, nb, d, qn, bn, metric, out, ldo,
                        (int)rt_m, (int)rt_n, flt);
 }

@@ -175,7 +175,7 @@ def test_scan_lds_plan_keeps_every_region_inside_the_allocation(capi):
             if M == 48 and not lut_fp16:
                 layouts.append(2)
             for layout in layouts:
-                for k in (1, 10, 100, 129, 320, 1000, 1024, 2048):
+                for k in (1, 10, 100, 128, 129, 160, 256, 300, 320, 384, 385, 1000, 1024, 1408, 1409, 2048):
                     for nprobe, nsplit in ((1, 1), (16, 1), (64, 8), (256, 1), (2048, 1), (2048, 8), (100, 3)):
                         for waves, shared in ((0, 0), (4, 0), (8, 0), (8, 1), (16, 1)):
                             d = M * 4
