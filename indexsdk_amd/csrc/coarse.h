@@ -49,14 +49,15 @@ bool launch_score_ring_bf16(const uint16_t *Q, int64_t nq, const uint16_t *B, in
 // The same two launches with the query tile resident in LDS and the split centroids read from matrix-core order
 // (coarse_resident.hip): Bt = the base-side split rows tiled as flat_i8.h describes (rows of 2 d3 bytes, whole tiles of
 // 256 rows, zero rows behind the last), cn_padded = |c|^2 per row (zeros for inner product) padded to whole tiles with
-// +inf.  The records hold DOT PRODUCTS, not scores: the folds below take them with raw = true.  test_scratch: nq
-// floats.  Return false (nothing launched) for split rows they have no instance for.
+// +inf.  The records hold DOT PRODUCTS, not scores: the folds below take them with raw = true.  test: the per-row
+// values of record_test_value (launch_tau_from_minima writes them).  Return false (nothing launched) for split rows
+// they have no instance for.
 bool resident_coarse_serves(int d3);
 bool launch_resident_bf16_minima(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, int64_t nb, int d3, const float *qn,
                                  const float *cn_padded, int metric, float *out, int64_t ldo, hipStream_t s);
 bool launch_resident_bf16_records(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, int64_t nb, int d3, const float *qn,
-                                  const float *cn_padded, int metric, float cmax, float *test_scratch,
-                                  ScoreFilter<float> flt, hipStream_t s);
+                                  const float *cn_padded, int metric, const float *test, ScoreFilter<float> flt,
+                                  hipStream_t s);
 
 // Record mode of the bf16 ring kernel: nothing is stored; every run of four consecutive base rows (first
 // row a multiple of four) whose smallest score is at or below flt.tau[row] is appended to the row's
@@ -71,7 +72,31 @@ bool launch_score_ring_bf16_records(const uint16_t *Q, int64_t nq, const uint16_
 bool launch_score_ring_bf16_minima(const uint16_t *Q, int64_t nq, const uint16_t *B, int64_t nb, int d, const float *qn,
                                    const float *bn, int metric, float *out, int64_t ldo, hipStream_t s);
 // tau[row] = the rank-th smallest (1-based) of gm[row * G .. + G); G <= 512.
-void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s);
+// With `test`, test->out[row] also receives the value the resident-query record launch compares against
+// (record_test_value below), so that launch needs no kernel of its own in front of it.
+//   A run is recorded when some u = g - |c|^2 / 2 of its four reaches the test value.
+//   L2: score v = fl(fl(fl(|q|^2 + |c|^2) - g) - g) <= tau.  v differs from |q|^2 + |c|^2 - 2 g by at most three
+//   roundings of numbers no larger than |q|^2 + |c|^2 + 2 |g| <= 2 (|q|^2 + |c|^2): 6 x 2^-24 (|q|^2 + |c|^2); u differs
+//   from g - |c|^2 / 2 by one rounding, at most 2^-24 (|q|^2 + |c|^2).  So v <= tau implies
+//   u >= (|q|^2 - tau) / 2 - 4 x 2^-24 (|q|^2 + |c|^2); the test value lies another factor of two below that, with
+//   |c| <= cmax, and below its own rounding.
+//   Inner product: v = -g <= tau  <=>  g >= -tau, and u = g exactly (the norms handed to the kernel are zero).
+__host__ __device__ inline float record_test_value(float qn, float tau, float cmax, bool l2)
+{
+    if (l2) {
+        const float mag = qn + cmax * cmax + (tau < 0.f ? -tau : tau);
+        return 0.5f * (qn - tau) - 4.8e-7f * mag;   // 2^-21 = 4.77e-7
+    }
+    return -tau - 4.8e-7f * (tau < 0.f ? -tau : tau);
+}
+struct RecordTest {
+    const float *qn;   // |q|^2 per row
+    float cmax;        // largest centroid norm
+    int metric;
+    float *out;
+};
+void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s,
+                            const RecordTest *test = nullptr);
 
 // Largest k of launch_fold_records.
 constexpr int kFoldMaxK = 384;
@@ -98,6 +123,8 @@ void launch_fold_refine_boundary(const float *Q, int64_t nq, const float *C, int
 // out[row] = [hi | hi | lo] (query side) or [hi | lo | hi] (base side) of x[row], each segment
 // zero-padded from d to dp elements of bf16 (stored as uint16_t); out has n * 3 * dp elements.
 void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s);
+// launch_sqnorm_rows(x -> norms) and the query-side launch_split_bf16x3(x -> split) in one launch
+void launch_sqnorm_and_split_bf16x3(const float *x, int64_t n, int d, int dp, float *norms, uint16_t *split, hipStream_t s);
 
 // Sets *flag = 1 if some query's approximate candidate list (running[nq][ncand], ascending keys) is
 // not provably a superset of its best nout centroids; see score_ring.hip.

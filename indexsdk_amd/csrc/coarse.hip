@@ -39,12 +39,12 @@ __global__ __launch_bounds__(256) void sqnorm_rows_kernel(const float *__restric
 // them at a time (four 128-bit loads per lane, 256 contiguous bytes per row), transpose the chunk
 // through LDS, and lanes 0..15 each add their own row's 64 squares in column order; the next chunk's
 // loads are in flight meanwhile.  The order of additions per row is unchanged.
-__global__ __launch_bounds__(256) void sqnorm_rows_tiled_kernel(const float *__restrict__ x, int64_t n, int d,
-                                                                float *__restrict__ out)
+__device__ __forceinline__ void sqnorm_rows_tiled_block(const float *__restrict__ x, int64_t n, int d,
+                                                        float *__restrict__ out, int64_t block)
 {
     __shared__ float tile[4][16][65];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 16;
+    const int64_t row0 = (block * 4 + wave) * 16;
     if (row0 >= n) {
         return;
     }
@@ -91,6 +91,12 @@ __global__ __launch_bounds__(256) void sqnorm_rows_tiled_kernel(const float *__r
     }
 }
 
+__global__ __launch_bounds__(256) void sqnorm_rows_tiled_kernel(const float *__restrict__ x, int64_t n, int d,
+                                                                float *__restrict__ out)
+{
+    sqnorm_rows_tiled_block(x, n, d, out, blockIdx.x);
+}
+
 void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_t s)
 {
     if (n == 0) {
@@ -100,6 +106,80 @@ void launch_sqnorm_rows(const float *x, int64_t n, int d, float *out, hipStream_
         hipLaunchKernelGGL(sqnorm_rows_tiled_kernel, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, s, x, n, d, out);
     } else {
         hipLaunchKernelGGL(sqnorm_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, n, d, out);
+    }
+}
+
+// ---- bf16 x 3 split --------------------------------------------------------------------------------
+// x = hi + lo + rest with hi = bf16(x), lo = bf16(x - hi) (both round-to-nearest-even), so
+// |lo| <= 2^-9 |x| and |rest| <= 2^-18 |x|.  A dot product over the concatenated rows
+// [hi | hi | lo] . [hi | lo | hi]  = hi.hi + hi.lo + lo.hi  misses lo.lo + rest.y + x.rest, at most
+// 3 * 2^-18 * sum |x_i y_i|, at three bf16 MFMAs (16x the fp32 matrix rate each) per fp32 product.
+// Rows are zero-padded to dp (a multiple of 32) per segment.
+__device__ __forceinline__ uint16_t bf16_rne(float v)
+{
+    uint32_t u = __float_as_uint(v);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ void split_bf16x3_block(const float *__restrict__ x, int64_t n, int d, int dp, int base_side,
+                                                   uint16_t *__restrict__ out, int64_t block)
+{
+    const int64_t e = block * 256 + threadIdx.x;
+    if (e >= n * dp) {
+        return;
+    }
+    const int64_t row = e / dp;
+    const int j = (int)(e % dp);
+    const float v = j < d ? x[row * d + j] : 0.f;
+    const uint16_t hi = bf16_rne(v);
+    const float hif = __uint_as_float((uint32_t)hi << 16);
+    const uint16_t lo = bf16_rne(v - hif);
+    uint16_t *o = out + row * 3 * dp + j;
+    o[0] = hi;
+    o[dp] = base_side ? lo : hi;
+    o[2 * dp] = base_side ? hi : lo;
+}
+
+__global__ __launch_bounds__(256) void split_bf16x3_kernel(const float *__restrict__ x, int64_t n, int d, int dp,
+                                                           int base_side, uint16_t *__restrict__ out)
+{
+    split_bf16x3_block(x, n, d, dp, base_side, out, blockIdx.x);
+}
+
+// Both of the above in one launch (the first blocks add up the norms, the others split): what a search does to its
+// queries before the coarse stage's first score launch.
+__global__ __launch_bounds__(256) void sqnorm_and_split_kernel(const float *__restrict__ x, int64_t n, int d, int dp,
+                                                               float *__restrict__ norms, uint16_t *__restrict__ split,
+                                                               unsigned norm_blocks)
+{
+    if (blockIdx.x < norm_blocks) {
+        sqnorm_rows_tiled_block(x, n, d, norms, blockIdx.x);
+    } else {
+        split_bf16x3_block(x, n, d, dp, 0, split, blockIdx.x - norm_blocks);
+    }
+}
+
+void launch_sqnorm_and_split_bf16x3(const float *x, int64_t n, int d, int dp, float *norms, uint16_t *split, hipStream_t s)
+{
+    if (n == 0) {
+        return;
+    }
+    if (d % 4 == 0 && d >= 32 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        const unsigned norm_blocks = (unsigned)((n + 63) / 64), split_blocks = (unsigned)((n * dp + 255) / 256);
+        hipLaunchKernelGGL(sqnorm_and_split_kernel, dim3(norm_blocks + split_blocks), dim3(256), 0, s, x, n, d, dp, norms,
+                           split, norm_blocks);
+    } else {
+        launch_sqnorm_rows(x, n, d, norms, s);
+        launch_split_bf16x3(x, n, d, dp, false, split, s);
+    }
+}
+
+void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(split_bf16x3_kernel, dim3((unsigned)((n * dp + 255) / 256)), dim3(256), 0, s, x, n, d, dp,
+                           base_side ? 1 : 0, out);
     }
 }
 
@@ -919,7 +999,7 @@ void launch_fold_records(unsigned long long *running, int k, ScoreFilter<float> 
 // registers, bisection over the ordered score bits.  G <= 64 E.
 template <int E>
 __global__ __launch_bounds__(256) void tau_from_minima_kernel(const float *__restrict__ gm, int G, int rank, int64_t n,
-                                                              float *__restrict__ tau)
+                                                              float *__restrict__ tau, RecordTest test)
 {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -943,25 +1023,30 @@ __global__ __launch_bounds__(256) void tau_from_minima_kernel(const float *__res
         p = below < rank ? c : p;
     }
     if (lane == 0) {
-        tau[row] = unordered_bits(p);
+        const float t = unordered_bits(p);
+        tau[row] = t;
+        if (test.out) {
+            test.out[row] = record_test_value(test.qn[row], t, test.cmax, test.metric == kMetricL2);
+        }
     }
 }
 
-void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s)
+void launch_tau_from_minima(const float *gm, int G, int rank, int64_t nq, float *tau, hipStream_t s, const RecordTest *test)
 {
+    const RecordTest rt = test ? *test : RecordTest{nullptr, 0.f, 0, nullptr};
     if (nq == 0) {
         return;
     }
     IXA_REQUIRE(G >= 1 && G <= 512 && rank >= 1 && rank <= G, kErrInner, "rank %d of %d group minima", rank, G);
     const dim3 grid((unsigned)((nq + 3) / 4)), block(256);
     if (G <= 64) {
-        hipLaunchKernelGGL(tau_from_minima_kernel<1>, grid, block, 0, s, gm, G, rank, nq, tau);
+        hipLaunchKernelGGL(tau_from_minima_kernel<1>, grid, block, 0, s, gm, G, rank, nq, tau, rt);
     } else if (G <= 128) {
-        hipLaunchKernelGGL(tau_from_minima_kernel<2>, grid, block, 0, s, gm, G, rank, nq, tau);
+        hipLaunchKernelGGL(tau_from_minima_kernel<2>, grid, block, 0, s, gm, G, rank, nq, tau, rt);
     } else if (G <= 256) {
-        hipLaunchKernelGGL(tau_from_minima_kernel<4>, grid, block, 0, s, gm, G, rank, nq, tau);
+        hipLaunchKernelGGL(tau_from_minima_kernel<4>, grid, block, 0, s, gm, G, rank, nq, tau, rt);
     } else {
-        hipLaunchKernelGGL(tau_from_minima_kernel<8>, grid, block, 0, s, gm, G, rank, nq, tau);
+        hipLaunchKernelGGL(tau_from_minima_kernel<8>, grid, block, 0, s, gm, G, rank, nq, tau, rt);
     }
 }
 

@@ -356,28 +356,6 @@ bool launch_for_row(int d3, const uint16_t *Qs, int64_t nq, const uint16_t *Bt, 
     }
 }
 
-// test[i] for the RECORDS launch: a run is recorded when some u = g - |c|^2 / 2 of its four reaches test[i].
-//   L2: score v = fl(fl(fl(|q|^2 + |c|^2) - g) - g) <= tau.  v differs from |q|^2 + |c|^2 - 2 g by at most three
-//   roundings of numbers no larger than |q|^2 + |c|^2 + 2 |g| <= 2 (|q|^2 + |c|^2): 6 x 2^-24 (|q|^2 + |c|^2); u differs
-//   from g - |c|^2 / 2 by one rounding, at most 2^-24 (|q|^2 + |c|^2).  So v <= tau implies
-//   u >= (|q|^2 - tau) / 2 - 4 x 2^-24 (|q|^2 + |c|^2); the test value lies another factor of two below that, with
-//   |c| <= cmax, and below its own rounding.
-//   Inner product: v = -g <= tau  <=>  g >= -tau, and u = g exactly (the norms handed to the kernel are zero).
-__global__ __launch_bounds__(256) void record_test_value_kernel(const float *__restrict__ qn, const float *__restrict__ tau,
-                                                                float cmax, int metric, int64_t n, float *__restrict__ out)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) {
-        const float t = tau[i];
-        if (metric == kMetricL2) {
-            const float mag = qn[i] + cmax * cmax + fabsf(t);
-            out[i] = 0.5f * (qn[i] - t) - 4.8e-7f * mag;   // 2^-21 = 4.77e-7
-        } else {
-            out[i] = -t - 4.8e-7f * fabsf(t);
-        }
-    }
-}
-
 }  // namespace
 
 bool resident_coarse_serves(int d3) { return d3 == 192 || d3 == 288 || d3 == 384; }
@@ -393,16 +371,15 @@ bool launch_resident_bf16_minima(const uint16_t *Qs, int64_t nq, const uint16_t 
 }
 
 bool launch_resident_bf16_records(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, int64_t nb, int d3, const float *qn,
-                                  const float *cn_padded, int metric, float cmax, float *test_scratch,
-                                  ScoreFilter<float> flt, hipStream_t s)
+                                  const float *cn_padded, int metric, const float *test, ScoreFilter<float> flt,
+                                  hipStream_t s)
 {
-    if (nq <= 0 || nb <= 0 || nb % 4 != 0 || !resident_coarse_serves(d3) || reinterpret_cast<uintptr_t>(Qs) % 16 != 0 ||
-        reinterpret_cast<uintptr_t>(Bt) % 16 != 0 || reinterpret_cast<uintptr_t>(cn_padded) % 16 != 0) {
+    if (nq <= 0 || nb <= 0 || nb % 4 != 0 || !test || !resident_coarse_serves(d3) ||
+        reinterpret_cast<uintptr_t>(Qs) % 16 != 0 || reinterpret_cast<uintptr_t>(Bt) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(cn_padded) % 16 != 0) {
         return false;
     }
-    hipLaunchKernelGGL(record_test_value_kernel, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, s, qn, flt.tau, cmax,
-                       metric, nq, test_scratch);
-    return launch_for_row<kRecords>(d3, Qs, nq, Bt, cn_padded, nb, qn, test_scratch, metric, nullptr, 0, flt, s);
+    return launch_for_row<kRecords>(d3, Qs, nq, Bt, cn_padded, nb, qn, test, metric, nullptr, 0, flt, s);
 }
 
 }  // namespace ixa

@@ -868,7 +868,12 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
         return;
     }
     ws_qn_.resize((size_t)n);
-    launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
+    if (cfg_.coarse_bf16) {   // the queries' norms and their bf16 x 3 split in one launch
+        ws_xsplit_.resize((size_t)n * 3 * dp_);
+        launch_sqnorm_and_split_bf16x3(x_dev, n, d_, dp_, ws_qn_.data(), ws_xsplit_.data(), stream_);
+    } else {
+        launch_sqnorm_rows(x_dev, n, d_, ws_qn_.data(), stream_);
+    }
     int ncand = (int)std::min<int64_t>(nlist_, (int64_t)nout + 16 + nout / 8);
     // flag[0] counts the queries without proof and is zero between calls: coarse_finish() clears it
     // when it was not, so the common case needs no fill in front of the kernels that append to it
@@ -885,8 +890,6 @@ void IvfpqIndex::coarse_select(const float *x_dev, int64_t n, int nout, int sele
     last_coarse_n_ = n;
     if (cfg_.coarse_bf16) {
         ws_running_.resize((size_t)n * ncand);
-        ws_xsplit_.resize((size_t)n * 3 * dp_);
-        launch_split_bf16x3(x_dev, n, d_, dp_, false, ws_xsplit_.data(), stream_);
         // large products: admission bound from a seed stretch, result proven by count, nothing but the seed's
         // scores written (rows without proof join the list of queries that coarse_finish() redoes exactly)
         const bool set_wanted = set_only && !out_dist && ncand > nout;   // search: only the SET of lists matters

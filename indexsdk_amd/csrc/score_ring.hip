@@ -714,46 +714,6 @@ bool launch_score_ring_bf16_records(const uint16_t *Q, int64_t nq, const uint16_
     return launch_ring<Bf16Traits>(Q, nq, B, nb, d, qn, bn, metric, nullptr, 0, 2, flt, s);
 }
 
-// ---- bf16 x 3 split --------------------------------------------------------------------------------
-// x = hi + lo + rest with hi = bf16(x), lo = bf16(x - hi) (both round-to-nearest-even), so
-// |lo| <= 2^-9 |x| and |rest| <= 2^-18 |x|.  A dot product over the concatenated rows
-// [hi | hi | lo] . [hi | lo | hi]  = hi.hi + hi.lo + lo.hi  misses lo.lo + rest.y + x.rest, at most
-// 3 * 2^-18 * sum |x_i y_i|, at three bf16 MFMAs (16x the fp32 matrix rate each) per fp32 product.
-// Rows are zero-padded to dp (a multiple of 32) per segment.
-__device__ __forceinline__ uint16_t bf16_rne(float v)
-{
-    uint32_t u = __float_as_uint(v);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
-
-__global__ __launch_bounds__(256) void split_bf16x3_kernel(const float *__restrict__ x, int64_t n, int d, int dp,
-                                                           int base_side, uint16_t *__restrict__ out)
-{
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (e >= n * dp) {
-        return;
-    }
-    const int64_t row = e / dp;
-    const int j = (int)(e % dp);
-    const float v = j < d ? x[row * d + j] : 0.f;
-    const uint16_t hi = bf16_rne(v);
-    const float hif = __uint_as_float((uint32_t)hi << 16);
-    const uint16_t lo = bf16_rne(v - hif);
-    uint16_t *o = out + row * 3 * dp + j;
-    o[0] = hi;
-    o[dp] = base_side ? lo : hi;
-    o[2 * dp] = base_side ? hi : lo;
-}
-
-void launch_split_bf16x3(const float *x, int64_t n, int d, int dp, bool base_side, uint16_t *out, hipStream_t s)
-{
-    if (n > 0) {
-        hipLaunchKernelGGL(split_bf16x3_kernel, dim3((unsigned)((n * dp + 255) / 256)), dim3(256), 0, s, x, n, d, dp,
-                           base_side ? 1 : 0, out);
-    }
-}
-
 // Appends a query to the list flag[1 + flag[0]++] unless, for that query, no centroid outside its approximate candidate list can beat
 // its nout-th exact score: (approximate score of the last candidate) - err > (nout-th exact score),
 // err = err_scale * |q| * max|c| + round_scale * (|q| + max|c|)^2.  Rows whose candidate list is not full hold every centroid.

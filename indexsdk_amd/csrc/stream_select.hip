@@ -447,10 +447,11 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uin
                            : launch_score_ring_bf16_minima(Qs + q0 * d3, nq, Bs, seed, d3, qn + q0, bn, metric,
                                                            ws.scores.data(), G, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
-        launch_tau_from_minima(ws.scores.data(), G, j, nq, ws.tau.data() + q0, s);
+        const RecordTest rt{qn + q0, resident ? resident->cmax : 0.f, metric, resident ? ws.thr.data() + q0 : nullptr};
+        launch_tau_from_minima(ws.scores.data(), G, j, nq, ws.tau.data() + q0, s, resident ? &rt : nullptr);
         ScoreFilter<float> flt{ws.tau.data() + q0, nullptr, ws.cnt.data() + q0, ws.filter.data(), cap, 0};
         ok = resident ? launch_resident_bf16_records(Qs + q0 * d3, nq, resident->Bt, nb_total, d3, qn + q0,
-                                                     resident->cn_padded, metric, resident->cmax, ws.thr.data() + q0, flt, s)
+                                                     resident->cn_padded, metric, ws.thr.data() + q0, flt, s)
                       : launch_score_ring_bf16_records(Qs + q0 * d3, nq, Bs, nb_total, d3, qn + q0, bn, metric, flt, s);
         IXA_REQUIRE(ok, kErrInner, "bf16 score kernel rejected a shape it had accepted");
         // the resident-query launch records dot products; the folds form the scores
