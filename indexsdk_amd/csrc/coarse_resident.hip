@@ -42,7 +42,7 @@ template <int NHS, int PF, int RA, int MODE>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void resident_bf16_kernel(
     const uint16_t *__restrict__ Qs, int64_t nq, const uint16_t *__restrict__ Bt, const float *__restrict__ cnp, int64_t nb,
     const float *__restrict__ qn, const float *__restrict__ test, int metric, float *__restrict__ out, int64_t ldo,
-    ScoreFilter<float> flt, int tiles_m, int ntiles, int seg_tiles)
+    ScoreFilter<float> flt, int tiles_m, int ntiles, int seg_tiles, int own_resident)
 {
     constexpr int D = NHS * 32, QT = RA * 32;   // bytes of a split row, queries of a tile
     constexpr int kStepLds = QT * 32;           // LDS bytes of one K-step: two chunks of QT x 16 bytes
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, l32 = lane & 31;
     const int xcd = blockIdx.x & 7, wi = blockIdx.x >> 3, wpx = gridDim.x >> 3;
-    const ResidentItems sched(tiles_m, ntiles, seg_tiles, xcd, wpx);
+    const ResidentItems sched(tiles_m, ntiles, seg_tiles, xcd, wpx, own_resident != 0);
     const int S = sched.S;
     const int first_item = sched.next(wi);
     if (first_item < 0) {
@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
     float *perq = reinterpret_cast<float *>(lds + QT * D);   // per query: the test value (RECORDS) or |q|^2 (MINIMA)
     const unsigned char *Bb = reinterpret_cast<const unsigned char *>(Bt);
     const unsigned char *Qb = reinterpret_cast<const unsigned char *>(Qs);
-    auto block_row0 = [&](int j) { return (xcd + 8 * (int64_t)j) * kI8TileRows + wave * 32; };
+    auto block_row0 = [&](int j) { return sched.streamed_tile(j) * kI8TileRows + wave * 32; };
     auto block_ptr = [&](int j) { return Bb + block_row0(j) * (int64_t)D + lane * 16; };
 
     v16f acc[RA];
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 
                 best = fminf(best, __shfl_xor(best, 32));   // both halves: the wave's 32 centroids
                 const int64_t row = (int64_t)tm * QT + ra * 32 + l32;
                 if (half == 0 && row < nq) {
-                    out[row * ldo + ((xcd + 8 * (int64_t)j) * 8 + wave)] = best;
+                    out[row * ldo + (sched.streamed_tile(j) * 8 + wave)] = best;
                 }
             }
         } else {
@@ -269,18 +269,21 @@ int device_cus()
     return cus;
 }
 
-// rounds of work items x (loading the query tile + walking a segment), in units of one block-row of matrix work
-double plan_cost(int64_t tiles_m, int64_t own_n, int64_t wpx, int ra, int64_t seg)
+// rounds of work items x (loading the query tile + walking a segment), in units of one block-row of matrix work;
+// load = what a query tile costs to load, in tiles' time (measured inside the kernel: 1.6 where a tile has the record
+// epilogue behind it, about 3 where it has the minima's)
+double plan_cost(int64_t tiles_m, int64_t own_n, int64_t wpx, int ra, int64_t seg, double load)
 {
-    const int64_t S = wpx / tiles_m > 1 ? wpx / tiles_m : 1;
+    const int64_t S = tiles_m > 0 && wpx / tiles_m > 1 ? wpx / tiles_m : 1;
     const int64_t nseg = (own_n + S * seg - 1) / (S * seg) * S;
     const int64_t rounds = (tiles_m * nseg + wpx - 1) / wpx;
-    return (double)rounds * ra * (0.6 + (double)seg);   // a query tile costs about 0.6 tiles' time to load
+    return (double)rounds * ra * (load + (double)seg);
 }
 
 template <int NHS, int PF, int RA, int MODE>
 void launch_shape(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const float *cnp, int64_t nb, const float *qn,
-                  const float *test, int metric, float *out, int64_t ldo, ScoreFilter<float> flt, int seg, hipStream_t s)
+                  const float *test, int metric, float *out, int64_t ldo, ScoreFilter<float> flt, int seg, bool own_resident,
+                  hipStream_t s)
 {
     constexpr int QT = RA * 32;
     constexpr size_t smem = (size_t)QT * NHS * 32 + QT * 4 + (MODE == kRecords ? kWaves * kQueueRecords * 32 : 0);
@@ -301,7 +304,7 @@ void launch_shape(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const floa
     const int64_t tiles_m = (nq + QT - 1) / QT, ntiles = (nb + kI8TileRows - 1) / kI8TileRows;
     const unsigned grid = (unsigned)((device_cus() + 7) / 8 * 8);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kWaves * 64), smem, s, Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt,
-                       (int)tiles_m, (int)ntiles, seg);
+                       (int)tiles_m, (int)ntiles, seg, own_resident ? 1 : 0);
     }
 }
 
@@ -309,36 +312,43 @@ template <int NHS, int PF, int MODE>
 void launch_ra(const uint16_t *Qs, int64_t nq, const uint16_t *Bt, const float *cnp, int64_t nb, const float *qn,
                const float *test, int metric, float *out, int64_t ldo, ScoreFilter<float> flt, hipStream_t s)
 {
-    // tile height and segment length by the number of rounds the launch will take
-    const int64_t wpx = (device_cus() + 7) / 8, own_n = ((nb + kI8TileRows - 1) / kI8TileRows + 7) / 8;
+    // tile height, segment length and which operand's tiles an XCD owns, by the number of rounds the launch will take
+    const int64_t wpx = (device_cus() + 7) / 8, ntiles = (nb + kI8TileRows - 1) / kI8TileRows;
+    const double load = MODE == kRecords ? 1.6 : 3.0;
     int best_ra = 4;
     int64_t best_seg = 1;
+    bool best_own = false;
     double best = 1e300;
     for (int ra = 4; ra <= 6; ra++) {
         if ((size_t)ra * 32 * NHS * 32 + ra * 128 + (MODE == kRecords ? kWaves * kQueueRecords * 32 : 0) > 160 * 1024) {
             continue;
         }
         const int64_t tiles_m = (nq + ra * 32 - 1) / (ra * 32);
-        for (int64_t seg = 1;; seg *= 2) {
-            const int64_t sg = seg < own_n ? seg : own_n;   // 1, 2, 4, ... and the XCD's whole share
-            const double c = plan_cost(tiles_m, own_n, wpx, ra, sg);
-            if (c < best) {
-                best = c;
-                best_ra = ra;
-                best_seg = sg;
-            }
-            if (seg >= own_n) {
-                break;
+        for (int own = 0; own < 2; own++) {
+            // the XCD with most to do: every resident tile and an eighth of the streamed ones, or the other way round
+            const int64_t tm = own ? (tiles_m + 7) / 8 : tiles_m, tn = own ? ntiles : (ntiles + 7) / 8;
+            for (int64_t seg = 1;; seg *= 2) {
+                const int64_t sg = seg < tn ? seg : tn;   // 1, 2, 4, ... and the XCD's whole share
+                const double c = plan_cost(tm, tn, wpx, ra, sg, load);
+                if (c < best) {
+                    best = c;
+                    best_ra = ra;
+                    best_seg = sg;
+                    best_own = own != 0;
+                }
+                if (seg >= tn) {
+                    break;
+                }
             }
         }
     }
     const int seg = (int)best_seg;
     if (best_ra == 4) {
-        launch_shape<NHS, PF, 4, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, s);
+        launch_shape<NHS, PF, 4, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, best_own, s);
     } else if (best_ra == 5) {
-        launch_shape<NHS, PF, 5, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, s);
+        launch_shape<NHS, PF, 5, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, best_own, s);
     } else {
-        launch_shape<NHS, PF, 6, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, s);
+        launch_shape<NHS, PF, 6, MODE>(Qs, nq, Bt, cnp, nb, qn, test, metric, out, ldo, flt, seg, best_own, s);
     }
 }
 

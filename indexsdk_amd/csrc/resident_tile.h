@@ -50,7 +50,7 @@ __device__ __forceinline__ void lds_wait_group(V (&f)[N])
 // contiguous bytes of every row on the memory side, 256 contiguous bytes per chunk on the LDS side (a four-way bank
 // conflict; row-fastest would read 16 bytes per row, chunk-fastest would put 64 lanes on four banks), and a
 // thread issues eight loads before the first store, so the tile costs a few memory round trips, not one per step.
-template <int QT, int D, int NT>
+template <int QT, int D, int NT, int kBatch = 8>
 __device__ __forceinline__ void load_resident_tile(unsigned char *lds, const unsigned char *__restrict__ rows, int64_t first,
                                                    int64_t nrows, int tid)
 {
@@ -60,7 +60,7 @@ __device__ __forceinline__ void load_resident_tile(unsigned char *lds, const uns
     constexpr int kPerWave = (kSteps + kWavesT - 1) / kWavesT;
     const int lane = tid & 63, wave = tid >> 6;
     const int qq = lane & 15, cc = lane >> 4;
-    constexpr int kBatch = 8;   // loads in flight per thread: registers are scarce where this is called
+    // kBatch = loads in flight per thread (8 where registers are scarce at the call)
 #pragma unroll
     for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
         uint4 v[kBatch];
@@ -90,21 +90,33 @@ __device__ __forceinline__ void load_resident_tile(unsigned char *lds, const uns
 // XCD's workgroups.  The S = wpx / tiles_m segments that are in flight together INTERLEAVE tile by tile inside a
 // group of S * seg_tiles tiles (segment `sub` of group g takes tiles g * S * seg_tiles + sub, + S, + 2 S, ...): all
 // workgroups of the XCD then read the same few tiles at any moment and its L2 holds them for every reader.
+// With own_resident the roles are swapped: XCD x owns the RESIDENT tiles x, x + 8, ... and walks every streamed tile
+// (fewer, longer items: the choice for launches with few streamed tiles per XCD, where loading the resident tile
+// costs more than walking a segment).  streamed_tile(j) / the tm that range() returns are the tiles' real numbers.
 struct ResidentItems {
     int tiles_m, own_n, wpx, S, group_tiles, items;
-    __device__ ResidentItems(int tiles_m_, int ntiles, int seg_tiles, int xcd, int wpx_)
+    int tm_add, tm_mul, j_add, j_mul;
+    __device__ ResidentItems(int tiles_m_, int ntiles, int seg_tiles, int xcd, int wpx_, bool own_resident = false)
     {
-        tiles_m = tiles_m_;
         wpx = wpx_;
-        own_n = ntiles > xcd ? (ntiles - xcd + 7) / 8 : 0;
-        S = wpx / tiles_m > 1 ? wpx / tiles_m : 1;
+        if (own_resident) {
+            tiles_m = tiles_m_ > xcd ? (tiles_m_ - xcd + 7) / 8 : 0;
+            own_n = ntiles;
+            tm_add = xcd, tm_mul = 8, j_add = 0, j_mul = 1;
+        } else {
+            tiles_m = tiles_m_;
+            own_n = ntiles > xcd ? (ntiles - xcd + 7) / 8 : 0;
+            tm_add = 0, tm_mul = 1, j_add = xcd, j_mul = 8;
+        }
+        S = tiles_m > 0 && wpx / tiles_m > 1 ? wpx / tiles_m : 1;
         group_tiles = S * seg_tiles;
         items = tiles_m * ((own_n + group_tiles - 1) / group_tiles * S);
     }
+    __device__ int64_t streamed_tile(int j) const { return j_add + (int64_t)j_mul * j; }
     // resident tile, first streamed tile, tile after the last of an item (tiles advance by S); may be empty
     __device__ void range(int it, int &tm, int &j0, int &j1) const
     {
-        tm = it % tiles_m;
+        tm = tm_add + tm_mul * (it % tiles_m);
         const int seg = it / tiles_m, g = seg / S, sub = seg % S;
         j0 = g * group_tiles + sub;
         j1 = (g + 1) * group_tiles < own_n ? (g + 1) * group_tiles : own_n;
