@@ -947,3 +947,27 @@ def test_coarse_training_step_is_the_lloyd_update_in_sample_order(ix, oracle, sp
         want = (want.astype(np.float64) / norm[:, None]).astype(np.float32)
     assert empties >= 1, "the data should leave clusters empty"
     assert np.array_equal(want.view(np.uint32), after.view(np.uint32))
+
+
+def test_host_batch_beyond_the_staging_buffer_equals_its_pieces(ix, oracle):
+    """Host searches of up to 256 MB of queries + results go through the index's page-locked staging buffer (the
+    kernels write the results into it, the copy-out is shared by threads); larger ones are copied by the runtime.
+    Both routes, and the pieces of a batch searched on their own, give the same bits."""
+    d, nlist, M, n, nq, k = 32, 64, 8, 20000, 450_000, 40
+    assert nq * (d * 4 + k * 12) > 256 << 20
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    cent, _ = oracle.kmeans(x[:4000], nlist, niter=3, seed=5)
+    cb = oracle.train_pq(x[:4000], M, niter=3, seed=5)
+    gpu = ix.AscendIndexIVFPQ(d, ix.METRIC_L2, nlist, M, 8)
+    gpu.set_trained(cent, cb)
+    gpu.add(x)
+    gpu.setNumProbes(8)
+    D, I = gpu.search(q, k)
+    for a, m in ((0, 3000), (200_000, 150_000), (nq - 2500, 2500)):     # a small piece, a multi-threaded copy-out, the tail
+        Dp, Ip = gpu.search(q[a:a + m], k)
+        assert np.array_equal(Ip, I[a:a + m]) and np.array_equal(Dp.view(np.uint32), D[a:a + m].view(np.uint32))
+    ref = oracle.CsrIndex.build(d, M, ix.METRIC_L2, cent, cb, x, np.arange(n, dtype=np.int64))
+    Dr, Ir = ref.search(q[:500], k, 8)
+    assert_topk_parity(oracle, ref, q[:500], D[:500], I[:500], Dr, Ir, TOL_FP32)
