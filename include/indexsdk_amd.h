@@ -18,11 +18,12 @@
  *   - metric: 0 = inner product, 1 = L2 (faiss::MetricType values).
  *   - missing results: label -1, distance FLT_MAX for L2 and -FLT_MAX for inner product
  *     (FR/ascenddaemon/impl/IndexIVFPQ.cpp:2202-2219; FR/ascend/impl/AscendIndexImpl.cpp:587-650).
- *   - every handle may be used from several threads.  An IVFPQ handle locks as the reference does under
- *     MX_INDEX_MULTITHREAD (FR/ascend/impl/AscendIndexImpl.h:62, 230; AscendIndexImpl.cpp:204, 508-564):
- *     ivfpq_search, ivfpq_search_device and ivfpq_search_probes_device take the lock shared and up to four of
- *     them run side by side, each on a stream and workspaces of its own; every other call takes it
- *     exclusively.  Calls on one Flat handle are serialised.  Different handles never wait for each other.
+ *   - every handle may be used from several threads.  A handle locks as the reference does under
+ *     MX_INDEX_MULTITHREAD (FR/ascend/impl/AscendIndexImpl.h:62, 230; AscendIndexImpl.cpp:204, 508-564): the
+ *     searches (ivfpq_search, ivfpq_search_device, ivfpq_search_probes_device; flat_search, flat_search_device,
+ *     flat_search_with_masks and their flat_i8_ forms) take the lock shared and up to four of them run side by
+ *     side, each on a stream and workspaces of its own; every other call takes it exclusively.  Different
+ *     handles never wait for each other.
  *   - there is no CPU fallback: every entry point fails with IXA_ERR_INDEX_NOT_INIT when no
  *     HIP device is present.
  */

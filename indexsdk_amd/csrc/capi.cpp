@@ -22,41 +22,43 @@ void write_faiss_ivfpq(const IvfpqIndex &idx, const char *path);
 std::unique_ptr<IvfpqIndex> read_faiss_ivfpq(const char *path, const IvfpqConfig &cfg);
 }  // namespace ixa
 
-// The handle owns the index through a pointer so that a loader can hand over a finished one.
 // Locking follows the reference's MX_INDEX_MULTITHREAD mode (FR/ascend/impl/AscendIndexImpl.h:62, 230;
 // AscendIndexImpl.cpp:204, 508-564), always on here: a search takes the handle's lock shared, everything that
 // changes the index takes it exclusively.  A search needs a stream and workspaces of its own, so each runs on a
-// lane: lane 0 is the index itself, lanes 1..kSearchViews are views that read the index's trained state and lists
-// in place (IvfpqIndex::borrow_from), made on first need.  A search that finds every lane taken waits for one.
-struct ivfpq_index {
+// lane: lane 0 is the index itself, lanes 1..kSearchViews are views that read the index's data in place
+// (borrow_from), made on first need.  A search that finds every lane taken waits for one.
+template <typename Index>
+struct Lanes {
     static constexpr int kSearchViews = 3;
     mutable std::shared_mutex mu;
-    std::unique_ptr<ixa::IvfpqIndex> owned;
-    ixa::IvfpqIndex &impl;
-    // lanes (guarded by lane_mu)
-    mutable std::mutex lane_mu;
+    mutable std::mutex lane_mu;                       // guards what follows
     mutable std::condition_variable lane_cv;
-    mutable std::unique_ptr<ixa::IvfpqIndex> views[kSearchViews];
+    mutable std::unique_ptr<Index> views[kSearchViews];
     mutable uint64_t view_version[kSearchViews] = {0, 0, 0};
     mutable uint64_t version = 1;       // counts the calls that may have changed the index
     mutable unsigned busy = 0;          // bit l = lane l is searching
-    mutable ixa::IvfpqIndex *last;      // lane of the search that finished last: "the last search" of the statistics
-    ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
-        : owned(new ixa::IvfpqIndex(d, metric, nlist, M, nbits, c)), impl(*owned), last(owned.get())
-    {
-    }
-    explicit ivfpq_index(std::unique_ptr<ixa::IvfpqIndex> p) : owned(std::move(p)), impl(*owned), last(owned.get()) {}
+    mutable Index *last = nullptr;      // lane of the search that finished last: "the last search" of the statistics
 };
 
-struct flat_index {
-    mutable std::mutex mu;
-    ixa::FlatIndex impl;
-    flat_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
+// The IVFPQ handle owns the index through a pointer so that a loader can hand over a finished one.
+struct ivfpq_index : Lanes<ixa::IvfpqIndex> {
+    std::unique_ptr<ixa::IvfpqIndex> owned;
+    ixa::IvfpqIndex &impl;
+    ivfpq_index(int d, int metric, int64_t nlist, int M, int nbits, const ixa::IvfpqConfig &c)
+        : owned(new ixa::IvfpqIndex(d, metric, nlist, M, nbits, c)), impl(*owned)
+    {
+        last = owned.get();
+    }
+    explicit ivfpq_index(std::unique_ptr<ixa::IvfpqIndex> p) : owned(std::move(p)), impl(*owned) { last = owned.get(); }
 };
-struct flat_i8_index {
-    mutable std::mutex mu;
+
+struct flat_index : Lanes<ixa::FlatIndex> {
+    ixa::FlatIndex impl;
+    flat_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) { last = &impl; }
+};
+struct flat_i8_index : Lanes<ixa::FlatI8Index> {
     ixa::FlatI8Index impl;
-    flat_i8_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) {}
+    flat_i8_index(int d, int metric, int64_t scratch) : impl(d, metric, scratch) { last = &impl; }
 };
 
 namespace {
@@ -87,24 +89,30 @@ int guarded(F &&f, bool uses_gpu = true)
     }
 }
 
-// Exclusive use of a handle.  For an IVFPQ handle: the statistics a view still owes refer to lists that the call
-// may move, so they are worked out first; a call that may change the index makes every view borrow again.
+ixa::IvfpqIndex *make_view(const ixa::IvfpqIndex &o)
+{
+    return new ixa::IvfpqIndex(o.d(), o.metric(), o.nlist(), o.M(), 8, o.config());
+}
+ixa::FlatIndex *make_view(const ixa::FlatIndex &o) { return new ixa::FlatIndex(o.d(), o.metric(), o.scratch_bytes()); }
+ixa::FlatI8Index *make_view(const ixa::FlatI8Index &o) { return new ixa::FlatI8Index(o.d(), o.metric(), o.scratch_bytes()); }
+// what a view still owes before the data it refers to may move
+void settle_view(ixa::IvfpqIndex &v) { v.flush_pending_stats(); }
+void settle_view(ixa::FlatIndex &) {}
+void settle_view(ixa::FlatI8Index &) {}
+
+// Exclusive use of a handle.  The statistics a view still owes refer to data that the call may move, so they are
+// worked out first; a call that may change the index makes every view borrow again.
 template <typename H>
 struct Exclusive {
-    std::unique_lock<decltype(H::mu)> lock;
-    Exclusive(const H *h, bool) : lock(h->mu) {}
-};
-template <>
-struct Exclusive<ivfpq_index> {
     std::unique_lock<std::shared_mutex> lock;
-    const ivfpq_index *h;
+    const H *h;
     bool changes;
-    Exclusive(const ivfpq_index *handle, bool may_change) : lock(handle->mu), h(handle), changes(may_change)
+    Exclusive(const H *handle, bool may_change) : lock(handle->mu), h(handle), changes(may_change)
     {
         if (changes) {
             for (auto &v : h->views) {
                 if (v) {
-                    v->flush_pending_stats();
+                    settle_view(*v);
                 }
             }
         }
@@ -118,13 +126,15 @@ struct Exclusive<ivfpq_index> {
     }
 };
 
-// One search on an IVFPQ handle: the lock shared, and a lane for as long as the search runs.
-class SearchLane {
+// One search on a handle: the lock shared, and a lane for as long as the search runs.
+template <typename H>
+class SearchLaneOf {
 public:
-    explicit SearchLane(const ivfpq_index *handle) : shared_(handle->mu), h_(handle)
+    using Index = std::remove_reference_t<decltype(std::declval<H>().impl)>;
+    explicit SearchLaneOf(const H *handle) : shared_(handle->mu), h_(handle)
     {
         std::unique_lock<std::mutex> g(h_->lane_mu);
-        const unsigned all = (1u << (1 + ivfpq_index::kSearchViews)) - 1;
+        const unsigned all = (1u << (1 + H::kSearchViews)) - 1;
         h_->lane_cv.wait(g, [&] { return (h_->busy & all) != all; });
         while (h_->busy >> lane_ & 1u) {
             lane_++;
@@ -132,8 +142,7 @@ public:
         if (lane_ > 0) {
             auto &view = h_->views[lane_ - 1];
             if (!view) {
-                const ixa::IvfpqIndex &o = h_->impl;
-                view.reset(new ixa::IvfpqIndex(o.d(), o.metric(), o.nlist(), o.M(), 8, o.config()));
+                view.reset(make_view(h_->impl));
             }
             if (h_->view_version[lane_ - 1] != h_->version) {
                 view->borrow_from(h_->impl);
@@ -142,7 +151,7 @@ public:
         }
         h_->busy |= 1u << lane_;
     }
-    ~SearchLane()
+    ~SearchLaneOf()
     {
         {
             std::lock_guard<std::mutex> g(h_->lane_mu);
@@ -151,13 +160,13 @@ public:
         }
         h_->lane_cv.notify_one();
     }
-    SearchLane(const SearchLane &) = delete;
-    SearchLane &operator=(const SearchLane &) = delete;
-    ixa::IvfpqIndex &index() const { return lane_ == 0 ? h_->impl : *h_->views[lane_ - 1]; }
+    SearchLaneOf(const SearchLaneOf &) = delete;
+    SearchLaneOf &operator=(const SearchLaneOf &) = delete;
+    Index &index() const { return lane_ == 0 ? const_cast<Index &>(h_->impl) : *h_->views[lane_ - 1]; }
 
 private:
     std::shared_lock<std::shared_mutex> shared_;
-    const ivfpq_index *h_;
+    const H *h_;
     int lane_ = 0;
 };
 
@@ -168,7 +177,7 @@ private:
 #define IXA_HANDLE_READS(h) IXA_HANDLE_AS(h, false)  // one that only reads it (but uses its stream or workspaces)
 #define IXA_SEARCH_LANE(h)                                                                        \
     IXA_REQUIRE((h) != nullptr, ixa::kErrInvalidParam, "index handle can not be nullptr.");      \
-    SearchLane ixa_lane(h)
+    SearchLaneOf<std::remove_cv_t<std::remove_pointer_t<decltype(h)>>> ixa_lane(h)
 
 ixa::IvfpqConfig to_config(const ivfpq_config_t *cfg)
 {
@@ -513,11 +522,11 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
     }                                                                                                             \
     IXA_EXPORT int PFX##_get_base(const HT *h, int64_t offset, int64_t n, ET *out)                               \
     {                                                                                                             \
-        return guarded([&] { IXA_HANDLE(h); h->impl.get_base(offset, n, out); });                                 \
+        return guarded([&] { IXA_HANDLE_READS(h); h->impl.get_base(offset, n, out); });                                 \
     }                                                                                                             \
     IXA_EXPORT int PFX##_get_ids(const HT *h, int64_t offset, int64_t n, int64_t *out)                           \
     {                                                                                                             \
-        return guarded([&] { IXA_HANDLE(h); h->impl.get_ids(offset, n, out); });                                  \
+        return guarded([&] { IXA_HANDLE_READS(h); h->impl.get_ids(offset, n, out); });                                  \
     }                                                                                                             \
     IXA_EXPORT int PFX##_remove_ids(HT *h, int64_t n, const int64_t *ids, int64_t *removed)                      \
     {                                                                                                             \
@@ -542,7 +551,7 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
     IXA_EXPORT int PFX##_ntotal(const HT *h, int64_t *out)                                                        \
     {                                                                                                             \
         return guarded([&] {                                                                                      \
-            IXA_HANDLE(h);                                                                                        \
+            IXA_HANDLE_READS(h);                                                                                  \
             IXA_REQUIRE(out, ixa::kErrInvalidParam, "out can not be nullptr.");                                   \
             *out = h->impl.ntotal();                                                                              \
         });                                                                                                       \
@@ -550,7 +559,7 @@ static void copy_stats(const ixa::FlatStats &s, flat_search_stats_t *out)
     IXA_EXPORT int PFX##_reset(HT *h) { return guarded([&] { IXA_HANDLE(h); h->impl.reset(); }); }                \
     IXA_EXPORT int PFX##_last_search_stats(const HT *h, flat_search_stats_t *out)                                 \
     {                                                                                                             \
-        return guarded([&] { IXA_HANDLE(h); copy_stats(h->impl.stats(), out); });                                 \
+        return guarded([&] { IXA_HANDLE_READS(h); copy_stats(h->last->stats(), out); });                                 \
     }
 
 IXA_FLAT_COMMON(flat, flat_index_t, float)
@@ -704,32 +713,32 @@ IXA_EXPORT int ixa_read_probe(const void *src_dev, int64_t bytes, int passes, do
 }
 IXA_EXPORT int flat_search(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances, int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, false); });
 }
 IXA_EXPORT int flat_search_with_masks(flat_index_t *h, int64_t n, const float *x, int64_t k, const uint8_t *mask,
                                       float *distances, int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search_with_masks(n, x, k, mask, distances, labels); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search_with_masks(n, x, k, mask, distances, labels); });
 }
 IXA_EXPORT int flat_search_device(flat_index_t *h, int64_t n, const float *x, int64_t k, float *distances,
                                   int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, true); });
 }
 IXA_EXPORT int flat_i8_search(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances,
                               int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, false); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, false); });
 }
 IXA_EXPORT int flat_i8_search_with_masks(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, const uint8_t *mask,
                                          int32_t *distances, int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search_with_masks(n, x, k, mask, distances, labels); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search_with_masks(n, x, k, mask, distances, labels); });
 }
 IXA_EXPORT int flat_i8_search_device(flat_i8_index_t *h, int64_t n, const int8_t *x, int64_t k, int32_t *distances,
                                      int64_t *labels)
 {
-    return guarded([&] { IXA_HANDLE(h); h->impl.search(n, x, k, distances, labels, true); });
+    return guarded([&] { IXA_SEARCH_LANE(h); ixa_lane.index().search(n, x, k, distances, labels, true); });
 }
 
 }  // extern "C"

@@ -35,6 +35,8 @@ public:
     int d() const { return d_; }
     int metric() const { return metric_; }
     int64_t ntotal() const { return ntotal_; }
+    int64_t scratch_bytes() const { return scratch_bytes_; }
+    hipStream_t stream() const { return stream_; }
     void add(int64_t n, const T *x, const int64_t *ids, bool on_device);
     void get_base(int64_t offset, int64_t n, T *out) const;   // host output
     void get_ids(int64_t offset, int64_t n, int64_t *out) const;
@@ -42,6 +44,14 @@ public:
     const FlatStats &stats() const { return stats_; }
 
 protected:
+    // this index becomes a search view of `owner`: it reads the owner's vectors and ids in place (see IvfpqIndex::borrow_from)
+    void borrow_base(const FlatBase &owner)
+    {
+        ntotal_ = owner.ntotal_;
+        capacity_ = owner.capacity_;
+        base_.borrow(owner.base_);
+        ids_.borrow(owner.ids_);
+    }
     void reserve(int64_t n);
     // How the vectors lie in base_: row-major here; FlatI8Index keeps them in matrix-core order (flat_i8.h).
     // new_base <- the first ntotal_ vectors of base_, with room for cap
@@ -77,6 +87,12 @@ public:
     int64_t remove_ids(int64_t n, const int64_t *ids);       // host ids; returns the number of vectors removed
     int64_t remove_range(int64_t imin, int64_t imax);        // ids in [imin, imax)
     void reset();
+    void borrow_from(const FlatIndex &owner)   // a view serves searches only
+    {
+        borrow_base(owner);
+        norms_.borrow(owner.norms_);
+        bmax_ = owner.bmax_;
+    }
 
 private:
     // exact results for the listed query rows, from canonical scores of the whole base
@@ -100,6 +116,11 @@ public:
     int64_t remove_ids(int64_t n, const int64_t *ids);
     int64_t remove_range(int64_t imin, int64_t imax);
     void reset();
+    void borrow_from(const FlatI8Index &owner)   // a view serves searches only
+    {
+        borrow_base(owner);
+        norms_.borrow(owner.norms_);
+    }
 
 private:
     void search_masked(int64_t n, const int8_t *x, int64_t k, int32_t *dist, int64_t *labels, bool on_device,

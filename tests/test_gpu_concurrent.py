@@ -121,6 +121,51 @@ def test_searches_beside_adds_and_removes_stay_valid(ix, oracle):
     concurrent_equal_serial(gpu, [np.ascontiguousarray(q[:16]), np.ascontiguousarray(q[16:17])], 5, 4, 10)
 
 
+@pytest.mark.parametrize("kind", ["int8", "fp32"])
+def test_flat_searches_side_by_side_equal_searches_alone(ix, oracle, kind):
+    """The Flat handles lock the same way: searches share the lock and run on lanes of their own, changes are exclusive."""
+    rng = np.random.default_rng(5)
+    d, n = 64, 30000
+    if kind == "int8":
+        base = rng.integers(-127, 128, size=(n, d), dtype=np.int8)
+        q = rng.integers(-127, 128, size=(300, d), dtype=np.int8)
+        index = ix.AscendIndexInt8Flat(d, ix.METRIC_L2)
+        search = index.search_int32
+        ref = lambda qq, kk, b, i: oracle.flat_i8(b, qq, kk, ids=i)
+    else:
+        base = rng.standard_normal((n, d)).astype(np.float32)
+        q = rng.standard_normal((300, d)).astype(np.float32)
+        index = ix.AscendIndexFlat(d, ix.METRIC_L2)
+        search = index.search
+        ref = lambda qq, kk, b, i: oracle.flat_f32(b, qq, kk, ids=i)
+    ids = np.arange(n, dtype=np.int64) * 3 + 1
+    index.add_with_ids(base[:20000], ids[:20000])
+    queries = [np.ascontiguousarray(q[a:b]) for a, b in ((0, 1), (1, 9), (9, 50), (50, 300))]
+    k = 10
+
+    def check(b, i):
+        want = [search(qq, k) for qq in queries]
+
+        def body(t):
+            for r in range(20):
+                j = (t + r) % len(queries)
+                D, I = search(queries[j], k)
+                assert np.array_equal(I, want[j][1]) and np.array_equal(D.view(np.uint32), want[j][0].view(np.uint32)), (t, r, j)
+
+        run_threads(5, body)
+        Dr, Ir = ref(queries[2], k, b, i)
+        assert np.array_equal(want[2][1], Ir) and np.array_equal(want[2][0].view(np.uint32), np.asarray(Dr).view(np.uint32))
+
+    check(base[:20000], ids[:20000])
+    index.add_with_ids(base[20000:], ids[20000:])       # the base is reallocated: every lane borrows again
+    check(base, ids)
+    assert index.remove_ids(ids[:100]) == 100
+    D, I = search(queries[3], k)
+    assert not np.isin(I, ids[:100]).any()
+    want = [search(qq, k) for qq in queries]
+    run_threads(4, lambda t: [np.testing.assert_array_equal(search(queries[(t + r) % 4], k)[1], want[(t + r) % 4][1]) for r in range(10)])
+
+
 @pytest.fixture(scope="module")
 def ix():
     import indexsdk_amd
