@@ -415,11 +415,16 @@ int stream_select_bf16x3_sampled(const uint16_t *Qs, int64_t nq_total, const uin
     }
     // expected scores <= tau per row: a group's minimum is <= tau with probability j / G
     const double admitted = (1.0 - std::pow(1.0 - (double)j / G, 1.0 / 32.0)) * (double)nb_total;
-    if (r + 2.0 * admitted > 2048.0) {
+    // How many a row may admit: tau is the j-th of G order statistics, so the share of groups below it scatters by
+    // about 1 / sqrt(j) of its mean -- twice the expectation is five deviations at j = 27 (a search for 64 lists) and
+    // fewer than three at j = 7 (an assignment among 65536 centroids: 0.6 % of the rows overflowed their records
+    // and were redone exactly), so small j get more room.
+    const double slack = std::max(2.0, 1.0 + 6.0 / std::sqrt((double)j));
+    if (r + slack * admitted > 2048.0) {
         return -1;   // more than a fold holds
     }
-    const int capk = (int)std::ceil(r + 2.0 * admitted);                     // scores <= tau a row may have
-    const int cap = std::max(256, pow2_ceil((int)std::ceil(2.0 * admitted)));   // records per row
+    const int capk = (int)std::ceil(r + slack * admitted);                     // scores <= tau a row may have
+    const int cap = std::max(256, pow2_ceil((int)std::ceil(slack * admitted)));   // records per row
     int64_t qb = std::min<int64_t>(round_up(nq_total, 128), 16384);
     if (scratch_bytes / ((int64_t)cap * 32) < qb) {   // the records of a query block stay inside the scratch budget
         qb = scratch_bytes / ((int64_t)cap * 32) / 128 * 128;
