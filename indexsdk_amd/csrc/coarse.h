@@ -32,8 +32,11 @@ void launch_score_tiles_filtered(const float *Q, int64_t nq, const float *C, int
 // cnt[row] and raises *overflow when a row had appended more than cap keys.
 void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<float> flt, float *tau, int64_t nq,
                              int *overflow, hipStream_t s);
+// thr (may be null): thr[row] = min(new tau, max_bound) - qn[row] is written along with tau[row], the threshold form the
+// int8 score kernels filter by
 void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter<int32_t> flt, int32_t *tau,
-                                 int64_t nq, int *overflow, hipStream_t s);
+                                 int64_t nq, int *overflow, hipStream_t s, int32_t *thr = nullptr,
+                                 const int32_t *qn = nullptr, int32_t max_bound = 0);
 
 // Persistent ring kernels (score_ring.hip): same results as the tile kernels, at a much higher
 // matrix-core rate.  Return false when the shape does not qualify (d not a multiple of one K-step,

@@ -391,7 +391,8 @@ void launch_score_tiles_filtered(const float *Q, int64_t nq, const float *C, int
 // Merge of filtered candidates into the running best-k keys of each row (one workgroup per row).
 template <typename S>
 __global__ __launch_bounds__(256) void merge_candidates_kernel(key_t *__restrict__ running, int k, ScoreFilter<S> flt,
-                                                               S *__restrict__ tau, int *__restrict__ overflow)
+                                                               S *__restrict__ tau, int *__restrict__ overflow,
+                                                               S *__restrict__ thr, const S *__restrict__ qn, S max_bound)
 {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     key_t *buf = reinterpret_cast<key_t *>(smem_raw);
@@ -423,14 +424,18 @@ __global__ __launch_bounds__(256) void merge_candidates_kernel(key_t *__restrict
     if (tid == 0) {
         flt.cnt[row] = 0;
         if (buf[k - 1] != kEmptyKey) {
-            tau[row] = key_score_as<S>(buf[k - 1]);
+            const S t = key_score_as<S>(buf[k - 1]);
+            tau[row] = t;
+            if (thr) {   // the next filtered launch's threshold (exact integer scores): min(tau, max_bound) - |q|^2
+                thr[row] = (t < max_bound ? t : max_bound) - qn[row];
+            }
         }
     }
 }
 
 template <typename S>
 static void launch_merge_candidates_t(key_t *running, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *overflow,
-                                      hipStream_t s)
+                                      hipStream_t s, S *thr = nullptr, const S *qn = nullptr, S max_bound = S())
 {
     if (nq == 0) {
         return;
@@ -439,7 +444,7 @@ static void launch_merge_candidates_t(key_t *running, int k, ScoreFilter<S> flt,
     IXA_REQUIRE(smem <= 160 * 1024, kErrInvalidParam, "candidate merge of %d + %d keys exceeds LDS", k, flt.cap);
     require_dynamic_lds(reinterpret_cast<const void *>(merge_candidates_kernel<S>), smem);
     hipLaunchKernelGGL(merge_candidates_kernel<S>, dim3((unsigned)nq), dim3(256), smem, s, running, k, flt, tau,
-                       overflow);
+                       overflow, thr, qn, max_bound);
 }
 
 void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<float> flt, float *tau, int64_t nq,
@@ -449,9 +454,10 @@ void launch_merge_candidates(unsigned long long *running, int k, ScoreFilter<flo
 }
 
 void launch_merge_candidates_i32(unsigned long long *running, int k, ScoreFilter<int32_t> flt, int32_t *tau,
-                                 int64_t nq, int *overflow, hipStream_t s)
+                                 int64_t nq, int *overflow, hipStream_t s, int32_t *thr, const int32_t *qn,
+                                 int32_t max_bound)
 {
-    launch_merge_candidates_t<int32_t>(running, k, flt, tau, nq, overflow, s);
+    launch_merge_candidates_t<int32_t>(running, k, flt, tau, nq, overflow, s, thr, qn, max_bound);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -120,7 +120,8 @@ struct F32Ops {
     {
         launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
-    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    static constexpr bool kMergeKeepsThreshold = false;
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int64_t, int *ovf, hipStream_t s) const
     {
         launch_merge_candidates(run, k, flt, tau, nq, ovf, s);
     }
@@ -152,7 +153,8 @@ struct Bf16Ops {
     {
         launch_select_rows(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
-    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    static constexpr bool kMergeKeepsThreshold = false;
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int64_t, int *ovf, hipStream_t s) const
     {
         launch_merge_candidates(run, k, flt, tau, nq, ovf, s);
     }
@@ -191,9 +193,11 @@ struct I8Ops {
     {
         launch_select_rows_i32(sc, nq, ld, nc, k, nullptr, base, run, s, fresh);
     }
-    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int *ovf, hipStream_t s) const
+    // the merge writes the next launch's thresholds along with the new bounds
+    static constexpr bool kMergeKeepsThreshold = true;
+    void merge(key_t *run, int k, ScoreFilter<S> flt, S *tau, int64_t nq, int64_t q0, int *ovf, hipStream_t s) const
     {
-        launch_merge_candidates_i32(run, k, flt, tau, nq, ovf, s);
+        launch_merge_candidates_i32(run, k, flt, tau, nq, ovf, s, const_cast<S *>(flt.thr), qn + q0, kI8MaxBound);
     }
 };
 
@@ -301,12 +305,17 @@ int stream_select(const Ops &ops, const typename Ops::T *Q, int64_t nq_total, co
             hipLaunchKernelGGL(tau_from_running_kernel<S>, dim3(blocks_for(nq)), dim3(256), 0, s,
                                running + q0 * ncand, ncand, nq, ws.tau.data() + q0);
             int64_t seen = head;
+            const S *thr = nullptr;
+            bool first_chunk = true;
             while (seen < nb_total) {
                 const int64_t nbc = std::min<int64_t>({nb_total - seen, seen * growth, (int64_t)1 << 23});
-                ScoreFilter<S> flt{ws.tau.data() + q0, ops.threshold(ws, q0, nq, s), ws.cnt.data() + q0, ws.filter.data(), cap,
-                                   seen};
+                if (first_chunk || !Ops::kMergeKeepsThreshold) {
+                    thr = ops.threshold(ws, q0, nq, s);
+                    first_chunk = false;
+                }
+                ScoreFilter<S> flt{ws.tau.data() + q0, thr, ws.cnt.data() + q0, ws.filter.data(), cap, seen};
                 ops.filtered(Q + q0 * d, nq, q0, B, nbc, seen, d, flt, s);
-                ops.merge(running + q0 * ncand, ncand, flt, ws.tau.data() + q0, nq, overflow, s);
+                ops.merge(running + q0 * ncand, ncand, flt, ws.tau.data() + q0, nq, q0, overflow, s);
                 launches++;
                 seen += nbc;
             }
